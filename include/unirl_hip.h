@@ -1,0 +1,272 @@
+/*
+ * unirl_hip.h -- C ABI of libunirl_hip.so: the per-sample RL-math hot path of
+ * UniRL as single-pass fused HIP kernels for gfx950 (MI355X).
+ *
+ * The reference has no FFI layer: the path is eager torch inside plain Python
+ * functions.  Each entry point below therefore names the Python function (file
+ * and line in the reference tree) whose arithmetic it replaces; the Python
+ * package `unirl_amd` keeps those functions' signatures and calls these entry
+ * points through ctypes.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless its comment says "host";
+ *   - tensors are dense and row-major; `B` is the leading (per-sample) extent
+ *     and `D` the product of all remaining extents;
+ *   - `dtype` arguments take UNIRL_F32 / UNIRL_BF16 / UNIRL_F16;
+ *   - `stream` is a hipStream_t passed as void*; every call only enqueues work
+ *     on it and returns (asynchronous, no host synchronisation);
+ *   - `workspace` is caller-owned device memory of at least
+ *     unirl_workspace_bytes() bytes that was zero-filled ONCE after allocation
+ *     (unirl_workspace_init does that).  Kernels leave it ready for the next
+ *     call.  Two calls that may overlap in time (different streams) need
+ *     different workspaces;
+ *   - the library allocates nothing, frees nothing and keeps no global state;
+ *   - return value: 0 = ok, < 0 = invalid argument (UNIRL_E_*), > 0 = the
+ *     hipError_t of a failed launch.  No C++ exception crosses this boundary.
+ */
+#ifndef UNIRL_HIP_H_
+#define UNIRL_HIP_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define UNIRL_ABI_VERSION 1
+
+enum unirl_dtype { UNIRL_F32 = 0, UNIRL_BF16 = 1, UNIRL_F16 = 2 };
+
+/* SDE transition family: unirl/sde/kernels.py:185 (flow), :239 (cps), :282 (dance). */
+enum unirl_sde_kind { UNIRL_SDE_FLOW = 0, UNIRL_SDE_DANCE = 1, UNIRL_SDE_CPS = 2 };
+
+enum unirl_status {
+  UNIRL_OK = 0,
+  UNIRL_E_NULL = -1,      /* a required pointer is NULL */
+  UNIRL_E_SHAPE = -2,     /* negative / inconsistent extent */
+  UNIRL_E_DTYPE = -3,     /* unknown dtype / kind / mode */
+  UNIRL_E_WORKSPACE = -4, /* workspace missing or too small */
+  UNIRL_E_ALIGN = -5,     /* pointer not aligned to its element size */
+  UNIRL_E_LIMIT = -6      /* extent beyond a documented limit */
+};
+
+#define UNIRL_MAX_ROLLOUT_STEPS 64
+
+int unirl_abi_version(void);
+const char* unirl_status_string(int status);
+
+/* Bytes of device workspace every reducing entry point expects. */
+size_t unirl_workspace_bytes(void);
+/* Zero-fill a freshly allocated workspace (a fill kernel on `stream`). */
+int unirl_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * One SDE transition + per-sample Gaussian log-prob.
+ * Replaces StepStrategy.denoise -> SDEStrategy.step -> _finalize_logp
+ * (unirl/sde/kernels.py:43-99, :154-177, :207-236, :255-279, :304-333).
+ *
+ *   noise_pred  [B,D] dtype_v          model velocity
+ *   sample      [B,D] dtype_x          current latent; dtype_x is the
+ *                                      "input dtype" of the round trip
+ *   prev_sample [B,D] dtype_x or NULL  NULL = sampling, else replay
+ *   noise       [B,D] f32 or NULL      sampling only; NULL = no noise term
+ *   sigma, sigma_next  f32, one value (stride 0) or one per sample (stride 1)
+ *   sigma_max_ptr      f32 device scalar or NULL (then sigma_max_val is used)
+ *   eta                python-side float; eta < 1e-7 skips the log-prob
+ *   prev_out    [B,D] f32 or NULL      prev_sample after the dtype round trip
+ *   mean_out    [B,D] f32 or NULL      prev_sample_mean
+ *   logp_out    [B]   f32 or NULL      mean over D of the element log-prob
+ *                                      (logp_sum != 0: sum over D instead)
+ * ---------------------------------------------------------------------- */
+int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const void* sample, int dtype_x,
+                        const void* prev_sample, const float* noise, const float* sigma,
+                        const float* sigma_next, int sigma_stride, const float* sigma_max_ptr,
+                        float sigma_max_val, double eta, int kind, int64_t B, int64_t D,
+                        float* prev_out, float* mean_out, float* logp_out, int logp_sum,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* Backward of unirl_sde_step_logp with respect to noise_pred and sample, for
+ * the autograd graph the reference builds through kernels.py:225-228 and
+ * :200-204 (prev_sample is detached there).  Inputs as in the forward call;
+ * g_logp [B] f32 (NULL = 0), g_mean [B,D] f32 (NULL = 0), g_prev [B,D] f32
+ * (sampling only, NULL = 0).  Outputs grad_v / grad_x are f32 [B,D], either
+ * may be NULL. */
+int unirl_sde_step_logp_bwd(const void* noise_pred, int dtype_v, const void* sample, int dtype_x,
+                            const void* prev_sample, const float* noise, const float* sigma,
+                            const float* sigma_next, int sigma_stride, const float* sigma_max_ptr,
+                            float sigma_max_val, double eta, int kind, int64_t B, int64_t D,
+                            const float* g_logp, const float* g_mean, const float* g_prev,
+                            int logp_sum, float* grad_v, float* grad_x, void* stream);
+
+/* ------------------------------------------------------------------------
+ * S chained SDE transitions with the latent held in registers: the loop of
+ * DiffusionStage.diffuse around StepStrategy.denoise
+ * (unirl/models/sd3/diffusion.py:366-390) for velocities that are already
+ * known.  Step k uses sigmas[k] -> sigmas[k+1] and etas[k].
+ *
+ *   x0          [B,D] dtype_x
+ *   v_steps     host array of S device pointers, each [B,D] dtype_v
+ *   noise_steps host array of S device pointers, each [B,D] f32 (entries may
+ *               be NULL for steps with eta < 1e-7)
+ *   sigmas      device f32 [S+1];  etas  host double [S]
+ *   x_out       [B,D] f32  final latent
+ *   traj_out    NULL or [S,B,D] f32: latent after every step
+ *   logp_out    [B,S] f32; steps with eta < 1e-7 hold NaN
+ * ---------------------------------------------------------------------- */
+int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* const* v_steps, int dtype_v,
+                           const float* const* noise_steps, const float* sigmas,
+                           const double* etas, int S, const float* sigma_max_ptr,
+                           float sigma_max_val, int kind, int64_t B, int64_t D, float* x_out,
+                           float* traj_out, float* logp_out, int logp_sum, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Gaussian KL between transition means, reduced per (sample, step), and the
+ * trust-region mask.  Replaces _gaussian_kl_div + the reduction and compare
+ * of _flowdppo_kl_adv_loss (unirl/algorithms/flowdppo.py:43-51, :92-96).
+ *
+ *   p, q     [R,D] dtype       new / old means, R = B*S' rows
+ *   sigma    f32 [n_sigma]     row r uses sigma[r % n_sigma]  (n_sigma = S'
+ *                              for the reference's [1,S',1,1,1]; 1 = scalar)
+ *   kl_out   [R] f32           mean over D of (p-q)^2 / (2 sigma^2), computed
+ *                              with torch's type promotion: 16-bit inputs
+ *                              subtract and square in that dtype, then divide
+ *                              in f32
+ *   mask_out [R] u8 or NULL    kl < threshold  (torch.bool layout)
+ * ---------------------------------------------------------------------- */
+int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, const float* sigma,
+                           int64_t n_sigma, int64_t R, int64_t D, float threshold, float* kl_out,
+                           uint8_t* mask_out, void* workspace, size_t workspace_bytes,
+                           void* stream);
+
+/* Element-wise form of the same quantity (flowdppo.py:51), f32 output [R,D]. */
+int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, const float* sigma,
+                           int64_t n_sigma, int64_t R, int64_t D, float* out, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Token log-prob and entropy over the vocabulary.  Replaces _logp_chunk
+ * (unirl/models/qwen3/ar.py:82-85) and the log_softmax(...).gather sites
+ * (qwen3/ar.py:144-174, qwen_vl/ar.py:334-335, hunyuan_image3/ar.py:509-510).
+ *
+ *   logits   [rows, V] dtype, consecutive rows `row_stride` elements apart
+ *   ids      [rows] int64      target token per row
+ *   temperature                values <= 0 mean 1 (qwen3/ar.py:78)
+ *   logp_out [rows] f32 or NULL   (x[id] - logsumexp(x)) with x = logits/T
+ *   ent_out  [rows] f32 or NULL   -sum softmax(x) log_softmax(x)
+ *   lse_out  [rows] f32 or NULL   logsumexp(x), kept for the backward
+ * An id outside [0,V) yields NaN in logp_out for that row.
+ * ---------------------------------------------------------------------- */
+int unirl_token_logp_entropy(const void* logits, int dtype, int64_t rows, int64_t V,
+                             int64_t row_stride, const int64_t* ids, float temperature,
+                             float* logp_out, float* ent_out, float* lse_out, void* stream);
+
+/* grad_logits[r, j] = g_logp[r] * (1[j == ids[r]] - softmax(x)[r, j]) / T in
+ * `dtype`, the gradient autograd gives through qwen3/ar.py:83-85. */
+int unirl_token_logp_bwd(const void* logits, int dtype, int64_t rows, int64_t V,
+                         int64_t row_stride, const int64_t* ids, float temperature,
+                         const float* lse, const float* g_logp, void* grad_logits,
+                         int64_t grad_row_stride, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Token-level ratio losses with every metric reduction fused in.
+ * Replaces _grpo_clip_loss (unirl/algorithms/base.py:115-157), _drpo_loss
+ * (unirl/algorithms/drpo.py:97-159), rollout_replay_logp_absdiff
+ * (base.py:83-103), GRPO._expand_advantages_to_tokens (grpo.py:172-198) and
+ * the aggregation in grpo.py:148-155 / drpo.py:318-330.
+ *
+ * Token layout (new_logp / old_logp are f32; n_tok = number of slots):
+ *   padded  : seq_stride > 0: [n_seq, seq_stride]; `lengths` is int64 [n_seq]
+ *             and row r holds lengths[r] valid tokens first
+ *   packed  : seq_stride == 0: `lengths` is the int64 PREFIX SUM cu_seqlens
+ *             [n_seq+1] (cu[0] = 0, cu[n_seq] = n_tok); sequence r owns tokens
+ *             [cu[r], cu[r+1])
+ *   flat    : lengths == NULL: one run of n_tok tokens (n_seq ignored); needs
+ *             per-token advantages and token-mean aggregation
+ * Advantages: adv_per_token != 0 -> one per token (same layout as the
+ * log-probs); else one per sequence (requires lengths).
+ * loss_mask: NULL or f32 per token, multiplied into the loss (drpo.py:319-321).
+ * ---------------------------------------------------------------------- */
+enum unirl_loss_kind { UNIRL_LOSS_GRPO = 0, UNIRL_LOSS_DRPO = 1 };
+enum unirl_agg_mode {
+  UNIRL_AGG_TOKEN_MEAN = 0,        /* sum over tokens / token count        */
+  UNIRL_AGG_SEQ_MEAN_TOKEN_SUM = 1,/* mean_seq(sum_tok) / horizon           */
+  UNIRL_AGG_SEQ_MEAN_TOKEN_MEAN = 2/* mean_seq(mean_tok), empty seq -> 0    */
+};
+
+/* Slots of the f32 metrics vector written by unirl_ratio_loss_fwd. */
+enum unirl_metric_slot {
+  UNIRL_M_LOSS = 0,           /* aggregated loss                              */
+  UNIRL_M_RATIO_MEAN = 1,
+  UNIRL_M_RATIO_STD = 2,      /* unbiased; 0 when fewer than two tokens       */
+  UNIRL_M_RATIO_MIN = 3,
+  UNIRL_M_RATIO_MAX = 4,
+  UNIRL_M_CLIP_FRACTION = 5,  /* GRPO: mean(max(gt, lt))                      */
+  UNIRL_M_CLIPFRAC_HI = 6,    /* GRPO clipfrac_gt_one / DRPO clipfrac_upper   */
+  UNIRL_M_CLIPFRAC_LO = 7,    /* GRPO clipfrac_lt_one / DRPO clipfrac_lower   */
+  UNIRL_M_APPROX_KL = 8,      /* GRPO 0.5*ld^2 ; DRPO (r-1)-ld                */
+  UNIRL_M_PENALTY_MEAN = 9,   /* DRPO drpo_penalty_mean                       */
+  UNIRL_M_ABSDIFF_MEAN = 10,  /* mean |new-old|                               */
+  UNIRL_M_ABSDIFF_MAX = 11,
+  UNIRL_M_NUM_TOKENS = 12,    /* valid-token count as f32                     */
+  UNIRL_M_COUNT = 16
+};
+
+struct unirl_ratio_loss_params {
+  int kind;            /* unirl_loss_kind                                     */
+  int agg_mode;        /* unirl_agg_mode                                      */
+  float clip_low;      /* GRPO clip_range                                     */
+  float clip_high;     /* GRPO clip_range_high (= clip_low when symmetric)    */
+  float drpo_epsilon;  /* DRPO epsilon                                        */
+  int mu_weighted;     /* DRPO penalty weight mu = exp(old) (1) or 1 (0)      */
+  float horizon;       /* UNIRL_AGG_SEQ_MEAN_TOKEN_SUM divisor                */
+  int adv_per_token;
+};
+
+int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp, const float* advantages,
+                         const int64_t* lengths, const float* loss_mask, int64_t n_seq,
+                         int64_t seq_stride, int64_t n_tok,
+                         const struct unirl_ratio_loss_params* params /* host */,
+                         float* loss_per_elem /* NULL or same layout as new_logp */,
+                         float* metrics /* [UNIRL_M_COUNT] f32 */, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
+/* grad_new = g_scale * w_tok * dloss/dnew, where w_tok is the aggregation
+ * weight of the token (1/N, 1/(n_seq*horizon) or 1/(n_seq*len)), times
+ * g_elem per token when that is not NULL (the caller reduced loss_per_elem
+ * itself).  Padded slots past a sequence's length receive 0. */
+int unirl_ratio_loss_bwd(const float* new_logp, const float* old_logp, const float* advantages,
+                         const int64_t* lengths, const float* loss_mask, int64_t n_seq,
+                         int64_t seq_stride, int64_t n_tok,
+                         const struct unirl_ratio_loss_params* params /* host */,
+                         const float* g_scale /* device scalar or NULL (=1) */,
+                         const float* g_elem, int aggregate,
+                         const float* n_valid /* device scalar: metrics[UNIRL_M_NUM_TOKENS]
+                                                 of the forward; token-mean only */,
+                         float* grad_new, void* stream);
+
+/* ------------------------------------------------------------------------
+ * Group-normalised advantages.  Replaces RolloutTrack.compute_advantages
+ * (unirl/types/rollout_resp.py:277-333) for n = n_groups * branch rewards in
+ * group-by-parent order.
+ *   scope_global  != 0: (r - mean_all) / (std_unbiased_all + eps)
+ *   use_global_std!= 0: (r - mean_g)   / (std_unbiased_all + eps)
+ *   otherwise          : (r - mean_g)   / sqrt(var_pop_g + eps)
+ *   normalize == 0     : centring only
+ * ---------------------------------------------------------------------- */
+int unirl_group_advantages(const float* rewards, int64_t n_groups, int64_t branch, int normalize,
+                           float eps, int scope_global, int use_global_std, float* adv_out,
+                           void* stream);
+
+/* ------------------------------------------------------------------------
+ * out[b, j, :] = src[b, positions[j], :] -- the copy behind gather_sde_field
+ * (unirl/algorithms/base.py:70,80).  inner_bytes is the byte size of one
+ * [b, s] slice; positions is a device int64 array with values in [0, S).
+ * ---------------------------------------------------------------------- */
+int unirl_gather_steps(const void* src, int64_t B, int64_t S, int64_t inner_bytes,
+                       const int64_t* positions, int64_t n_pos, void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* UNIRL_HIP_H_ */

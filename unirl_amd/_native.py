@@ -1,0 +1,197 @@
+"""ctypes binding of libunirl_hip.so (the C ABI declared in include/unirl_hip.h).
+
+There is no CPU implementation behind this module: if the shared library has
+not been built, or a tensor does not live on a HIP device, the call raises.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+from ctypes import POINTER, Structure, c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
+from pathlib import Path
+from typing import Dict, Optional, Tuple
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libunirl_hip.so"
+
+# enum unirl_dtype
+F32, BF16, F16 = 0, 1, 2
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+
+# enum unirl_sde_kind
+SDE_FLOW, SDE_DANCE, SDE_CPS = 0, 1, 2
+
+# enum unirl_loss_kind / unirl_agg_mode
+LOSS_GRPO, LOSS_DRPO = 0, 1
+AGG_TOKEN_MEAN, AGG_SEQ_MEAN_TOKEN_SUM, AGG_SEQ_MEAN_TOKEN_MEAN = 0, 1, 2
+AGG_MODES = {
+    "token-mean": AGG_TOKEN_MEAN,
+    "seq-mean-token-sum-norm": AGG_SEQ_MEAN_TOKEN_SUM,
+    "seq-mean-token-mean": AGG_SEQ_MEAN_TOKEN_MEAN,
+}
+
+# enum unirl_metric_slot
+M_LOSS, M_RATIO_MEAN, M_RATIO_STD, M_RATIO_MIN, M_RATIO_MAX = 0, 1, 2, 3, 4
+M_CLIP_FRACTION, M_CLIPFRAC_HI, M_CLIPFRAC_LO, M_APPROX_KL, M_PENALTY_MEAN = 5, 6, 7, 8, 9
+M_ABSDIFF_MEAN, M_ABSDIFF_MAX, M_NUM_TOKENS, M_COUNT = 10, 11, 12, 16
+
+MAX_ROLLOUT_STEPS = 64
+
+
+class RatioLossParams(Structure):
+    """struct unirl_ratio_loss_params."""
+
+    _fields_ = [
+        ("kind", c_int),
+        ("agg_mode", c_int),
+        ("clip_low", c_float),
+        ("clip_high", c_float),
+        ("drpo_epsilon", c_float),
+        ("mu_weighted", c_int),
+        ("horizon", c_float),
+        ("adv_per_token", c_int),
+    ]
+
+
+_SIGNATURES = {
+    "unirl_abi_version": (c_int, []),
+    "unirl_status_string": (c_char_p, [c_int]),
+    "unirl_workspace_bytes": (c_size_t, []),
+    "unirl_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
+    "unirl_sde_step_logp": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,
+         c_double, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "unirl_sde_step_logp_bwd": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,
+         c_double, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+    ),
+    "unirl_sde_rollout_logp": (
+        c_int,
+        [c_void_p, c_int, POINTER(c_void_p), c_int, POINTER(c_void_p), c_void_p, POINTER(c_double), c_int,
+         c_void_p, c_float, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t,
+         c_void_p],
+    ),
+    "unirl_gaussian_kl_mask": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p,
+         c_size_t, c_void_p],
+    ),
+    "unirl_gaussian_kl_elem": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p],
+    ),
+    "unirl_token_logp_entropy": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
+    "unirl_token_logp_bwd": (
+        c_int,
+        [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int64,
+         c_void_p],
+    ),
+    "unirl_ratio_loss_fwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, POINTER(RatioLossParams),
+         c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    ),
+    "unirl_ratio_loss_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, POINTER(RatioLossParams),
+         c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+    ),
+    "unirl_group_advantages": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
+    ),
+    "unirl_gather_steps": (
+        c_int,
+        [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p],
+    ),
+}
+
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+_lib: Optional[ctypes.CDLL] = None
+_lib_lock = threading.Lock()
+
+
+class UnirlHipError(RuntimeError):
+    """A C-ABI call returned a non-zero status."""
+
+
+def lib() -> ctypes.CDLL:
+    """Load the shared library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lib_lock:
+        if _lib is None:
+            if not LIB_PATH.exists():
+                raise RuntimeError(
+                    f"{LIB_PATH} is missing: build it with `python -m unirl_amd.build` "
+                    "(hipcc, gfx950). unirl_amd has no CPU or eager-torch path behind its kernels."
+                )
+            handle = ctypes.CDLL(str(LIB_PATH))
+            for name, (restype, argtypes) in _SIGNATURES.items():
+                fn = getattr(handle, name)
+                fn.restype = restype
+                fn.argtypes = argtypes
+            _lib = handle
+    return _lib
+
+
+def check(status: int, what: str) -> None:
+    """Turn a C-ABI status into an exception: ValueError for argument errors,
+    UnirlHipError for a failed launch."""
+    if status == 0:
+        return
+    msg = lib().unirl_status_string(int(status)).decode()
+    if status < 0:
+        raise ValueError(f"{what}: {msg} (status {status})")
+    raise UnirlHipError(f"{what}: HIP error {status}: {msg}")
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {dtype}; expected float32, bfloat16 or float16") from None
+
+
+def require_device(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(
+            f"{name} lives on {t.device}: unirl_amd kernels run on a HIP device only "
+            "(there is no CPU fallback; use the torch reference for CPU tensors)"
+        )
+
+
+def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def current_stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+_workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
+
+
+def workspace(device: torch.device) -> Tuple[torch.Tensor, int]:
+    """Zero-initialised scratch for the reducing kernels, one per (device, stream).
+
+    The kernels leave it zeroed again, so it is allocated and cleared once.
+    """
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    key = (index, current_stream(device))
+    ws = _workspaces.get(key)
+    if ws is None:
+        nbytes = int(lib().unirl_workspace_bytes())
+        ws = torch.zeros(nbytes, dtype=torch.uint8, device=torch.device("cuda", index))
+        _workspaces[key] = ws
+    return ws, ws.numel()

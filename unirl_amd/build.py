@@ -1,0 +1,96 @@
+"""Build libunirl_hip.so for gfx950 with hipcc, in-tree.
+
+    python -m unirl_amd.build            # compile every csrc/*.hip and link
+
+hipcc cross-compiles without a GPU.  Objects go to ``unirl_amd/lib/obj`` and the
+shared library to ``unirl_amd/lib/libunirl_hip.so``; both are git-ignored build
+products.
+"""
+
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+from pathlib import Path
+from typing import List
+
+PKG_DIR = Path(__file__).resolve().parent
+CSRC_DIR = PKG_DIR / "csrc"
+LIB_DIR = PKG_DIR / "lib"
+OBJ_DIR = LIB_DIR / "obj"
+LIB_PATH = LIB_DIR / "libunirl_hip.so"
+
+ARCH = "gfx950"
+
+# -ffp-contract=off: a*b+c stays two roundings like eager torch; the kernels
+#   spell out fmaf() where a fused multiply-add is wanted.
+# -packed-fp32-ops off: keep the compiler from forming v_pk_{add,mul,fma}_f32.
+HIPCC_FLAGS: List[str] = [
+    f"--offload-arch={ARCH}",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    "-ffp-contract=off",
+    "-Xclang",
+    "-target-feature",
+    "-Xclang",
+    "-packed-fp32-ops",
+    "-Wall",
+    "-Wno-unused-function",
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not Path(exe).exists():
+        raise RuntimeError("hipcc not found (looked on PATH and in /opt/rocm/bin)")
+    return exe
+
+
+def _run(cmd: List[str]) -> None:
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    # The host pass of hipcc does not know the packed-fp32 target feature and says so.
+    noise = "is not a recognized feature for this target"
+    out = "\n".join(line for line in proc.stdout.splitlines() if noise not in line)
+    if proc.returncode != 0:
+        raise RuntimeError(f"command failed ({proc.returncode}): {' '.join(cmd)}\n{out}")
+    if out.strip():
+        print(out, file=sys.stderr)
+
+
+def sources() -> List[Path]:
+    return sorted(CSRC_DIR.glob("*.hip"))
+
+
+def build(verbose: bool = True, jobs: int | None = None) -> Path:
+    """Compile every kernel source and link the shared library. Always recompiles."""
+    hipcc = _hipcc()
+    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    srcs = sources()
+    if not srcs:
+        raise RuntimeError(f"no .hip sources under {CSRC_DIR}")
+    objs = [OBJ_DIR / (s.stem + ".o") for s in srcs]
+    jobs = jobs or min(len(srcs), max(1, (os.cpu_count() or 2) // 2))
+
+    def compile_one(pair):
+        src, obj = pair
+        if verbose:
+            print(f"[unirl_amd.build] hipcc {src.name}", flush=True)
+        _run([hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)])
+
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        list(pool.map(compile_one, zip(srcs, objs)))
+
+    tmp = LIB_PATH.with_suffix(".so.tmp")
+    _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)])
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print(f"[unirl_amd.build] linked {LIB_PATH}", flush=True)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()

@@ -1,0 +1,241 @@
+// Gaussian KL between old and new transition means, reduced per (sample, step)
+// row and thresholded into the Flow-DPPO trust-region mask.
+//
+// Replaces unirl/algorithms/flowdppo.py:
+//   _gaussian_kl_div          :43-51   (p - q)**2 / (2 * sigma**2)
+//   kl_per_sample / kl_mask   :92-96   mean over dims >= 2, then `< threshold`
+// torch's type promotion is reproduced: with 16-bit means and an f32 sigma
+// tensor, the subtraction and the square each round to the 16-bit dtype and
+// only the division runs in f32.  The kernel sums the squares (f32 per lane,
+// f64 across lanes and workgroups, fixed order) and divides once per row.
+//
+// HBM traffic: 2 * D * sizeof(T) bytes read per row, 5 bytes written per row.
+
+#include "common.cuh"
+#include "unirl_internal.h"
+
+namespace unirl {
+
+constexpr int kKlThreads = 256;
+
+struct KlArgs {
+  const void* p;
+  const void* q;
+  const float* sigma;
+  int64_t n_sigma;
+  int64_t row0;  // global index of the first row of this launch (for the sigma lookup)
+  int64_t D;
+  float threshold;
+  float* kl;
+  uint8_t* mask;
+  float* elem_out;
+  double* partials;
+  unsigned int* counters;
+};
+
+template <typename T>
+__device__ __forceinline__ float kl_sq(float p, float q) {
+  const float d = Elem<T>::round_trip(p - q);
+  return Elem<T>::round_trip(d * d);
+}
+
+__device__ __forceinline__ float kl_den(const KlArgs& A, int64_t row) {
+  const float s = A.sigma[(A.row0 + row) % A.n_sigma];
+  return 2.0f * (s * s);
+}
+
+__device__ __forceinline__ void kl_finish(const KlArgs& A, int64_t row, double q) {
+  const float kl = (float)((q / (double)kl_den(A, row)) / (double)A.D);
+  A.kl[row] = kl;
+  if (A.mask) A.mask[row] = (kl < A.threshold) ? 1 : 0;
+}
+
+template <typename T, int VEC, int ITEMS>
+__global__ __launch_bounds__(kKlThreads) void gaussian_kl_kernel(KlArgs A) {
+  __shared__ double lds[kKlThreads / kWave];
+  __shared__ int lds_flag;
+  const int64_t row = blockIdx.y;
+  const int64_t D = A.D;
+  const T* __restrict__ pp = reinterpret_cast<const T*>(A.p) + row * D;
+  const T* __restrict__ qp = reinterpret_cast<const T*>(A.q) + row * D;
+  const int64_t nvec = D / VEC;
+  const int64_t stride = (int64_t)gridDim.x * kKlThreads;
+  float acc = 0.0f;
+  for (int64_t i0 = (int64_t)blockIdx.x * kKlThreads + threadIdx.x; i0 < nvec; i0 += stride * ITEMS) {
+    float a[ITEMS][VEC], b[ITEMS][VEC];
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t i = i0 + it * stride;
+      if (i < nvec) {
+        Vec<T, VEC>::load(pp + i * VEC, a[it]);
+        Vec<T, VEC>::load(qp + i * VEC, b[it]);
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t i = i0 + it * stride;
+      if (i < nvec) {
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) acc += kl_sq<T>(a[it][k], b[it][k]);
+      }
+    }
+  }
+  const double part = block_sum<double>((double)acc, lds);
+  if (gridDim.x == 1) {
+    if (threadIdx.x == 0) kl_finish(A, row, part);
+    return;
+  }
+  if (threadIdx.x == 0) A.partials[row * gridDim.x + blockIdx.x] = part;
+  if (!arrive_and_check_last(A.counters + row, gridDim.x, &lds_flag)) return;
+  double q = 0.0;
+  for (unsigned int j = threadIdx.x; j < gridDim.x; j += kKlThreads)
+    q += __builtin_nontemporal_load(A.partials + row * gridDim.x + j);
+  q = block_sum<double>(q, lds);
+  if (threadIdx.x == 0) kl_finish(A, row, q);
+}
+
+template <typename T, int VEC>
+__global__ __launch_bounds__(kKlThreads) void gaussian_kl_elem_kernel(KlArgs A) {
+  const int64_t row = blockIdx.y;
+  const int64_t D = A.D;
+  const T* __restrict__ pp = reinterpret_cast<const T*>(A.p) + row * D;
+  const T* __restrict__ qp = reinterpret_cast<const T*>(A.q) + row * D;
+  float* __restrict__ op = A.elem_out + row * D;
+  const float den = kl_den(A, row);
+  const int64_t nvec = D / VEC;
+  const int64_t stride = (int64_t)gridDim.x * kKlThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kKlThreads + threadIdx.x; i < nvec; i += stride) {
+    float a[VEC], b[VEC], o[VEC];
+    Vec<T, VEC>::load(pp + i * VEC, a);
+    Vec<T, VEC>::load(qp + i * VEC, b);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) o[k] = kl_sq<T>(a[k], b[k]) / den;
+    Vec<float, VEC>::store(op + i * VEC, o);
+  }
+}
+
+static unsigned int kl_blocks_per_row(int64_t nvec, int items, int64_t R) {
+  const int64_t per_pass = (int64_t)kKlThreads * items;
+  int64_t nblk = (nvec + per_pass - 1) / per_pass;
+  const int64_t cap = tune_int("UNIRL_KL_MAX_BLOCKS", 4096);
+  int64_t max_per_row = cap / (R > 0 ? R : 1);
+  if (max_per_row < 1) max_per_row = 1;
+  if (nblk > max_per_row) nblk = max_per_row;
+  if (nblk > kMaxPartialBlocks) nblk = kMaxPartialBlocks;
+  if (nblk < 1) nblk = 1;
+  return (unsigned int)nblk;
+}
+
+template <typename T>
+static int launch_kl(const KlArgs& A, int64_t R, int vec, unsigned int nblk, int items, hipStream_t st) {
+  dim3 grid(nblk, (unsigned int)R), block(kKlThreads);
+  if (vec == 4) {
+    if (items >= 4)
+      hipLaunchKernelGGL((gaussian_kl_kernel<T, 4, 4>), grid, block, 0, st, A);
+    else if (items >= 2)
+      hipLaunchKernelGGL((gaussian_kl_kernel<T, 4, 2>), grid, block, 0, st, A);
+    else
+      hipLaunchKernelGGL((gaussian_kl_kernel<T, 4, 1>), grid, block, 0, st, A);
+  } else {
+    hipLaunchKernelGGL((gaussian_kl_kernel<T, 1, 2>), grid, block, 0, st, A);
+  }
+  return (int)hipGetLastError();
+}
+
+template <typename T>
+static int launch_kl_elem(const KlArgs& A, int64_t R, int vec, hipStream_t st) {
+  int64_t nblk = (A.D / vec + kKlThreads - 1) / kKlThreads;
+  if (nblk > 2048) nblk = 2048;
+  if (nblk < 1) nblk = 1;
+  dim3 grid((unsigned int)nblk, (unsigned int)R), block(kKlThreads);
+  if (vec == 4)
+    hipLaunchKernelGGL((gaussian_kl_elem_kernel<T, 4>), grid, block, 0, st, A);
+  else
+    hipLaunchKernelGGL((gaussian_kl_elem_kernel<T, 1>), grid, block, 0, st, A);
+  return (int)hipGetLastError();
+}
+
+}  // namespace unirl
+
+using namespace unirl;
+
+extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, const float* sigma, int64_t n_sigma,
+                                      int64_t R, int64_t D, float threshold, float* kl_out, uint8_t* mask_out,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  if (!dtype_ok(dtype)) return UNIRL_E_DTYPE;
+  if (R < 0 || D <= 0 || n_sigma <= 0) return UNIRL_E_SHAPE;
+  if (R == 0) return UNIRL_OK;
+  if (!p || !q || !sigma || !kl_out) return UNIRL_E_NULL;
+  if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
+  const size_t sz = dtype_size(dtype);
+  if (!aligned_to(p, sz) || !aligned_to(q, sz)) return UNIRL_E_ALIGN;
+  int vec = 4;
+  if (D % 4 != 0 || !aligned_to(p, 4 * sz) || !aligned_to(q, 4 * sz)) vec = 1;
+  const int items = (vec == 4) ? (int)tune_int("UNIRL_KL_ITEMS", 4) : 2;
+  const unsigned int nblk = kl_blocks_per_row(D / vec, items, R);
+  int64_t per_launch = kPartialCapacity / nblk;
+  if (per_launch > kMaxCounters) per_launch = kMaxCounters;
+  hipStream_t st = (hipStream_t)stream;
+  for (int64_t r0 = 0; r0 < R; r0 += per_launch) {
+    const int64_t nr = (R - r0 < per_launch) ? (R - r0) : per_launch;
+    KlArgs A;
+    A.p = offset_ptr(p, r0 * D, sz);
+    A.q = offset_ptr(q, r0 * D, sz);
+    A.sigma = sigma;
+    A.n_sigma = n_sigma;
+    A.row0 = r0;
+    A.D = D;
+    A.threshold = threshold;
+    A.kl = kl_out + r0;
+    A.mask = mask_out ? mask_out + r0 : nullptr;
+    A.elem_out = nullptr;
+    A.partials = ws_partials(workspace);
+    A.counters = ws_counters(workspace);
+    int rc = UNIRL_E_DTYPE;
+    switch (dtype) {
+      case UNIRL_F32: rc = launch_kl<float>(A, nr, vec, nblk, items, st); break;
+      case UNIRL_BF16: rc = launch_kl<bf16_t>(A, nr, vec, nblk, items, st); break;
+      case UNIRL_F16: rc = launch_kl<f16_t>(A, nr, vec, nblk, items, st); break;
+    }
+    if (rc != 0) return rc;
+  }
+  return UNIRL_OK;
+}
+
+extern "C" int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, const float* sigma, int64_t n_sigma,
+                                      int64_t R, int64_t D, float* out, void* stream) {
+  if (!dtype_ok(dtype)) return UNIRL_E_DTYPE;
+  if (R < 0 || D <= 0 || n_sigma <= 0) return UNIRL_E_SHAPE;
+  if (R == 0) return UNIRL_OK;
+  if (!p || !q || !sigma || !out) return UNIRL_E_NULL;
+  const size_t sz = dtype_size(dtype);
+  if (!aligned_to(p, sz) || !aligned_to(q, sz) || !aligned_to(out, 4)) return UNIRL_E_ALIGN;
+  int vec = 4;
+  if (D % 4 != 0 || !aligned_to(p, 4 * sz) || !aligned_to(q, 4 * sz) || !aligned_to(out, 16)) vec = 1;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t per_launch = 32768;
+  for (int64_t r0 = 0; r0 < R; r0 += per_launch) {
+    const int64_t nr = (R - r0 < per_launch) ? (R - r0) : per_launch;
+    KlArgs A;
+    A.p = offset_ptr(p, r0 * D, sz);
+    A.q = offset_ptr(q, r0 * D, sz);
+    A.sigma = sigma;
+    A.n_sigma = n_sigma;
+    A.row0 = r0;
+    A.D = D;
+    A.threshold = 0.0f;
+    A.kl = nullptr;
+    A.mask = nullptr;
+    A.elem_out = out + r0 * D;
+    A.partials = nullptr;
+    A.counters = nullptr;
+    int rc = UNIRL_E_DTYPE;
+    switch (dtype) {
+      case UNIRL_F32: rc = launch_kl_elem<float>(A, nr, vec, st); break;
+      case UNIRL_BF16: rc = launch_kl_elem<bf16_t>(A, nr, vec, st); break;
+      case UNIRL_F16: rc = launch_kl_elem<f16_t>(A, nr, vec, st); break;
+    }
+    if (rc != 0) return rc;
+  }
+  return UNIRL_OK;
+}

@@ -1,0 +1,175 @@
+// Small kernels around the hot path: group-normalised advantages and the
+// step gather.
+
+#include "common.cuh"
+#include "unirl_internal.h"
+
+namespace unirl {
+
+// ---------------------------------------------------------------------------
+// Group advantages: unirl/types/rollout_resp.py:277-283 (global scope) and
+// :314-333 (group scope).  One workgroup; statistics in fp64, rounded to f32 at
+// the points where the reference holds f32 tensors (mean, var/std), then the
+// same f32 operations: `+ eps`, `.sqrt()`, `(r - mean) / std`.
+// ---------------------------------------------------------------------------
+constexpr int kAdvThreads = 256;
+
+struct AdvArgs {
+  const float* r;
+  int64_t n_groups, branch;
+  int normalize, scope_global, use_global_std;
+  float eps;
+  float* out;
+};
+
+__global__ __launch_bounds__(kAdvThreads) void group_advantages_kernel(AdvArgs A) {
+  __shared__ double lds[kAdvThreads / kWave];
+  const int64_t n = A.n_groups * A.branch;
+  float g_mean = 0.0f, g_std = 1.0f;
+  if (A.scope_global || (A.normalize && A.use_global_std)) {
+    double s = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += kAdvThreads) s += (double)A.r[i];
+    s = block_sum<double>(s, lds);
+    const double mean = s / (double)n;
+    double q = 0.0;
+    for (int64_t i = threadIdx.x; i < n; i += kAdvThreads) {
+      const double d = (double)A.r[i] - mean;
+      q += d * d;
+    }
+    q = block_sum<double>(q, lds);
+    g_mean = (float)mean;
+    const float std_unbiased = (float)sqrt(q / (double)(n - 1));  // n == 1 -> NaN, as torch.std
+    g_std = std_unbiased + A.eps;
+  }
+  if (A.scope_global) {
+    for (int64_t i = threadIdx.x; i < n; i += kAdvThreads) {
+      const float c = A.r[i] - g_mean;
+      A.out[i] = A.normalize ? c / g_std : c;
+    }
+    return;
+  }
+  // one lane per group; groups are short (the branching factor of a prompt)
+  for (int64_t g = threadIdx.x; g < A.n_groups; g += kAdvThreads) {
+    const float* rg = A.r + g * A.branch;
+    double s = 0.0;
+    for (int64_t j = 0; j < A.branch; ++j) s += (double)rg[j];
+    const double mean = s / (double)A.branch;
+    const float mean_f = (float)mean;
+    float std_f = 1.0f;
+    if (A.normalize) {
+      if (A.use_global_std) {
+        std_f = g_std;
+      } else {
+        double q = 0.0;
+        for (int64_t j = 0; j < A.branch; ++j) {
+          const double d = (double)rg[j] - mean;
+          q += d * d;
+        }
+        const float var_pop = (float)(q / (double)A.branch);
+        std_f = sqrtf(var_pop + A.eps);
+      }
+    }
+    for (int64_t j = 0; j < A.branch; ++j) {
+      const float c = rg[j] - mean_f;
+      A.out[g * A.branch + j] = A.normalize ? c / std_f : c;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// out[b, j, :] = src[b, pos[j], :]   (unirl/algorithms/base.py:70,80)
+// ---------------------------------------------------------------------------
+constexpr int kGatherThreads = 256;
+
+template <typename W>
+__global__ __launch_bounds__(kGatherThreads) void gather_steps_kernel(const W* __restrict__ src, int64_t S,
+                                                                      int64_t inner, const int64_t* __restrict__ pos,
+                                                                      int64_t n_pos, W* __restrict__ out) {
+  const int64_t bj = blockIdx.y;  // b * n_pos + j
+  const int64_t b = bj / n_pos, j = bj % n_pos;
+  const int64_t p = pos[j];
+  if (p < 0 || p >= S) return;  // validated on the host; never read out of bounds
+  const W* s = src + (b * S + p) * inner;
+  W* o = out + bj * inner;
+  const int64_t stride = (int64_t)gridDim.x * kGatherThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x; i < inner; i += stride) o[i] = s[i];
+}
+
+}  // namespace unirl
+
+using namespace unirl;
+
+extern "C" int unirl_group_advantages(const float* rewards, int64_t n_groups, int64_t branch, int normalize,
+                                      float eps, int scope_global, int use_global_std, float* adv_out,
+                                      void* stream) {
+  if (n_groups < 0 || branch < 0) return UNIRL_E_SHAPE;
+  if (n_groups == 0 || branch == 0) return UNIRL_OK;
+  if (!rewards || !adv_out) return UNIRL_E_NULL;
+  if (!aligned_to(rewards, 4) || !aligned_to(adv_out, 4)) return UNIRL_E_ALIGN;
+  AdvArgs A;
+  A.r = rewards;
+  A.n_groups = n_groups;
+  A.branch = branch;
+  A.normalize = normalize;
+  A.scope_global = scope_global;
+  A.use_global_std = use_global_std;
+  A.eps = eps;
+  A.out = adv_out;
+  hipLaunchKernelGGL(group_advantages_kernel, dim3(1), dim3(kAdvThreads), 0, (hipStream_t)stream, A);
+  return (int)hipGetLastError();
+}
+
+extern "C" int unirl_gather_steps(const void* src, int64_t B, int64_t S, int64_t inner_bytes,
+                                  const int64_t* positions, int64_t n_pos, void* out, void* stream) {
+  if (B < 0 || S < 0 || inner_bytes < 0 || n_pos < 0) return UNIRL_E_SHAPE;
+  if (B == 0 || n_pos == 0 || inner_bytes == 0) return UNIRL_OK;
+  if (!src || !positions || !out) return UNIRL_E_NULL;
+  if (S == 0) return UNIRL_E_SHAPE;
+  if (!aligned_to(positions, 8)) return UNIRL_E_ALIGN;
+  hipStream_t st = (hipStream_t)stream;
+  // widest word that divides the slice size and both base addresses
+  int w = 16;
+  while (w > 1 && (inner_bytes % w != 0 || !aligned_to(src, w) || !aligned_to(out, w))) w >>= 1;
+  const int64_t inner = inner_bytes / w;
+  int64_t nbx = (inner + kGatherThreads * 4 - 1) / (kGatherThreads * 4);
+  if (nbx > 1024) nbx = 1024;
+  if (nbx < 1) nbx = 1;
+  const int64_t rows_total = B * n_pos;
+  const int64_t per_launch = 32768;
+  const int64_t b_per_launch = (per_launch / n_pos) > 0 ? (per_launch / n_pos) : 0;
+  if (b_per_launch == 0) return UNIRL_E_LIMIT;  // more than 32768 positions
+  (void)rows_total;
+  for (int64_t b0 = 0; b0 < B; b0 += b_per_launch) {
+    const int64_t nb = (B - b0 < b_per_launch) ? (B - b0) : b_per_launch;
+    const char* s = reinterpret_cast<const char*>(src) + b0 * S * inner_bytes;
+    char* o = reinterpret_cast<char*>(out) + b0 * n_pos * inner_bytes;
+    dim3 grid((unsigned int)nbx, (unsigned int)(nb * n_pos)), block(kGatherThreads);
+    switch (w) {
+      case 16:
+        hipLaunchKernelGGL((gather_steps_kernel<uint4>), grid, block, 0, st, reinterpret_cast<const uint4*>(s), S,
+                           inner, positions, n_pos, reinterpret_cast<uint4*>(o));
+        break;
+      case 8:
+        hipLaunchKernelGGL((gather_steps_kernel<uint2>), grid, block, 0, st, reinterpret_cast<const uint2*>(s), S,
+                           inner, positions, n_pos, reinterpret_cast<uint2*>(o));
+        break;
+      case 4:
+        hipLaunchKernelGGL((gather_steps_kernel<uint32_t>), grid, block, 0, st,
+                           reinterpret_cast<const uint32_t*>(s), S, inner, positions, n_pos,
+                           reinterpret_cast<uint32_t*>(o));
+        break;
+      case 2:
+        hipLaunchKernelGGL((gather_steps_kernel<uint16_t>), grid, block, 0, st,
+                           reinterpret_cast<const uint16_t*>(s), S, inner, positions, n_pos,
+                           reinterpret_cast<uint16_t*>(o));
+        break;
+      default:
+        hipLaunchKernelGGL((gather_steps_kernel<uint8_t>), grid, block, 0, st, reinterpret_cast<const uint8_t*>(s),
+                           S, inner, positions, n_pos, reinterpret_cast<uint8_t*>(o));
+        break;
+    }
+    const int rc = (int)hipGetLastError();
+    if (rc != 0) return rc;
+  }
+  return UNIRL_OK;
+}

@@ -1,0 +1,754 @@
+// Flow-matching SDE transition + per-sample Gaussian log-prob, fused.
+//
+// Arithmetic follows unirl/sde/kernels.py of the reference op for op in fp32:
+//   FlowSDEStrategy.step            :207-236
+//   DanceSDEStrategy.step           :304-333
+//   CPSSDEStrategy.step             :255-279
+//   compute_log_prob                :193-205 / :247-253 / :290-302
+//   SDEStrategy._finalize_logp      :154-177 (dtype round trip, mean over D)
+// The scalar coefficients (one set per sample) are evaluated in the kernel with
+// the same fp32 operation order torch uses on the [1,1,..] sigma tensors, so
+// prev_sample and prev_sample_mean come out bit-identical to eager torch on the
+// CPU.  The log-prob accumulates sum((prev-mean)^2) per lane in fp32 over a few
+// elements, then in fp64 across lanes / wavefronts / workgroups in a fixed
+// order.
+//
+// HBM traffic per element (fp32, sampling): read v, x, noise; write prev, mean
+// = 20 bytes; replay with the mean kept: read v, x, prev; write mean = 16.
+
+#include "common.cuh"
+#include "unirl_internal.h"
+
+namespace unirl {
+
+constexpr int kSdeThreads = 256;
+constexpr float kHalfLog2Pi = 0.9189385332046727f;  // 0.5*log(2*pi) as torch casts it to f32
+
+struct SdeCoef {
+  // flow / dance: mean = x*a + (v*b)*dt ; prev = mean + s_noise*n
+  // cps         : mean = (x - sigma*v)*om_sn + (x + v*om_s)*c2 ; prev = mean + s_noise*n
+  float a, b, dt, s_noise;
+  float sigma, om_s, om_sn, c2;
+  float den;   // 2*std_var^2   (flow / dance log-prob denominator)
+  float logs;  // log(std_var)
+};
+
+struct SdeScalars {
+  float eta;      // (float)eta
+  float eta2;     // (float)(eta*eta)            -- dance: python computes eta**2 in double
+  float sin_eta;  // (float)sin(eta*pi/2)        -- cps
+};
+
+// Correctly rounded f32 divide / sqrt through f64 (53 >= 2*24+2 bits, so the
+// double rounding is innocuous); independent of how the compiler lowers the
+// f32 forms.
+__device__ __forceinline__ float div_rn(float a, float b) { return (float)((double)a / (double)b); }
+__device__ __forceinline__ float sqrt_rn(float a) { return (float)sqrt((double)a); }
+
+__device__ __forceinline__ SdeCoef sde_coef(int kind, float s, float sn, float smax, SdeScalars sc) {
+  SdeCoef c;
+  c.sigma = s;
+  c.om_s = 1.0f - s;
+  c.om_sn = 1.0f - sn;
+  c.dt = sn - s;
+  c.a = 1.0f;
+  c.b = 1.0f;
+  c.c2 = 0.0f;
+  if (kind == UNIRL_SDE_FLOW) {
+    const float den0 = 1.0f - ((s == 1.0f) ? smax : s);
+    const float std_dev = sqrt_rn(div_rn(s, den0)) * sc.eta;
+    const float std2 = std_dev * std_dev;
+    c.a = 1.0f + div_rn(std2, 2.0f * s) * c.dt;
+    c.b = 1.0f + div_rn(std2 * (1.0f - s), 2.0f * s);
+    c.s_noise = std_dev * sqrt_rn(-c.dt);
+  } else if (kind == UNIRL_SDE_DANCE) {
+    // eta**2 / (2*sigma) is float.__truediv__(tensor) = tensor.reciprocal() * scalar
+    c.a = 1.0f + (div_rn(1.0f, 2.0f * s) * sc.eta2) * c.dt;
+    c.b = 1.0f + div_rn((1.0f - s) * sc.eta2, 2.0f * s);
+    c.s_noise = sqrt_rn(-c.dt) * sc.eta;
+  } else {  // CPS
+    const float std_dev = sn * sc.sin_eta;
+    c.c2 = sqrt_rn(sn * sn - std_dev * std_dev);
+    c.s_noise = std_dev;
+  }
+  const float sv = c.s_noise;
+  c.den = 2.0f * (sv * sv);
+  c.logs = (float)log((double)sv);  // correctly rounded f32 log
+  return c;
+}
+
+// One element of the transition.  Returns prev - mean (the log-prob residual).
+template <typename TX, bool SAMPLING>
+__device__ __forceinline__ float sde_elem(int kind, const SdeCoef& c, float v, float x, float third,
+                                          float& mean, float& prev) {
+  if (kind == UNIRL_SDE_CPS) {
+    const float po = x - c.sigma * v;
+    const float ne = x + v * c.om_s;
+    mean = po * c.om_sn + ne * c.c2;
+  } else {
+    mean = x * c.a + (v * c.b) * c.dt;
+  }
+  if (SAMPLING) {
+    prev = mean + c.s_noise * third;
+  } else {
+    prev = third;
+  }
+  prev = Elem<TX>::round_trip(prev);
+  return prev - mean;
+}
+
+// Final per-sample log-prob from sum((prev-mean)^2) over D elements.
+__device__ __forceinline__ float sde_finish_logp(int kind, const SdeCoef& c, double q, double D, int logp_sum) {
+  double lp;
+  if (kind == UNIRL_SDE_CPS) {
+    lp = -(q / D);
+  } else {
+    lp = -(q / D) / (double)c.den - (double)c.logs - (double)kHalfLog2Pi;
+  }
+  if (logp_sum) lp *= D;
+  return (float)lp;
+}
+
+struct SdeStepArgs {
+  const void* v;
+  const void* x;
+  const void* third;  // noise (f32) when sampling, prev_sample (TX) when replaying; may be null when sampling
+  const float* sigma;
+  const float* sigma_next;
+  const float* sigma_max_ptr;
+  float sigma_max_val;
+  int sigma_stride;
+  SdeScalars sc;
+  int kind;
+  int want_logp;
+  int logp_sum;
+  int64_t D;
+  float* prev_out;
+  float* mean_out;
+  float* logp_out;
+  double* partials;        // [B][gridDim.x]
+  unsigned int* counters;  // [B]
+  unsigned int nblk;       // host only: grid.x
+  int items;               // host only: vectors in flight per lane
+};
+
+template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING>
+__global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
+  __shared__ double lds[kSdeThreads / kWave];
+  __shared__ int lds_flag;
+  using T3 = typename std::conditional<SAMPLING, float, TX>::type;
+
+  const int64_t b = blockIdx.y;
+  const int64_t D = A.D;
+  const float s = A.sigma[b * A.sigma_stride];
+  const float sn = A.sigma_next[b * A.sigma_stride];
+  const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
+  const int kind = A.kind;
+  const SdeCoef c = sde_coef(kind, s, sn, smax, A.sc);
+
+  const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + b * D;
+  const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + b * D;
+  const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + b * D : nullptr;
+  float* __restrict__ po = A.prev_out ? A.prev_out + b * D : nullptr;
+  float* __restrict__ mo = A.mean_out ? A.mean_out + b * D : nullptr;
+
+  const int64_t nvec = D / VEC;  // VEC == 1 or D % VEC == 0 (checked on the host)
+  const int64_t stride = (int64_t)gridDim.x * kSdeThreads;
+  float acc = 0.0f;
+
+  for (int64_t i0 = (int64_t)blockIdx.x * kSdeThreads + threadIdx.x; i0 < nvec; i0 += stride * ITEMS) {
+    float v[ITEMS][VEC], x[ITEMS][VEC], t[ITEMS][VEC];
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t i = i0 + it * stride;
+      if (i < nvec) {
+        Vec<TV, VEC>::load(vp + i * VEC, v[it]);
+        Vec<TX, VEC>::load(xp + i * VEC, x[it]);
+        if (tp) {
+          Vec<T3, VEC>::load(tp + i * VEC, t[it]);
+        } else {
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) t[it][k] = 0.0f;
+        }
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t i = i0 + it * stride;
+      if (i < nvec) {
+        float mean[VEC], prev[VEC];
+#pragma unroll
+        for (int k = 0; k < VEC; ++k) {
+          const float d = sde_elem<TX, SAMPLING>(kind, c, v[it][k], x[it][k], t[it][k], mean[k], prev[k]);
+          acc = fmaf(d, d, acc);
+        }
+        if (po) Vec<float, VEC>::store(po + i * VEC, prev);
+        if (mo) Vec<float, VEC>::store(mo + i * VEC, mean);
+      }
+    }
+  }
+
+  if (!A.want_logp) return;  // uniform across the grid
+
+  const double part = block_sum<double>((double)acc, lds);
+  if (gridDim.x == 1) {
+    if (threadIdx.x == 0) A.logp_out[b] = sde_finish_logp(kind, c, part, (double)D, A.logp_sum);
+    return;
+  }
+  if (threadIdx.x == 0) A.partials[b * gridDim.x + blockIdx.x] = part;
+  if (!arrive_and_check_last(A.counters + b, gridDim.x, &lds_flag)) return;
+  double q = 0.0;
+  for (unsigned int j = threadIdx.x; j < gridDim.x; j += kSdeThreads)
+    q += __builtin_nontemporal_load(A.partials + b * gridDim.x + j);
+  q = block_sum<double>(q, lds);
+  if (threadIdx.x == 0) A.logp_out[b] = sde_finish_logp(kind, c, q, (double)D, A.logp_sum);
+}
+
+// ---------------------------------------------------------------------------
+// Backward.  With r = prev - mean (prev detached) and, for flow / dance,
+//   logp_b = mean_D( -r^2/den ) + const      => dlogp/dmean = 2 r / (den * D)
+//   mean   = x*a + v*(b*dt)                  => dmean/dv = b*dt, dmean/dx = a
+// cps: dlogp/dmean = 2 r / D ; dmean/dv = -sigma*om_sn + om_s*c2 ; dmean/dx = om_sn + c2.
+// In sampling mode prev = mean + s*n also carries g_prev, and prev is detached
+// inside the log-prob, so r contributes no second path.
+// ---------------------------------------------------------------------------
+struct SdeBwdArgs {
+  const void* v;
+  const void* x;
+  const void* third;
+  const float* sigma;
+  const float* sigma_next;
+  const float* sigma_max_ptr;
+  float sigma_max_val;
+  int sigma_stride;
+  SdeScalars sc;
+  int kind;
+  int logp_sum;
+  int64_t D;
+  const float* g_logp;
+  const float* g_mean;
+  const float* g_prev;
+  float* grad_v;
+  float* grad_x;
+};
+
+template <typename TV, typename TX, int VEC, bool SAMPLING>
+__global__ __launch_bounds__(kSdeThreads) void sde_step_bwd_kernel(SdeBwdArgs A) {
+  using T3 = typename std::conditional<SAMPLING, float, TX>::type;
+  const int64_t b = blockIdx.y;
+  const int64_t D = A.D;
+  const float s = A.sigma[b * A.sigma_stride];
+  const float sn = A.sigma_next[b * A.sigma_stride];
+  const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
+  const int kind = A.kind;
+  const SdeCoef c = sde_coef(kind, s, sn, smax, A.sc);
+
+  const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + b * D;
+  const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + b * D;
+  const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + b * D : nullptr;
+  const float* __restrict__ gm = A.g_mean ? A.g_mean + b * D : nullptr;
+  const float* __restrict__ gp = A.g_prev ? A.g_prev + b * D : nullptr;
+  float* __restrict__ gv = A.grad_v ? A.grad_v + b * D : nullptr;
+  float* __restrict__ gx = A.grad_x ? A.grad_x + b * D : nullptr;
+
+  float dmean_dv, dmean_dx, k_lp;
+  const float glp = A.g_logp ? A.g_logp[b] : 0.0f;
+  const float scale = A.logp_sum ? 1.0f : 1.0f / (float)D;
+  if (kind == UNIRL_SDE_CPS) {
+    dmean_dv = c.om_s * c.c2 - c.sigma * c.om_sn;
+    dmean_dx = c.om_sn + c.c2;
+    k_lp = 2.0f * glp * scale;
+  } else {
+    dmean_dv = c.b * c.dt;
+    dmean_dx = c.a;
+    k_lp = 2.0f * glp * scale / c.den;
+  }
+
+  const int64_t nvec = D / VEC;
+  const int64_t stride = (int64_t)gridDim.x * kSdeThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kSdeThreads + threadIdx.x; i < nvec; i += stride) {
+    float v[VEC], x[VEC], t[VEC], g1[VEC], g2[VEC], ov[VEC], ox[VEC];
+    Vec<TV, VEC>::load(vp + i * VEC, v);
+    Vec<TX, VEC>::load(xp + i * VEC, x);
+    if (tp) {
+      Vec<T3, VEC>::load(tp + i * VEC, t);
+    } else {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) t[k] = 0.0f;
+    }
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) g1[k] = g2[k] = 0.0f;
+    if (gm) Vec<float, VEC>::load(gm + i * VEC, g1);
+    if (gp) Vec<float, VEC>::load(gp + i * VEC, g2);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      float mean, prev;
+      const float r = sde_elem<TX, SAMPLING>(kind, c, v[k], x[k], t[k], mean, prev);
+      float g = k_lp * r + g1[k];
+      if (SAMPLING) g += g2[k];
+      ov[k] = g * dmean_dv;
+      ox[k] = g * dmean_dx;
+    }
+    if (gv) Vec<float, VEC>::store(gv + i * VEC, ov);
+    if (gx) Vec<float, VEC>::store(gx + i * VEC, ox);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// S chained transitions, latent in registers.
+// ---------------------------------------------------------------------------
+struct SdeRolloutArgs {
+  const void* x0;
+  const void* v[UNIRL_MAX_ROLLOUT_STEPS];
+  const float* n[UNIRL_MAX_ROLLOUT_STEPS];
+  SdeScalars sc[UNIRL_MAX_ROLLOUT_STEPS];
+  unsigned char want_logp[UNIRL_MAX_ROLLOUT_STEPS];
+  const float* sigmas;
+  const float* sigma_max_ptr;
+  float sigma_max_val;
+  int S;
+  int kind;
+  int logp_sum;
+  int64_t D;
+  int64_t BD;
+  float* x_out;
+  float* traj_out;
+  float* logp_out;         // [B][S]
+  double* partials;        // [B][S][gridDim.x]
+  unsigned int* counters;  // [B]
+  unsigned int nblk;       // host only: grid.x
+  int items;               // host only: vectors per lane (one pass covers a sample)
+};
+
+template <typename TV, typename TX, int VEC, int ITEMS>
+__global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs A) {
+  constexpr int NW = kSdeThreads / kWave;
+  __shared__ double lds_q[UNIRL_MAX_ROLLOUT_STEPS][NW];
+  __shared__ double lds[NW];
+  __shared__ int lds_flag;
+
+  const int64_t b = blockIdx.y;
+  const int64_t D = A.D;
+  const int S = A.S;
+  const int kind = A.kind;
+  const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wid = threadIdx.x / kWave;
+
+  const int64_t nvec = D / VEC;
+  const int64_t stride = (int64_t)gridDim.x * kSdeThreads;
+  const int64_t i_first = (int64_t)blockIdx.x * kSdeThreads + threadIdx.x;
+  // host guarantees gridDim.x * kSdeThreads * ITEMS >= nvec: one pass covers the sample.
+
+  float x[ITEMS][VEC];
+  const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x0) + b * D;
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int64_t i = i_first + it * stride;
+    if (i < nvec) Vec<TX, VEC>::load(xp + i * VEC, x[it]);
+  }
+
+  for (int k = 0; k < S; ++k) {
+    const SdeCoef c = sde_coef(kind, A.sigmas[k], A.sigmas[k + 1], smax, A.sc[k]);
+    const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v[k]) + b * D;
+    const float* __restrict__ np = A.n[k] ? A.n[k] + b * D : nullptr;
+    float* __restrict__ tj = A.traj_out ? A.traj_out + (int64_t)k * A.BD + b * D : nullptr;
+    float v[ITEMS][VEC], n[ITEMS][VEC];
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t i = i_first + it * stride;
+      if (i < nvec) {
+        Vec<TV, VEC>::load(vp + i * VEC, v[it]);
+        if (np) {
+          Vec<float, VEC>::load(np + i * VEC, n[it]);
+        } else {
+#pragma unroll
+          for (int e = 0; e < VEC; ++e) n[it][e] = 0.0f;
+        }
+      }
+    }
+    float acc = 0.0f;
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t i = i_first + it * stride;
+      if (i < nvec) {
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+          float mean, prev;
+          const float d = sde_elem<TX, true>(kind, c, v[it][e], x[it][e], n[it][e], mean, prev);
+          acc = fmaf(d, d, acc);
+          x[it][e] = prev;
+        }
+        if (tj) Vec<float, VEC>::store(tj + i * VEC, x[it]);
+      }
+    }
+    const double w = wave_sum<double>((double)acc);
+    if (lane == 0) lds_q[k][wid] = w;
+  }
+
+  float* __restrict__ xo = A.x_out + b * D;
+#pragma unroll
+  for (int it = 0; it < ITEMS; ++it) {
+    const int64_t i = i_first + it * stride;
+    if (i < nvec) Vec<float, VEC>::store(xo + i * VEC, x[it]);
+  }
+
+  __syncthreads();
+  const unsigned int nblk = gridDim.x;
+  // workgroup totals per step, summed in wave order
+  if ((int)threadIdx.x < S) {
+    double q = 0.0;
+#pragma unroll
+    for (int w = 0; w < NW; ++w) q += lds_q[threadIdx.x][w];
+    if (nblk == 1) {
+      if (A.want_logp[threadIdx.x]) {
+        const SdeCoef c =
+            sde_coef(kind, A.sigmas[threadIdx.x], A.sigmas[threadIdx.x + 1], smax, A.sc[threadIdx.x]);
+        A.logp_out[b * S + threadIdx.x] = sde_finish_logp(kind, c, q, (double)D, A.logp_sum);
+      } else {
+        A.logp_out[b * S + threadIdx.x] = __uint_as_float(0x7fc00000u);
+      }
+    } else {
+      A.partials[((int64_t)b * S + threadIdx.x) * nblk + blockIdx.x] = q;
+    }
+  }
+  if (nblk == 1) return;
+  if (!arrive_and_check_last(A.counters + b, nblk, &lds_flag)) return;
+  for (int k = 0; k < S; ++k) {
+    double q = 0.0;
+    const double* pp = A.partials + ((int64_t)b * S + k) * nblk;
+    for (unsigned int j = threadIdx.x; j < nblk; j += kSdeThreads) q += __builtin_nontemporal_load(pp + j);
+    q = block_sum<double>(q, lds);
+    if (threadIdx.x == 0) {
+      if (A.want_logp[k]) {
+        const SdeCoef c = sde_coef(kind, A.sigmas[k], A.sigmas[k + 1], smax, A.sc[k]);
+        A.logp_out[b * S + k] = sde_finish_logp(kind, c, q, (double)D, A.logp_sum);
+      } else {
+        A.logp_out[b * S + k] = __uint_as_float(0x7fc00000u);
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Host side
+// ---------------------------------------------------------------------------
+static SdeScalars make_scalars(double eta) {
+  SdeScalars sc;
+  sc.eta = (float)eta;
+  sc.eta2 = (float)(eta * eta);
+  sc.sin_eta = (float)sin(eta * 3.141592653589793 / 2.0);
+  return sc;
+}
+
+// Workgroups per sample: enough that each lane keeps ITEMS vectors in flight
+// in one pass, capped so a launch stays a few waves of workgroups over the chip.
+static unsigned int sde_blocks_per_sample(int64_t nvec, int items, int64_t B) {
+  const int64_t per_pass = (int64_t)kSdeThreads * items;
+  int64_t nblk = (nvec + per_pass - 1) / per_pass;
+  const int64_t cap = tune_int("UNIRL_SDE_MAX_BLOCKS", 4096);
+  int64_t max_per_sample = cap / (B > 0 ? B : 1);
+  if (max_per_sample < 1) max_per_sample = 1;
+  if (nblk > max_per_sample) nblk = max_per_sample;
+  if (nblk > kMaxPartialBlocks) nblk = kMaxPartialBlocks;
+  if (nblk < 1) nblk = 1;
+  return (unsigned int)nblk;
+}
+
+// Samples per launch so that counters and partials fit the workspace.
+static int64_t sde_samples_per_launch(int64_t B, int64_t partials_per_sample) {
+  int64_t nb = kPartialCapacity / (partials_per_sample > 0 ? partials_per_sample : 1);
+  if (nb > kMaxCounters) nb = kMaxCounters;
+  if (nb > B) nb = B;
+  return nb < 1 ? 1 : nb;
+}
+
+template <typename TV, typename TX, bool SAMPLING>
+static int launch_step(const SdeStepArgs& A, int64_t B, int vec, hipStream_t st) {
+  const int items = A.items;
+  dim3 grid(A.nblk, (unsigned int)B), block(kSdeThreads);
+  if (vec == 4) {
+    if (items >= 4)
+      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 4, SAMPLING>), grid, block, 0, st, A);
+    else if (items >= 2)
+      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 2, SAMPLING>), grid, block, 0, st, A);
+    else
+      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 1, SAMPLING>), grid, block, 0, st, A);
+  } else {
+    hipLaunchKernelGGL((sde_step_kernel<TV, TX, 1, 2, SAMPLING>), grid, block, 0, st, A);
+  }
+  return (int)hipGetLastError();
+}
+
+template <typename TV, typename TX>
+static int launch_step_mode(const SdeStepArgs& A, int64_t B, int vec, bool sampling, hipStream_t st) {
+  return sampling ? launch_step<TV, TX, true>(A, B, vec, st) : launch_step<TV, TX, false>(A, B, vec, st);
+}
+
+template <typename TV>
+static int launch_step_x(const SdeStepArgs& A, int dtype_x, int64_t B, int vec, bool sampling, hipStream_t st) {
+  switch (dtype_x) {
+    case UNIRL_F32: return launch_step_mode<TV, float>(A, B, vec, sampling, st);
+    case UNIRL_BF16: return launch_step_mode<TV, bf16_t>(A, B, vec, sampling, st);
+    case UNIRL_F16: return launch_step_mode<TV, f16_t>(A, B, vec, sampling, st);
+  }
+  return UNIRL_E_DTYPE;
+}
+
+template <typename TV, typename TX, bool SAMPLING>
+static int launch_bwd(const SdeBwdArgs& A, int64_t B, int vec, hipStream_t st) {
+  const int64_t nvec = A.D / vec;
+  const unsigned int nblk = sde_blocks_per_sample(nvec, 1, B);
+  dim3 grid(nblk, (unsigned int)B), block(kSdeThreads);
+  if (vec == 4)
+    hipLaunchKernelGGL((sde_step_bwd_kernel<TV, TX, 4, SAMPLING>), grid, block, 0, st, A);
+  else
+    hipLaunchKernelGGL((sde_step_bwd_kernel<TV, TX, 1, SAMPLING>), grid, block, 0, st, A);
+  return (int)hipGetLastError();
+}
+
+template <typename TV>
+static int launch_bwd_x(const SdeBwdArgs& A, int dtype_x, int64_t B, int vec, bool sampling, hipStream_t st) {
+  switch (dtype_x) {
+    case UNIRL_F32:
+      return sampling ? launch_bwd<TV, float, true>(A, B, vec, st) : launch_bwd<TV, float, false>(A, B, vec, st);
+    case UNIRL_BF16:
+      return sampling ? launch_bwd<TV, bf16_t, true>(A, B, vec, st) : launch_bwd<TV, bf16_t, false>(A, B, vec, st);
+    case UNIRL_F16:
+      return sampling ? launch_bwd<TV, f16_t, true>(A, B, vec, st) : launch_bwd<TV, f16_t, false>(A, B, vec, st);
+  }
+  return UNIRL_E_DTYPE;
+}
+
+template <typename TV, typename TX>
+static int launch_rollout(const SdeRolloutArgs& A, int64_t B, int vec, hipStream_t st) {
+  dim3 grid(A.nblk, (unsigned int)B), block(kSdeThreads);
+  const int items = A.items;
+  if (vec == 4) {
+    if (items >= 4)
+      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 4, 4>), grid, block, 0, st, A);
+    else if (items == 2)
+      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 4, 2>), grid, block, 0, st, A);
+    else
+      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 4, 1>), grid, block, 0, st, A);
+  } else {
+    if (items >= 4)
+      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 1, 4>), grid, block, 0, st, A);
+    else if (items == 2)
+      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 1, 2>), grid, block, 0, st, A);
+    else
+      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 1, 1>), grid, block, 0, st, A);
+  }
+  return (int)hipGetLastError();
+}
+
+template <typename TV>
+static int launch_rollout_x(const SdeRolloutArgs& A, int dtype_x, int64_t B, int vec, hipStream_t st) {
+  switch (dtype_x) {
+    case UNIRL_F32: return launch_rollout<TV, float>(A, B, vec, st);
+    case UNIRL_BF16: return launch_rollout<TV, bf16_t>(A, B, vec, st);
+    case UNIRL_F16: return launch_rollout<TV, f16_t>(A, B, vec, st);
+  }
+  return UNIRL_E_DTYPE;
+}
+
+}  // namespace unirl
+
+using namespace unirl;
+
+extern "C" int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const void* sample, int dtype_x,
+                                   const void* prev_sample, const float* noise, const float* sigma,
+                                   const float* sigma_next, int sigma_stride, const float* sigma_max_ptr,
+                                   float sigma_max_val, double eta, int kind, int64_t B, int64_t D,
+                                   float* prev_out, float* mean_out, float* logp_out, int logp_sum,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+  if (!dtype_ok(dtype_v) || !dtype_ok(dtype_x)) return UNIRL_E_DTYPE;
+  if (kind < UNIRL_SDE_FLOW || kind > UNIRL_SDE_CPS) return UNIRL_E_DTYPE;
+  if (B < 0 || D <= 0 || (sigma_stride != 0 && sigma_stride != 1)) return UNIRL_E_SHAPE;
+  if (B == 0) return UNIRL_OK;
+  if (!noise_pred || !sample || !sigma || !sigma_next) return UNIRL_E_NULL;
+  const bool sampling = (prev_sample == nullptr);
+  const bool want_logp = (logp_out != nullptr) && !(eta < 1e-7);
+  if (want_logp && (!workspace || workspace_bytes < kWorkspaceBytes)) return UNIRL_E_WORKSPACE;
+  const size_t sv = dtype_size(dtype_v), sx = dtype_size(dtype_x);
+  if (!aligned_to(noise_pred, sv) || !aligned_to(sample, sx) || !aligned_to(prev_sample, sx) ||
+      !aligned_to(noise, 4) || !aligned_to(prev_out, 4) || !aligned_to(mean_out, 4))
+    return UNIRL_E_ALIGN;
+
+  // 4-element vectors need every per-sample base to keep the vector alignment.
+  int vec = 4;
+  if (D % 4 != 0 || !aligned_to(noise_pred, 4 * sv) || !aligned_to(sample, 4 * sx) ||
+      !aligned_to(prev_sample, 4 * sx) || !aligned_to(noise, 16) || !aligned_to(prev_out, 16) ||
+      !aligned_to(mean_out, 16))
+    vec = 1;
+
+  const int items = (vec == 4) ? (int)tune_int("UNIRL_SDE_ITEMS", 2) : 2;
+  const unsigned int nblk = sde_blocks_per_sample(D / vec, items, B);
+  const int64_t per_launch = sde_samples_per_launch(B, nblk);
+  hipStream_t st = (hipStream_t)stream;
+
+  for (int64_t b0 = 0; b0 < B; b0 += per_launch) {
+    const int64_t nb = (B - b0 < per_launch) ? (B - b0) : per_launch;
+    const int64_t off = b0 * D;
+    SdeStepArgs A;
+    A.v = offset_ptr(noise_pred, off, sv);
+    A.x = offset_ptr(sample, off, sx);
+    A.third = sampling ? (const void*)offset_f32(noise, off) : offset_ptr(prev_sample, off, sx);
+    A.sigma = sigma + b0 * sigma_stride;
+    A.sigma_next = sigma_next + b0 * sigma_stride;
+    A.sigma_max_ptr = sigma_max_ptr;
+    A.sigma_max_val = sigma_max_val;
+    A.sigma_stride = sigma_stride;
+    A.sc = make_scalars(eta);
+    A.kind = kind;
+    A.want_logp = want_logp ? 1 : 0;
+    A.logp_sum = logp_sum;
+    A.D = D;
+    A.prev_out = offset_f32(prev_out, off);
+    A.mean_out = offset_f32(mean_out, off);
+    A.logp_out = offset_f32(logp_out, b0);
+    A.partials = ws_partials(workspace);
+    A.counters = ws_counters(workspace);
+    A.nblk = nblk;
+    A.items = items;
+    int rc = UNIRL_E_DTYPE;
+    switch (dtype_v) {
+      case UNIRL_F32: rc = launch_step_x<float>(A, dtype_x, nb, vec, sampling, st); break;
+      case UNIRL_BF16: rc = launch_step_x<bf16_t>(A, dtype_x, nb, vec, sampling, st); break;
+      case UNIRL_F16: rc = launch_step_x<f16_t>(A, dtype_x, nb, vec, sampling, st); break;
+    }
+    if (rc != 0) return rc;
+  }
+  return UNIRL_OK;
+}
+
+extern "C" int unirl_sde_step_logp_bwd(const void* noise_pred, int dtype_v, const void* sample, int dtype_x,
+                                       const void* prev_sample, const float* noise, const float* sigma,
+                                       const float* sigma_next, int sigma_stride, const float* sigma_max_ptr,
+                                       float sigma_max_val, double eta, int kind, int64_t B, int64_t D,
+                                       const float* g_logp, const float* g_mean, const float* g_prev,
+                                       int logp_sum, float* grad_v, float* grad_x, void* stream) {
+  if (!dtype_ok(dtype_v) || !dtype_ok(dtype_x)) return UNIRL_E_DTYPE;
+  if (kind < UNIRL_SDE_FLOW || kind > UNIRL_SDE_CPS) return UNIRL_E_DTYPE;
+  if (B < 0 || D <= 0 || (sigma_stride != 0 && sigma_stride != 1)) return UNIRL_E_SHAPE;
+  if (B == 0) return UNIRL_OK;
+  if (!noise_pred || !sample || !sigma || !sigma_next) return UNIRL_E_NULL;
+  if (!grad_v && !grad_x) return UNIRL_OK;
+  const bool sampling = (prev_sample == nullptr);
+  const size_t sv = dtype_size(dtype_v), sx = dtype_size(dtype_x);
+  if (!aligned_to(noise_pred, sv) || !aligned_to(sample, sx) || !aligned_to(prev_sample, sx) ||
+      !aligned_to(noise, 4) || !aligned_to(g_mean, 4) || !aligned_to(g_prev, 4) || !aligned_to(grad_v, 4) ||
+      !aligned_to(grad_x, 4))
+    return UNIRL_E_ALIGN;
+  int vec = 4;
+  if (D % 4 != 0 || !aligned_to(noise_pred, 4 * sv) || !aligned_to(sample, 4 * sx) ||
+      !aligned_to(prev_sample, 4 * sx) || !aligned_to(noise, 16) || !aligned_to(g_mean, 16) ||
+      !aligned_to(g_prev, 16) || !aligned_to(grad_v, 16) || !aligned_to(grad_x, 16))
+    vec = 1;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t per_launch = 32768;  // grid.y limit is 65535
+  for (int64_t b0 = 0; b0 < B; b0 += per_launch) {
+    const int64_t nb = (B - b0 < per_launch) ? (B - b0) : per_launch;
+    const int64_t off = b0 * D;
+    SdeBwdArgs A;
+    A.v = offset_ptr(noise_pred, off, sv);
+    A.x = offset_ptr(sample, off, sx);
+    A.third = sampling ? (const void*)offset_f32(noise, off) : offset_ptr(prev_sample, off, sx);
+    A.sigma = sigma + b0 * sigma_stride;
+    A.sigma_next = sigma_next + b0 * sigma_stride;
+    A.sigma_max_ptr = sigma_max_ptr;
+    A.sigma_max_val = sigma_max_val;
+    A.sigma_stride = sigma_stride;
+    A.sc = make_scalars(eta);
+    A.kind = kind;
+    A.logp_sum = logp_sum;
+    A.D = D;
+    A.g_logp = (eta < 1e-7) ? nullptr : offset_f32(g_logp, b0);
+    A.g_mean = offset_f32(g_mean, off);
+    A.g_prev = offset_f32(g_prev, off);
+    A.grad_v = offset_f32(grad_v, off);
+    A.grad_x = offset_f32(grad_x, off);
+    int rc = UNIRL_E_DTYPE;
+    switch (dtype_v) {
+      case UNIRL_F32: rc = launch_bwd_x<float>(A, dtype_x, nb, vec, sampling, st); break;
+      case UNIRL_BF16: rc = launch_bwd_x<bf16_t>(A, dtype_x, nb, vec, sampling, st); break;
+      case UNIRL_F16: rc = launch_bwd_x<f16_t>(A, dtype_x, nb, vec, sampling, st); break;
+    }
+    if (rc != 0) return rc;
+  }
+  return UNIRL_OK;
+}
+
+extern "C" int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* const* v_steps, int dtype_v,
+                                      const float* const* noise_steps, const float* sigmas, const double* etas,
+                                      int S, const float* sigma_max_ptr, float sigma_max_val, int kind, int64_t B,
+                                      int64_t D, float* x_out, float* traj_out, float* logp_out, int logp_sum,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  if (!dtype_ok(dtype_v) || !dtype_ok(dtype_x)) return UNIRL_E_DTYPE;
+  if (kind < UNIRL_SDE_FLOW || kind > UNIRL_SDE_CPS) return UNIRL_E_DTYPE;
+  if (B < 0 || D <= 0 || S < 1) return UNIRL_E_SHAPE;
+  if (S > UNIRL_MAX_ROLLOUT_STEPS) return UNIRL_E_LIMIT;
+  if (B == 0) return UNIRL_OK;
+  if (!x0 || !x_out || !logp_out || !v_steps || !noise_steps || !sigmas || !etas) return UNIRL_E_NULL;
+  if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
+  const size_t sv = dtype_size(dtype_v), sx = dtype_size(dtype_x);
+  if (!aligned_to(x0, sx) || !aligned_to(x_out, 4) || !aligned_to(traj_out, 4)) return UNIRL_E_ALIGN;
+
+  int vec = 4;
+  if (D % 4 != 0 || !aligned_to(x0, 4 * sx) || !aligned_to(x_out, 16) || !aligned_to(traj_out, 16)) vec = 1;
+  for (int k = 0; k < S; ++k) {
+    if (!v_steps[k]) return UNIRL_E_NULL;
+    if (!aligned_to(v_steps[k], sv) || !aligned_to(noise_steps[k], 4)) return UNIRL_E_ALIGN;
+    if (!aligned_to(v_steps[k], 4 * sv) || !aligned_to(noise_steps[k], 16)) vec = 1;
+  }
+
+  // One pass must cover a sample (the latent lives in registers): pick the
+  // vectors per lane, the workgroup count follows.
+  const int64_t nvec = D / vec;
+  int items = (int)tune_int("UNIRL_ROLLOUT_ITEMS", 1);
+  if (items != 1 && items != 2 && items != 4) items = 1;
+  int64_t nblk = (nvec + (int64_t)kSdeThreads * items - 1) / ((int64_t)kSdeThreads * items);
+  while (nblk * S > kPartialCapacity && items < 4) {
+    items *= 2;
+    nblk = (nvec + (int64_t)kSdeThreads * items - 1) / ((int64_t)kSdeThreads * items);
+  }
+  if (nblk * S > kPartialCapacity) return UNIRL_E_LIMIT;
+  const int64_t per_launch = sde_samples_per_launch(B, nblk * S);
+  hipStream_t st = (hipStream_t)stream;
+
+  for (int64_t b0 = 0; b0 < B; b0 += per_launch) {
+    const int64_t nb = (B - b0 < per_launch) ? (B - b0) : per_launch;
+    const int64_t off = b0 * D;
+    SdeRolloutArgs A;
+    for (int k = 0; k < S; ++k) {
+      A.v[k] = offset_ptr(v_steps[k], off, sv);
+      A.n[k] = offset_f32(noise_steps[k], off);
+      A.sc[k] = make_scalars(etas[k]);
+      A.want_logp[k] = !(etas[k] < 1e-7);
+    }
+    A.x0 = offset_ptr(x0, off, sx);
+    A.sigmas = sigmas;
+    A.sigma_max_ptr = sigma_max_ptr;
+    A.sigma_max_val = sigma_max_val;
+    A.S = S;
+    A.kind = kind;
+    A.logp_sum = logp_sum;
+    A.D = D;
+    A.BD = B * D;
+    A.x_out = offset_f32(x_out, off);
+    A.traj_out = offset_f32(traj_out, off);
+    A.logp_out = offset_f32(logp_out, b0 * S);
+    A.partials = ws_partials(workspace);
+    A.counters = ws_counters(workspace);
+    A.nblk = (unsigned int)nblk;
+    A.items = items;
+    int rc = UNIRL_E_DTYPE;
+    switch (dtype_v) {
+      case UNIRL_F32: rc = launch_rollout_x<float>(A, dtype_x, nb, vec, st); break;
+      case UNIRL_BF16: rc = launch_rollout_x<bf16_t>(A, dtype_x, nb, vec, st); break;
+      case UNIRL_F16: rc = launch_rollout_x<f16_t>(A, dtype_x, nb, vec, st); break;
+    }
+    if (rc != 0) return rc;
+  }
+  return UNIRL_OK;
+}

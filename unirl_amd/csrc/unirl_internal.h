@@ -1,0 +1,45 @@
+// Host-side declarations shared by the translation units of libunirl_hip.so.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <type_traits>
+
+#include "../../include/unirl_hip.h"
+
+namespace unirl {
+
+// Workspace layout: [ticket counters | fp64 partials].
+constexpr int64_t kMaxCounters = 16384;                // uint32 each
+constexpr int64_t kMaxPartialBlocks = 2048;            // workgroups per reduced row
+constexpr int64_t kPartialCapacity = 512 * 1024;       // doubles
+constexpr size_t kCounterBytes = (size_t)kMaxCounters * sizeof(unsigned int);
+constexpr size_t kWorkspaceBytes = kCounterBytes + (size_t)kPartialCapacity * sizeof(double);
+
+inline unsigned int* ws_counters(void* ws) { return reinterpret_cast<unsigned int*>(ws); }
+inline double* ws_partials(void* ws) {
+  return ws ? reinterpret_cast<double*>(reinterpret_cast<char*>(ws) + kCounterBytes) : nullptr;
+}
+
+// Launch-shape knobs for measurement sweeps; read from the environment at every
+// call (a getenv is nanoseconds next to a kernel launch).  Unset = default.
+inline int64_t tune_int(const char* name, int64_t dflt) {
+  const char* s = getenv(name);
+  if (!s || !*s) return dflt;
+  char* end = nullptr;
+  const long long v = strtoll(s, &end, 10);
+  return (end && *end == '\0' && v > 0) ? (int64_t)v : dflt;
+}
+
+inline size_t dtype_size(int dt) { return dt == UNIRL_F32 ? 4 : 2; }
+inline bool dtype_ok(int dt) { return dt == UNIRL_F32 || dt == UNIRL_BF16 || dt == UNIRL_F16; }
+// NULL counts as aligned: optional pointers are checked only when present.
+inline bool aligned_to(const void* p, size_t a) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) % a) == 0; }
+inline const void* offset_ptr(const void* p, int64_t elems, size_t elem_size) {
+  return p ? (const void*)(reinterpret_cast<const char*>(p) + elems * (int64_t)elem_size) : nullptr;
+}
+inline float* offset_f32(float* p, int64_t elems) { return p ? p + elems : nullptr; }
+inline const float* offset_f32(const float* p, int64_t elems) { return p ? p + elems : nullptr; }
+
+}  // namespace unirl

@@ -1,0 +1,612 @@
+"""Tensor-level wrappers over the C ABI: validate, allocate outputs, launch.
+
+Every function takes HIP tensors, enqueues one fused kernel on the current
+torch stream and returns without synchronising.  The reference-shaped Python
+API (``unirl_amd.sde``, ``unirl_amd.algorithms``, ...) is built on these.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import math
+from typing import Dict, List, Optional, Sequence, Tuple, Union
+
+import torch
+
+from . import _native as N
+
+SDE_KINDS = {"flow": N.SDE_FLOW, "dance": N.SDE_DANCE, "cps": N.SDE_CPS}
+
+
+def _flat2(t: torch.Tensor, name: str) -> torch.Tensor:
+    N.require_device(t, name)
+    return t if t.is_contiguous() else t.contiguous()
+
+
+def _sigma_arg(sigma: torch.Tensor, B: int, device: torch.device, name: str) -> Tuple[torch.Tensor, int]:
+    """f32 device tensor with 1 or B values, and the per-sample stride (0 or 1)."""
+    s = sigma.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    if s.numel() == 1:
+        return s, 0
+    if s.numel() == B:
+        return s, 1
+    raise ValueError(f"{name} must hold one value or one per sample ({B}); got {tuple(sigma.shape)}")
+
+
+def _sigma_max_arg(sigma_max, device: torch.device):
+    """(device tensor or None, float value)."""
+    if isinstance(sigma_max, torch.Tensor):
+        if sigma_max.is_cuda:
+            t = sigma_max.detach().to(device=device, dtype=torch.float32).reshape(-1)[:1].contiguous()
+            return t, 0.0
+        return None, float(sigma_max)
+    return None, float(sigma_max)
+
+
+def sde_step_logp(
+    noise_pred: torch.Tensor,
+    sample: torch.Tensor,
+    sigma: torch.Tensor,
+    sigma_next: torch.Tensor,
+    *,
+    kind: str = "flow",
+    eta: float = 1.0,
+    prev_sample: Optional[torch.Tensor] = None,
+    noise: Optional[torch.Tensor] = None,
+    sigma_max: Union[float, torch.Tensor] = 0.99,
+    want_prev: bool = True,
+    want_mean: bool = True,
+    want_logp: bool = True,
+    logp_sum: bool = False,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """One fused SDE transition. Returns ``(prev f32, logp [B] f32 or None, mean f32)``.
+
+    ``prev_sample`` given = replay, else sampling with ``noise`` (f32, same shape;
+    ``None`` adds no noise).  ``sample.dtype`` is the dtype of the round trip applied
+    to ``prev`` before the log-prob.
+    """
+    if sample.dim() < 2:
+        raise ValueError(f"sample needs a batch dimension and at least one more; got {tuple(sample.shape)}")
+    if noise_pred.shape != sample.shape:
+        raise ValueError(f"noise_pred {tuple(noise_pred.shape)} != sample {tuple(sample.shape)}")
+    device = sample.device
+    v = _flat2(noise_pred.detach(), "noise_pred")
+    x = _flat2(sample.detach(), "sample")
+    if v.dtype not in N._DTYPE_CODE:
+        v = v.float()
+    if x.dtype not in N._DTYPE_CODE:
+        x = x.float()
+    B = x.shape[0]
+    D = x.numel() // B if B else 0
+    prev_in = None
+    if prev_sample is not None:
+        if prev_sample.shape != sample.shape:
+            raise ValueError(f"prev_sample {tuple(prev_sample.shape)} != sample {tuple(sample.shape)}")
+        # prev.float().to(x.dtype) == prev.to(x.dtype): casting here is the reference's round trip
+        prev_in = _flat2(prev_sample.detach(), "prev_sample").to(x.dtype)
+    nz = None
+    if noise is not None and prev_sample is None:
+        if noise.shape != sample.shape:
+            raise ValueError(f"noise {tuple(noise.shape)} != sample {tuple(sample.shape)}")
+        nz = _flat2(noise.detach(), "noise").float()
+    sig, stride = _sigma_arg(sigma, B, device, "sigma")
+    sig_n, stride_n = _sigma_arg(sigma_next, B, device, "sigma_next")
+    if stride != stride_n:
+        if stride == 0:
+            sig, stride = sig.expand(B).contiguous(), 1
+        else:
+            sig_n = sig_n.expand(B).contiguous()
+    smax_t, smax_v = _sigma_max_arg(sigma_max, device)
+
+    logp_wanted = want_logp and not (eta < 1e-7)
+    prev_out = torch.empty(x.shape, dtype=torch.float32, device=device) if want_prev else None
+    mean_out = torch.empty(x.shape, dtype=torch.float32, device=device) if want_mean else None
+    logp_out = torch.empty(B, dtype=torch.float32, device=device) if logp_wanted else None
+    if B == 0 or D == 0:
+        if logp_out is not None:
+            logp_out.fill_(float("nan"))
+        return prev_out, logp_out, mean_out
+    ws, ws_bytes = N.workspace(device)
+    with torch.cuda.device(device):
+        rc = N.lib().unirl_sde_step_logp(
+            N.ptr(v), N.dtype_code(v.dtype), N.ptr(x), N.dtype_code(x.dtype), N.ptr(prev_in), N.ptr(nz),
+            N.ptr(sig), N.ptr(sig_n), stride, N.ptr(smax_t), smax_v, float(eta), SDE_KINDS[kind], B, D,
+            N.ptr(prev_out), N.ptr(mean_out), N.ptr(logp_out), int(bool(logp_sum)), N.ptr(ws), ws_bytes,
+            N.current_stream(device),
+        )
+    N.check(rc, "unirl_sde_step_logp")
+    return prev_out, logp_out, mean_out
+
+
+def sde_step_logp_bwd(
+    noise_pred: torch.Tensor,
+    sample: torch.Tensor,
+    sigma: torch.Tensor,
+    sigma_next: torch.Tensor,
+    *,
+    kind: str,
+    eta: float,
+    prev_sample: Optional[torch.Tensor],
+    noise: Optional[torch.Tensor],
+    sigma_max,
+    g_logp: Optional[torch.Tensor],
+    g_mean: Optional[torch.Tensor],
+    g_prev: Optional[torch.Tensor],
+    need_grad_v: bool,
+    need_grad_x: bool,
+    logp_sum: bool = False,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Gradients of :func:`sde_step_logp` w.r.t. ``noise_pred`` and ``sample`` (f32)."""
+    device = sample.device
+    v = _flat2(noise_pred.detach(), "noise_pred")
+    x = _flat2(sample.detach(), "sample")
+    if v.dtype not in N._DTYPE_CODE:
+        v = v.float()
+    if x.dtype not in N._DTYPE_CODE:
+        x = x.float()
+    B = x.shape[0]
+    D = x.numel() // B if B else 0
+    prev_in = None if prev_sample is None else _flat2(prev_sample.detach(), "prev_sample").to(x.dtype)
+    nz = None if (noise is None or prev_sample is not None) else _flat2(noise.detach(), "noise").float()
+    sig, stride = _sigma_arg(sigma, B, device, "sigma")
+    sig_n, stride_n = _sigma_arg(sigma_next, B, device, "sigma_next")
+    if stride != stride_n:
+        if stride == 0:
+            sig, stride = sig.expand(B).contiguous(), 1
+        else:
+            sig_n = sig_n.expand(B).contiguous()
+    smax_t, smax_v = _sigma_max_arg(sigma_max, device)
+
+    def f32c(t):
+        return None if t is None else t.detach().to(device=device, dtype=torch.float32).contiguous()
+
+    gl, gm, gp = f32c(g_logp), f32c(g_mean), f32c(g_prev)
+    grad_v = torch.empty(x.shape, dtype=torch.float32, device=device) if need_grad_v else None
+    grad_x = torch.empty(x.shape, dtype=torch.float32, device=device) if need_grad_x else None
+    if B == 0 or D == 0 or (grad_v is None and grad_x is None):
+        return grad_v, grad_x
+    with torch.cuda.device(device):
+        rc = N.lib().unirl_sde_step_logp_bwd(
+            N.ptr(v), N.dtype_code(v.dtype), N.ptr(x), N.dtype_code(x.dtype), N.ptr(prev_in), N.ptr(nz),
+            N.ptr(sig), N.ptr(sig_n), stride, N.ptr(smax_t), smax_v, float(eta), SDE_KINDS[kind], B, D,
+            N.ptr(gl), N.ptr(gm), N.ptr(gp), int(bool(logp_sum)), N.ptr(grad_v), N.ptr(grad_x),
+            N.current_stream(device),
+        )
+    N.check(rc, "unirl_sde_step_logp_bwd")
+    return grad_v, grad_x
+
+
+def sde_rollout_logp(
+    x0: torch.Tensor,
+    velocities: Sequence[torch.Tensor],
+    noises: Sequence[Optional[torch.Tensor]],
+    sigmas: torch.Tensor,
+    etas: Union[float, Sequence[float]],
+    *,
+    kind: str = "flow",
+    sigma_max: Union[float, torch.Tensor, None] = None,
+    want_trajectory: bool = False,
+    logp_sum: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """``S = len(velocities)`` chained transitions in one launch.
+
+    Step ``k`` moves ``sigmas[k] -> sigmas[k+1]`` with ``velocities[k]``, ``noises[k]``
+    and ``etas[k]``.  ``sigma_max=None`` takes ``sigmas[1]`` like the reference's stage
+    loop.  Returns ``(x_final f32, logp [B,S] f32 (NaN where eta<1e-7), trajectory
+    [S,B,...] f32 or None)``.
+    """
+    S = len(velocities)
+    if S < 1 or S > N.MAX_ROLLOUT_STEPS:
+        raise ValueError(f"number of steps must be in [1, {N.MAX_ROLLOUT_STEPS}]; got {S}")
+    if len(noises) != S:
+        raise ValueError(f"{S} velocities but {len(noises)} noises")
+    if isinstance(etas, (int, float)):
+        etas = [float(etas)] * S
+    if len(etas) != S:
+        raise ValueError(f"{S} velocities but {len(etas)} etas")
+    device = x0.device
+    x = _flat2(x0.detach(), "x0")
+    if x.dtype not in N._DTYPE_CODE:
+        x = x.float()
+    B = x.shape[0]
+    D = x.numel() // B if B else 0
+    sig = sigmas.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    if sig.numel() < S + 1:
+        raise ValueError(f"sigmas needs {S + 1} values for {S} steps; got {sig.numel()}")
+    if sigma_max is None:
+        smax_t, smax_v = sig[1:2], 0.0
+    else:
+        smax_t, smax_v = _sigma_max_arg(sigma_max, device)
+    vs: List[torch.Tensor] = []
+    ns: List[Optional[torch.Tensor]] = []
+    vdtype = None
+    for k in range(S):
+        vk = _flat2(velocities[k].detach(), f"velocities[{k}]")
+        if vk.shape != x.shape:
+            raise ValueError(f"velocities[{k}] {tuple(vk.shape)} != x0 {tuple(x.shape)}")
+        if vk.dtype not in N._DTYPE_CODE:
+            vk = vk.float()
+        if vdtype is None:
+            vdtype = vk.dtype
+        elif vk.dtype != vdtype:
+            vk = vk.to(vdtype)
+        vs.append(vk)
+        nk = noises[k]
+        if nk is not None:
+            if nk.shape != x.shape:
+                raise ValueError(f"noises[{k}] {tuple(nk.shape)} != x0 {tuple(x.shape)}")
+            nk = _flat2(nk.detach(), f"noises[{k}]").float()
+        ns.append(nk)
+    x_out = torch.empty(x.shape, dtype=torch.float32, device=device)
+    logp = torch.empty((B, S), dtype=torch.float32, device=device)
+    traj = torch.empty((S,) + tuple(x.shape), dtype=torch.float32, device=device) if want_trajectory else None
+    if B == 0 or D == 0:
+        return x_out, logp, traj
+    v_arr = (ctypes.c_void_p * S)(*[t.data_ptr() for t in vs])
+    n_arr = (ctypes.c_void_p * S)(*[(t.data_ptr() if t is not None else None) for t in ns])
+    e_arr = (ctypes.c_double * S)(*[float(e) for e in etas])
+    ws, ws_bytes = N.workspace(device)
+    with torch.cuda.device(device):
+        rc = N.lib().unirl_sde_rollout_logp(
+            N.ptr(x), N.dtype_code(x.dtype), v_arr, N.dtype_code(vdtype), n_arr, N.ptr(sig), e_arr, S,
+            N.ptr(smax_t), smax_v, SDE_KINDS[kind], B, D, N.ptr(x_out), N.ptr(traj), N.ptr(logp),
+            int(bool(logp_sum)), N.ptr(ws), ws_bytes, N.current_stream(device),
+        )
+    N.check(rc, "unirl_sde_rollout_logp")
+    return x_out, logp, traj
+
+
+def gaussian_kl_mask(
+    p: torch.Tensor,
+    q: torch.Tensor,
+    sigma: torch.Tensor,
+    threshold: float,
+    *,
+    reduce_from_dim: int = 2,
+    want_mask: bool = True,
+) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Per-row mean of ``(p-q)^2 / (2 sigma^2)`` and ``kl < threshold``.
+
+    Rows are the leading ``reduce_from_dim`` dimensions of ``p``; ``sigma`` holds one
+    value, or one per index of the LAST leading dimension (``[1,S',1,...]``).
+    """
+    if p.shape != q.shape:
+        raise ValueError(f"p {tuple(p.shape)} != q {tuple(q.shape)}")
+    if p.dim() <= reduce_from_dim:
+        raise ValueError(f"need more than {reduce_from_dim} dims to reduce over; got {tuple(p.shape)}")
+    device = p.device
+    pc = _flat2(p.detach(), "p")
+    qc = _flat2(q.detach(), "q").to(pc.dtype)
+    if pc.dtype not in N._DTYPE_CODE:
+        pc, qc = pc.float(), qc.float()
+    lead = tuple(pc.shape[:reduce_from_dim])
+    R = int(math.prod(lead))
+    D = pc.numel() // R if R else 0
+    sig = sigma.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    if sig.numel() not in (1, lead[-1]):
+        raise ValueError(f"sigma must hold 1 or {lead[-1]} values; got {tuple(sigma.shape)}")
+    kl = torch.empty(lead, dtype=torch.float32, device=device)
+    mask = torch.empty(lead, dtype=torch.bool, device=device) if want_mask else None
+    if R == 0 or D == 0:
+        return kl, mask
+    ws, ws_bytes = N.workspace(device)
+    with torch.cuda.device(device):
+        rc = N.lib().unirl_gaussian_kl_mask(
+            N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, float(threshold),
+            N.ptr(kl), N.ptr(mask), N.ptr(ws), ws_bytes, N.current_stream(device),
+        )
+    N.check(rc, "unirl_gaussian_kl_mask")
+    return kl, mask
+
+
+def gaussian_kl_elem(p: torch.Tensor, q: torch.Tensor, sigma: torch.Tensor, *, sigma_dim: int = 1) -> torch.Tensor:
+    """Element-wise ``(p-q)^2 / (2 sigma^2)`` as f32; sigma broadcast along ``sigma_dim``."""
+    if p.shape != q.shape:
+        raise ValueError(f"p {tuple(p.shape)} != q {tuple(q.shape)}")
+    device = p.device
+    pc = _flat2(p.detach(), "p")
+    qc = _flat2(q.detach(), "q").to(pc.dtype)
+    if pc.dtype not in N._DTYPE_CODE:
+        pc, qc = pc.float(), qc.float()
+    sig = sigma.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    if sig.numel() == 1:
+        R, D = 1, pc.numel()
+    else:
+        if pc.dim() <= sigma_dim or sig.numel() != pc.shape[sigma_dim]:
+            raise ValueError(f"sigma {tuple(sigma.shape)} does not match dim {sigma_dim} of {tuple(p.shape)}")
+        R = int(math.prod(pc.shape[: sigma_dim + 1]))
+        D = pc.numel() // R if R else 0
+    out = torch.empty(pc.shape, dtype=torch.float32, device=device)
+    if pc.numel() == 0:
+        return out
+    with torch.cuda.device(device):
+        rc = N.lib().unirl_gaussian_kl_elem(
+            N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, N.ptr(out),
+            N.current_stream(device),
+        )
+    N.check(rc, "unirl_gaussian_kl_elem")
+    return out
+
+
+def token_logp_entropy(
+    logits: torch.Tensor,
+    ids: Optional[torch.Tensor],
+    temperature: float = 1.0,
+    *,
+    want_logp: bool = True,
+    want_entropy: bool = True,
+    want_lse: bool = False,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """``(logp, entropy, logsumexp)`` per row of ``logits [..., V]``, each f32 ``[...]``."""
+    N.require_device(logits, "logits")
+    if logits.dim() < 1:
+        raise ValueError("logits needs a vocabulary dimension")
+    device = logits.device
+    V = logits.shape[-1]
+    lead = tuple(logits.shape[:-1])
+    x = logits.detach()
+    if x.dtype not in N._DTYPE_CODE:
+        x = x.float()
+    x2 = x.reshape(-1, V)
+    if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < V):
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    row_stride = x2.stride(0) if rows > 1 else V
+    idc = None
+    if want_logp:
+        if ids is None:
+            raise ValueError("ids is required for the log-prob")
+        if tuple(ids.shape) != lead:
+            raise ValueError(f"ids {tuple(ids.shape)} does not match logits rows {lead}")
+        idc = ids.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
+    logp = torch.empty(lead, dtype=torch.float32, device=device) if want_logp else None
+    ent = torch.empty(lead, dtype=torch.float32, device=device) if want_entropy else None
+    lse = torch.empty(lead, dtype=torch.float32, device=device) if want_lse else None
+    if rows == 0:
+        return logp, ent, lse
+    if V == 0:
+        raise ValueError("empty vocabulary")
+    with torch.cuda.device(device):
+        rc = N.lib().unirl_token_logp_entropy(
+            N.ptr(x2), N.dtype_code(x2.dtype), rows, V, row_stride, N.ptr(idc), float(temperature),
+            N.ptr(logp), N.ptr(ent), N.ptr(lse), N.current_stream(device),
+        )
+    N.check(rc, "unirl_token_logp_entropy")
+    return logp, ent, lse
+
+
+def token_logp_bwd(
+    logits: torch.Tensor, ids: torch.Tensor, temperature: float, lse: torch.Tensor, g_logp: torch.Tensor
+) -> torch.Tensor:
+    """``d logp / d logits`` contracted with ``g_logp``, in the dtype of ``logits``."""
+    N.require_device(logits, "logits")
+    device = logits.device
+    V = logits.shape[-1]
+    x = logits.detach()
+    orig_dtype = x.dtype
+    if x.dtype not in N._DTYPE_CODE:
+        x = x.float()
+    x2 = x.reshape(-1, V)
+    if not x2.is_contiguous():
+        x2 = x2.contiguous()
+    rows = x2.shape[0]
+    idc = ids.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
+    lsec = lse.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    gc = g_logp.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    grad = torch.empty_like(x2)
+    if rows and V:
+        with torch.cuda.device(device):
+            rc = N.lib().unirl_token_logp_bwd(
+                N.ptr(x2), N.dtype_code(x2.dtype), rows, V, V, N.ptr(idc), float(temperature), N.ptr(lsec),
+                N.ptr(gc), N.ptr(grad), V, N.current_stream(device),
+            )
+        N.check(rc, "unirl_token_logp_bwd")
+    grad = grad.reshape(logits.shape)
+    return grad if grad.dtype == orig_dtype else grad.to(orig_dtype)
+
+
+def _ratio_params(
+    kind: int,
+    agg_mode: str,
+    clip_low: float,
+    clip_high: float,
+    drpo_epsilon: float,
+    mu_weighted: bool,
+    horizon: float,
+    adv_per_token: bool,
+) -> N.RatioLossParams:
+    if agg_mode not in N.AGG_MODES:
+        raise ValueError(f"loss_agg_mode must be one of {sorted(N.AGG_MODES)}; got {agg_mode!r}")
+    return N.RatioLossParams(
+        kind=kind,
+        agg_mode=N.AGG_MODES[agg_mode],
+        clip_low=float(clip_low),
+        clip_high=float(clip_high),
+        drpo_epsilon=float(drpo_epsilon),
+        mu_weighted=int(bool(mu_weighted)),
+        horizon=float(horizon),
+        adv_per_token=int(bool(adv_per_token)),
+    )
+
+
+class RatioLossPlan:
+    """Validated, device-ready arguments of one ratio-loss call (forward and backward share them)."""
+
+    def __init__(
+        self,
+        new_logp: torch.Tensor,
+        old_logp: torch.Tensor,
+        advantages: torch.Tensor,
+        *,
+        kind: int,
+        lengths: Optional[torch.Tensor] = None,
+        cu_seqlens: Optional[torch.Tensor] = None,
+        loss_mask: Optional[torch.Tensor] = None,
+        agg_mode: str = "token-mean",
+        clip_low: float = 0.2,
+        clip_high: Optional[float] = None,
+        drpo_epsilon: float = 12.5,
+        mu_weighted: bool = True,
+        horizon: float = 8192,
+    ) -> None:
+        N.require_device(new_logp, "new_logp")
+        if new_logp.shape != old_logp.shape:
+            raise ValueError(f"new_logp {tuple(new_logp.shape)} != old_logp {tuple(old_logp.shape)}")
+        device = new_logp.device
+        self.device = device
+        self.shape = tuple(new_logp.shape)
+        self.nw = new_logp.detach().to(torch.float32).contiguous()
+        self.od = old_logp.detach().to(device=device, dtype=torch.float32).contiguous()
+        self.n_tok = self.nw.numel()
+        adv = advantages.detach().to(device=device, dtype=torch.float32).contiguous()
+        self.seq = None
+        self.n_seq = 0
+        self.seq_stride = 0
+        if lengths is not None and cu_seqlens is not None:
+            raise ValueError("pass lengths (padded layout) or cu_seqlens (packed layout), not both")
+        if lengths is not None:
+            if new_logp.dim() != 2:
+                raise ValueError("the padded layout needs [n_seq, max_len] log-probs")
+            self.n_seq, self.seq_stride = self.shape
+            self.seq = lengths.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
+            if self.seq.numel() != self.n_seq:
+                raise ValueError(f"lengths has {self.seq.numel()} entries for {self.n_seq} sequences")
+        elif cu_seqlens is not None:
+            self.seq = cu_seqlens.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
+            self.n_seq = self.seq.numel() - 1
+            if self.n_seq < 0:
+                raise ValueError("cu_seqlens needs n_seq + 1 entries")
+        if adv.shape == self.nw.shape or (adv.numel() == self.n_tok and self.seq is None):
+            adv_per_token = True
+        elif self.seq is not None and adv.numel() == self.n_seq:
+            adv_per_token = False
+        else:
+            raise ValueError(
+                f"advantages {tuple(advantages.shape)} match neither the tokens {self.shape} "
+                f"nor the {self.n_seq} sequences"
+            )
+        self.adv = adv
+        self.mask = None
+        if loss_mask is not None:
+            if loss_mask.numel() != self.n_tok:
+                raise ValueError(f"loss_mask {tuple(loss_mask.shape)} does not match tokens {self.shape}")
+            self.mask = loss_mask.detach().to(device=device, dtype=torch.float32).contiguous()
+        self.params = _ratio_params(
+            kind, agg_mode, clip_low, clip_low if clip_high is None else clip_high, drpo_epsilon, mu_weighted,
+            horizon, adv_per_token,
+        )
+
+    def forward(self, want_elem: bool) -> Tuple[Optional[torch.Tensor], torch.Tensor]:
+        """Launch the forward kernel: ``(loss_per_elem or None, metrics [16] f32)``."""
+        device = self.device
+        metrics = torch.empty(N.M_COUNT, dtype=torch.float32, device=device)
+        elem = torch.empty(self.shape, dtype=torch.float32, device=device) if want_elem else None
+        if self.n_tok == 0:
+            metrics.fill_(float("nan"))
+            metrics[N.M_NUM_TOKENS] = 0.0
+            return elem, metrics
+        ws, ws_bytes = N.workspace(device)
+        with torch.cuda.device(device):
+            rc = N.lib().unirl_ratio_loss_fwd(
+                N.ptr(self.nw), N.ptr(self.od), N.ptr(self.adv), N.ptr(self.seq), N.ptr(self.mask), self.n_seq,
+                self.seq_stride, self.n_tok, ctypes.byref(self.params), N.ptr(elem), N.ptr(metrics), N.ptr(ws),
+                ws_bytes, N.current_stream(device),
+            )
+        N.check(rc, "unirl_ratio_loss_fwd")
+        return elem, metrics
+
+    def backward(
+        self,
+        *,
+        g_scale: Optional[torch.Tensor],
+        g_elem: Optional[torch.Tensor],
+        aggregate: bool,
+        n_valid: Optional[torch.Tensor],
+    ) -> torch.Tensor:
+        """Launch the backward kernel: gradient w.r.t. ``new_logp`` (f32, same shape)."""
+        device = self.device
+        grad = torch.empty(self.shape, dtype=torch.float32, device=device)
+        if self.n_tok == 0:
+            return grad
+        gs = None if g_scale is None else g_scale.detach().to(device=device, dtype=torch.float32).reshape(-1)[:1].contiguous()
+        ge = None if g_elem is None else g_elem.detach().to(device=device, dtype=torch.float32).contiguous()
+        nv = None if n_valid is None else n_valid.detach().reshape(-1)[:1].contiguous()
+        with torch.cuda.device(device):
+            rc = N.lib().unirl_ratio_loss_bwd(
+                N.ptr(self.nw), N.ptr(self.od), N.ptr(self.adv), N.ptr(self.seq), N.ptr(self.mask), self.n_seq,
+                self.seq_stride, self.n_tok, ctypes.byref(self.params), N.ptr(gs), N.ptr(ge),
+                int(bool(aggregate)), N.ptr(nv), N.ptr(grad), N.current_stream(device),
+            )
+        N.check(rc, "unirl_ratio_loss_bwd")
+        return grad
+
+
+def group_advantages(
+    rewards: torch.Tensor,
+    n_groups: int,
+    *,
+    normalize: bool = True,
+    eps: float = 1e-8,
+    scope: str = "group",
+    use_global_std: bool = False,
+) -> torch.Tensor:
+    """Advantages of ``n_groups`` contiguous equal-size groups of ``rewards [n]`` (f32 ``[n]``)."""
+    N.require_device(rewards, "rewards")
+    if scope not in ("group", "global"):
+        raise ValueError(f"scope must be 'group' or 'global'; got {scope!r}")
+    r = rewards.detach().to(torch.float32).reshape(-1).contiguous()
+    n = r.numel()
+    out = torch.empty(n, dtype=torch.float32, device=r.device)
+    if n == 0:
+        return out
+    if n_groups <= 0 or n % n_groups != 0:
+        raise ValueError(f"non-uniform group sizes (n={n}, n_groups={n_groups})")
+    with torch.cuda.device(r.device):
+        rc = N.lib().unirl_group_advantages(
+            N.ptr(r), n_groups, n // n_groups, int(bool(normalize)), float(eps), int(scope == "global"),
+            int(bool(use_global_std)), N.ptr(out), N.current_stream(r.device),
+        )
+    N.check(rc, "unirl_group_advantages")
+    return out
+
+
+def gather_steps(tensor: torch.Tensor, positions: Sequence[int]) -> torch.Tensor:
+    """``tensor[:, positions]`` for a ``[B, S, ...]`` tensor, as one gather kernel."""
+    N.require_device(tensor, "tensor")
+    if tensor.dim() < 2:
+        raise ValueError(f"need a [B, S, ...] tensor; got {tuple(tensor.shape)}")
+    t = tensor if tensor.is_contiguous() else tensor.contiguous()
+    B, S = t.shape[0], t.shape[1]
+    pos = [int(p) for p in positions]
+    for p in pos:
+        if p < -S or p >= S:
+            raise IndexError(f"index {p} is out of bounds for dimension 1 with size {S}")
+    pos = [p % S for p in pos] if S else pos
+    out = torch.empty((B, len(pos)) + tuple(t.shape[2:]), dtype=t.dtype, device=t.device)
+    inner_bytes = (t.numel() // (B * S)) * t.element_size() if B * S else 0
+    if out.numel() == 0:
+        return out
+    pos_t = torch.tensor(pos, dtype=torch.int64, device=t.device)
+    with torch.cuda.device(t.device):
+        rc = N.lib().unirl_gather_steps(
+            N.ptr(t), B, S, inner_bytes, N.ptr(pos_t), len(pos), N.ptr(out), N.current_stream(t.device)
+        )
+    N.check(rc, "unirl_gather_steps")
+    return out
+
+
+METRIC_SLOTS: Dict[str, int] = {
+    "loss": N.M_LOSS,
+    "ratio_mean": N.M_RATIO_MEAN,
+    "ratio_std": N.M_RATIO_STD,
+    "ratio_min": N.M_RATIO_MIN,
+    "ratio_max": N.M_RATIO_MAX,
+    "clip_fraction": N.M_CLIP_FRACTION,
+    "clipfrac_hi": N.M_CLIPFRAC_HI,
+    "clipfrac_lo": N.M_CLIPFRAC_LO,
+    "approx_kl": N.M_APPROX_KL,
+    "penalty_mean": N.M_PENALTY_MEAN,
+    "absdiff_mean": N.M_ABSDIFF_MEAN,
+    "absdiff_max": N.M_ABSDIFF_MAX,
+    "num_tokens": N.M_NUM_TOKENS,
+}
