@@ -140,6 +140,18 @@ int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, const float*
                            uint8_t* mask_out, void* workspace, size_t workspace_bytes,
                            void* stream);
 
+/* The [B,S'] part of _flowdppo_kl_adv_loss (flowdppo.py:86-137) given the row
+ * KLs from unirl_gaussian_kl_mask: ratio, the KL / advantage-sign masks,
+ * loss_elem = where(keep, -A*ratio, 0) and the logged metrics.  All arrays are
+ * f32 [n].  metrics [16] f32: 0 ratio_mean, 1 ratio_std, 2 ratio_min,
+ * 3 ratio_max, 4 approx_kl, 5 kl_new_old_mean, 6 kl_new_old_max,
+ * 7 kl_mask_fraction, 8 pos_rm_fraction, 9 neg_rm_fraction, 10 masked_fraction,
+ * 11 unmasked_fraction, 12 mean(loss_elem).  d loss_elem / d new_logp equals
+ * loss_elem itself, so no separate backward entry point exists. */
+int unirl_flowdppo_loss(const float* new_logp, const float* old_logp, const float* advantages,
+                        const float* kl, int64_t n, float threshold, float* loss_elem,
+                        float* metrics, void* stream);
+
 /* Element-wise form of the same quantity (flowdppo.py:51), f32 output [R,D]. */
 int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, const float* sigma,
                            int64_t n_sigma, int64_t R, int64_t D, float* out, void* stream);
@@ -245,6 +257,12 @@ int unirl_ratio_loss_bwd(const float* new_logp, const float* old_logp, const flo
                                                  of the forward; token-mean only */,
                          float* grad_new, void* stream);
 
+/* out[t] = vals[r] for every token t of sequence r (packed layout, cu_seqlens
+ * int64 [n_seq+1]): GRPO._expand_advantages_to_tokens
+ * (unirl/algorithms/grpo.py:187-198) as one kernel. */
+int unirl_expand_per_seq(const float* vals, const int64_t* cu_seqlens, int64_t n_seq,
+                         int64_t n_tok, float* out, void* stream);
+
 /* ------------------------------------------------------------------------
  * Group-normalised advantages.  Replaces RolloutTrack.compute_advantages
  * (unirl/types/rollout_resp.py:277-333) for n = n_groups * branch rewards in
@@ -257,6 +275,19 @@ int unirl_ratio_loss_bwd(const float* new_logp, const float* old_logp, const flo
 int unirl_group_advantages(const float* rewards, int64_t n_groups, int64_t branch, int normalize,
                            float eps, int scope_global, int use_global_std, float* adv_out,
                            void* stream);
+
+/* Grouped normalisation over arbitrary index lists, normalize_grouped
+ * (unirl/algorithms/normalizers.py:8-59).  `members` int64 concatenates the
+ * groups' sample indices (each in [0,n), validated by the caller), `offsets`
+ * int64 [n_groups+1] delimits them.  out must be zero-filled by the caller:
+ * samples in no group keep 0.  Statistics: mean and unbiased std (+ eps) of
+ * the group, of its trimmed core when trim_ratio > 0 (k = int(len*ratio)
+ * members dropped from each end, only if len > 2 and 0 < 2k < len), or one
+ * batch-wide unbiased std + eps when use_global_std != 0. */
+int unirl_normalize_grouped(const float* rewards, int64_t n, const int64_t* members,
+                            const int64_t* offsets, int64_t n_groups, float eps, float trim_ratio,
+                            int use_global_std, int has_clip, float clip_max, float* out,
+                            void* stream);
 
 /* ------------------------------------------------------------------------
  * out[b, j, :] = src[b, positions[j], :] -- the copy behind gather_sde_field

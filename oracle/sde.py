@@ -7,6 +7,14 @@ Eager-torch CPU restatement of unirl/sde/kernels.py:
   dance  step / log-prob        :319-333 / :297-301
   cps    step / log-prob        :270-279 / :253
 The only deviation: sampling noise is an argument instead of being drawn inside.
+
+``ieee_sqrt=True`` evaluates the square roots of the scalar coefficients with
+numpy (hardware sqrt, correctly rounded on every CPU) instead of ``torch.sqrt``,
+whose CPU path goes through a vendor math library that returns a 1-ulp-different
+fp32 root on some hosts (seen: sqrt(0x3c47ce40) = 0x3de22a0a, the correctly
+rounded value, on one CPU and 0x3de22a09 on another).  Every other operation in
+the chain is an IEEE add / sub / mul / div, so with this switch the element-wise
+outputs are reproducible bit for bit across machines.
 """
 
 from __future__ import annotations
@@ -14,9 +22,16 @@ from __future__ import annotations
 import math
 from typing import Optional, Tuple
 
+import numpy as np
 import torch
 
 KINDS = ("flow", "dance", "cps")
+
+
+def _sqrt(t: torch.Tensor, ieee: bool) -> torch.Tensor:
+    if ieee and t.dtype == torch.float32 and not t.requires_grad:
+        return torch.from_numpy(np.sqrt(t.detach().contiguous().numpy()))
+    return torch.sqrt(t)
 
 
 def _broadcast_sigma(s: torch.Tensor, ndim: int) -> torch.Tensor:
@@ -38,19 +53,20 @@ def sde_step(
     prev_sample: Optional[torch.Tensor],
     noise: Optional[torch.Tensor],
     sigma_max,
+    ieee_sqrt: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """(prev_sample, prev_sample_mean, std_var) on fp32 inputs with broadcast sigmas."""
     if kind == "cps":
         std_dev_t = sigma_next * math.sin(eta * math.pi / 2)
         pred_original = sample - sigma * noise_pred
         noise_estimate = sample + noise_pred * (1 - sigma)
-        mean = pred_original * (1 - sigma_next) + noise_estimate * torch.sqrt(sigma_next**2 - std_dev_t**2)
+        mean = pred_original * (1 - sigma_next) + noise_estimate * _sqrt(sigma_next**2 - std_dev_t**2, ieee_sqrt)
         if prev_sample is None:
             prev_sample = mean + std_dev_t * noise
         return prev_sample, mean, std_dev_t
     dt = sigma_next - sigma
     if kind == "flow":
-        std_dev_t = torch.sqrt(sigma / (1 - torch.where(sigma == 1, sigma_max, sigma))) * eta
+        std_dev_t = _sqrt(sigma / (1 - torch.where(sigma == 1, sigma_max, sigma)), ieee_sqrt) * eta
     elif kind == "dance":
         std_dev_t = eta
     else:
@@ -59,15 +75,18 @@ def sde_step(
         1 + std_dev_t**2 * (1 - sigma) / (2 * sigma)
     ) * dt
     if prev_sample is None:
-        prev_sample = mean + std_dev_t * torch.sqrt(-dt) * noise
-    std_var = std_dev_t * torch.sqrt(-dt)
+        prev_sample = mean + std_dev_t * _sqrt(-dt, ieee_sqrt) * noise
+    std_var = std_dev_t * _sqrt(-dt, ieee_sqrt)
     return prev_sample, mean, std_var
 
 
 def elem_log_prob(kind: str, prev_sample: torch.Tensor, mean: torch.Tensor, std_var) -> torch.Tensor:
+    # the sample is detached: gradients reach the log-prob through the mean only
     if kind == "cps":
-        return -((prev_sample - mean) ** 2)
-    return -((prev_sample - mean) ** 2) / (2 * std_var**2) - torch.log(std_var) - 0.5 * math.log(2 * math.pi)
+        return -((prev_sample.detach() - mean) ** 2)
+    return (
+        -((prev_sample.detach() - mean) ** 2) / (2 * std_var**2) - torch.log(std_var) - 0.5 * math.log(2 * math.pi)
+    )
 
 
 def sde_denoise(
@@ -81,6 +100,7 @@ def sde_denoise(
     prev_sample: Optional[torch.Tensor] = None,
     noise: Optional[torch.Tensor] = None,
     sigma_max=0.99,
+    ieee_sqrt: bool = False,
 ) -> Tuple[torch.Tensor, Optional[torch.Tensor], torch.Tensor]:
     """Full denoise: returns (prev_sample fp32, log_prob [B] or None, prev_sample_mean fp32)."""
     input_dtype = sample.dtype
@@ -92,7 +112,9 @@ def sde_denoise(
         noise = torch.zeros_like(sample)
     sigma = _broadcast_sigma(sigma, sample.dim())
     sigma_next = _broadcast_sigma(sigma_next, sample.dim())
-    prev, mean, std_var = sde_step(kind, noise_pred, sample, sigma, sigma_next, eta, prev_sample, noise, sigma_max)
+    prev, mean, std_var = sde_step(
+        kind, noise_pred, sample, sigma, sigma_next, eta, prev_sample, noise, sigma_max, ieee_sqrt
+    )
     if eta < 1e-7:
         return prev, None, mean
     prev = prev.to(dtype=input_dtype).float()
@@ -109,6 +131,7 @@ def sde_rollout(
     sigmas: torch.Tensor,
     etas,
     sigma_max=None,
+    ieee_sqrt: bool = False,
 ):
     """Chain of denoise calls as in the stage loop (unirl/models/sd3/diffusion.py:364-390):
     sigma_max = sigmas[1]; the latent is cast back to the trajectory dtype (= x0.dtype)
@@ -122,7 +145,8 @@ def sde_rollout(
     cols, traj = [], []
     for k in range(S):
         prev, lp, _ = sde_denoise(
-            kind, velocities[k], x, sigmas[k], sigmas[k + 1], eta=etas[k], noise=noises[k], sigma_max=sigma_max
+            kind, velocities[k], x, sigmas[k], sigmas[k + 1], eta=etas[k], noise=noises[k], sigma_max=sigma_max,
+            ieee_sqrt=ieee_sqrt,
         )
         if lp is None:
             lp = torch.full((x0.shape[0],), float("nan"))

@@ -1,0 +1,221 @@
+"""CPU-only checks: the C-ABI library loads and exports what include/unirl_hip.h declares,
+argument errors come back as statuses (no kernel is launched), and the host-side logic of the
+Python layer (validation, index math, error types, loud failure without a device)."""
+
+import ctypes
+import math
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from oracle import flowdppo as ofd
+from oracle import schedule as osch
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "unirl_hip.h"
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(unirl_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound(built_lib):
+    from unirl_amd import _native
+
+    names = declared_symbols()
+    assert len(names) >= 18
+    handle = ctypes.CDLL(str(built_lib))
+    for name in names:
+        assert hasattr(handle, name), f"{name} declared in the header but not exported"
+    assert sorted(_native.EXPORTED_SYMBOLS) == names, "ctypes signature table and header disagree"
+
+
+def test_version_status_strings_and_workspace(built_lib):
+    from unirl_amd import _native as N
+
+    L = N.lib()
+    assert L.unirl_abi_version() == 1
+    assert L.unirl_workspace_bytes() >= 64 * 1024
+    assert L.unirl_status_string(0) == b"ok"
+    for code in range(-6, 0):
+        assert L.unirl_status_string(code) not in (b"ok", b"unknown status")
+    assert L.unirl_status_string(-99) == b"unknown status"
+
+
+def test_argument_errors_return_statuses_without_launching(built_lib):
+    from unirl_amd import _native as N
+
+    L = N.lib()
+    # bad dtype / kind / shape / null pointers: rejected before any HIP call
+    assert L.unirl_token_logp_entropy(None, 7, 1, 10, 10, None, 1.0, None, None, None, None) == -3
+    assert L.unirl_token_logp_entropy(None, N.BF16, 1, 0, 0, None, 1.0, None, None, None, None) == -2
+    assert L.unirl_token_logp_entropy(None, N.BF16, 1, 10, 10, None, 1.0, None, None, None, None) == -1
+    assert L.unirl_token_logp_entropy(None, N.BF16, 0, 10, 10, None, 1.0, None, None, None, None) == 0
+    args = [None, N.F32, None, N.F32, None, None, None, None, 0, None, 0.99, 0.7, N.SDE_FLOW, 2, 16, None, None,
+            None, 0, None, 0, None]
+    assert L.unirl_sde_step_logp(*args) == -1
+    args[12] = 9
+    assert L.unirl_sde_step_logp(*args) == -3
+    args[12] = N.SDE_FLOW
+    args[14] = 0
+    assert L.unirl_sde_step_logp(*args) == -2
+    assert L.unirl_gaussian_kl_mask(None, None, N.BF16, None, 1, 2, 8, 0.01, None, None, None, 0, None) == -1
+    assert L.unirl_gaussian_kl_mask(None, None, N.BF16, None, 0, 2, 8, 0.01, None, None, None, 0, None) == -2
+    assert L.unirl_workspace_init(None, 0, None) == -1
+    p = N.RatioLossParams(kind=5)
+    assert L.unirl_ratio_loss_fwd(None, None, None, None, None, 1, 0, 4, ctypes.byref(p), None, None, None, 0,
+                                  None) == -3
+    assert L.unirl_group_advantages(None, 2, 2, 1, 1e-8, 0, 0, None, None) == -1
+    assert L.unirl_group_advantages(None, 0, 2, 1, 1e-8, 0, 0, None, None) == 0
+    # misaligned pointer
+    assert L.unirl_token_logp_entropy(ctypes.c_void_p(0x1001), N.BF16, 1, 10, 10, ctypes.c_void_p(0x1000), 1.0,
+                                      ctypes.c_void_p(0x2000), None, None, None) == -5
+
+
+def test_status_to_exception_mapping(built_lib):
+    from unirl_amd import _native as N
+
+    N.check(0, "x")
+    with pytest.raises(ValueError):
+        N.check(-2, "x")
+    with pytest.raises(N.UnirlHipError):
+        N.check(1, "x")
+    with pytest.raises(TypeError):
+        N.dtype_code(torch.float64)
+
+
+def test_missing_library_fails_loudly(monkeypatch, tmp_path):
+    from unirl_amd import _native as N
+
+    monkeypatch.setattr(N, "_lib", None)
+    monkeypatch.setattr(N, "LIB_PATH", tmp_path / "libunirl_hip.so")
+    with pytest.raises(RuntimeError, match="no CPU or eager-torch path"):
+        N.lib()
+
+
+def test_cpu_tensors_are_refused_not_emulated(built_lib):
+    from unirl_amd import models, ops, sde
+    from unirl_amd.algorithms import _drpo_loss, _grpo_clip_loss
+
+    x = torch.randn(2, 4, 4)
+    s = torch.tensor(0.5)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        sde.FlowSDEStrategy().denoise(x, x, s, s * 0.9, eta=0.7)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        models.token_logp(torch.randn(3, 10), torch.zeros(3, dtype=torch.int64))
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _grpo_clip_loss(new_logp=x, old_logp=x, advantages=x, clip_range=0.2)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        _drpo_loss(new_logp=x, old_logp=x, advantages=x, epsilon=5.0)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        ops.gaussian_kl_mask(x, x, s, 0.01, reduce_from_dim=1)
+
+
+def test_sigma_schedule_matches_oracle():
+    from unirl_amd.sde import calculate_dynamic_mu, get_sigma_schedule
+
+    for T, shift in ((28, 3.0), (10, 3.0), (14, 5.0), (12, 1.0)):
+        assert torch.equal(get_sigma_schedule(T, shift), osch.sigma_schedule(T, shift))
+    assert get_sigma_schedule(4).shape == (5,)
+    # linear in the sequence length between (256, 0.5) and (4096, 1.15)
+    assert abs(calculate_dynamic_mu(256) - 0.5) < 1e-12 and abs(calculate_dynamic_mu(4096) - 1.15) < 1e-12
+    assert abs(calculate_dynamic_mu(2176) - 0.825) < 1e-12
+
+
+def test_strategy_surface():
+    from unirl_amd import sde
+
+    assert sde.FlowSDEStrategy.canonical_name == "flow"
+    assert sde.DanceSDEStrategy.canonical_name == "dance"
+    assert sde.CPSSDEStrategy.canonical_name == "cps"
+    for cls in sde.STRATEGIES.values():
+        obj = cls(config=None)
+        assert isinstance(obj, sde.SDEStrategy) and isinstance(obj, sde.StepStrategy)
+        obj.reset()
+        obj.init_schedule(torch.ones(3))
+    with pytest.raises(TypeError):
+        sde.FlowSDEStrategy(None)  # config is keyword-only
+
+
+def test_clip_schedule():
+    from unirl_amd.algorithms import _resolve_clip_range_from_schedule as f
+
+    assert f(0.2, "constant", 0.7) == 0.2
+    assert abs(f(0.2, "linear_decay", 0.5) - 0.15) < 1e-12
+    assert abs(f(0.2, "cosine_decay", 0.5) - 0.1) < 1e-12
+    assert abs(f(0.2, "cosine_decay", 1.0)) < 1e-12 and f(0.2, "anything-else", 1.0) == 0.2
+
+
+def test_gather_sde_field_host_path_and_errors():
+    from unirl_amd.algorithms import gather_sde_field
+
+    g = torch.Generator().manual_seed(0)
+    t = torch.randn(3, 5, 2, 4, generator=g)
+    idx = torch.tensor([7, 2, 9, 0, 4])
+    for target in ([2, 9], [0, 4, 7], [9], [4, 4], []):
+        got = gather_sde_field(t, idx, target, field_name="sde_means")
+        if target:
+            assert torch.equal(got, ofd.gather_by_lookup(t, idx, target))
+            assert torch.equal(got, ofd.gather_sde_field(t, idx, target))
+        else:
+            assert got.shape == (3, 0, 2, 4)
+    with pytest.raises(ValueError, match=r"target steps \[3\] not in sde_indices"):
+        gather_sde_field(t, idx, [2, 3], field_name="sde_logp")
+    with pytest.raises(ValueError, match="is None"):
+        gather_sde_field(None, idx, [2])
+    with pytest.raises(ValueError, match="is None"):
+        gather_sde_field(t, None, [2])
+
+
+def test_compute_advantages_validation_needs_no_device():
+    from unirl_amd.types import RolloutTrack, compute_advantages
+
+    r = torch.tensor([1.0, 0.0, 1.0, 0.0, 1.0, 0.0])
+    with pytest.raises(ValueError, match="not in group-by-parent contiguous order"):
+        compute_advantages(r, ["a", "b", "a", "b", "a", "b"])
+    with pytest.raises(ValueError, match="non-uniform group sizes"):
+        compute_advantages(r[:5], ["a", "a", "a", "b", "b"])
+    assert compute_advantages(r, None).tolist() == [0.0] * 6  # root track: zeros, no kernel
+    assert compute_advantages(r[:0], []).shape == (0,)
+    with pytest.raises(ValueError, match="no rewards"):
+        RolloutTrack(sample_ids=["a"], parent_ids=["p"]).compute_advantages()
+    empty = RolloutTrack(sample_ids=[], parent_ids=[], rewards=torch.zeros(0))
+    assert empty.compute_advantages() is empty
+
+
+def test_expand_advantages_validation():
+    from unirl_amd.algorithms import GRPO
+
+    with pytest.raises(ValueError, match="advantages batch=3 != lengths=2"):
+        GRPO._expand_advantages_to_tokens(torch.zeros(3), torch.ones(2, dtype=torch.int64), dtype=torch.float32,
+                                          device=torch.device("cpu"))
+
+
+def test_algorithm_constructors_validate():
+    from unirl_amd.algorithms import DRPO, GRPO, FlowDPPO, FlowGRPO
+
+    with pytest.raises(ValueError):
+        GRPO()
+    with pytest.raises(ValueError):
+        DRPO()
+    with pytest.raises(ValueError):
+        FlowGRPO(params=None)
+    with pytest.raises(ValueError):
+        FlowDPPO(params=None)
+
+    class P:
+        ar = object()
+        diffusion = object()
+
+    with pytest.raises(ValueError):
+        DRPO(pipeline=P(), old_logp_source="nope")
+    with pytest.raises(ValueError):
+        FlowDPPO(params=None, pipeline=P(), old_logp_source="nope")
+    g = GRPO(pipeline=P(), clip_range=0.2, clip_range_high=0.28)
+    assert g.stage is P.ar and g.sampling_temperature == 0.7 and g.supports_multi_update
+    assert FlowDPPO(params=None, pipeline=P()).recomputes_anchor()
+    assert not FlowGRPO(params=None, pipeline=P()).recomputes_anchor()
+    assert FlowGRPO(params=None, pipeline=P(), old_logp_source="replay").recomputes_anchor()

@@ -81,6 +81,14 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p,
          c_size_t, c_void_p],
     ),
+    "unirl_flowdppo_loss": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_float, c_void_p, c_void_p, c_void_p],
+    ),
+    "unirl_expand_per_seq": (
+        c_int,
+        [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p],
+    ),
     "unirl_gaussian_kl_elem": (
         c_int,
         [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p],
@@ -107,6 +115,11 @@ _SIGNATURES = {
     "unirl_group_advantages": (
         c_int,
         [c_void_p, c_int64, c_int64, c_int, c_float, c_int, c_int, c_void_p, c_void_p],
+    ),
+    "unirl_normalize_grouped": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_float, c_float, c_int, c_int, c_float, c_void_p,
+         c_void_p],
     ),
     "unirl_gather_steps": (
         c_int,

@@ -1,0 +1,154 @@
+"""Shared loss helpers and the stage-algorithm contract.
+
+Keeps the call signatures of ``unirl/algorithms/base.py``:
+``gather_sde_field`` (:46-80), ``rollout_replay_logp_absdiff`` (:83-103),
+``_resolve_clip_range_from_schedule`` (:106-112), ``_grpo_clip_loss`` (:115-157),
+``AlgorithmStepResult`` (:160-171) and the ``StageAlgorithm`` hooks (:182-298).
+The element-wise chain and its eight metric reductions are one kernel launch
+(``unirl_ratio_loss_fwd``); autograd gets a one-kernel backward.
+"""
+
+from __future__ import annotations
+
+import math
+from abc import ABC, abstractmethod
+from dataclasses import dataclass
+from typing import Any, Dict, List, Mapping, Optional, Tuple, Type
+
+import torch
+
+from .. import _native as N
+from .. import ops
+from ._fused import ABSDIFF_METRICS, GRPO_METRICS, elem_loss, metric_tensors
+
+
+def typed_conditions(conditions: Mapping[str, Any], conditions_cls: Optional[Type[Any]]) -> Any:
+    """The stage's typed conditions container, or the mapping itself when no class is given."""
+    return conditions if conditions_cls is None else conditions_cls.from_dict(dict(conditions))
+
+
+def gather_sde_field(
+    tensor: Optional[torch.Tensor],
+    sde_indices: Optional[torch.Tensor],
+    target_steps: List[int],
+    *,
+    field_name: str = "field",
+) -> torch.Tensor:
+    """``tensor[:, slots]`` where ``slots`` are the positions of ``target_steps`` in ``sde_indices``.
+
+    ``sde_indices`` need not be sorted.  A device tensor is gathered by one copy kernel;
+    a host tensor is indexed where its bytes are (the caller uploads only the gathered
+    slices, as the reference does).
+    """
+    if tensor is None or sde_indices is None:
+        raise ValueError(
+            f"gather_sde_field: {field_name} or sde_indices is None "
+            f"(ensure prepare_segment ran before compute_loss_and_backward)."
+        )
+    recorded = [int(i) for i in sde_indices.tolist()]
+    slot_of: Dict[int, int] = {}
+    for slot, step in enumerate(recorded):
+        slot_of.setdefault(step, slot)
+    missing = [int(t) for t in target_steps if int(t) not in slot_of]
+    if missing:
+        raise ValueError(
+            f"gather_sde_field({field_name}): target steps {missing} not in sde_indices={sorted(recorded)}"
+        )
+    positions = [slot_of[int(t)] for t in target_steps]
+    if tensor.is_cuda:
+        return ops.gather_steps(tensor, positions)
+    return tensor[:, positions]
+
+
+def rollout_replay_logp_absdiff(new_logp: torch.Tensor, old_logp: torch.Tensor) -> Dict[str, float]:
+    """``mean|new-old|`` and ``max|new-old|`` over all tokens, as python floats (one sync)."""
+    with torch.no_grad():
+        flat_new = new_logp.detach().reshape(-1)
+        # advantages only feed the loss; reuse new_logp as a same-shape stand-in
+        plan = ops.RatioLossPlan(flat_new, old_logp.detach().reshape(-1), flat_new, kind=N.LOSS_GRPO)
+        _, metrics = plan.forward(want_elem=False)
+        mean_v, max_v = metrics[N.M_ABSDIFF_MEAN : N.M_ABSDIFF_MAX + 1].tolist()
+    return {"rollout_replay_logp_absdiff_mean": float(mean_v), "rollout_replay_logp_absdiff_max": float(max_v)}
+
+
+def _resolve_clip_range_from_schedule(clip_range: float, schedule: str, progress: float) -> float:
+    if schedule == "linear_decay":
+        return clip_range * (1.0 - 0.5 * float(progress))
+    if schedule == "cosine_decay":
+        return clip_range * (0.5 * (1.0 + math.cos(math.pi * float(progress))))
+    return clip_range
+
+
+def _grpo_clip_loss(
+    *,
+    new_logp: torch.Tensor,
+    old_logp: torch.Tensor,
+    advantages: torch.Tensor,
+    clip_range: float,
+    clip_range_high: Optional[float] = None,
+) -> Tuple[torch.Tensor, Dict[str, torch.Tensor]]:
+    """PPO clipped objective per element plus the ratio metrics.
+
+    ``clip_range`` is the lower epsilon, ``clip_range_high`` the upper one (``None`` =
+    symmetric).  Returns ``(loss_per_elem, metrics)``; ``loss_per_elem`` is differentiable
+    w.r.t. ``new_logp`` and the metrics are detached 0-dim tensors.
+    """
+    adv = advantages.detach()
+    if adv.shape != new_logp.shape:
+        adv = adv.expand(new_logp.shape)
+    plan = ops.RatioLossPlan(
+        new_logp, old_logp, adv, kind=N.LOSS_GRPO, clip_low=clip_range, clip_high=clip_range_high
+    )
+    elem, metrics = elem_loss(new_logp, plan)
+    return elem, metric_tensors(metrics, GRPO_METRICS)
+
+
+@dataclass(frozen=True)
+class AlgorithmStepResult:
+    """One micro-step: scalar loss, logged metrics, step / token count, whether backward ran."""
+
+    loss: float
+    metrics: Mapping[str, Any]
+    num_steps_or_tokens: int
+    has_backward: bool
+
+
+class BaseAlgorithmConfig(ABC):
+    """Marker base of the per-stage algorithm config dataclasses."""
+
+
+class StageAlgorithm(ABC):
+    """``(conditions, segment, advantages) -> loss``; holds the stage whose ``replay`` it calls."""
+
+    requires_ema_rollout: bool = False
+    supports_multi_update: bool = False
+    anchor_fields: Tuple[str, ...] = ()
+
+    def recomputes_anchor(self) -> bool:
+        return False
+
+    def prepare_segment(self, *, conditions: Mapping[str, Any], segment: Any) -> None:
+        return None
+
+    @abstractmethod
+    def compute_loss_and_backward(
+        self,
+        *,
+        conditions: Mapping[str, Any],
+        segment: Any,
+        advantages: torch.Tensor,
+        training_progress: float,
+        loss_scale: float,
+    ) -> AlgorithmStepResult:
+        ...
+
+
+__all__ = [
+    "ABSDIFF_METRICS",
+    "AlgorithmStepResult",
+    "BaseAlgorithmConfig",
+    "StageAlgorithm",
+    "gather_sde_field",
+    "rollout_replay_logp_absdiff",
+    "typed_conditions",
+]

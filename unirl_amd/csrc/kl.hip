@@ -155,9 +155,110 @@ static int launch_kl_elem(const KlArgs& A, int64_t R, int vec, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
+// ---------------------------------------------------------------------------
+// KL-ADV masked loss over the [B,S'] log-probs (unirl/algorithms/flowdppo.py:86-137):
+// ratio, masks, where(keep, -A*r, 0) and the twelve logged metrics, one workgroup.
+// ---------------------------------------------------------------------------
+struct DppoArgs {
+  const float* nw;
+  const float* od;
+  const float* adv;
+  const float* kl;
+  int64_t n;
+  float threshold;
+  float* loss_elem;
+  float* metrics;
+};
+
+enum { D_SR = 0, D_SR2, D_LD2, D_KL, D_LOSS, D_NKL, D_POS, D_NEG, D_RM, D_SUMS, D_RMIN = D_SUMS, D_RMAX, D_KLMAX, D_VALS };
+
+__global__ __launch_bounds__(kKlThreads) void flowdppo_loss_kernel(DppoArgs A) {
+  __shared__ double lds[kKlThreads / kWave];
+  __shared__ float ldsf[kKlThreads / kWave];
+  double acc[D_SUMS];
+#pragma unroll
+  for (int v = 0; v < D_SUMS; ++v) acc[v] = 0.0;
+  float rmin = INFINITY, rmax = -INFINITY, klmax = -INFINITY;
+  for (int64_t i = threadIdx.x; i < A.n; i += kKlThreads) {
+    const float ld = A.nw[i] - A.od[i];
+    const float r = expf(ld);
+    const float a = A.adv[i];
+    const float kl = A.kl[i];
+    const bool low_kl = kl < A.threshold;
+    const bool pos = !low_kl && (r > 1.0f) && (a > 0.0f);
+    const bool neg = !low_kl && (r < 1.0f) && (a < 0.0f);
+    const bool rm = pos || neg;
+    const float loss = rm ? 0.0f : (-a) * r;
+    A.loss_elem[i] = loss;
+    acc[D_SR] += (double)r;
+    acc[D_SR2] += (double)r * (double)r;
+    acc[D_LD2] += (double)(0.5f * (ld * ld));
+    acc[D_KL] += (double)kl;
+    acc[D_LOSS] += (double)loss;
+    acc[D_NKL] += low_kl ? 0.0 : 1.0;
+    acc[D_POS] += pos ? 1.0 : 0.0;
+    acc[D_NEG] += neg ? 1.0 : 0.0;
+    acc[D_RM] += rm ? 1.0 : 0.0;
+    rmin = fminf(rmin, r);
+    rmax = fmaxf(rmax, r);
+    klmax = fmaxf(klmax, kl);
+  }
+  double tot[D_SUMS];
+#pragma unroll
+  for (int v = 0; v < D_SUMS; ++v) tot[v] = block_sum<double>(acc[v], lds);
+  rmin = block_min(rmin, ldsf);
+  rmax = block_max(rmax, ldsf);
+  klmax = block_max(klmax, ldsf);
+  if (threadIdx.x != 0) return;
+  const double N = (double)A.n;
+  double var = 0.0;
+  if (A.n > 1) {
+    var = (tot[D_SR2] - tot[D_SR] * tot[D_SR] / N) / (N - 1.0);
+    if (var < 0.0) var = 0.0;
+  }
+  float* M = A.metrics;
+  const float nf = (float)A.n;
+  M[0] = (float)(tot[D_SR] / N);
+  M[1] = (float)sqrt(var);
+  M[2] = rmin;
+  M[3] = rmax;
+  M[4] = (float)(tot[D_LD2] / N);
+  M[5] = (float)(tot[D_KL] / N);
+  M[6] = klmax;
+  M[7] = (float)tot[D_NKL] / nf;
+  M[8] = (float)tot[D_POS] / nf;
+  M[9] = (float)tot[D_NEG] / nf;
+  M[10] = (float)tot[D_RM] / nf;
+  M[11] = (float)(N - tot[D_RM]) / nf;
+  M[12] = (float)(tot[D_LOSS] / N);
+  M[13] = M[14] = M[15] = 0.0f;
+}
+
 }  // namespace unirl
 
 using namespace unirl;
+
+extern "C" int unirl_flowdppo_loss(const float* new_logp, const float* old_logp, const float* advantages,
+                                   const float* kl, int64_t n, float threshold, float* loss_elem, float* metrics,
+                                   void* stream) {
+  if (n < 0) return UNIRL_E_SHAPE;
+  if (!metrics) return UNIRL_E_NULL;
+  if (n > 0 && (!new_logp || !old_logp || !advantages || !kl || !loss_elem)) return UNIRL_E_NULL;
+  if (!aligned_to(new_logp, 4) || !aligned_to(old_logp, 4) || !aligned_to(advantages, 4) || !aligned_to(kl, 4) ||
+      !aligned_to(loss_elem, 4) || !aligned_to(metrics, 4))
+    return UNIRL_E_ALIGN;
+  DppoArgs A;
+  A.nw = new_logp;
+  A.od = old_logp;
+  A.adv = advantages;
+  A.kl = kl;
+  A.n = n;
+  A.threshold = threshold;
+  A.loss_elem = loss_elem;
+  A.metrics = metrics;
+  hipLaunchKernelGGL(flowdppo_loss_kernel, dim3(1), dim3(kKlThreads), 0, (hipStream_t)stream, A);
+  return (int)hipGetLastError();
+}
 
 extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, const float* sigma, int64_t n_sigma,
                                       int64_t R, int64_t D, float threshold, float* kl_out, uint8_t* mask_out,

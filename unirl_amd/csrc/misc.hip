@@ -95,6 +95,126 @@ __global__ __launch_bounds__(kGatherThreads) void gather_steps_kernel(const W* _
   for (int64_t i = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x; i < inner; i += stride) o[i] = s[i];
 }
 
+// ---------------------------------------------------------------------------
+// out[t] = vals[seq(t)] for packed tokens: the per-token expansion of per-sample
+// advantages (unirl/algorithms/grpo.py:187-198) without a host loop.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(kGatherThreads) void expand_per_seq_kernel(const float* __restrict__ vals,
+                                                                        const int64_t* __restrict__ cu, int64_t n_seq,
+                                                                        int64_t n_tok, float* __restrict__ out) {
+  const int64_t stride = (int64_t)gridDim.x * kGatherThreads;
+  int64_t end = -1;
+  float v = 0.0f;
+  for (int64_t t = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x; t < n_tok; t += stride) {
+    if (t >= end) {
+      int64_t lo = 0, hi = n_seq;  // cu[lo] <= t < cu[hi]
+      while (hi - lo > 1) {
+        const int64_t mid = (lo + hi) >> 1;
+        if (cu[mid] <= t) lo = mid; else hi = mid;
+      }
+      end = cu[lo + 1];
+      v = vals[lo];
+    }
+    out[t] = v;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Grouped normalisation over arbitrary index lists (CSR), with optional trimmed
+// statistics and clipping: unirl/algorithms/normalizers.py:32-59.  One lane per
+// group.  Trimming drops the k smallest and k largest members from the
+// statistics; membership is decided by rank (ties broken by position, i.e. a
+// stable sort), so no per-lane sort buffer is needed.
+// ---------------------------------------------------------------------------
+struct NormArgs {
+  const float* r;
+  int64_t n;
+  const int64_t* members;  // concatenated group members
+  const int64_t* offsets;  // [n_groups + 1]
+  int64_t n_groups;
+  float eps;
+  float trim_ratio;
+  int use_global_std;
+  int has_clip;
+  float clip_max;
+  float* out;
+};
+
+__global__ __launch_bounds__(kAdvThreads) void normalize_grouped_kernel(NormArgs A) {
+  __shared__ double lds[kAdvThreads / kWave];
+  float batch_std = 1.0f;
+  if (A.use_global_std) {
+    double s = 0.0;
+    for (int64_t i = threadIdx.x; i < A.n; i += kAdvThreads) s += (double)A.r[i];
+    s = block_sum<double>(s, lds);
+    const double mean = s / (double)A.n;
+    double q = 0.0;
+    for (int64_t i = threadIdx.x; i < A.n; i += kAdvThreads) {
+      const double d = (double)A.r[i] - mean;
+      q += d * d;
+    }
+    q = block_sum<double>(q, lds);
+    batch_std = (float)sqrt(q / (double)(A.n - 1)) + A.eps;
+  }
+  for (int64_t g = threadIdx.x; g < A.n_groups; g += kAdvThreads) {
+    const int64_t lo = A.offsets[g], hi = A.offsets[g + 1];
+    const int64_t m = hi - lo;
+    if (m <= 0) continue;
+    int64_t k = 0;
+    if (A.trim_ratio > 0.0f && m > 2) {
+      k = (int64_t)((double)m * (double)A.trim_ratio);  // int(len * ratio)
+      if (!(k > 0 && 2 * k < m)) k = 0;
+    }
+    // pass 1: mean over the kept ranks
+    double s = 0.0;
+    int64_t kept = 0;
+    for (int64_t a = lo; a < hi; ++a) {
+      const float va = A.r[A.members[a]];
+      bool keep = true;
+      if (k > 0) {
+        int64_t rank = 0;
+        for (int64_t b = lo; b < hi; ++b) {
+          const float vb = A.r[A.members[b]];
+          rank += (vb < va || (vb == va && b < a)) ? 1 : 0;
+        }
+        keep = (rank >= k) && (rank < m - k);
+      }
+      if (keep) {
+        s += (double)va;
+        ++kept;
+      }
+    }
+    const double mean = s / (double)kept;
+    float scale = batch_std;
+    if (!A.use_global_std) {
+      double q = 0.0;
+      for (int64_t a = lo; a < hi; ++a) {
+        const float va = A.r[A.members[a]];
+        bool keep = true;
+        if (k > 0) {
+          int64_t rank = 0;
+          for (int64_t b = lo; b < hi; ++b) {
+            const float vb = A.r[A.members[b]];
+            rank += (vb < va || (vb == va && b < a)) ? 1 : 0;
+          }
+          keep = (rank >= k) && (rank < m - k);
+        }
+        if (keep) {
+          const double d = (double)va - mean;
+          q += d * d;
+        }
+      }
+      scale = (float)sqrt(q / (double)(kept - 1)) + A.eps;  // one kept member -> NaN, as torch.std
+    }
+    const float mean_f = (float)mean;
+    for (int64_t a = lo; a < hi; ++a) {
+      float v = (A.r[A.members[a]] - mean_f) / scale;
+      if (A.has_clip) v = fminf(fmaxf(v, -A.clip_max), A.clip_max);
+      A.out[A.members[a]] = v;
+    }
+  }
+}
+
 }  // namespace unirl
 
 using namespace unirl;
@@ -172,4 +292,43 @@ extern "C" int unirl_gather_steps(const void* src, int64_t B, int64_t S, int64_t
     if (rc != 0) return rc;
   }
   return UNIRL_OK;
+}
+
+extern "C" int unirl_expand_per_seq(const float* vals, const int64_t* cu_seqlens, int64_t n_seq, int64_t n_tok,
+                                    float* out, void* stream) {
+  if (n_seq < 0 || n_tok < 0) return UNIRL_E_SHAPE;
+  if (n_tok == 0) return UNIRL_OK;
+  if (!vals || !cu_seqlens || !out) return UNIRL_E_NULL;
+  if (n_seq == 0) return UNIRL_E_SHAPE;
+  if (!aligned_to(vals, 4) || !aligned_to(cu_seqlens, 8) || !aligned_to(out, 4)) return UNIRL_E_ALIGN;
+  int64_t nb = (n_tok + kGatherThreads * 4 - 1) / (kGatherThreads * 4);
+  if (nb > 4096) nb = 4096;
+  hipLaunchKernelGGL(expand_per_seq_kernel, dim3((unsigned int)nb), dim3(kGatherThreads), 0, (hipStream_t)stream,
+                     vals, cu_seqlens, n_seq, n_tok, out);
+  return (int)hipGetLastError();
+}
+
+extern "C" int unirl_normalize_grouped(const float* rewards, int64_t n, const int64_t* members,
+                                       const int64_t* offsets, int64_t n_groups, float eps, float trim_ratio,
+                                       int use_global_std, int has_clip, float clip_max, float* out,
+                                       void* stream) {
+  if (n < 0 || n_groups < 0) return UNIRL_E_SHAPE;
+  if (n == 0 || n_groups == 0) return UNIRL_OK;
+  if (!rewards || !members || !offsets || !out) return UNIRL_E_NULL;
+  if (!aligned_to(rewards, 4) || !aligned_to(out, 4) || !aligned_to(members, 8) || !aligned_to(offsets, 8))
+    return UNIRL_E_ALIGN;
+  NormArgs A;
+  A.r = rewards;
+  A.n = n;
+  A.members = members;
+  A.offsets = offsets;
+  A.n_groups = n_groups;
+  A.eps = eps;
+  A.trim_ratio = trim_ratio;
+  A.use_global_std = use_global_std;
+  A.has_clip = has_clip;
+  A.clip_max = clip_max;
+  A.out = out;
+  hipLaunchKernelGGL(normalize_grouped_kernel, dim3(1), dim3(kAdvThreads), 0, (hipStream_t)stream, A);
+  return (int)hipGetLastError();
 }

@@ -1,0 +1,136 @@
+"""Token log-probs (and entropy) from logits, fused.
+
+Drop-in for the log-prob sites of the reference's AR stages:
+
+* replay -- ``_logp_chunk`` inside ``_replay_aware_forward``
+  (``unirl/models/qwen3/ar.py:78-99``): ``lf = lm_head(h).float() / T``,
+  ``lf[tok] - logsumexp(lf)``, chunked over the response and checkpointed;
+* sampling -- the behaviour log-prob of ``Qwen3ARStep.step``
+  (``unirl/models/qwen3/ar.py:138-175``; same arithmetic in ``qwen_vl/ar.py:334-335``
+  and ``hunyuan_image3/ar.py:509-510``).
+
+The reference materialises ``.float()`` and ``/ T`` copies of the ``[B, chunk, V]``
+logits and reads them again for the gather and the logsumexp; here the logits are
+read once in their own dtype and only ``[B, chunk]`` floats are written.  Under
+autograd the backward is one more pass that writes ``(onehot - softmax) * g / T``
+in the logits' dtype, so the chunk needs no activation checkpoint of an fp32 copy.
+"""
+
+from __future__ import annotations
+
+from typing import Any, Callable, List, Optional, Tuple
+
+import torch
+
+from .. import ops
+
+
+class _TokenLogpFn(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits: torch.Tensor, tokens: torch.Tensor, temperature: float):
+        logp, _, lse = ops.token_logp_entropy(
+            logits, tokens, temperature, want_logp=True, want_entropy=False, want_lse=True
+        )
+        ctx.save_for_backward(logits, tokens, lse)
+        ctx.temperature = temperature
+        return logp
+
+    @staticmethod
+    def backward(ctx, g_logp):
+        logits, tokens, lse = ctx.saved_tensors
+        return ops.token_logp_bwd(logits, tokens, ctx.temperature, lse, g_logp), None, None
+
+
+def token_logp(logits: torch.Tensor, tokens: torch.Tensor, temperature: float = 1.0) -> torch.Tensor:
+    """fp32 ``log_softmax(logits.float() / T)[..., tokens]`` with shape ``logits.shape[:-1]``.
+
+    ``temperature <= 0`` means 1 (greedy decoding reports the untempered log-prob).
+    Differentiable w.r.t. ``logits``.
+    """
+    T = float(temperature) if float(temperature) > 0.0 else 1.0
+    if torch.is_grad_enabled() and logits.requires_grad:
+        return _TokenLogpFn.apply(logits, tokens, T)
+    logp, _, _ = ops.token_logp_entropy(logits, tokens, T, want_logp=True, want_entropy=False)
+    return logp
+
+
+def token_logp_entropy(
+    logits: torch.Tensor, tokens: torch.Tensor, temperature: float = 1.0
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """``(log-prob of tokens, entropy of softmax(logits / T))`` per row, both fp32, one pass.
+
+    The log-prob is differentiable w.r.t. ``logits``; the entropy is returned detached.
+    """
+    T = float(temperature) if float(temperature) > 0.0 else 1.0
+    if torch.is_grad_enabled() and logits.requires_grad:
+        logp = _TokenLogpFn.apply(logits, tokens, T)
+        _, ent, _ = ops.token_logp_entropy(logits, None, T, want_logp=False, want_entropy=True)
+        return logp, ent
+    logp, ent, _ = ops.token_logp_entropy(logits, tokens, T, want_logp=True, want_entropy=True)
+    return logp, ent
+
+
+def token_entropy(logits: torch.Tensor, temperature: float = 1.0) -> torch.Tensor:
+    """Entropy of ``softmax(logits.float() / T)`` per row (fp32, detached)."""
+    T = float(temperature) if float(temperature) > 0.0 else 1.0
+    _, ent, _ = ops.token_logp_entropy(logits, None, T, want_logp=False, want_entropy=True)
+    return ent
+
+
+def chunked_replay_logp(
+    lm_head: Callable[[torch.Tensor], torch.Tensor],
+    resp_hidden: torch.Tensor,
+    response_tokens: torch.Tensor,
+    temperature: float = 1.0,
+    chunk: Optional[int] = None,
+) -> torch.Tensor:
+    """Padded ``[B, T_max]`` fp32 log-probs of ``response_tokens`` under ``lm_head(resp_hidden)``.
+
+    Same chunking rule as the reference (``chunk = max(64, 2048 // B)``), so the
+    ``[B, chunk, V]`` logits block -- the only large transient -- stays bounded; each
+    block is consumed by the fused kernel in the dtype ``lm_head`` produced.
+    """
+    bsz, t_max = int(resp_hidden.size(0)), int(response_tokens.size(1))
+    if t_max == 0:
+        return resp_hidden.new_zeros((bsz, 0), dtype=torch.float32)
+    step = int(chunk) if chunk is not None else max(64, 2048 // max(1, bsz))
+    parts: List[torch.Tensor] = []
+    for s in range(0, t_max, step):
+        logits = lm_head(resp_hidden[:, s : s + step, :])
+        parts.append(token_logp(logits, response_tokens[:, s : s + step], temperature))
+    return torch.cat(parts, dim=1)
+
+
+class ARLogprobStep:
+    """Per-token sampling step: pick the next token and report its log-prob under the
+    temperature-scaled full softmax (before top-k / top-p truncation), as
+    ``Qwen3ARStep.step`` does.  Token selection uses torch's sampling primitives; the
+    log-prob is the fused kernel."""
+
+    def __init__(self, *, temperature: float = 1.0, top_p: float = 1.0, top_k: int = 0) -> None:
+        self.temperature = float(temperature)
+        self.top_p = float(top_p)
+        self.top_k = int(top_k)
+
+    def step(self, logits: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        if logits.dim() != 2:
+            raise ValueError(f"ARLogprobStep.step: expected logits shape [B, vocab], got {tuple(logits.shape)}")
+        if self.temperature <= 0.0:
+            token_id = logits.argmax(dim=-1)
+            return token_id, token_logp(logits, token_id, 1.0)
+        scaled = logits.float() / self.temperature
+        if 0 < self.top_k < scaled.shape[-1]:
+            kth = torch.topk(scaled, self.top_k, dim=-1).values[..., -1, None]
+            scaled = scaled.masked_fill(scaled < kth, float("-inf"))
+        if self.top_p < 1.0:
+            sorted_vals, sorted_idx = torch.sort(scaled, dim=-1, descending=True)
+            cum = torch.softmax(sorted_vals, dim=-1).cumsum(dim=-1)
+            drop = torch.zeros_like(cum, dtype=torch.bool)
+            drop[..., 1:] = cum[..., :-1] > self.top_p
+            sorted_vals = sorted_vals.masked_fill(drop, float("-inf"))
+            scaled = torch.full_like(scaled, float("-inf")).scatter(-1, sorted_idx, sorted_vals)
+        token_id = torch.multinomial(torch.softmax(scaled, dim=-1), num_samples=1).squeeze(-1)
+        return token_id, token_logp(logits, token_id, self.temperature)
+
+
+__all__ = ["ARLogprobStep", "chunked_replay_logp", "token_entropy", "token_logp", "token_logp_entropy"]

@@ -299,6 +299,68 @@ def gaussian_kl_mask(
     return kl, mask
 
 
+FLOWDPPO_METRIC_SLOTS = {
+    "ratio_mean": 0,
+    "ratio_std": 1,
+    "ratio_min": 2,
+    "ratio_max": 3,
+    "approx_kl": 4,
+    "kl_new_old_mean": 5,
+    "kl_new_old_max": 6,
+    "kl_mask_fraction": 7,
+    "pos_rm_fraction": 8,
+    "neg_rm_fraction": 9,
+    "masked_fraction": 10,
+    "unmasked_fraction": 11,
+    "loss_mean": 12,
+}
+
+
+def flowdppo_loss(
+    new_logp: torch.Tensor, old_logp: torch.Tensor, advantages: torch.Tensor, kl: torch.Tensor, threshold: float
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """KL-ADV masked loss per element (same shape as ``new_logp``) and the metrics vector [16]."""
+    N.require_device(new_logp, "new_logp")
+    device = new_logp.device
+    shape = tuple(new_logp.shape)
+
+    def f32c(t, name):
+        t = t.detach().to(device=device, dtype=torch.float32)
+        if tuple(t.shape) != shape:
+            t = t.expand(shape)
+        return t.contiguous()
+
+    nw, od = f32c(new_logp, "new_logp"), f32c(old_logp, "old_logp")
+    ad, klc = f32c(advantages, "advantages"), f32c(kl, "kl")
+    elem = torch.empty(shape, dtype=torch.float32, device=device)
+    metrics = torch.empty(N.M_COUNT, dtype=torch.float32, device=device)
+    with torch.cuda.device(device):
+        rc = N.lib().unirl_flowdppo_loss(
+            N.ptr(nw), N.ptr(od), N.ptr(ad), N.ptr(klc), nw.numel(), float(threshold), N.ptr(elem),
+            N.ptr(metrics), N.current_stream(device),
+        )
+    N.check(rc, "unirl_flowdppo_loss")
+    return elem, metrics
+
+
+def expand_per_seq(values: torch.Tensor, cu_seqlens: torch.Tensor, n_tok: int) -> torch.Tensor:
+    """``out[t] = values[r]`` for the tokens of packed sequence ``r`` (f32 ``[n_tok]``)."""
+    N.require_device(values, "values")
+    device = values.device
+    v = values.detach().to(torch.float32).reshape(-1).contiguous()
+    cu = cu_seqlens.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
+    if cu.numel() != v.numel() + 1:
+        raise ValueError(f"cu_seqlens needs {v.numel() + 1} entries; got {cu.numel()}")
+    out = torch.empty(int(n_tok), dtype=torch.float32, device=device)
+    if n_tok:
+        with torch.cuda.device(device):
+            rc = N.lib().unirl_expand_per_seq(
+                N.ptr(v), N.ptr(cu), v.numel(), int(n_tok), N.ptr(out), N.current_stream(device)
+            )
+        N.check(rc, "unirl_expand_per_seq")
+    return out
+
+
 def gaussian_kl_elem(p: torch.Tensor, q: torch.Tensor, sigma: torch.Tensor, *, sigma_dim: int = 1) -> torch.Tensor:
     """Element-wise ``(p-q)^2 / (2 sigma^2)`` as f32; sigma broadcast along ``sigma_dim``."""
     if p.shape != q.shape:
@@ -567,6 +629,45 @@ def group_advantages(
             int(bool(use_global_std)), N.ptr(out), N.current_stream(r.device),
         )
     N.check(rc, "unirl_group_advantages")
+    return out
+
+
+def normalize_grouped(
+    rewards: torch.Tensor,
+    group_indices: Sequence[Sequence[int]],
+    *,
+    eps: float = 1e-8,
+    clip_max: Optional[float] = None,
+    trim_outliers_ratio: float = 0.0,
+    use_global_std: bool = False,
+) -> torch.Tensor:
+    """Grouped normalisation of ``rewards [n]`` over arbitrary index lists (f32 ``[n]``)."""
+    N.require_device(rewards, "rewards")
+    device = rewards.device
+    r = rewards.detach().to(torch.float32).reshape(-1).contiguous()
+    n = r.numel()
+    out = torch.zeros(n, dtype=torch.float32, device=device)
+    members: List[int] = []
+    offsets: List[int] = [0]
+    for g in group_indices:
+        for i in g:
+            i = int(i)
+            if i < -n or i >= n:
+                raise IndexError(f"index {i} is out of bounds for dimension 0 with size {n}")
+            members.append(i % n)
+        offsets.append(len(members))
+    n_groups = len(offsets) - 1
+    if n == 0 or n_groups == 0 or not members:
+        return out
+    mem_t = torch.tensor(members, dtype=torch.int64, device=device)
+    off_t = torch.tensor(offsets, dtype=torch.int64, device=device)
+    with torch.cuda.device(device):
+        rc = N.lib().unirl_normalize_grouped(
+            N.ptr(r), n, N.ptr(mem_t), N.ptr(off_t), n_groups, float(eps), float(trim_outliers_ratio),
+            int(bool(use_global_std)), int(clip_max is not None), float(clip_max or 0.0), N.ptr(out),
+            N.current_stream(device),
+        )
+    N.check(rc, "unirl_normalize_grouped")
     return out
 
 

@@ -1,0 +1,24 @@
+"""Flow-matching SDE transition kernels and the sigma schedule."""
+
+from .kernels import (
+    STRATEGIES,
+    CPSSDEStrategy,
+    DanceSDEStrategy,
+    FlowSDEStrategy,
+    SDEStrategy,
+    StepStrategy,
+    sde_rollout,
+)
+from .runtime import calculate_dynamic_mu, get_sigma_schedule
+
+__all__ = [
+    "CPSSDEStrategy",
+    "DanceSDEStrategy",
+    "FlowSDEStrategy",
+    "SDEStrategy",
+    "STRATEGIES",
+    "StepStrategy",
+    "calculate_dynamic_mu",
+    "get_sigma_schedule",
+    "sde_rollout",
+]

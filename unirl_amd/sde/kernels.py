@@ -1,0 +1,300 @@
+"""SDE step strategies with the reference's call contract, on fused HIP kernels.
+
+Mirrors the public surface of ``unirl/sde/kernels.py`` (``StepStrategy.denoise``
+:43-99, ``SDEStrategy`` :115-177, ``FlowSDEStrategy`` :185, ``CPSSDEStrategy``
+:239, ``DanceSDEStrategy`` :282): same class names, ``canonical_name`` values,
+constructor and method signatures, return tuples and ``None`` rules, so a recipe
+``_target_`` can point here.  Where the reference runs ~15 eager element-wise
+ops and a reduction per call, ``denoise`` here is one kernel launch
+(``unirl_sde_step_logp``) that reads each operand once and writes ``prev_sample``,
+``prev_sample_mean`` and the per-sample log-prob; under autograd a second kernel
+(``unirl_sde_step_logp_bwd``) produces the gradients w.r.t. ``noise_pred`` and
+``sample``.
+
+Additions over the reference signature (keyword-only, optional): ``noise`` lets
+the caller supply the sampling noise instead of drawing it inside the step.
+
+The DPM2 ODE solver of the reference (eval-only, no log-prob) is not part of
+this package.
+"""
+
+from __future__ import annotations
+
+import math
+from abc import ABC, abstractmethod
+from typing import Any, ClassVar, Optional, Tuple, Union
+
+import torch
+
+from .. import ops
+
+SigmaMax = Union[float, torch.Tensor]
+
+
+class _SdeStepFn(torch.autograd.Function):
+    """Differentiable fused step: gradients flow to ``noise_pred`` and ``sample`` through
+    ``prev_sample_mean``, the log-prob and (when sampling) ``prev_sample``."""
+
+    @staticmethod
+    def forward(ctx, noise_pred, sample, prev_sample, noise, sigma, sigma_next, sigma_max, eta, kind):
+        prev, logp, mean = ops.sde_step_logp(
+            noise_pred, sample, sigma, sigma_next, kind=kind, eta=eta, prev_sample=prev_sample, noise=noise,
+            sigma_max=sigma_max,
+        )
+        ctx.kind, ctx.eta = kind, eta
+        ctx.sampling = prev_sample is None
+        ctx.has_logp = logp is not None
+        ctx.sigma_max = sigma_max
+        ctx.saved = (noise_pred.detach(), sample.detach(), None if prev_sample is None else prev_sample.detach(),
+                     None if noise is None else noise.detach(), sigma.detach(), sigma_next.detach())
+        if not ctx.sampling:
+            ctx.mark_non_differentiable(prev)
+        if logp is None:
+            logp = torch.empty(0, device=sample.device)
+            ctx.mark_non_differentiable(logp)
+        return prev, logp, mean
+
+    @staticmethod
+    def backward(ctx, g_prev, g_logp, g_mean):
+        v, x, prev_sample, noise, sigma, sigma_next = ctx.saved
+        grad_v, grad_x = ops.sde_step_logp_bwd(
+            v, x, sigma, sigma_next, kind=ctx.kind, eta=ctx.eta, prev_sample=prev_sample, noise=noise,
+            sigma_max=ctx.sigma_max, g_logp=g_logp if ctx.has_logp else None, g_mean=g_mean,
+            g_prev=g_prev if ctx.sampling else None, need_grad_v=ctx.needs_input_grad[0],
+            need_grad_x=ctx.needs_input_grad[1],
+        )
+        if grad_v is not None and grad_v.dtype != v.dtype:
+            grad_v = grad_v.to(v.dtype)
+        if grad_x is not None and grad_x.dtype != x.dtype:
+            grad_x = grad_x.to(x.dtype)
+        return grad_v, grad_x, None, None, None, None, None, None, None
+
+
+class StepStrategy(ABC):
+    """Base class of all sampling step strategies."""
+
+    #: kernel family; ``None`` for strategies without a fused kernel
+    _kind: ClassVar[Optional[str]] = None
+
+    @abstractmethod
+    def step(
+        self,
+        noise_pred: torch.Tensor,
+        sample: torch.Tensor,
+        sigma: torch.Tensor,
+        sigma_next: torch.Tensor,
+        eta: float = 1.0,
+        prev_sample: Optional[torch.Tensor] = None,
+        generator: Optional[torch.Generator] = None,
+        sigma_max: SigmaMax = 0.99,
+        step_index: int = 0,
+    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """One sampling step: ``(prev_sample, prev_sample_mean, std_var)``."""
+
+    def reset(self) -> None:
+        """Stateless strategies have nothing to reset."""
+
+    def init_schedule(self, sigmas: torch.Tensor) -> None:
+        """Stateless strategies ignore the full schedule."""
+
+    def denoise(
+        self,
+        noise_pred: torch.Tensor,
+        sample: torch.Tensor,
+        sigma: torch.Tensor,
+        sigma_next: torch.Tensor,
+        *,
+        eta: float = 1.0,
+        prev_sample: Optional[torch.Tensor] = None,
+        sigma_max: SigmaMax = 0.99,
+        step_index: int = 0,
+        noise: Optional[torch.Tensor] = None,
+    ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+        """One denoising transition: ``(prev_sample, log_prob, prev_sample_mean)``, all fp32.
+
+        ``prev_sample=None`` samples (noise is drawn on the device unless given);
+        otherwise the log-prob of the stored transition is replayed.  ``log_prob``
+        is ``None`` when ``eta < 1e-7``.
+        """
+        del step_index
+        kind = self._kind
+        if kind is None:
+            raise NotImplementedError(f"{type(self).__name__} has no fused kernel")
+        if not sample.is_cuda:
+            raise RuntimeError(
+                f"{type(self).__name__}.denoise: sample lives on {sample.device}; the fused SDE kernel "
+                "runs on a HIP device only and there is no CPU fallback"
+            )
+        if prev_sample is None and noise is None and float(eta) != 0.0:
+            # the reference draws with generator=None on noise_pred's device, in fp32
+            noise = torch.randn(sample.shape, device=sample.device, dtype=torch.float32)
+        needs_grad = torch.is_grad_enabled() and (noise_pred.requires_grad or sample.requires_grad)
+        if needs_grad:
+            prev, logp, mean = _SdeStepFn.apply(
+                noise_pred, sample, prev_sample, noise, sigma, sigma_next, sigma_max, float(eta), kind
+            )
+            if eta < 1e-7:
+                logp = None
+        else:
+            prev, logp, mean = ops.sde_step_logp(
+                noise_pred, sample, sigma, sigma_next, kind=kind, eta=float(eta), prev_sample=prev_sample,
+                noise=noise, sigma_max=sigma_max,
+            )
+        if prev_sample is not None and prev_sample.dtype == torch.float32 and sample.dtype == torch.float32:
+            # the reference's .float() / .to(float32) are no-ops here: hand the caller's tensor back
+            prev = prev_sample
+        return prev, logp, mean
+
+
+class SDEStrategy(StepStrategy, ABC):
+    """Stochastic strategies: a transition mean, a noise scale and a Gaussian log-prob."""
+
+    @abstractmethod
+    def compute_log_prob(self, prev_sample: torch.Tensor, prev_sample_mean: torch.Tensor, **kwargs) -> torch.Tensor:
+        """Element-wise log-prob of ``prev_sample`` under the transition."""
+
+    def _coefficients(self, sigma, sigma_next, eta, sigma_max, ndim, device):
+        """std_var with the reference's fp32 operation order, broadcast to ``ndim`` dims."""
+        raise NotImplementedError
+
+    def step(
+        self,
+        noise_pred: torch.Tensor,
+        sample: torch.Tensor,
+        sigma: torch.Tensor,
+        sigma_next: torch.Tensor,
+        eta: float = 1.0,
+        prev_sample: Optional[torch.Tensor] = None,
+        generator: Optional[torch.Generator] = None,
+        sigma_max: SigmaMax = 0.99,
+        step_index: int = 0,
+    ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+        """``(prev_sample, prev_sample_mean, std_var)`` without the log-prob or the dtype
+        round trip; the same fused kernel with the reduction switched off."""
+        del step_index
+        noise = None
+        if prev_sample is None:
+            noise = torch.randn(sample.shape, generator=generator, device=sample.device, dtype=torch.float32)
+        prev, _, mean = ops.sde_step_logp(
+            noise_pred.float(), sample.float(), sigma, sigma_next, kind=self._kind, eta=float(eta),
+            prev_sample=None if prev_sample is None else prev_sample.float(), noise=noise, sigma_max=sigma_max,
+            want_logp=False,
+        )
+        if prev_sample is not None:
+            prev = prev_sample
+        std_var = self._coefficients(sigma, sigma_next, float(eta), sigma_max, sample.dim(), sample.device)
+        return prev, mean, std_var
+
+
+def _as_broadcast(s: torch.Tensor, ndim: int, device) -> torch.Tensor:
+    s = s.detach().to(device=device, dtype=torch.float32)
+    if s.dim() == 0:
+        s = s.unsqueeze(0)
+    while s.dim() < ndim:
+        s = s.unsqueeze(-1)
+    return s
+
+
+def _gaussian_elem_log_prob(prev_sample, prev_sample_mean, std_var):
+    return (
+        -((prev_sample.detach() - prev_sample_mean) ** 2) / (2 * std_var**2)
+        - torch.log(std_var)
+        - 0.5 * math.log(2 * math.pi)
+    )
+
+
+class FlowSDEStrategy(SDEStrategy):
+    """FlowGRPO's SDE: ``std = sqrt(sigma / (1 - sigma)) * eta`` (``sigma_max`` where sigma is 1)."""
+
+    canonical_name: ClassVar[str] = "flow"
+    _kind: ClassVar[str] = "flow"
+
+    def __init__(self, *, config: Optional[Any] = None) -> None:
+        del config
+
+    def compute_log_prob(self, prev_sample, prev_sample_mean, std_var, **kwargs) -> torch.Tensor:
+        return _gaussian_elem_log_prob(prev_sample, prev_sample_mean, std_var)
+
+    def _coefficients(self, sigma, sigma_next, eta, sigma_max, ndim, device):
+        s = _as_broadcast(sigma, ndim, device)
+        sn = _as_broadcast(sigma_next, ndim, device)
+        if isinstance(sigma_max, torch.Tensor):
+            sigma_max = sigma_max.to(device)
+        std_dev_t = torch.sqrt(s / (1 - torch.where(s == 1, sigma_max, s))) * eta
+        return std_dev_t * torch.sqrt(-(sn - s))
+
+
+class DanceSDEStrategy(SDEStrategy):
+    """DanceGRPO's SDE: constant ``std = eta``."""
+
+    canonical_name: ClassVar[str] = "dance"
+    _kind: ClassVar[str] = "dance"
+
+    def __init__(self, *, config: Optional[Any] = None) -> None:
+        del config
+
+    def compute_log_prob(self, prev_sample, prev_sample_mean, std_var, **kwargs) -> torch.Tensor:
+        return _gaussian_elem_log_prob(prev_sample, prev_sample_mean, std_var)
+
+    def _coefficients(self, sigma, sigma_next, eta, sigma_max, ndim, device):
+        s = _as_broadcast(sigma, ndim, device)
+        sn = _as_broadcast(sigma_next, ndim, device)
+        return eta * torch.sqrt(-(sn - s))
+
+
+class CPSSDEStrategy(SDEStrategy):
+    """Coefficient-preserving sampling: ``std = sigma_next * sin(eta*pi/2)``, un-normalised log-prob."""
+
+    canonical_name: ClassVar[str] = "cps"
+    _kind: ClassVar[str] = "cps"
+
+    def __init__(self, *, config: Optional[Any] = None) -> None:
+        del config
+
+    def compute_log_prob(self, prev_sample, prev_sample_mean, **kwargs) -> torch.Tensor:
+        return -((prev_sample.detach() - prev_sample_mean) ** 2)
+
+    def _coefficients(self, sigma, sigma_next, eta, sigma_max, ndim, device):
+        sn = _as_broadcast(sigma_next, ndim, device)
+        return sn * math.sin(eta * math.pi / 2)
+
+
+STRATEGIES = {cls.canonical_name: cls for cls in (FlowSDEStrategy, DanceSDEStrategy, CPSSDEStrategy)}
+
+
+def sde_rollout(
+    strategy: SDEStrategy,
+    latents: torch.Tensor,
+    velocities,
+    sigmas: torch.Tensor,
+    etas,
+    *,
+    noises=None,
+    sigma_max: Optional[SigmaMax] = None,
+    return_trajectory: bool = False,
+):
+    """``S`` chained ``denoise`` calls for known velocities in ONE launch, the latent
+    held in registers between steps (the loop at ``unirl/models/sd3/diffusion.py:366-390``
+    with ``predict_noise`` factored out).  ``etas`` is one float or one per step; steps
+    with ``eta < 1e-7`` are Euler steps and report NaN in their log-prob column.
+    Returns ``(final latent fp32, log_probs [B,S] fp32, trajectory [S,B,...] or None)``.
+    """
+    S = len(velocities)
+    if noises is None:
+        noises = [torch.randn(latents.shape, device=latents.device, dtype=torch.float32) for _ in range(S)]
+    x, logp, traj = ops.sde_rollout_logp(
+        latents, velocities, noises, sigmas, etas, kind=strategy._kind, sigma_max=sigma_max,
+        want_trajectory=return_trajectory,
+    )
+    return x, logp, traj
+
+
+__all__ = [
+    "CPSSDEStrategy",
+    "DanceSDEStrategy",
+    "FlowSDEStrategy",
+    "SDEStrategy",
+    "STRATEGIES",
+    "StepStrategy",
+    "sde_rollout",
+]
