@@ -1,0 +1,388 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused RL-math kernels on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  The headline (`value`) is the fused token log-prob + entropy
+kernel on bf16 logits [8192, 151936] -- the second configuration of BASELINE.json, the
+one large enough to be cleanly HBM-bound -- as algorithmic GB/s over exactly K timed
+steps with the inputs resident in HBM.  `roofline` prices that kernel against the
+8 TB/s HBM peak from HIP-event timing of the same launches; `shapes` carries the same
+figures for all five synthetic shapes (small ones timed as back-to-back launches inside
+a HIP graph over rotating buffer sets, so neither the launch path nor the 256 MB
+last-level cache hides the kernel time); `cpu_baseline` is the eager-torch CPU oracle of
+the headline path on a bounded row sample, timed on this host's cores.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, published peak
+L2_PLUS_MALL_BYTES = 256 * 2**20 + 32 * 2**20
+
+
+def log(msg: str) -> None:
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+# ----------------------------------------------------------------------------------------------
+# timing helpers
+# ----------------------------------------------------------------------------------------------
+def time_steps(torch, fn, steps: int, warmup: int):
+    """(wall ms per step, HIP-event ms per step) over exactly `steps` calls of fn(i)."""
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        fn(i)
+    stop.record()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    return (t1 - t0) * 1e3 / steps, start.elapsed_time(stop) / steps
+
+
+def time_in_graph(torch, fn, n_sets: int, launches: int = 64, replays: int = 7):
+    """Median per-launch microseconds of `launches` back-to-back calls captured in a HIP graph."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(n_sets):  # warm up on the capture stream (workspace, code objects)
+            fn(i)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        for i in range(launches):
+            fn(i % n_sets)
+    torch.cuda.synchronize()
+    graph.replay()
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(replays):
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        graph.replay()
+        stop.record()
+        torch.cuda.synchronize()
+        times.append(start.elapsed_time(stop) * 1e3 / launches)
+    del graph
+    return statistics.median(times)
+
+
+def time_cpu(fn, reps: int = 5, warmup: int = 2):
+    for _ in range(warmup):
+        fn()
+    out = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        out.append(time.perf_counter() - t0)
+    return statistics.median(out) * 1e3
+
+
+def wrapper_latency_us(torch, fn, reps: int = 20):
+    """End-to-end call + synchronise, microseconds (median)."""
+    out = []
+    for i in range(reps):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        fn(i)
+        torch.cuda.synchronize()
+        out.append((time.perf_counter() - t0) * 1e6)
+    return statistics.median(out)
+
+
+# ----------------------------------------------------------------------------------------------
+# the five synthetic shapes of BASELINE.json
+# ----------------------------------------------------------------------------------------------
+def n_sets_for(bytes_per_set: int) -> int:
+    """Enough rotating input sets that consecutive launches cannot be served from cache."""
+    return max(2, min(16, math.ceil(1.5 * L2_PLUS_MALL_BYTES / max(1, bytes_per_set))))
+
+
+def make_shapes(torch, dev):
+    from oracle import advantages as oadv
+    from oracle import flowdppo as ofd
+    from oracle import losses as olos
+    from oracle import schedule as osch
+    from oracle import sde as osde
+    from unirl_amd import _native as N
+    from unirl_amd import ops
+
+    sig = osch.sigma_schedule(28, 3.0)
+    sig_d = sig.to(dev)
+    shapes = []
+
+    # -- config 1: SDE step + log-prob, SD3 latents fp32 [8,16,128,128], step 10 of 28 ------------
+    g = torch.Generator().manual_seed(1001)
+    shp = (8, 16, 128, 128)
+    host1 = [torch.randn(shp, generator=g) for _ in range(3)]  # x, v, noise
+    numel = host1[0].numel()
+    bytes1 = 5 * numel * 4
+    ns = n_sets_for(bytes1)
+    sets1 = [[t.to(dev) + 0.0 * k for t in host1] for k in range(ns)]
+    s10, s11, smax = sig_d[10], sig_d[11], sig_d[1]
+
+    def run1(i):
+        x, v, n = sets1[i % ns]
+        return ops.sde_step_logp(v, x, s10, s11, kind="flow", eta=0.7, noise=n, sigma_max=smax)
+
+    shapes.append(dict(
+        name="sde_step_logp", config=1, shape="fp32 [8,16,128,128], step 10/28, shift 3, eta 0.7, sampling",
+        bytes=bytes1, elements=numel, run=run1, sets=ns,
+        cpu=lambda: osde.sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7, noise=host1[2],
+                                     sigma_max=sig[1]),
+        cpu_bytes=bytes1,
+    ))
+
+    # -- config 3: GRPO / DRPO token loss, fp32 [256, 8192], lengths U[512, 8192] -----------------
+    g = torch.Generator().manual_seed(1003)
+    old = -8 * torch.rand(256, 8192, generator=g)
+    new = old + 0.05 * torch.randn(256, 8192, generator=g)
+    lengths = torch.randint(512, 8193, (256,), generator=g)
+    rewards = (torch.rand(256, generator=g) < 0.5).float()
+    adv = oadv.compute_advantages(rewards, [i // 16 for i in range(256)])
+    n_valid = int(lengths.sum())
+    bytes3_padded = 2 * new.numel() * 4
+    bytes3_valid = 2 * n_valid * 4
+    ns3 = n_sets_for(bytes3_padded)
+    sets3 = [(new.to(dev) + 0.0 * k, old.to(dev) + 0.0 * k) for k in range(ns3)]
+    len_d, adv_d = lengths.to(dev), adv.to(dev)
+    plans = {}
+    for kind, code, kw in (("grpo", N.LOSS_GRPO, dict(clip_low=0.2, clip_high=0.28)),
+                           ("drpo", N.LOSS_DRPO, dict(drpo_epsilon=5.0))):
+        plans[kind] = [ops.RatioLossPlan(a, b, adv_d, kind=code, lengths=len_d, **kw) for a, b in sets3]
+    newp, oldp = olos.pack_padded(new, lengths), olos.pack_padded(old, lengths)
+    for kind, okw in (("grpo", dict(clip_range=0.2, clip_range_high=0.28)), ("drpo", dict(epsilon=5.0))):
+        shapes.append(dict(
+            name=f"ratio_loss_{kind}", config=3,
+            shape=f"fp32 [256,8192] padded, {n_valid} valid tokens, 16x16 groups, token-mean",
+            bytes=bytes3_valid, bytes_padded=bytes3_padded, elements=n_valid,
+            run=(lambda i, k=kind: plans[k][i % ns3].forward(False)), sets=ns3,
+            cpu=(lambda k=kind, o=okw: olos.token_loss(k, newp, oldp, adv, lengths, **o)), cpu_bytes=bytes3_valid,
+        ))
+
+    # -- config 4: Flow-DPPO KL mask, WAN bf16 [2,16,21,60,104] -----------------------------------
+    g = torch.Generator().manual_seed(1004)
+    shp4 = (2, 1, 16, 21, 60, 104)
+    base = torch.randn(shp4, generator=g)
+    old_m = (base + 0.01 * torch.randn(shp4, generator=g)).bfloat16()
+    new_m = (base + 0.01 * torch.randn(shp4, generator=g)).bfloat16()
+    step = int((sig - 0.5).abs().argmin())
+    sig_t = torch.tensor(0.7 * math.sqrt(float(sig[step] - sig[step + 1])))
+    bytes4 = 2 * old_m.numel() * 2
+    ns4 = n_sets_for(bytes4)
+    sets4 = [(new_m.to(dev).clone(), old_m.to(dev).clone()) for _ in range(ns4)]
+    sig_t_d = sig_t.to(dev)
+
+    def run4(i):
+        p, q = sets4[i % ns4]
+        return ops.gaussian_kl_mask(p, q, sig_t_d, 0.01)
+
+    shapes.append(dict(
+        name="gaussian_kl_mask", config=4, shape="bf16 [2,16,21,60,104] old/new means, threshold 0.01",
+        bytes=bytes4, elements=old_m.numel(), run=run4, sets=ns4,
+        cpu=lambda: ofd.kl_per_sample(new_m, old_m, sig_t.reshape(1, 1, 1, 1, 1, 1)) < 0.01, cpu_bytes=bytes4,
+    ))
+
+    # -- config 5: 10-step rollout, Qwen-Image packed latents fp32 [16,4096,64] -------------------
+    g = torch.Generator().manual_seed(1005)
+    shp5 = (16, 4096, 64)
+    x0 = torch.randn(shp5, generator=g)
+    vs = [torch.randn(shp5, generator=g) for _ in range(10)]
+    nz = [torch.randn(shp5, generator=g) for _ in range(10)]
+    bytes5 = 22 * x0.numel() * 4
+    x0_d, vs_d, nz_d = x0.to(dev), [t.to(dev) for t in vs], [t.to(dev) for t in nz]
+
+    def run5(i):
+        return ops.sde_rollout_logp(x0_d, vs_d, nz_d, sig_d, 0.7, kind="flow")
+
+    shapes.append(dict(
+        name="sde_rollout_logp", config=5, shape="fp32 [16,4096,64], 10 steps from step 0, eta 0.7",
+        bytes=bytes5, elements=10 * x0.numel(), run=run5, sets=1,
+        cpu=lambda: osde.sde_rollout("flow", x0, vs, nz, sig, 0.7), cpu_bytes=bytes5, cpu_reps=3,
+    ))
+    return shapes
+
+
+def make_headline(torch, dev, rows: int, vocab: int):
+    """Config 2: logits bf16 [rows, vocab] ~ N(0, 2) with 1% of the rows holding one +15 spike."""
+    g = torch.Generator(device=dev).manual_seed(1002)
+    x = torch.empty(rows, vocab, dtype=torch.bfloat16, device=dev)
+    for s in range(0, rows, 512):
+        n = min(512, rows - s)
+        x[s : s + n] = (2 * torch.randn(n, vocab, generator=g, device=dev)).bfloat16()
+    n_spike = max(1, rows // 100)
+    spiked = torch.randperm(rows, generator=g, device=dev)[:n_spike]
+    x[spiked, torch.randint(0, vocab, (n_spike,), generator=g, device=dev)] = 15.0
+    ids = torch.randint(0, vocab, (rows,), generator=g, device=dev)
+    return x, ids, spiked
+
+
+# ----------------------------------------------------------------------------------------------
+def main() -> int:
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--rows", type=int, default=8192, help="token rows of the headline workload")
+    ap.add_argument("--vocab", type=int, default=151936)
+    ap.add_argument("--cpu-rows", type=int, default=512, help="rows of the bounded CPU-baseline sample")
+    ap.add_argument("--skip-shapes", action="store_true", help="headline only")
+    ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this path runs on ONE GPU (independent per-sample work, no cross-GPU exchange); "
+              "run it with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no HIP device visible", file=sys.stderr)
+        return 1
+    from unirl_amd import _native as N
+
+    if not N.LIB_PATH.exists():
+        from unirl_amd.build import build
+
+        build(verbose=False)
+    from oracle import token_logp as otok
+    from unirl_amd import ops
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    log(f"device {torch.cuda.get_device_name(0)}, torch {torch.__version__}, host threads {torch.get_num_threads()}")
+
+    # ---------------- headline: token log-prob + entropy ----------------
+    x, ids, spiked = make_headline(torch, dev, args.rows, args.vocab)
+    alg_bytes = x.numel() * 2 + ids.numel() * 8 + 2 * args.rows * 4
+
+    def step(i):
+        return ops.token_logp_entropy(x, ids, 1.0, want_logp=True, want_entropy=True)
+
+    wall_ms, event_ms = time_steps(torch, step, args.steps, args.warmup)
+    value = alg_bytes / (wall_ms * 1e-3) / 1e9
+    achieved = alg_bytes / (event_ms * 1e-3) / 1e9
+    log(f"token_logp_entropy: {wall_ms:.4f} ms/step wall, {event_ms:.4f} ms/launch (events), "
+        f"{achieved:.1f} GB/s = {achieved / HBM_PEAK_GBPS:.1%} of peak")
+
+    # parity + CPU baseline on a bounded, spike-including row sample
+    lp, ent, _ = step(0)
+    sample = torch.cat([spiked[: min(8, spiked.numel())],
+                        torch.arange(0, args.rows, max(1, args.rows // args.cpu_rows), device=dev)])[: args.cpu_rows]
+    xs, ids_s = x[sample].cpu(), ids[sample].cpu()
+    ref_lp, ref_ent = otok.token_logp_entropy_chunked(xs, ids_s, 1.0, chunk=512)
+    parity = {
+        "rows_checked": int(sample.numel()),
+        "logp_max_rel": float(((lp[sample].cpu() - ref_lp).abs() / ref_lp.abs().clamp_min(1e-6)).max()),
+        "entropy_max_rel": float(((ent[sample].cpu() - ref_ent).abs() / ref_ent.abs().clamp_min(1e-6)).max()),
+    }
+    cpu_baseline = None
+    if not args.skip_cpu:
+        def cpu_fn():
+            for s in range(0, xs.shape[0], 512):
+                blk, idb = xs[s : s + 512], ids_s[s : s + 512]
+                otok.token_logp(blk, idb, 1.0)
+                otok.token_entropy_fp32(blk, 1.0)
+
+        cpu_ms = time_cpu(cpu_fn)
+        cpu_bytes = xs.numel() * 2 + ids_s.numel() * 8 + 2 * xs.shape[0] * 4
+        cpu_baseline = {
+            "value": round(cpu_bytes / (cpu_ms * 1e-3) / 1e9, 3), "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{xs.shape[0]} of {args.rows} rows x {args.vocab} bf16 logits, eager-torch fp32 log-prob + "
+                      f"entropy in 512-row chunks, median of 5 runs ({cpu_ms:.0f} ms each)",
+        }
+        log(f"cpu baseline: {cpu_baseline['value']} GB/s on {cpu_baseline['cores']} threads")
+
+    # ---------------- the other four shapes ----------------
+    shapes_out = [{
+        "name": "token_logp_entropy", "config": 2, "shape": f"bf16 [{args.rows},{args.vocab}] + int64 ids",
+        "algorithmic_bytes": alg_bytes, "elements": x.numel(), "kernel_us": round(event_ms * 1e3, 2),
+        "gbps": round(achieved, 1), "frac_of_peak": round(achieved / HBM_PEAK_GBPS, 4),
+        "elements_per_s": round(x.numel() / (event_ms * 1e-3), 0), "timing": "hip events over the timed steps",
+        "cpu_gbps": None if cpu_baseline is None else cpu_baseline["value"],
+    }]
+    if not args.skip_shapes:
+        del lp, ent
+        for sh in make_shapes(torch, dev):
+            try:
+                us = time_in_graph(torch, sh["run"], sh["sets"])
+                method = f"hip graph, 64 back-to-back launches over {sh['sets']} input sets"
+            except Exception as exc:  # graph capture unavailable: fall back to stream-ordered events
+                log(f"{sh['name']}: graph timing failed ({type(exc).__name__}: {exc}); using event loop")
+                _, ms = time_steps(torch, sh["run"], 200, 20)
+                us, method = ms * 1e3, "hip events over 200 stream-ordered launches (launch-bound)"
+            lat = wrapper_latency_us(torch, sh["run"])
+            gbps = sh["bytes"] / (us * 1e-6) / 1e9
+            row = {
+                "name": sh["name"], "config": sh["config"], "shape": sh["shape"], "algorithmic_bytes": sh["bytes"],
+                "elements": sh["elements"], "kernel_us": round(us, 2), "gbps": round(gbps, 1),
+                "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4),
+                "elements_per_s": round(sh["elements"] / (us * 1e-6), 0), "wrapper_latency_us": round(lat, 1),
+                "timing": method,
+            }
+            if "bytes_padded" in sh:
+                row["gbps_padded_bytes"] = round(sh["bytes_padded"] / (us * 1e-6) / 1e9, 1)
+            if not args.skip_cpu:
+                cms = time_cpu(sh["cpu"], reps=sh.get("cpu_reps", 5), warmup=1)
+                row["cpu_ms"] = round(cms, 2)
+                row["cpu_gbps"] = round(sh["cpu_bytes"] / (cms * 1e-3) / 1e9, 3)
+                row["cpu_cores"] = torch.get_num_threads()
+            log(f"{sh['name']}: {us:.2f} us/launch, {gbps:.0f} GB/s = {gbps / HBM_PEAK_GBPS:.1%} of peak, "
+                f"wrapper {lat:.0f} us")
+            shapes_out.append(row)
+
+    result = {
+        "metric": "fused-kernel HBM GB/s (token log-prob + entropy)",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"token log-prob + entropy, logits bf16 [{args.rows},{args.vocab}] ~N(0,2) with 1% spiked "
+                        f"rows, int64 target ids, T=1 (BASELINE.json configs[1])",
+            "rows": args.rows, "vocab": args.vocab,
+        },
+        "roofline": {
+            "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+            "kernel": "token_logp_entropy_kernel<bf16>", "algorithmic_bytes_per_launch": alg_bytes,
+            "launch_ms": round(event_ms, 4),
+        },
+        "cpu_baseline": cpu_baseline,
+        "parity": parity,
+        "shapes": shapes_out,
+        "device": torch.cuda.get_device_name(0),
+    }
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -16,10 +16,11 @@
  *   - `stream` is a hipStream_t passed as void*; every call only enqueues work
  *     on it and returns (asynchronous, no host synchronisation);
  *   - `workspace` is caller-owned device memory of at least
- *     unirl_workspace_bytes() bytes that was zero-filled ONCE after allocation
- *     (unirl_workspace_init does that).  Kernels leave it ready for the next
- *     call.  Two calls that may overlap in time (different streams) need
- *     different workspaces;
+ *     unirl_workspace_bytes() bytes.  A reducing entry point stores one fp64
+ *     partial per workgroup there and a small second kernel, enqueued by the
+ *     same call, adds them in a fixed order; nothing is carried from call to
+ *     call and no initialisation is required.  Two calls that may overlap in
+ *     time (different streams) need different workspaces;
  *   - the library allocates nothing, frees nothing and keeps no global state;
  *   - return value: 0 = ok, < 0 = invalid argument (UNIRL_E_*), > 0 = the
  *     hipError_t of a failed launch.  No C++ exception crosses this boundary.
@@ -58,7 +59,7 @@ const char* unirl_status_string(int status);
 
 /* Bytes of device workspace every reducing entry point expects. */
 size_t unirl_workspace_bytes(void);
-/* Zero-fill a freshly allocated workspace (a fill kernel on `stream`). */
+/* Optional: zero-fill a workspace (a fill kernel on `stream`); no entry point needs it. */
 int unirl_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 
 /* ------------------------------------------------------------------------

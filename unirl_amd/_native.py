@@ -196,10 +196,8 @@ _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
 def workspace(device: torch.device) -> Tuple[torch.Tensor, int]:
-    """Zero-initialised scratch for the reducing kernels, one per (device, stream).
-
-    The kernels leave it zeroed again, so it is allocated and cleared once.
-    """
+    """Scratch for the reducing kernels (per-workgroup partial sums), one per (device, stream):
+    calls on different streams may overlap and must not share it."""
     index = device.index if device.index is not None else torch.cuda.current_device()
     key = (index, current_stream(device))
     ws = _workspaces.get(key)

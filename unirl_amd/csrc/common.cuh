@@ -6,8 +6,9 @@
 //     roundings exactly like eager torch; fused multiply-adds are written as
 //     fmaf()/fma() where they are wanted (the reductions);
 //   * cross-lane reductions use wave shuffles, then one LDS hop across the
-//     waves of a workgroup, then (for grid-wide sums) a fixed-order pass by
-//     the last workgroup to arrive, so results do not depend on scheduling.
+//     waves of a workgroup, then (for grid-wide sums) a fixed-order pass over
+//     per-workgroup partials in a small second kernel, so results do not
+//     depend on scheduling.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -234,25 +235,20 @@ __device__ __forceinline__ float block_min(float v, float* lds) {
 }
 
 // ---------------------------------------------------------------------------
-// "Last workgroup finalises": every workgroup of a group publishes its partial
-// results, then takes a ticket; the one that draws the last ticket sees all
-// partials and reduces them in index order.  The ticket counter is left at zero
-// for the next launch, so the workspace needs zeroing only once.
-// Returns true (in every thread of the workgroup) for the last arrival.
+// Grid-wide sums are two launches: the streaming kernel stores one partial per
+// workgroup (plain stores), and a finalize kernel of a few wavefronts -- ordered
+// after it on the stream -- adds them in index order.  In-kernel alternatives
+// were measured and dropped: a device-scope release fence per workgroup writes
+// back the XCD's whole L2 (20x slower than the kernel itself), and "last
+// arrival finalises" tickets serialise at ~90 ns per same-address atomic,
+// which exceeds the ~2 us cost of the second launch beyond ~25 workgroups.
 // ---------------------------------------------------------------------------
-__device__ __forceinline__ bool arrive_and_check_last(unsigned int* counter, unsigned int expected, int* lds_flag) {
-  __threadfence();  // partials written by this workgroup are visible device-wide
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    const unsigned int ticket = atomicAdd(counter, 1u);
-    const int last = (ticket == expected - 1u);
-    if (last) *counter = 0u;  // nobody else touches it again in this launch
-    *lds_flag = last;
-  }
-  __syncthreads();
-  const bool last = (*lds_flag != 0);
-  if (last) __threadfence();  // order the reads of other workgroups' partials
-  return last;
+// Sum of `n` partials at `p`, added in a fixed order by one wavefront; valid in every lane.
+__device__ __forceinline__ double wave_ordered_sum(const double* __restrict__ p, int64_t n) {
+  const int lane = threadIdx.x & (kWave - 1);
+  double q = 0.0;
+  for (int64_t j = lane; j < n; j += kWave) q += p[j];
+  return wave_sum<double>(q);
 }
 
 }  // namespace unirl

@@ -36,7 +36,8 @@ extern "C" int unirl_workspace_init(void* workspace, size_t workspace_bytes, voi
   if (!workspace) return UNIRL_E_NULL;
   if (workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
   if (!aligned_to(workspace, 16)) return UNIRL_E_ALIGN;
-  // A fill kernel rather than a memset node, so the call is safe to capture in a graph.
+  // Nothing in the library depends on the contents; the fill only gives a fresh allocation defined
+  // values.  A fill kernel rather than a memset node, so the call is safe to capture in a graph.
   hipLaunchKernelGGL(fill_zero_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream,
                      reinterpret_cast<uint32_t*>(workspace), workspace_bytes / 4);
   return (int)hipGetLastError();

@@ -30,7 +30,6 @@ struct KlArgs {
   uint8_t* mask;
   float* elem_out;
   double* partials;
-  unsigned int* counters;
 };
 
 template <typename T>
@@ -53,7 +52,6 @@ __device__ __forceinline__ void kl_finish(const KlArgs& A, int64_t row, double q
 template <typename T, int VEC, int ITEMS>
 __global__ __launch_bounds__(kKlThreads) void gaussian_kl_kernel(KlArgs A) {
   __shared__ double lds[kKlThreads / kWave];
-  __shared__ int lds_flag;
   const int64_t row = blockIdx.y;
   const int64_t D = A.D;
   const T* __restrict__ pp = reinterpret_cast<const T*>(A.p) + row * D;
@@ -81,17 +79,20 @@ __global__ __launch_bounds__(kKlThreads) void gaussian_kl_kernel(KlArgs A) {
     }
   }
   const double part = block_sum<double>((double)acc, lds);
+  if (threadIdx.x != 0) return;
   if (gridDim.x == 1) {
-    if (threadIdx.x == 0) kl_finish(A, row, part);
-    return;
+    kl_finish(A, row, part);
+  } else {
+    A.partials[row * gridDim.x + blockIdx.x] = part;  // summed by gaussian_kl_finalize_kernel
   }
-  if (threadIdx.x == 0) A.partials[row * gridDim.x + blockIdx.x] = part;
-  if (!arrive_and_check_last(A.counters + row, gridDim.x, &lds_flag)) return;
-  double q = 0.0;
-  for (unsigned int j = threadIdx.x; j < gridDim.x; j += kKlThreads)
-    q += __builtin_nontemporal_load(A.partials + row * gridDim.x + j);
-  q = block_sum<double>(q, lds);
-  if (threadIdx.x == 0) kl_finish(A, row, q);
+}
+
+// One wavefront per row: adds the workgroup partials in index order, divides, thresholds.
+__global__ __launch_bounds__(kKlThreads) void gaussian_kl_finalize_kernel(KlArgs A, int64_t R, unsigned int nblk) {
+  const int64_t row = (int64_t)blockIdx.x * (kKlThreads / kWave) + threadIdx.x / kWave;
+  if (row >= R) return;
+  const double q = wave_ordered_sum(A.partials + row * nblk, nblk);
+  if ((threadIdx.x & (kWave - 1)) == 0) kl_finish(A, row, q);
 }
 
 template <typename T, int VEC>
@@ -275,7 +276,7 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
   const int items = (vec == 4) ? (int)tune_int("UNIRL_KL_ITEMS", 4) : 2;
   const unsigned int nblk = kl_blocks_per_row(D / vec, items, R);
   int64_t per_launch = kPartialCapacity / nblk;
-  if (per_launch > kMaxCounters) per_launch = kMaxCounters;
+  if (per_launch > 32768) per_launch = 32768;
   hipStream_t st = (hipStream_t)stream;
   for (int64_t r0 = 0; r0 < R; r0 += per_launch) {
     const int64_t nr = (R - r0 < per_launch) ? (R - r0) : per_launch;
@@ -291,7 +292,6 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
     A.mask = mask_out ? mask_out + r0 : nullptr;
     A.elem_out = nullptr;
     A.partials = ws_partials(workspace);
-    A.counters = ws_counters(workspace);
     int rc = UNIRL_E_DTYPE;
     switch (dtype) {
       case UNIRL_F32: rc = launch_kl<float>(A, nr, vec, nblk, items, st); break;
@@ -299,6 +299,13 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
       case UNIRL_F16: rc = launch_kl<f16_t>(A, nr, vec, nblk, items, st); break;
     }
     if (rc != 0) return rc;
+    if (nblk > 1) {
+      const int per_block = kKlThreads / kWave;
+      hipLaunchKernelGGL(gaussian_kl_finalize_kernel, dim3((unsigned int)((nr + per_block - 1) / per_block)),
+                         dim3(kKlThreads), 0, st, A, nr, nblk);
+      rc = (int)hipGetLastError();
+      if (rc != 0) return rc;
+    }
   }
   return UNIRL_OK;
 }
@@ -329,7 +336,6 @@ extern "C" int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, c
     A.mask = nullptr;
     A.elem_out = out + r0 * D;
     A.partials = nullptr;
-    A.counters = nullptr;
     int rc = UNIRL_E_DTYPE;
     switch (dtype) {
       case UNIRL_F32: rc = launch_kl_elem<float>(A, nr, vec, st); break;

@@ -55,7 +55,6 @@ struct RatioArgs {
   float* loss_elem;
   float* metrics;
   double* partials;
-  unsigned int* counters;
   // backward only
   const float* g_scale;
   const float* g_elem;
@@ -107,6 +106,11 @@ __device__ __forceinline__ TokVals ratio_token(float nw, float od, float A, cons
   return o;
 }
 
+// min for the ratio minimum, max for the two maxima, sum for everything else
+__device__ __forceinline__ double combine(int v, double x, double y) {
+  return (v == P_RMIN) ? fmin(x, y) : ((v == P_RMAX || v == P_AMAX) ? fmax(x, y) : x + y);
+}
+
 struct Acc {
   double sr = 0.0, sr2 = 0.0;
   float loss = 0.0f, kl = 0.0f, pen = 0.0f, ab = 0.0f;
@@ -134,8 +138,6 @@ template <int KIND, int VEC>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A) {
   constexpr int NW = kRlThreads / kWave;
   __shared__ double lds_v[NW][kRlVals];
-  __shared__ double lds_fin[kRlThreads];
-  __shared__ int lds_flag;
   const RatioConsts C = A.C;
 
   Acc acc;
@@ -232,10 +234,11 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
   double vals[kRlVals];
   vals[P_SR] = wave_sum<double>(acc.sr);
   vals[P_SR2] = wave_sum<double>(acc.sr2);
-  vals[P_LOSS] = wave_sum<double>((double)acc.loss);
-  vals[P_KL] = wave_sum<double>((double)acc.kl);
-  vals[P_PEN] = wave_sum<double>((double)acc.pen);
-  vals[P_ABS] = wave_sum<double>((double)acc.ab);
+  // 64 lanes x a handful of tokens: an fp32 shuffle tree keeps full accuracy at half the shuffles
+  vals[P_LOSS] = (double)wave_sum<float>(acc.loss);
+  vals[P_KL] = (double)wave_sum<float>(acc.kl);
+  vals[P_PEN] = (double)wave_sum<float>(acc.pen);
+  vals[P_ABS] = (double)wave_sum<float>(acc.ab);
   vals[P_CNT] = (double)wave_sum<unsigned int>(acc.cnt);
   vals[P_CHI] = (double)wave_sum<unsigned int>(acc.chi);
   vals[P_CLO] = (double)wave_sum<unsigned int>(acc.clo);
@@ -251,38 +254,32 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
     for (int v = 0; v < kRlVals; ++v) lds_v[wid][v] = vals[v];
   }
   __syncthreads();
-  const unsigned int nblk = gridDim.x * gridDim.y;
   const unsigned int blk = blockIdx.y * gridDim.x + blockIdx.x;
   if (threadIdx.x < kRlVals) {
     const int v = threadIdx.x;
     double x = lds_v[0][v];
-    for (int w = 1; w < NW; ++w) {
-      const double y = lds_v[w][v];
-      x = (v == P_RMIN) ? fmin(x, y) : ((v == P_RMAX || v == P_AMAX) ? fmax(x, y) : x + y);
-    }
-    A.partials[(int64_t)blk * kRlVals + v] = x;
+    for (int w = 1; w < NW; ++w) x = combine(v, x, lds_v[w][v]);
+    A.partials[(int64_t)blk * kRlVals + v] = x;  // reduced by ratio_loss_finalize_kernel
   }
-  if (!arrive_and_check_last(A.counters, nblk, &lds_flag)) return;
+}
 
-  // ---- last workgroup: fixed-order reduction over all workgroups ----------
+// One workgroup: fixed-order reduction of every workgroup's partial vector, then the metrics.
+__global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioArgs A, unsigned int nblk) {
+  __shared__ double lds_fin[kRlThreads];
+  const RatioConsts C = A.C;
   {
     const int v = threadIdx.x % kRlVals;
     const int j0 = threadIdx.x / kRlVals;  // 0..15
     double x = (v == P_RMIN) ? (double)INFINITY : ((v == P_RMAX || v == P_AMAX) ? -(double)INFINITY : 0.0);
-    for (unsigned int j = j0; j < nblk; j += kRlThreads / kRlVals) {
-      const double y = __builtin_nontemporal_load(A.partials + (int64_t)j * kRlVals + v);
-      x = (v == P_RMIN) ? fmin(x, y) : ((v == P_RMAX || v == P_AMAX) ? fmax(x, y) : x + y);
-    }
+    for (unsigned int j = j0; j < nblk; j += kRlThreads / kRlVals)
+      x = combine(v, x, A.partials[(int64_t)j * kRlVals + v]);
     lds_fin[threadIdx.x] = x;
   }
   __syncthreads();
   if (threadIdx.x < kRlVals) {
     const int v = threadIdx.x;
     double x = lds_fin[v];
-    for (int j = 1; j < kRlThreads / kRlVals; ++j) {
-      const double y = lds_fin[j * kRlVals + v];
-      x = (v == P_RMIN) ? fmin(x, y) : ((v == P_RMAX || v == P_AMAX) ? fmax(x, y) : x + y);
-    }
+    for (int j = 1; j < kRlThreads / kRlVals; ++j) x = combine(v, x, lds_fin[j * kRlVals + v]);
     lds_fin[v] = x;
   }
   __syncthreads();
@@ -499,7 +496,6 @@ extern "C" int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp
   A.loss_elem = loss_per_elem;
   A.metrics = metrics;
   A.partials = ws_partials(workspace);
-  A.counters = ws_counters(workspace);
   RatioShape S;
   plan(A, false, S);
   if ((int64_t)S.grid.x * S.grid.y * kRlVals > kPartialCapacity) return UNIRL_E_LIMIT;
@@ -516,6 +512,9 @@ extern "C" int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp
     else
       hipLaunchKernelGGL((ratio_loss_fwd_kernel<UNIRL_LOSS_DRPO, 1>), S.grid, block, 0, st, A);
   }
+  const int launch_rc = (int)hipGetLastError();
+  if (launch_rc != 0) return launch_rc;
+  hipLaunchKernelGGL(ratio_loss_finalize_kernel, dim3(1), block, 0, st, A, S.grid.x * S.grid.y);
   return (int)hipGetLastError();
 }
 

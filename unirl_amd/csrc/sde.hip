@@ -127,7 +127,6 @@ struct SdeStepArgs {
   float* mean_out;
   float* logp_out;
   double* partials;        // [B][gridDim.x]
-  unsigned int* counters;  // [B]
   unsigned int nblk;       // host only: grid.x
   int items;               // host only: vectors in flight per lane
 };
@@ -135,7 +134,6 @@ struct SdeStepArgs {
 template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING>
 __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
   __shared__ double lds[kSdeThreads / kWave];
-  __shared__ int lds_flag;
   using T3 = typename std::conditional<SAMPLING, float, TX>::type;
 
   const int64_t b = blockIdx.y;
@@ -191,17 +189,25 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
   if (!A.want_logp) return;  // uniform across the grid
 
   const double part = block_sum<double>((double)acc, lds);
+  if (threadIdx.x != 0) return;
   if (gridDim.x == 1) {
-    if (threadIdx.x == 0) A.logp_out[b] = sde_finish_logp(kind, c, part, (double)D, A.logp_sum);
-    return;
+    A.logp_out[b] = sde_finish_logp(kind, c, part, (double)D, A.logp_sum);
+  } else {
+    A.partials[b * gridDim.x + blockIdx.x] = part;  // summed by sde_step_finalize_kernel
   }
-  if (threadIdx.x == 0) A.partials[b * gridDim.x + blockIdx.x] = part;
-  if (!arrive_and_check_last(A.counters + b, gridDim.x, &lds_flag)) return;
-  double q = 0.0;
-  for (unsigned int j = threadIdx.x; j < gridDim.x; j += kSdeThreads)
-    q += __builtin_nontemporal_load(A.partials + b * gridDim.x + j);
-  q = block_sum<double>(q, lds);
-  if (threadIdx.x == 0) A.logp_out[b] = sde_finish_logp(kind, c, q, (double)D, A.logp_sum);
+}
+
+// One wavefront per sample: adds the workgroup partials in index order and finishes the log-prob.
+__global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepArgs A, int64_t B, unsigned int nblk) {
+  const int64_t b = (int64_t)blockIdx.x * (kSdeThreads / kWave) + threadIdx.x / kWave;
+  if (b >= B) return;
+  const double q = wave_ordered_sum(A.partials + b * nblk, nblk);
+  if ((threadIdx.x & (kWave - 1)) != 0) return;
+  const float s = A.sigma[b * A.sigma_stride];
+  const float sn = A.sigma_next[b * A.sigma_stride];
+  const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
+  const SdeCoef c = sde_coef(A.kind, s, sn, smax, A.sc);
+  A.logp_out[b] = sde_finish_logp(A.kind, c, q, (double)A.D, A.logp_sum);
 }
 
 // ---------------------------------------------------------------------------
@@ -315,7 +321,6 @@ struct SdeRolloutArgs {
   float* traj_out;
   float* logp_out;         // [B][S]
   double* partials;        // [B][S][gridDim.x]
-  unsigned int* counters;  // [B]
   unsigned int nblk;       // host only: grid.x
   int items;               // host only: vectors per lane (one pass covers a sample)
 };
@@ -324,8 +329,6 @@ template <typename TV, typename TX, int VEC, int ITEMS>
 __global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs A) {
   constexpr int NW = kSdeThreads / kWave;
   __shared__ double lds_q[UNIRL_MAX_ROLLOUT_STEPS][NW];
-  __shared__ double lds[NW];
-  __shared__ int lds_flag;
 
   const int64_t b = blockIdx.y;
   const int64_t D = A.D;
@@ -409,24 +412,25 @@ __global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs
         A.logp_out[b * S + threadIdx.x] = __uint_as_float(0x7fc00000u);
       }
     } else {
-      A.partials[((int64_t)b * S + threadIdx.x) * nblk + blockIdx.x] = q;
+      A.partials[((int64_t)b * S + threadIdx.x) * nblk + blockIdx.x] = q;  // summed by sde_rollout_finalize_kernel
     }
   }
-  if (nblk == 1) return;
-  if (!arrive_and_check_last(A.counters + b, nblk, &lds_flag)) return;
-  for (int k = 0; k < S; ++k) {
-    double q = 0.0;
-    const double* pp = A.partials + ((int64_t)b * S + k) * nblk;
-    for (unsigned int j = threadIdx.x; j < nblk; j += kSdeThreads) q += __builtin_nontemporal_load(pp + j);
-    q = block_sum<double>(q, lds);
-    if (threadIdx.x == 0) {
-      if (A.want_logp[k]) {
-        const SdeCoef c = sde_coef(kind, A.sigmas[k], A.sigmas[k + 1], smax, A.sc[k]);
-        A.logp_out[b * S + k] = sde_finish_logp(kind, c, q, (double)D, A.logp_sum);
-      } else {
-        A.logp_out[b * S + k] = __uint_as_float(0x7fc00000u);
-      }
-    }
+}
+
+// One wavefront per (sample, step).
+__global__ __launch_bounds__(kSdeThreads) void sde_rollout_finalize_kernel(SdeRolloutArgs A, int64_t B,
+                                                                           unsigned int nblk) {
+  const int64_t row = (int64_t)blockIdx.x * (kSdeThreads / kWave) + threadIdx.x / kWave;  // b * S + k
+  if (row >= B * A.S) return;
+  const double q = wave_ordered_sum(A.partials + row * nblk, nblk);
+  if ((threadIdx.x & (kWave - 1)) != 0) return;
+  const int k = (int)(row % A.S);
+  if (A.want_logp[k]) {
+    const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
+    const SdeCoef c = sde_coef(A.kind, A.sigmas[k], A.sigmas[k + 1], smax, A.sc[k]);
+    A.logp_out[row] = sde_finish_logp(A.kind, c, q, (double)A.D, A.logp_sum);
+  } else {
+    A.logp_out[row] = __uint_as_float(0x7fc00000u);
   }
 }
 
@@ -455,10 +459,10 @@ static unsigned int sde_blocks_per_sample(int64_t nvec, int items, int64_t B) {
   return (unsigned int)nblk;
 }
 
-// Samples per launch so that counters and partials fit the workspace.
+// Samples per launch so that the partials fit the workspace (and grid.y its limit).
 static int64_t sde_samples_per_launch(int64_t B, int64_t partials_per_sample) {
   int64_t nb = kPartialCapacity / (partials_per_sample > 0 ? partials_per_sample : 1);
-  if (nb > kMaxCounters) nb = kMaxCounters;
+  if (nb > 32768) nb = 32768;
   if (nb > B) nb = B;
   return nb < 1 ? 1 : nb;
 }
@@ -608,7 +612,6 @@ extern "C" int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const vo
     A.mean_out = offset_f32(mean_out, off);
     A.logp_out = offset_f32(logp_out, b0);
     A.partials = ws_partials(workspace);
-    A.counters = ws_counters(workspace);
     A.nblk = nblk;
     A.items = items;
     int rc = UNIRL_E_DTYPE;
@@ -618,6 +621,13 @@ extern "C" int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const vo
       case UNIRL_F16: rc = launch_step_x<f16_t>(A, dtype_x, nb, vec, sampling, st); break;
     }
     if (rc != 0) return rc;
+    if (want_logp && nblk > 1) {
+      const int per_block = kSdeThreads / kWave;
+      hipLaunchKernelGGL(sde_step_finalize_kernel, dim3((unsigned int)((nb + per_block - 1) / per_block)),
+                         dim3(kSdeThreads), 0, st, A, nb, nblk);
+      rc = (int)hipGetLastError();
+      if (rc != 0) return rc;
+    }
   }
   return UNIRL_OK;
 }
@@ -739,7 +749,6 @@ extern "C" int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* c
     A.traj_out = offset_f32(traj_out, off);
     A.logp_out = offset_f32(logp_out, b0 * S);
     A.partials = ws_partials(workspace);
-    A.counters = ws_counters(workspace);
     A.nblk = (unsigned int)nblk;
     A.items = items;
     int rc = UNIRL_E_DTYPE;
@@ -749,6 +758,13 @@ extern "C" int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* c
       case UNIRL_F16: rc = launch_rollout_x<f16_t>(A, dtype_x, nb, vec, st); break;
     }
     if (rc != 0) return rc;
+    if (nblk > 1) {
+      const int per_block = kSdeThreads / kWave;
+      hipLaunchKernelGGL(sde_rollout_finalize_kernel, dim3((unsigned int)((nb * S + per_block - 1) / per_block)),
+                         dim3(kSdeThreads), 0, st, A, nb, (unsigned int)nblk);
+      rc = (int)hipGetLastError();
+      if (rc != 0) return rc;
+    }
   }
   return UNIRL_OK;
 }

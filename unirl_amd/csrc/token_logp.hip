@@ -8,12 +8,26 @@
 //          reference; equals torch.distributions.Categorical(logits=lf).entropy(),
 //          which clamps -inf logits to the lowest finite value)
 //
-// One workgroup owns one row.  Every lane keeps an online (max, sum e, sum e*x)
-// triple over 16-byte vectors, rescaling only when a vector raises the running
-// maximum; lanes merge by wavefront shuffles, wavefronts through LDS.  The
-// exponent is evaluated in base 2 with the temperature folded into one
-// constant: e = 2^(-(m - x)*c), c = log2(e)/T, and the entropy sum is kept as
-// sum e*(m - x) >= 0, so a row dominated by one logit loses no digits.
+// One workgroup owns one row and streams it with non-temporal 16-byte loads.
+// Each lane keeps online sums relative to a reference r = fl(m*c) shared by its
+// wavefront, m the largest logit the wavefront has seen and c = log2(e)/T:
+//     a_i = fma(x_i, c, -r)        one FMA; exact single rounding
+//     e_i = 2^a_i                  one v_exp_f32
+//     s  += e_i ,  t += e_i * a_i  (t <= ~0: every term has the same sign)
+// One DPP max-reduction per chunk of UNROLL vectors keeps m wave-uniform, so
+// raising the reference is a uniform, rarely taken branch (about ln(#chunks)
+// times per row; per-lane maxima would make some lane take it in almost every
+// chunk); inside that branch the elements equal to the new maximum are
+// counted apart (cnt) so that sum = cnt*2^r0 + s keeps full relative accuracy
+// when one logit dominates (sum = 1 + tiny), r0 = fma(m, c, -r) being the exact
+// residual of the rounded reference.  With sum and t:
+//     logsumexp = ln2*(r + log2 sum),  H = ln sum - ln2 * t/sum,
+//     logp = ln2*a_id - ln sum.
+// Lanes of a wavefront share the reference, so their sums just add; wavefronts
+// merge through LDS; the last few operations run in fp64 on one lane.
+//
+// The fast path spends no instruction on -inf / NaN logits; a row whose sums
+// come out non-finite is simply done again with clamping (SAFE = true).
 //
 // HBM traffic: V*sizeof(T) bytes read per row + 8 bytes of id + 4..12 bytes out.
 
@@ -26,73 +40,162 @@ namespace unirl {
 
 constexpr int kTokThreads = 256;
 constexpr float kLog2e = 1.4426950408889634f;
+constexpr double kLn2 = 0.6931471805599453;
 
-struct TokState {
-  float m;    // running maximum of the raw logits seen by this lane
-  float cnt;  // how many elements equalled m when m was last raised (their e is exactly 1)
-  float s;    // sum of e over every other element, e = 2^(-(m - x) * c) = exp((x - m)/T)
-  float t;    // sum e*(m - x) (every term >= 0: no cancellation for peaked rows)
+// Reference shared by the 64 lanes of a wavefront (wave-uniform, lives in scalar registers).
+struct TokRef {
+  float m;  // largest logit the wavefront has seen (-inf: none yet)
+  float r;  // fl(m * c)
 };
-// sum exp((x-m)/T) = cnt + s.  Keeping the exact ones apart from the small terms keeps
-// ln(sum) accurate when one logit dominates (sum = 1 + tiny).
+// Per-lane sums relative to the wavefront's reference.
+struct TokAcc {
+  float cnt;  // elements equal to m, counted when m was last raised
+  float s;    // sum of 2^(x*c - r) over all other elements
+  float t;    // sum of 2^a * a over them, a = x*c - r
+};
+// A whole state (one lane's, one wavefront's or one row's).
+struct TokState {
+  float m, r, cnt, s, t;
+};
 
-// Move a state to a higher maximum M: every e scales by f = 2^(-(M-m)c), (m - x)
-// grows by (M - m), and the former maxima join the ordinary terms.
-__device__ __forceinline__ void tok_raise(TokState& a, float M, float c) {
-  if (a.m == M) return;
-  if (a.m == -INFINITY) {  // nothing accumulated yet
-    a.s = 0.0f;
-    a.t = 0.0f;
-  } else {
-    const float dm = M - a.m;
-    const float f = __builtin_amdgcn_exp2f(-(dm * c));
-    const float all = a.s + a.cnt;
-    a.t = f * fmaf(dm, all, a.t);
-    a.s = f * all;
-  }
-  a.cnt = 0.0f;
-  a.m = M;
+__device__ __forceinline__ float tok_exp2(float a) { return __builtin_amdgcn_exp2f(a); }
+
+// Maximum over the 64 lanes, returned wave-uniform.  DPP row shifts build each 16-lane row's
+// maximum in its last lane, two row broadcasts carry them to lane 63, readlane makes it scalar.
+// Full-rate VALU, no LDS traffic.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float tok_dpp_max(float v) {
+  const int moved = __builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, ROW_MASK, 0xf, false);
+  return fmaxf(v, __int_as_float(moved));
+}
+__device__ __forceinline__ float wave_max_uniform(float v) {
+  v = tok_dpp_max<0x111, 0xf>(v);  // row_shr:1
+  v = tok_dpp_max<0x112, 0xf>(v);  // row_shr:2
+  v = tok_dpp_max<0x114, 0xf>(v);  // row_shr:4
+  v = tok_dpp_max<0x118, 0xf>(v);  // row_shr:8   -> lane 15 of each row holds the row maximum
+  v = tok_dpp_max<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
+  v = tok_dpp_max<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the maximum
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 
-template <int N>
-__device__ __forceinline__ void tok_update(TokState& st, float (&x)[N], float c) {
-  float vm = x[0];
+// Re-express sums relative to a higher maximum M.  (m, r) -> (M, fl(M*c)).
+__device__ __forceinline__ void tok_raise(float& m, float& r, TokAcc& acc, float M, float c) {
+  if (m == M) return;
+  const float R = M * c;
+  if (m == -INFINITY) {
+    acc.s = 0.0f;
+    acc.t = 0.0f;
+  } else {
+    // the former maxima become ordinary terms: each is 2^r0 with a = r0
+    const float r0 = fmaf(m, c, -r);
+    const float e0 = acc.cnt * tok_exp2(r0);
+    const float s_all = acc.s + e0;
+    const float t_all = fmaf(e0, r0, acc.t);
+    const float delta = r - R;  // < 0: every a shifts by delta, every e scales by 2^delta
+    const float f = tok_exp2(delta);
+    acc.s = f * s_all;
+    acc.t = f * fmaf(delta, s_all, t_all);
+  }
+  acc.cnt = 0.0f;
+  m = M;
+  r = R;
+}
+
+// One chunk of N elements per lane.  `active` is false for lanes past the end of the row.
+template <int N, bool SAFE>
+__device__ __forceinline__ void tok_update(TokRef& ref, TokAcc& acc, const float (&x)[N], bool active, float c) {
+  float cm = x[0];
 #pragma unroll
-  for (int k = 1; k < N; ++k) vm = fmaxf(vm, x[k]);
-  if (vm > st.m) {
-    // rare: this vector holds the lane's new maximum; split its exact maxima from the rest
-    tok_raise(st, vm, c);
+  for (int k = 1; k < N; ++k) cm = fmaxf(cm, x[k]);
+  const float wm = wave_max_uniform(active ? cm : -INFINITY);
+  if (__builtin_expect(wm > ref.m, 0)) {
+    // Wave-uniform and rare (about ln(chunks) times per row): move to the new maximum, then
+    // split this chunk's exact maxima from the rest.
+    tok_raise(ref.m, ref.r, acc, wm, c);
+    if (active) {
 #pragma unroll
-    for (int k = 0; k < N; ++k) {
-      const float d = fminf(st.m - x[k], FLT_MAX);
-      if (d == 0.0f) {
-        st.cnt += 1.0f;
-      } else {
-        const float e = __builtin_amdgcn_exp2f(-(d * c));
-        st.s += e;
-        st.t = fmaf(e, d, st.t);
+      for (int k = 0; k < N; ++k) {
+        if (x[k] == ref.m) {
+          acc.cnt += 1.0f;
+        } else {
+          float a = fmaf(x[k], c, -ref.r);
+          if (SAFE) a = (a < -FLT_MAX) ? -FLT_MAX : a;
+          const float e = tok_exp2(a);
+          acc.s += e;
+          acc.t = fmaf(e, a, acc.t);
+        }
       }
     }
-    return;
-  }
-  if (st.m == -INFINITY) return;  // nothing finite seen yet: every term is 0
+  } else if (active && ref.m != -INFINITY) {
 #pragma unroll
-  for (int k = 0; k < N; ++k) {
-    const float d = fminf(st.m - x[k], FLT_MAX);  // x = -inf contributes 0 to both sums
-    const float e = __builtin_amdgcn_exp2f(-(d * c));
-    st.s += e;
-    st.t = fmaf(e, d, st.t);
+    for (int k = 0; k < N; ++k) {
+      float a = fmaf(x[k], c, -ref.r);
+      if (SAFE) a = (a < -FLT_MAX) ? -FLT_MAX : a;  // -inf logit: e = 0 and e*a = 0; NaN stays NaN
+      const float e = tok_exp2(a);
+      acc.s += e;
+      acc.t = fmaf(e, a, acc.t);
+    }
   }
 }
 
-__device__ __forceinline__ void tok_merge(TokState& a, float m2, float c2, float s2, float t2, float c) {
-  TokState b{m2, c2, s2, t2};
+__device__ __forceinline__ void tok_merge(TokState& a, TokState b, float c) {
   const float M = fmaxf(a.m, b.m);
-  tok_raise(a, M, c);
-  tok_raise(b, M, c);
-  a.cnt += b.cnt;
-  a.s += b.s;
-  a.t += b.t;
+  TokAcc aa{a.cnt, a.s, a.t}, bb{b.cnt, b.s, b.t};
+  tok_raise(a.m, a.r, aa, M, c);
+  tok_raise(b.m, b.r, bb, M, c);
+  a.cnt = aa.cnt + bb.cnt;
+  a.s = aa.s + bb.s;
+  a.t = aa.t + bb.t;
+}
+
+// 16 bytes of logits -> floats
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+
+template <typename T>
+struct Stream16;
+template <>
+struct Stream16<float> {
+  static constexpr int N = 4;
+  static __device__ __forceinline__ void unpack(u32x4 v, float* o) {
+    o[0] = __uint_as_float(v.x);
+    o[1] = __uint_as_float(v.y);
+    o[2] = __uint_as_float(v.z);
+    o[3] = __uint_as_float(v.w);
+  }
+};
+template <>
+struct Stream16<bf16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(u32x4 v, float* o) {
+    o[0] = __uint_as_float(v.x << 16);
+    o[1] = __uint_as_float(v.x & 0xffff0000u);
+    o[2] = __uint_as_float(v.y << 16);
+    o[3] = __uint_as_float(v.y & 0xffff0000u);
+    o[4] = __uint_as_float(v.z << 16);
+    o[5] = __uint_as_float(v.z & 0xffff0000u);
+    o[6] = __uint_as_float(v.w << 16);
+    o[7] = __uint_as_float(v.w & 0xffff0000u);
+  }
+};
+template <>
+struct Stream16<f16_t> {
+  static constexpr int N = 8;
+  static __device__ __forceinline__ void unpack(u32x4 v, float* o) {
+    o[0] = f16_bits_to_f32(v.x & 0xffffu);
+    o[1] = f16_bits_to_f32(v.x >> 16);
+    o[2] = f16_bits_to_f32(v.y & 0xffffu);
+    o[3] = f16_bits_to_f32(v.y >> 16);
+    o[4] = f16_bits_to_f32(v.z & 0xffffu);
+    o[5] = f16_bits_to_f32(v.z >> 16);
+    o[6] = f16_bits_to_f32(v.w & 0xffffu);
+    o[7] = f16_bits_to_f32(v.w >> 16);
+  }
+};
+
+// streaming 16-byte load (non-temporal: a row is read exactly once)
+template <typename T>
+__device__ __forceinline__ u32x4 stream_load16(const T* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
 }
 
 struct TokArgs {
@@ -106,16 +209,12 @@ struct TokArgs {
   float* lse;
 };
 
-template <typename T, int UNROLL>
-__global__ __launch_bounds__(kTokThreads) void token_logp_entropy_kernel(TokArgs A) {
-  constexpr int VEC = 16 / sizeof(T);
+// One pass over the row; returns the workgroup's merged state in thread 0.
+template <typename T, int UNROLL, bool SAFE>
+__device__ __forceinline__ TokState tok_scan_row(const T* __restrict__ p, int64_t V, float c, float (*lds)[5]) {
+  constexpr int VEC = Stream16<T>::N;
   constexpr int NW = kTokThreads / kWave;
-  __shared__ float lm[NW], lc[NW], ls[NW], lt[NW];
-
-  const int64_t row = blockIdx.x;
-  const T* __restrict__ p = reinterpret_cast<const T*>(A.logits) + row * A.row_stride;
-  const int64_t V = A.V;
-  const float c = A.c;
+  constexpr int CHUNK = UNROLL * VEC;
 
   // peel to a 16-byte boundary
   int64_t head = (int64_t)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(p) & 15u)) & 15u) / sizeof(T));
@@ -123,64 +222,111 @@ __global__ __launch_bounds__(kTokThreads) void token_logp_entropy_kernel(TokArgs
   const int64_t nvec = (V - head) / VEC;
   const int64_t tail0 = head + nvec * VEC;
 
-  TokState st{-INFINITY, 0.0f, 0.0f, 0.0f};
-  if ((int64_t)threadIdx.x < head) {
-    float x[1] = {Elem<T>::load(p + threadIdx.x)};
-    tok_update<1>(st, x, c);
+  TokRef ref{-INFINITY, -INFINITY};
+  TokAcc acc{0.0f, 0.0f, 0.0f};
+  if (head > 0) {  // workgroup-uniform
+    const bool on = (int64_t)threadIdx.x < head;
+    const float x[1] = {on ? Elem<T>::load(p + threadIdx.x) : 0.0f};
+    tok_update<1, SAFE>(ref, acc, x, on, c);
   }
-  if (tail0 + (int64_t)threadIdx.x < V) {
-    float x[1] = {Elem<T>::load(p + tail0 + threadIdx.x)};
-    tok_update<1>(st, x, c);
+  if (tail0 < V) {
+    const bool on = tail0 + (int64_t)threadIdx.x < V;
+    const float x[1] = {on ? Elem<T>::load(p + tail0 + threadIdx.x) : 0.0f};
+    tok_update<1, SAFE>(ref, acc, x, on, c);
   }
 
   const T* __restrict__ pv = p + head;
-  for (int64_t i0 = threadIdx.x; i0 < nvec; i0 += (int64_t)kTokThreads * UNROLL) {
-    float x[UNROLL][VEC];
+  const int64_t per_iter = (int64_t)kTokThreads * UNROLL;
+  const int64_t n_full = nvec / per_iter;
+  // Unguarded body: UNROLL vectors per lane, the lanes of a wavefront on consecutive 16-byte
+  // words.  The next chunk's loads are issued before the current chunk is consumed.
+  if (n_full > 0) {
+    const T* __restrict__ q = pv + (int64_t)threadIdx.x * VEC;
+    u32x4 cur[UNROLL], nxt[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int64_t i = i0 + (int64_t)u * kTokThreads;
-      if (i < nvec) Vec<T, VEC>::load(pv + i * VEC, x[u]);
-    }
+    for (int u = 0; u < UNROLL; ++u) cur[u] = stream_load16(q + (int64_t)u * kTokThreads * VEC);
+    for (int64_t it = 1; it < n_full; ++it) {  // every pass but the last prefetches unconditionally
+      q += per_iter * VEC;
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) {
-      const int64_t i = i0 + (int64_t)u * kTokThreads;
-      if (i < nvec) tok_update<VEC>(st, x[u], c);
+      for (int u = 0; u < UNROLL; ++u) nxt[u] = stream_load16(q + (int64_t)u * kTokThreads * VEC);
+      float x[CHUNK];
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) Stream16<T>::unpack(cur[u], x + u * VEC);
+      tok_update<CHUNK, SAFE>(ref, acc, x, true, c);
+#pragma unroll
+      for (int u = 0; u < UNROLL; ++u) cur[u] = nxt[u];
     }
+    float x[CHUNK];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) Stream16<T>::unpack(cur[u], x + u * VEC);
+    tok_update<CHUNK, SAFE>(ref, acc, x, true, c);
+  }
+  // remainder: fewer than UNROLL vectors per lane; trip count is workgroup-uniform
+  for (int64_t i0 = n_full * per_iter; i0 < nvec; i0 += kTokThreads) {
+    const int64_t i = i0 + threadIdx.x;
+    const bool on = i < nvec;
+    float x[VEC];
+    if (on) {
+      Stream16<T>::unpack(stream_load16(pv + i * VEC), x);
+    } else {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) x[k] = 0.0f;
+    }
+    tok_update<VEC, SAFE>(ref, acc, x, on, c);
   }
 
-  // lanes -> wavefront
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) {
-    const float m2 = __shfl_xor(st.m, o, kWave);
-    const float c2 = __shfl_xor(st.cnt, o, kWave);
-    const float s2 = __shfl_xor(st.s, o, kWave);
-    const float t2 = __shfl_xor(st.t, o, kWave);
-    tok_merge(st, m2, c2, s2, t2, c);
-  }
+  // lanes -> wavefront: the lanes share (m, r), so the sums simply add
+  TokState st{ref.m, ref.r, wave_sum<float>(acc.cnt), wave_sum<float>(acc.s), wave_sum<float>(acc.t)};
   const int lane = threadIdx.x & (kWave - 1);
   const int wid = threadIdx.x / kWave;
+  __syncthreads();  // lds may still be read from a previous scan of this row
   if (lane == 0) {
-    lm[wid] = st.m;
-    lc[wid] = st.cnt;
-    ls[wid] = st.s;
-    lt[wid] = st.t;
+    lds[wid][0] = st.m;
+    lds[wid][1] = st.r;
+    lds[wid][2] = st.cnt;
+    lds[wid][3] = st.s;
+    lds[wid][4] = st.t;
   }
   __syncthreads();
-  if (threadIdx.x != 0) return;
+  if (threadIdx.x == 0) {
 #pragma unroll
-  for (int w = 1; w < NW; ++w) tok_merge(st, lm[w], lc[w], ls[w], lt[w], c);
+    for (int w = 1; w < NW; ++w) tok_merge(st, TokState{lds[w][0], lds[w][1], lds[w][2], lds[w][3], lds[w][4]}, c);
+  }
+  return st;
+}
 
-  // with lf = x/T:  logsumexp = m/T + ln s ;  H = ln s + (t/s)/T ;  logp = -(m - x_id)/T - ln s
-  // ln(cnt + s); cnt >= 1 whenever the row holds a finite logit
-  const double ln_s = log((double)st.cnt) + log1p((double)st.s / (double)st.cnt);
-  const double sum = (double)st.cnt + (double)st.s;
-  const double inv_t = (double)A.inv_t;
-  if (A.lse) A.lse[row] = (float)((double)st.m * inv_t + ln_s);
-  if (A.ent) A.ent[row] = (float)(ln_s + ((double)st.t / sum) * inv_t);
+template <typename T, int UNROLL>
+__global__ __launch_bounds__(kTokThreads) void token_logp_entropy_kernel(TokArgs A) {
+  __shared__ float lds[kTokThreads / kWave][5];
+  __shared__ int redo;
+
+  const int64_t row = blockIdx.x;
+  const T* __restrict__ p = reinterpret_cast<const T*>(A.logits) + row * A.row_stride;
+  const int64_t V = A.V;
+  const float c = A.c;
+
+  TokState st = tok_scan_row<T, UNROLL, false>(p, V, c, lds);
+  if (threadIdx.x == 0) redo = !(fabsf(st.s) <= FLT_MAX) || !(fabsf(st.t) <= FLT_MAX);  // inf or NaN
+  __syncthreads();
+  if (redo) st = tok_scan_row<T, 1, true>(p, V, c, lds);  // -inf (or NaN) logits in this row
+  if (threadIdx.x != 0) return;
+
+  // sum = cnt*2^r0 + s relative to the reference r;  ln sum = r0 ln2 + ln cnt + log1p(s 2^-r0 / cnt)
+  const double r0 = (double)fmaf(st.m, c, -st.r);
+  const double cnt = (double)st.cnt;
+  const double e0 = cnt * exp2(r0);
+  const double sum = e0 + (double)st.s;
+  const double ln_sum = r0 * kLn2 + log(cnt) + log1p((double)st.s * exp2(-r0) / cnt);
+  const double t_all = (double)st.t + e0 * r0;
+  if (A.lse) A.lse[row] = (float)(kLn2 * (double)st.r + ln_sum);
+  if (A.ent) A.ent[row] = (float)(ln_sum - kLn2 * t_all / sum);
   if (A.logp) {
     const int64_t id = A.ids[row];
     float out = __uint_as_float(0x7fc00000u);
-    if (id >= 0 && id < V) out = (float)(-(((double)st.m - (double)Elem<T>::load(p + id)) * inv_t) - ln_s);
+    if (id >= 0 && id < V) {
+      const double a_id = (double)Elem<T>::load(p + id) * (double)c - (double)st.r;
+      out = (float)(kLn2 * a_id - ln_sum);
+    }
     A.logp[row] = out;
   }
 }
@@ -208,7 +354,7 @@ __global__ __launch_bounds__(kTokThreads) void token_logp_bwd_kernel(TokBwdArgs 
   const int64_t stride = (int64_t)gridDim.x * kTokThreads;
   for (int64_t j = (int64_t)blockIdx.x * kTokThreads + threadIdx.x; j < A.V; j += stride) {
     const float x = Elem<T>::load(p + j);
-    const float prob = __builtin_amdgcn_exp2f(fmaf(x, A.c, -lse2));
+    const float prob = tok_exp2(fmaf(x, A.c, -lse2));
     const float one = (j == id) ? 1.0f : 0.0f;
     Elem<T>::store(gp + j, gs * (one - prob));
   }

@@ -10,17 +10,13 @@
 
 namespace unirl {
 
-// Workspace layout: [ticket counters | fp64 partials].
-constexpr int64_t kMaxCounters = 16384;                // uint32 each
-constexpr int64_t kMaxPartialBlocks = 2048;            // workgroups per reduced row
-constexpr int64_t kPartialCapacity = 512 * 1024;       // doubles
-constexpr size_t kCounterBytes = (size_t)kMaxCounters * sizeof(unsigned int);
-constexpr size_t kWorkspaceBytes = kCounterBytes + (size_t)kPartialCapacity * sizeof(double);
+// Workspace: fp64 per-workgroup partials, written by a streaming kernel and read
+// by its finalize kernel.  No state survives a call.
+constexpr int64_t kMaxPartialBlocks = 2048;       // workgroups per reduced row
+constexpr int64_t kPartialCapacity = 512 * 1024;  // doubles
+constexpr size_t kWorkspaceBytes = (size_t)kPartialCapacity * sizeof(double);
 
-inline unsigned int* ws_counters(void* ws) { return reinterpret_cast<unsigned int*>(ws); }
-inline double* ws_partials(void* ws) {
-  return ws ? reinterpret_cast<double*>(reinterpret_cast<char*>(ws) + kCounterBytes) : nullptr;
-}
+inline double* ws_partials(void* ws) { return reinterpret_cast<double*>(ws); }
 
 // Launch-shape knobs for measurement sweeps; read from the environment at every
 // call (a getenv is nanoseconds next to a kernel launch).  Unset = default.
