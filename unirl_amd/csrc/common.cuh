@@ -79,9 +79,23 @@ struct Elem<f16_t> {
   static __device__ __forceinline__ float round_trip(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
 };
 
+// Streaming (non-temporal) 8/16-byte accesses for data that is touched exactly once.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ u32x4 stream_load16(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
+}
+__device__ __forceinline__ u32x2 stream_load8(const void* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p));
+}
+__device__ __forceinline__ void stream_store16(void* p, u32x4 v) {
+  __builtin_nontemporal_store(v, reinterpret_cast<u32x4*>(p));
+}
+
 // ---------------------------------------------------------------------------
 // Vector loads: N consecutive elements of T -> N floats.  N*sizeof(T) is 8 or
-// 16 bytes and `p` is aligned to that, so one lane issues one dwordx2/x4.
+// 16 bytes and `p` is aligned to that, so one lane issues one dwordx2/x4.  The
+// 8- and 16-byte forms are streaming accesses.
 // ---------------------------------------------------------------------------
 template <typename T, int N>
 struct Vec;
@@ -89,14 +103,19 @@ struct Vec;
 template <>
 struct Vec<float, 4> {
   static __device__ __forceinline__ void load(const float* p, float (&o)[4]) {
-    const float4 v = *reinterpret_cast<const float4*>(p);
-    o[0] = v.x;
-    o[1] = v.y;
-    o[2] = v.z;
-    o[3] = v.w;
+    const u32x4 v = stream_load16(p);
+    o[0] = __uint_as_float(v.x);
+    o[1] = __uint_as_float(v.y);
+    o[2] = __uint_as_float(v.z);
+    o[3] = __uint_as_float(v.w);
   }
   static __device__ __forceinline__ void store(float* p, const float (&o)[4]) {
-    *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[3]);
+    u32x4 v;
+    v.x = __float_as_uint(o[0]);
+    v.y = __float_as_uint(o[1]);
+    v.z = __float_as_uint(o[2]);
+    v.w = __float_as_uint(o[3]);
+    stream_store16(p, v);
   }
 };
 template <>
@@ -108,7 +127,7 @@ struct Vec<float, 1> {
 template <>
 struct Vec<bf16_t, 4> {
   static __device__ __forceinline__ void load(const bf16_t* p, float (&o)[4]) {
-    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    const u32x2 v = stream_load8(p);
     o[0] = __uint_as_float(v.x << 16);
     o[1] = __uint_as_float(v.x & 0xffff0000u);
     o[2] = __uint_as_float(v.y << 16);
@@ -124,7 +143,7 @@ struct Vec<bf16_t, 4> {
 template <>
 struct Vec<bf16_t, 8> {
   static __device__ __forceinline__ void load(const bf16_t* p, float (&o)[8]) {
-    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    const u32x4 v = stream_load16(p);
     o[0] = __uint_as_float(v.x << 16);
     o[1] = __uint_as_float(v.x & 0xffff0000u);
     o[2] = __uint_as_float(v.y << 16);
@@ -144,7 +163,7 @@ struct Vec<bf16_t, 1> {
 template <>
 struct Vec<f16_t, 4> {
   static __device__ __forceinline__ void load(const f16_t* p, float (&o)[4]) {
-    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    const u32x2 v = stream_load8(p);
     o[0] = f16_bits_to_f32(v.x & 0xffffu);
     o[1] = f16_bits_to_f32(v.x >> 16);
     o[2] = f16_bits_to_f32(v.y & 0xffffu);
@@ -160,7 +179,7 @@ struct Vec<f16_t, 4> {
 template <>
 struct Vec<f16_t, 8> {
   static __device__ __forceinline__ void load(const f16_t* p, float (&o)[8]) {
-    const uint4 v = *reinterpret_cast<const uint4*>(p);
+    const u32x4 v = stream_load16(p);
     o[0] = f16_bits_to_f32(v.x & 0xffffu);
     o[1] = f16_bits_to_f32(v.x >> 16);
     o[2] = f16_bits_to_f32(v.y & 0xffffu);
@@ -179,59 +198,124 @@ struct Vec<f16_t, 1> {
 
 // ---------------------------------------------------------------------------
 // Wavefront / workgroup reductions.
+//
+// Wavefront reductions run on DPP (data-parallel primitives): four row shifts
+// leave each 16-lane row's total in its last lane, two row broadcasts carry the
+// totals to lane 63, and v_readlane returns it as a wave-uniform scalar.  Full
+// rate VALU, no LDS traffic, a fixed association order.  Every lane of the
+// wavefront must be active at the call.
 // ---------------------------------------------------------------------------
-template <typename T>
-__device__ __forceinline__ T wave_sum(T v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);
-  return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, kWave));
-  return v;
-}
-__device__ __forceinline__ float wave_min(float v) {
-#pragma unroll
-  for (int o = kWave / 2; o > 0; o >>= 1) v = fminf(v, __shfl_xor(v, o, kWave));
-  return v;
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int dpp_move(int identity, int v) {
+  // lanes without a valid source lane (or outside ROW_MASK) receive `identity`
+  return __builtin_amdgcn_update_dpp(identity, v, CTRL, ROW_MASK, 0xf, false);
 }
 
-// Sum of `v` over the workgroup, valid in every thread.  `lds` holds at least
-// blockDim.x/64 elements of T and may be reused after the call returns.
+#define UNIRL_DPP_REDUCE(v, OP, MOVE)          \
+  v = OP(v, MOVE<0x111, 0xf>(v)); /* shr 1  */ \
+  v = OP(v, MOVE<0x112, 0xf>(v)); /* shr 2  */ \
+  v = OP(v, MOVE<0x114, 0xf>(v)); /* shr 4  */ \
+  v = OP(v, MOVE<0x118, 0xf>(v)); /* shr 8  */ \
+  v = OP(v, MOVE<0x142, 0xa>(v)); /* bcast15 */ \
+  v = OP(v, MOVE<0x143, 0xc>(v)); /* bcast31 */
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f32_or_zero(float v) {
+  return __int_as_float(dpp_move<CTRL, ROW_MASK>(0, __float_as_int(v)));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_f32_or_self(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, ROW_MASK, 0xf, false));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ unsigned int dpp_u32_or_zero(unsigned int v) {
+  return (unsigned int)dpp_move<CTRL, ROW_MASK>(0, (int)v);
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_f64_or_zero(double v) {
+  const long long b = __double_as_longlong(v);
+  const unsigned int lo = (unsigned int)dpp_move<CTRL, ROW_MASK>(0, (int)(unsigned int)b);
+  const unsigned int hi = (unsigned int)dpp_move<CTRL, ROW_MASK>(0, (int)(unsigned int)((unsigned long long)b >> 32));
+  return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
+__device__ __forceinline__ float op_add(float a, float b) { return a + b; }
+__device__ __forceinline__ double op_add(double a, double b) { return a + b; }
+__device__ __forceinline__ unsigned int op_add(unsigned int a, unsigned int b) { return a + b; }
+__device__ __forceinline__ float op_max(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ float op_min(float a, float b) { return fminf(a, b); }
+
+__device__ __forceinline__ float last_lane(float v) {
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), kWave - 1));
+}
+__device__ __forceinline__ unsigned int last_lane(unsigned int v) {
+  return (unsigned int)__builtin_amdgcn_readlane((int)v, kWave - 1);
+}
+__device__ __forceinline__ double last_lane(double v) {
+  const long long b = __double_as_longlong(v);
+  const unsigned int lo = (unsigned int)__builtin_amdgcn_readlane((int)(unsigned int)b, kWave - 1);
+  const unsigned int hi = (unsigned int)__builtin_amdgcn_readlane((int)(unsigned int)((unsigned long long)b >> 32), kWave - 1);
+  return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
+// Wave-uniform results.
+__device__ __forceinline__ float wave_sum(float v) {
+  UNIRL_DPP_REDUCE(v, op_add, dpp_f32_or_zero)
+  return last_lane(v);
+}
+__device__ __forceinline__ double wave_sum(double v) {
+  UNIRL_DPP_REDUCE(v, op_add, dpp_f64_or_zero)
+  return last_lane(v);
+}
+__device__ __forceinline__ unsigned int wave_sum(unsigned int v) {
+  UNIRL_DPP_REDUCE(v, op_add, dpp_u32_or_zero)
+  return last_lane(v);
+}
+__device__ __forceinline__ float wave_max(float v) {
+  UNIRL_DPP_REDUCE(v, op_max, dpp_f32_or_self)
+  return last_lane(v);
+}
+__device__ __forceinline__ float wave_min(float v) {
+  UNIRL_DPP_REDUCE(v, op_min, dpp_f32_or_self)
+  return last_lane(v);
+}
+
+// Reduction over the workgroup, valid in every thread: wavefront totals meet in LDS and are
+// combined in wavefront order.  `lds` holds at least blockDim.x/64 elements and may be
+// reused after the call returns.  Must be called by every thread of the workgroup.
 template <typename T>
 __device__ __forceinline__ T block_sum(T v, T* lds) {
-  const int lane = threadIdx.x & (kWave - 1);
   const int wid = threadIdx.x / kWave;
   const int nw = blockDim.x / kWave;
   v = wave_sum(v);
   __syncthreads();  // protect lds from a previous use
-  if (lane == 0) lds[wid] = v;
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wid] = v;
   __syncthreads();
-  T r = (lane < nw) ? lds[lane] : T(0);
-  return wave_sum(r);
+  T r = lds[0];
+  for (int w = 1; w < nw; ++w) r += lds[w];
+  return r;
 }
 __device__ __forceinline__ float block_max(float v, float* lds) {
-  const int lane = threadIdx.x & (kWave - 1);
   const int wid = threadIdx.x / kWave;
   const int nw = blockDim.x / kWave;
   v = wave_max(v);
   __syncthreads();
-  if (lane == 0) lds[wid] = v;
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wid] = v;
   __syncthreads();
-  float r = (lane < nw) ? lds[lane] : -INFINITY;
-  return wave_max(r);
+  float r = lds[0];
+  for (int w = 1; w < nw; ++w) r = fmaxf(r, lds[w]);
+  return r;
 }
 __device__ __forceinline__ float block_min(float v, float* lds) {
-  const int lane = threadIdx.x & (kWave - 1);
   const int wid = threadIdx.x / kWave;
   const int nw = blockDim.x / kWave;
   v = wave_min(v);
   __syncthreads();
-  if (lane == 0) lds[wid] = v;
+  if ((threadIdx.x & (kWave - 1)) == 0) lds[wid] = v;
   __syncthreads();
-  float r = (lane < nw) ? lds[lane] : INFINITY;
-  return wave_min(r);
+  float r = lds[0];
+  for (int w = 1; w < nw; ++w) r = fminf(r, lds[w]);
+  return r;
 }
 
 // ---------------------------------------------------------------------------
@@ -248,7 +332,7 @@ __device__ __forceinline__ double wave_ordered_sum(const double* __restrict__ p,
   const int lane = threadIdx.x & (kWave - 1);
   double q = 0.0;
   for (int64_t j = lane; j < n; j += kWave) q += p[j];
-  return wave_sum<double>(q);
+  return wave_sum(q);
 }
 
 }  // namespace unirl

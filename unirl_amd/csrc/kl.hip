@@ -118,7 +118,7 @@ __global__ __launch_bounds__(kKlThreads) void gaussian_kl_elem_kernel(KlArgs A) 
 static unsigned int kl_blocks_per_row(int64_t nvec, int items, int64_t R) {
   const int64_t per_pass = (int64_t)kKlThreads * items;
   int64_t nblk = (nvec + per_pass - 1) / per_pass;
-  const int64_t cap = tune_int("UNIRL_KL_MAX_BLOCKS", 4096);
+  const int64_t cap = tune_int("UNIRL_KL_MAX_BLOCKS", 512);
   int64_t max_per_row = cap / (R > 0 ? R : 1);
   if (max_per_row < 1) max_per_row = 1;
   if (nblk > max_per_row) nblk = max_per_row;
@@ -130,6 +130,17 @@ static unsigned int kl_blocks_per_row(int64_t nvec, int items, int64_t R) {
 template <typename T>
 static int launch_kl(const KlArgs& A, int64_t R, int vec, unsigned int nblk, int items, hipStream_t st) {
   dim3 grid(nblk, (unsigned int)R), block(kKlThreads);
+  if constexpr (sizeof(T) == 2) {
+    if (vec == 8) {  // 16-byte loads of eight 16-bit values
+      if (items >= 4)
+        hipLaunchKernelGGL((gaussian_kl_kernel<T, 8, 4>), grid, block, 0, st, A);
+      else if (items >= 2)
+        hipLaunchKernelGGL((gaussian_kl_kernel<T, 8, 2>), grid, block, 0, st, A);
+      else
+        hipLaunchKernelGGL((gaussian_kl_kernel<T, 8, 1>), grid, block, 0, st, A);
+      return (int)hipGetLastError();
+    }
+  }
   if (vec == 4) {
     if (items >= 4)
       hipLaunchKernelGGL((gaussian_kl_kernel<T, 4, 4>), grid, block, 0, st, A);
@@ -273,7 +284,8 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
   if (!aligned_to(p, sz) || !aligned_to(q, sz)) return UNIRL_E_ALIGN;
   int vec = 4;
   if (D % 4 != 0 || !aligned_to(p, 4 * sz) || !aligned_to(q, 4 * sz)) vec = 1;
-  const int items = (vec == 4) ? (int)tune_int("UNIRL_KL_ITEMS", 4) : 2;
+  if (sz == 2 && D % 8 == 0 && aligned_to(p, 16) && aligned_to(q, 16)) vec = 8;
+  const int items = (vec >= 4) ? (int)tune_int("UNIRL_KL_ITEMS", 1) : 2;
   const unsigned int nblk = kl_blocks_per_row(D / vec, items, R);
   int64_t per_launch = kPartialCapacity / nblk;
   if (per_launch > 32768) per_launch = 32768;

@@ -134,18 +134,67 @@ __device__ __forceinline__ float seq_weight(const RatioConsts& C, int64_t len) {
   return (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_MEAN) ? 1.0f / (float)len : 1.0f;
 }
 
+// Per-lane context of the sequence a token belongs to.
+struct SeqCtx {
+  float adv = 0.0f;      // advantage of the current sequence (per-sequence advantages)
+  float w = 1.0f;        // aggregation weight of its tokens
+  int64_t cur_end = -1;  // packed layout: first token index past the current sequence
+};
+
+// One loaded vector of VEC tokens starting at row-relative index t0; tokens at or past `count`
+// are padding.  Accumulates into acc and leaves the per-token loss in out[].
+template <int KIND, int VEC>
+__device__ __forceinline__ void ratio_vec_fwd(const RatioArgs& A, const RatioConsts& C, int64_t t0, int64_t count,
+                                              const float (&nw)[VEC], const float (&od)[VEC],
+                                              const float (&ad)[VEC], const float (&mk)[VEC], SeqCtx& sq,
+                                              Acc& acc, float (&out)[VEC]) {
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) {
+    const int64_t t = t0 + k;
+    out[k] = 0.0f;
+    if (t < count) {
+      if (A.layout == LAYOUT_PACKED && t >= sq.cur_end) {
+        const int64_t s = find_seq(A.seq, A.n_seq, t);
+        sq.cur_end = A.seq[s + 1];
+        sq.w = seq_weight(C, sq.cur_end - A.seq[s]);
+        if (!C.adv_per_token) sq.adv = A.adv[s];
+      }
+      const float a = C.adv_per_token ? ad[k] : sq.adv;
+      const TokVals v = ratio_token<KIND>(nw[k], od[k], a, C);
+      out[k] = v.loss;
+      float lm = v.loss;
+      if (A.mask) lm = lm * mk[k];
+      acc.sr += (double)v.r;
+      acc.sr2 = fma((double)v.r, (double)v.r, acc.sr2);
+      acc.loss += lm * sq.w;
+      acc.kl += v.kterm;
+      acc.pen += v.pen;
+      const float ad0 = fabsf(v.d0);
+      acc.ab += ad0;
+      acc.rmin = fminf(acc.rmin, v.r);
+      acc.rmax = fmaxf(acc.rmax, v.r);
+      acc.amax = fmaxf(acc.amax, ad0);
+      acc.cnt += 1u;
+      acc.chi += v.hi ? 1u : 0u;
+      acc.clo += v.lo ? 1u : 0u;
+      acc.cany += (v.hi || v.lo) ? 1u : 0u;
+    }
+  }
+}
+
 template <int KIND, int VEC>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A) {
   constexpr int NW = kRlThreads / kWave;
+  constexpr int ITEMS = (VEC == 4) ? 4 : 2;  // vectors in flight per lane
   __shared__ double lds_v[NW][kRlVals];
   const RatioConsts C = A.C;
 
   Acc acc;
+  SeqCtx sq;
   const bool padded = (A.layout == LAYOUT_PADDED);
   const int64_t n_rows = padded ? A.n_seq : 1;
   const int64_t stride = (int64_t)gridDim.x * kRlThreads;
-  int64_t cur_end = -1;
-  float row_adv = 0.0f, row_w = 1.0f;
+  const int64_t first = (int64_t)blockIdx.x * kRlThreads + threadIdx.x;
 
   for (int64_t r = blockIdx.y; r < n_rows; r += gridDim.y) {
     // tokens [base, base+count) are valid; whole vectors may be loaded up to base+row_end
@@ -156,93 +205,73 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
       base = r * A.seq_stride;
       count = len;
       row_end = A.seq_stride;
-      if (!C.adv_per_token) row_adv = A.adv[r];
-      row_w = (len > 0) ? seq_weight(C, len) : 1.0f;
+      if (!C.adv_per_token) sq.adv = A.adv[r];
+      sq.w = (len > 0) ? seq_weight(C, len) : 1.0f;
     }
-    const int64_t nvec = (count + VEC - 1) / VEC;
-    const int64_t nvec_full = row_end / VEC;
+    const int64_t nvec = (count + VEC - 1) / VEC;  // vectors holding a valid token
+    const int64_t nvec_full = row_end / VEC;       // vectors that can be loaded whole
+    const int64_t nload = nvec < nvec_full ? nvec : nvec_full;
 
-    for (int64_t i = (int64_t)blockIdx.x * kRlThreads + threadIdx.x; i < nvec; i += stride) {
-      float nw[VEC], od[VEC], ad[VEC], mk[VEC], out[VEC];
-      const int64_t t0 = i * VEC;
-      const bool whole = (i < nvec_full);
-      if (VEC == 1 || whole) {
-        Vec<float, VEC>::load(A.nw + base + t0, nw);
-        Vec<float, VEC>::load(A.od + base + t0, od);
-        if (C.adv_per_token) Vec<float, VEC>::load(A.adv + base + t0, ad);
-        if (A.mask) Vec<float, VEC>::load(A.mask + base + t0, mk);
-      } else {
+    for (int64_t i0 = first; i0 < nload; i0 += stride * ITEMS) {
+      float nw[ITEMS][VEC], od[ITEMS][VEC], ad[ITEMS][VEC], mk[ITEMS][VEC];
 #pragma unroll
-        for (int k = 0; k < VEC; ++k) {
-          const bool ok = (t0 + k) < count;
-          nw[k] = ok ? A.nw[base + t0 + k] : 0.0f;
-          od[k] = ok ? A.od[base + t0 + k] : 0.0f;
-          if (C.adv_per_token) ad[k] = ok ? A.adv[base + t0 + k] : 0.0f;
-          if (A.mask) mk[k] = ok ? A.mask[base + t0 + k] : 0.0f;
+      for (int it = 0; it < ITEMS; ++it) {
+        const int64_t i = i0 + it * stride;
+        if (i < nload) {
+          Vec<float, VEC>::load(A.nw + base + i * VEC, nw[it]);
+          Vec<float, VEC>::load(A.od + base + i * VEC, od[it]);
+          if (C.adv_per_token) Vec<float, VEC>::load(A.adv + base + i * VEC, ad[it]);
+          if (A.mask) Vec<float, VEC>::load(A.mask + base + i * VEC, mk[it]);
         }
       }
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) {
+        const int64_t i = i0 + it * stride;
+        if (i < nload) {
+          float out[VEC];
+          ratio_vec_fwd<KIND, VEC>(A, C, i * VEC, count, nw[it], od[it], ad[it], mk[it], sq, acc, out);
+          if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + base + i * VEC, out);
+        }
+      }
+    }
+    // a row whose length is not a multiple of VEC ends in one vector that cannot be loaded whole
+    if (nvec > nvec_full && first == nvec_full % stride) {
+      const int64_t t0 = nvec_full * VEC;
+      float nw[VEC], od[VEC], ad[VEC], mk[VEC], out[VEC];
 #pragma unroll
       for (int k = 0; k < VEC; ++k) {
-        const int64_t t = t0 + k;
-        out[k] = 0.0f;
-        if (t < count) {
-          if (A.layout == LAYOUT_PACKED && t >= cur_end) {
-            const int64_t sq = find_seq(A.seq, A.n_seq, t);
-            cur_end = A.seq[sq + 1];
-            row_w = seq_weight(C, cur_end - A.seq[sq]);
-            if (!C.adv_per_token) row_adv = A.adv[sq];
-          }
-          const float a = C.adv_per_token ? ad[k] : row_adv;
-          const TokVals v = ratio_token<KIND>(nw[k], od[k], a, C);
-          out[k] = v.loss;
-          float lm = v.loss;
-          if (A.mask) lm = lm * mk[k];
-          acc.sr += (double)v.r;
-          acc.sr2 = fma((double)v.r, (double)v.r, acc.sr2);
-          acc.loss += lm * row_w;
-          acc.kl += v.kterm;
-          acc.pen += v.pen;
-          const float ad0 = fabsf(v.d0);
-          acc.ab += ad0;
-          acc.rmin = fminf(acc.rmin, v.r);
-          acc.rmax = fmaxf(acc.rmax, v.r);
-          acc.amax = fmaxf(acc.amax, ad0);
-          acc.cnt += 1u;
-          acc.chi += v.hi ? 1u : 0u;
-          acc.clo += v.lo ? 1u : 0u;
-          acc.cany += (v.hi || v.lo) ? 1u : 0u;
-        }
+        const bool ok = (t0 + k) < count;
+        nw[k] = ok ? A.nw[base + t0 + k] : 0.0f;
+        od[k] = ok ? A.od[base + t0 + k] : 0.0f;
+        ad[k] = (ok && C.adv_per_token) ? A.adv[base + t0 + k] : 0.0f;
+        mk[k] = (ok && A.mask) ? A.mask[base + t0 + k] : 0.0f;
       }
+      ratio_vec_fwd<KIND, VEC>(A, C, t0, count, nw, od, ad, mk, sq, acc, out);
       if (A.loss_elem) {
-        if (VEC == 1 || whole) {
-          Vec<float, VEC>::store(A.loss_elem + base + t0, out);
-        } else {
 #pragma unroll
-          for (int k = 0; k < VEC; ++k)
-            if (t0 + k < row_end) A.loss_elem[base + t0 + k] = out[k];
-        }
+        for (int k = 0; k < VEC; ++k)
+          if (t0 + k < row_end) A.loss_elem[base + t0 + k] = out[k];
       }
     }
     // padded layout: zero the loss of the slots past the sequence end
     if (A.loss_elem && padded) {
-      for (int64_t t = nvec * VEC + (int64_t)blockIdx.x * kRlThreads + threadIdx.x; t < row_end; t += stride)
-        A.loss_elem[base + t] = 0.0f;
+      for (int64_t t = nvec * VEC + first; t < row_end; t += stride) A.loss_elem[base + t] = 0.0f;
     }
   }
 
   // ---- workgroup partials -------------------------------------------------
   double vals[kRlVals];
-  vals[P_SR] = wave_sum<double>(acc.sr);
-  vals[P_SR2] = wave_sum<double>(acc.sr2);
+  vals[P_SR] = wave_sum(acc.sr);
+  vals[P_SR2] = wave_sum(acc.sr2);
   // 64 lanes x a handful of tokens: an fp32 shuffle tree keeps full accuracy at half the shuffles
-  vals[P_LOSS] = (double)wave_sum<float>(acc.loss);
-  vals[P_KL] = (double)wave_sum<float>(acc.kl);
-  vals[P_PEN] = (double)wave_sum<float>(acc.pen);
-  vals[P_ABS] = (double)wave_sum<float>(acc.ab);
-  vals[P_CNT] = (double)wave_sum<unsigned int>(acc.cnt);
-  vals[P_CHI] = (double)wave_sum<unsigned int>(acc.chi);
-  vals[P_CLO] = (double)wave_sum<unsigned int>(acc.clo);
-  vals[P_CANY] = (double)wave_sum<unsigned int>(acc.cany);
+  vals[P_LOSS] = (double)wave_sum(acc.loss);
+  vals[P_KL] = (double)wave_sum(acc.kl);
+  vals[P_PEN] = (double)wave_sum(acc.pen);
+  vals[P_ABS] = (double)wave_sum(acc.ab);
+  vals[P_CNT] = (double)wave_sum(acc.cnt);
+  vals[P_CHI] = (double)wave_sum(acc.chi);
+  vals[P_CLO] = (double)wave_sum(acc.clo);
+  vals[P_CANY] = (double)wave_sum(acc.cany);
   vals[P_RMIN] = (double)wave_min(acc.rmin);
   vals[P_RMAX] = (double)wave_max(acc.rmax);
   vals[P_AMAX] = (double)wave_max(acc.amax);
@@ -268,11 +297,23 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
   __shared__ double lds_fin[kRlThreads];
   const RatioConsts C = A.C;
   {
+    // thread = (value v, slice j0): 16 slices walk the workgroups' vectors, eight loads in flight each
     const int v = threadIdx.x % kRlVals;
     const int j0 = threadIdx.x / kRlVals;  // 0..15
+    constexpr int kSlices = kRlThreads / kRlVals;
+    constexpr int kBatch = 8;
     double x = (v == P_RMIN) ? (double)INFINITY : ((v == P_RMAX || v == P_AMAX) ? -(double)INFINITY : 0.0);
-    for (unsigned int j = j0; j < nblk; j += kRlThreads / kRlVals)
-      x = combine(v, x, A.partials[(int64_t)j * kRlVals + v]);
+    const double ident = x;
+    for (unsigned int j = j0; j < nblk; j += kSlices * kBatch) {
+      double y[kBatch];
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) {
+        const unsigned int jj = j + b * kSlices;
+        y[b] = (jj < nblk) ? A.partials[(int64_t)jj * kRlVals + v] : ident;
+      }
+#pragma unroll
+      for (int b = 0; b < kBatch; ++b) x = combine(v, x, y[b]);
+    }
     lds_fin[threadIdx.x] = x;
   }
   __syncthreads();
@@ -434,7 +475,7 @@ static int plan(const RatioArgs& A, bool bwd, RatioShape& S) {
   if (padded && A.seq_stride % 4 != 0) vec = 1;
   const int64_t row_tok = padded ? A.seq_stride : A.n_tok;
   const int64_t nvec = (row_tok + vec - 1) / vec;
-  const int64_t cap = bwd ? 16384 : tune_int("UNIRL_RATIO_MAX_BLOCKS", 2048);
+  const int64_t cap = bwd ? 16384 : tune_int("UNIRL_RATIO_MAX_BLOCKS", 512);
   int64_t rows = padded ? A.n_seq : 1;
   if (rows > cap) rows = cap;
   if (rows < 1) rows = 1;

@@ -385,7 +385,7 @@ __global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs
         if (tj) Vec<float, VEC>::store(tj + i * VEC, x[it]);
       }
     }
-    const double w = wave_sum<double>((double)acc);
+    const double w = wave_sum((double)acc);
     if (lane == 0) lds_q[k][wid] = w;
   }
 
@@ -586,7 +586,7 @@ extern "C" int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const vo
       !aligned_to(mean_out, 16))
     vec = 1;
 
-  const int items = (vec == 4) ? (int)tune_int("UNIRL_SDE_ITEMS", 2) : 2;
+  const int items = (vec == 4) ? (int)tune_int("UNIRL_SDE_ITEMS", 4) : 2;
   const unsigned int nblk = sde_blocks_per_sample(D / vec, items, B);
   const int64_t per_launch = sde_samples_per_launch(B, nblk);
   hipStream_t st = (hipStream_t)stream;
@@ -715,7 +715,7 @@ extern "C" int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* c
   // One pass must cover a sample (the latent lives in registers): pick the
   // vectors per lane, the workgroup count follows.
   const int64_t nvec = D / vec;
-  int items = (int)tune_int("UNIRL_ROLLOUT_ITEMS", 1);
+  int items = (int)tune_int("UNIRL_ROLLOUT_ITEMS", 4);
   if (items != 1 && items != 2 && items != 4) items = 1;
   int64_t nblk = (nvec + (int64_t)kSdeThreads * items - 1) / ((int64_t)kSdeThreads * items);
   while (nblk * S > kPartialCapacity && items < 4) {

@@ -60,24 +60,6 @@ struct TokState {
 
 __device__ __forceinline__ float tok_exp2(float a) { return __builtin_amdgcn_exp2f(a); }
 
-// Maximum over the 64 lanes, returned wave-uniform.  DPP row shifts build each 16-lane row's
-// maximum in its last lane, two row broadcasts carry them to lane 63, readlane makes it scalar.
-// Full-rate VALU, no LDS traffic.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ float tok_dpp_max(float v) {
-  const int moved = __builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, ROW_MASK, 0xf, false);
-  return fmaxf(v, __int_as_float(moved));
-}
-__device__ __forceinline__ float wave_max_uniform(float v) {
-  v = tok_dpp_max<0x111, 0xf>(v);  // row_shr:1
-  v = tok_dpp_max<0x112, 0xf>(v);  // row_shr:2
-  v = tok_dpp_max<0x114, 0xf>(v);  // row_shr:4
-  v = tok_dpp_max<0x118, 0xf>(v);  // row_shr:8   -> lane 15 of each row holds the row maximum
-  v = tok_dpp_max<0x142, 0xa>(v);  // row_bcast:15 into rows 1 and 3
-  v = tok_dpp_max<0x143, 0xc>(v);  // row_bcast:31 into rows 2 and 3 -> lane 63 holds the maximum
-  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
-}
-
 // Re-express sums relative to a higher maximum M.  (m, r) -> (M, fl(M*c)).
 __device__ __forceinline__ void tok_raise(float& m, float& r, TokAcc& acc, float M, float c) {
   if (m == M) return;
@@ -107,7 +89,7 @@ __device__ __forceinline__ void tok_update(TokRef& ref, TokAcc& acc, const float
   float cm = x[0];
 #pragma unroll
   for (int k = 1; k < N; ++k) cm = fmaxf(cm, x[k]);
-  const float wm = wave_max_uniform(active ? cm : -INFINITY);
+  const float wm = wave_max(active ? cm : -INFINITY);  // wave-uniform, DPP
   if (__builtin_expect(wm > ref.m, 0)) {
     // Wave-uniform and rare (about ln(chunks) times per row): move to the new maximum, then
     // split this chunk's exact maxima from the rest.
@@ -149,7 +131,6 @@ __device__ __forceinline__ void tok_merge(TokState& a, TokState b, float c) {
 }
 
 // 16 bytes of logits -> floats
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 template <typename T>
 struct Stream16;
@@ -191,12 +172,6 @@ struct Stream16<f16_t> {
     o[7] = f16_bits_to_f32(v.w >> 16);
   }
 };
-
-// streaming 16-byte load (non-temporal: a row is read exactly once)
-template <typename T>
-__device__ __forceinline__ u32x4 stream_load16(const T* p) {
-  return __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p));
-}
 
 struct TokArgs {
   const void* logits;
@@ -276,7 +251,7 @@ __device__ __forceinline__ TokState tok_scan_row(const T* __restrict__ p, int64_
   }
 
   // lanes -> wavefront: the lanes share (m, r), so the sums simply add
-  TokState st{ref.m, ref.r, wave_sum<float>(acc.cnt), wave_sum<float>(acc.s), wave_sum<float>(acc.t)};
+  TokState st{ref.m, ref.r, wave_sum(acc.cnt), wave_sum(acc.s), wave_sum(acc.t)};
   const int lane = threadIdx.x & (kWave - 1);
   const int wid = threadIdx.x / kWave;
   __syncthreads();  // lds may still be read from a previous scan of this row
