@@ -243,6 +243,9 @@ def main() -> int:
     ap.add_argument("--vocab", type=int, default=151936)
     ap.add_argument("--cpu-rows", type=int, default=512, help="rows of the bounded CPU-baseline sample")
     ap.add_argument("--spinup", type=float, default=0.5, help="seconds of untimed launches before the warm-up")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="run 3 calibration copies of 1 GiB and 3 headline launches, then exit "
+                         "(the command `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` is pointed at)")
     ap.add_argument("--skip-shapes", action="store_true", help="headline only")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
     args = ap.parse_args()
@@ -278,6 +281,18 @@ def main() -> int:
 
     def step(i):
         return ops.token_logp_entropy(x, ids, 1.0, want_logp=True, want_entropy=True)
+
+    if args.traffic_probe:
+        src = torch.empty(2**30, dtype=torch.uint8, device=dev).fill_(7)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            ops.calib_copy(src, dst)
+        for i in range(3):
+            step(i)
+        torch.cuda.synchronize()
+        print(json.dumps({"traffic_probe": {"calib_copy_bytes_each_way": 2**30,
+                                            "token_kernel_algorithmic_bytes": alg_bytes}}), flush=True)
+        return 0
 
     # Untimed spin-up: the device needs a few hundred milliseconds of work to reach its sustained
     # clocks (measured: 6.2 TB/s after 5 launches, 6.8 TB/s after 200).  Then W warm-up steps,
@@ -360,6 +375,17 @@ def main() -> int:
                 f"wrapper {lat:.0f} us")
             shapes_out.append(row)
 
+    # HBM bytes per launch from hardware counters, when a committed counter summary covers this workload
+    traffic = None
+    traffic_file = ROOT / "profiles" / "token_logp_entropy_traffic.json"
+    if traffic_file.exists():
+        try:
+            rec = json.loads(traffic_file.read_text())
+            if rec.get("rows") == args.rows and rec.get("vocab") == args.vocab:
+                traffic = rec.get("hbm_bytes_per_launch")
+        except (ValueError, OSError):
+            traffic = None
+
     result = {
         "metric": "fused-kernel HBM GB/s (token log-prob + entropy)",
         "value": round(value, 1),
@@ -380,7 +406,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": None,
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
             "kernel": "token_logp_entropy_kernel<bf16>", "algorithmic_bytes_per_launch": alg_bytes,
             "launch_ms": round(event_ms, 4),
         },

@@ -62,6 +62,11 @@ size_t unirl_workspace_bytes(void);
 /* Optional: zero-fill a workspace (a fill kernel on `stream`); no entry point needs it. */
 int unirl_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
 
+/* Measurement aid, no counterpart in the reference: a plain streaming copy of
+ * `bytes` (a multiple of 16, both pointers 16-byte aligned).  Hardware byte
+ * counters read for this kernel calibrate the ones read for the kernels below. */
+int unirl_calib_copy(const void* src, void* dst, size_t bytes, void* stream);
+
 /* ------------------------------------------------------------------------
  * One SDE transition + per-sample Gaussian log-prob.
  * Replaces StepStrategy.denoise -> SDEStrategy.step -> _finalize_logp

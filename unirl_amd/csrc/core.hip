@@ -10,6 +10,15 @@ __global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* p, size_t n_wo
   for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += stride) p[i] = 0u;
 }
 
+// Plain streaming copy, the yardstick for hardware byte counters: it moves exactly `n_vec`*16
+// bytes in and out.
+__global__ __launch_bounds__(256) void calib_copy_kernel(const u32x4* __restrict__ src, u32x4* __restrict__ dst,
+                                                         size_t n_vec) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_vec; i += stride)
+    stream_store16(dst + i, stream_load16(src + i));
+}
+
 }  // namespace unirl
 
 using namespace unirl;
@@ -40,5 +49,15 @@ extern "C" int unirl_workspace_init(void* workspace, size_t workspace_bytes, voi
   // values.  A fill kernel rather than a memset node, so the call is safe to capture in a graph.
   hipLaunchKernelGGL(fill_zero_kernel, dim3(256), dim3(256), 0, (hipStream_t)stream,
                      reinterpret_cast<uint32_t*>(workspace), workspace_bytes / 4);
+  return (int)hipGetLastError();
+}
+
+extern "C" int unirl_calib_copy(const void* src, void* dst, size_t bytes, void* stream) {
+  if (!src || !dst) return UNIRL_E_NULL;
+  if (bytes % 16 != 0) return UNIRL_E_SHAPE;
+  if (!aligned_to(src, 16) || !aligned_to(dst, 16)) return UNIRL_E_ALIGN;
+  if (bytes == 0) return UNIRL_OK;
+  hipLaunchKernelGGL(calib_copy_kernel, dim3(8192), dim3(256), 0, (hipStream_t)stream,
+                     reinterpret_cast<const u32x4*>(src), reinterpret_cast<u32x4*>(dst), bytes / 16);
   return (int)hipGetLastError();
 }

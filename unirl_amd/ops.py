@@ -671,6 +671,19 @@ def normalize_grouped(
     return out
 
 
+def calib_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """Plain streaming copy of ``src`` into ``dst`` (same byte size, a multiple of 16): the
+    reference kernel for calibrating hardware byte counters."""
+    N.require_device(src, "src")
+    N.require_device(dst, "dst")
+    nbytes = src.numel() * src.element_size()
+    if nbytes != dst.numel() * dst.element_size() or not (src.is_contiguous() and dst.is_contiguous()):
+        raise ValueError("calib_copy needs two contiguous tensors of the same byte size")
+    with torch.cuda.device(src.device):
+        rc = N.lib().unirl_calib_copy(N.ptr(src), N.ptr(dst), nbytes, N.current_stream(src.device))
+    N.check(rc, "unirl_calib_copy")
+
+
 def gather_steps(tensor: torch.Tensor, positions: Sequence[int]) -> torch.Tensor:
     """``tensor[:, positions]`` for a ``[B, S, ...]`` tensor, as one gather kernel."""
     N.require_device(tensor, "tensor")
