@@ -347,6 +347,20 @@ def main() -> int:
     }]
     if not args.skip_shapes:
         del lp, ent
+        # backward of the token log-prob at the same shape: reads the logits, writes their gradient
+        lse = ops.token_logp_entropy(x, ids, 1.0, want_logp=False, want_entropy=False, want_lse=True)[2]
+        g_lp = torch.randn(args.rows, device=dev)
+        _, bwd_ms = time_steps(torch, lambda i: ops.token_logp_bwd(x, ids, 1.0, lse, g_lp), args.steps, args.warmup)
+        bwd_bytes = 2 * x.numel() * 2 + args.rows * (8 + 4 + 4)
+        bwd_gbps = bwd_bytes / (bwd_ms * 1e-3) / 1e9
+        log(f"token_logp_bwd: {bwd_ms:.4f} ms/launch, {bwd_gbps:.0f} GB/s = {bwd_gbps / HBM_PEAK_GBPS:.1%} of peak")
+        shapes_out.append({
+            "name": "token_logp_bwd", "config": 2, "shape": f"bf16 [{args.rows},{args.vocab}] logits -> bf16 gradient",
+            "algorithmic_bytes": bwd_bytes, "elements": x.numel(), "kernel_us": round(bwd_ms * 1e3, 2),
+            "gbps": round(bwd_gbps, 1), "frac_of_peak": round(bwd_gbps / HBM_PEAK_GBPS, 4),
+            "elements_per_s": round(x.numel() / (bwd_ms * 1e-3), 0), "timing": "hip events over the timed steps",
+        })
+        del lse, g_lp
         for sh in make_shapes(torch, dev):
             try:
                 us = time_in_graph(torch, sh["run"], sh["sets"])

@@ -30,13 +30,26 @@ struct f16_t {
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-// Round-to-nearest-even fp32 -> bf16, NaN -> quiet NaN (what torch's
-// c10::BFloat16 conversion does).
+// Round-to-nearest-even fp32 -> bf16 on the hardware converter (v_cvt_pk_bf16_f32); NaN stays a
+// quiet NaN.  The pair form converts two values with one instruction.
+typedef __bf16 hw_bf16x2 __attribute__((ext_vector_type(2)));
+typedef float hw_f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+  const hw_f32x2 v = {lo, hi};
+  union {
+    hw_bf16x2 h;
+    uint32_t u;
+  } c;
+  c.h = __builtin_convertvector(v, hw_bf16x2);
+  return c.u;
+}
 __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return 0x7fc0u;
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return u >> 16;
+  union {
+    __bf16 h;
+    uint16_t u;
+  } c;
+  c.h = (__bf16)f;
+  return c.u;
 }
 
 __device__ __forceinline__ float f16_bits_to_f32(uint32_t h) {
@@ -135,8 +148,8 @@ struct Vec<bf16_t, 4> {
   }
   static __device__ __forceinline__ void store(bf16_t* p, const float (&o)[4]) {
     uint2 v;
-    v.x = f32_to_bf16_bits(o[0]) | (f32_to_bf16_bits(o[1]) << 16);
-    v.y = f32_to_bf16_bits(o[2]) | (f32_to_bf16_bits(o[3]) << 16);
+    v.x = f32x2_to_bf16x2_bits(o[0], o[1]);
+    v.y = f32x2_to_bf16x2_bits(o[2], o[3]);
     *reinterpret_cast<uint2*>(p) = v;
   }
 };

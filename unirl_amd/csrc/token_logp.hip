@@ -173,6 +173,43 @@ struct Stream16<f16_t> {
   }
 };
 
+// Inverse of Stream16<T>::unpack: N floats -> one 16-byte vector of T (round to nearest even).
+template <typename T>
+struct Pack16;
+template <>
+struct Pack16<float> {
+  static __device__ __forceinline__ u32x4 pack(const float* o) {
+    u32x4 v;
+    v.x = __float_as_uint(o[0]);
+    v.y = __float_as_uint(o[1]);
+    v.z = __float_as_uint(o[2]);
+    v.w = __float_as_uint(o[3]);
+    return v;
+  }
+};
+template <>
+struct Pack16<bf16_t> {
+  static __device__ __forceinline__ u32x4 pack(const float* o) {
+    u32x4 v;
+    v.x = f32x2_to_bf16x2_bits(o[0], o[1]);
+    v.y = f32x2_to_bf16x2_bits(o[2], o[3]);
+    v.z = f32x2_to_bf16x2_bits(o[4], o[5]);
+    v.w = f32x2_to_bf16x2_bits(o[6], o[7]);
+    return v;
+  }
+};
+template <>
+struct Pack16<f16_t> {
+  static __device__ __forceinline__ u32x4 pack(const float* o) {
+    u32x4 v;
+    v.x = f32_to_f16_bits(o[0]) | (f32_to_f16_bits(o[1]) << 16);
+    v.y = f32_to_f16_bits(o[2]) | (f32_to_f16_bits(o[3]) << 16);
+    v.z = f32_to_f16_bits(o[4]) | (f32_to_f16_bits(o[5]) << 16);
+    v.w = f32_to_f16_bits(o[6]) | (f32_to_f16_bits(o[7]) << 16);
+    return v;
+  }
+};
+
 struct TokArgs {
   const void* logits;
   const int64_t* ids;
@@ -318,20 +355,78 @@ struct TokBwdArgs {
   void* grad;
 };
 
-template <typename T>
+__device__ __forceinline__ float tok_bwd_elem(float x, float c, float lse2, float gs, float one) {
+  return gs * (one - tok_exp2(fmaf(x, c, -lse2)));
+}
+
+// One workgroup per row.  The row is read and its gradient written once, as 16-byte streaming
+// vectors when the logits row and the gradient row share their offset from a 16-byte boundary
+// (always, for contiguous tensors whose V*sizeof(T) is a multiple of 16), else element-wise.
+template <typename T, int UNROLL>
 __global__ __launch_bounds__(kTokThreads) void token_logp_bwd_kernel(TokBwdArgs A) {
-  const int64_t row = blockIdx.y;
+  constexpr int VEC = Stream16<T>::N;
+  const int64_t row = blockIdx.x;
   const T* __restrict__ p = reinterpret_cast<const T*>(A.logits) + row * A.row_stride;
   T* __restrict__ gp = reinterpret_cast<T*>(A.grad) + row * A.grad_row_stride;
   const float lse2 = A.lse[row] * kLog2e;
   const float gs = A.g[row] * A.inv_t;
+  const float c = A.c;
   const int64_t id = A.ids[row];
-  const int64_t stride = (int64_t)gridDim.x * kTokThreads;
-  for (int64_t j = (int64_t)blockIdx.x * kTokThreads + threadIdx.x; j < A.V; j += stride) {
-    const float x = Elem<T>::load(p + j);
-    const float prob = tok_exp2(fmaf(x, A.c, -lse2));
-    const float one = (j == id) ? 1.0f : 0.0f;
-    Elem<T>::store(gp + j, gs * (one - prob));
+  const int64_t V = A.V;
+  const int tid = threadIdx.x;
+
+  const unsigned mis_p = (unsigned)(reinterpret_cast<uintptr_t>(p) & 15u);
+  const unsigned mis_g = (unsigned)(reinterpret_cast<uintptr_t>(gp) & 15u);
+  if (mis_p != mis_g) {  // row-uniform
+    for (int64_t j = tid; j < V; j += kTokThreads)
+      Elem<T>::store(gp + j, tok_bwd_elem(Elem<T>::load(p + j), c, lse2, gs, (j == id) ? 1.0f : 0.0f));
+    return;
+  }
+  int64_t head = (int64_t)(((16u - mis_p) & 15u) / sizeof(T));
+  if (head > V) head = V;
+  const int64_t nvec = (V - head) / VEC;
+  const int64_t tail0 = head + nvec * VEC;
+  if (tid < head) Elem<T>::store(gp + tid, tok_bwd_elem(Elem<T>::load(p + tid), c, lse2, gs, (tid == id) ? 1.0f : 0.0f));
+  if (tail0 + tid < V) {
+    const int64_t j = tail0 + tid;
+    Elem<T>::store(gp + j, tok_bwd_elem(Elem<T>::load(p + j), c, lse2, gs, (j == id) ? 1.0f : 0.0f));
+  }
+
+  const T* __restrict__ pv = p + head;
+  T* __restrict__ gv = gp + head;
+  const int64_t idv = id - head;  // position of the gathered column in the vector region
+  const int64_t per_iter = (int64_t)kTokThreads * UNROLL;
+  const int64_t n_full = nvec / per_iter;
+  for (int64_t it = 0; it < n_full; ++it) {
+    const int64_t v0 = it * per_iter + tid;
+    u32x4 raw[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) raw[u] = stream_load16(pv + (v0 + (int64_t)u * kTokThreads) * VEC);
+#pragma unroll
+    for (int u = 0; u < UNROLL; ++u) {
+      const int64_t e0 = (v0 + (int64_t)u * kTokThreads) * VEC;
+      float x[VEC];
+      Stream16<T>::unpack(raw[u], x);
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) x[k] = tok_bwd_elem(x[k], c, lse2, gs, 0.0f);
+      if ((uint64_t)(idv - e0) < (uint64_t)VEC) {  // this vector holds the gathered column
+        float y[VEC];
+        Stream16<T>::unpack(raw[u], y);
+#pragma unroll
+        for (int k = 0; k < VEC; ++k)
+          if (idv - e0 == k) x[k] = tok_bwd_elem(y[k], c, lse2, gs, 1.0f);
+      }
+      stream_store16(gv + e0, Pack16<T>::pack(x));
+    }
+  }
+  for (int64_t v = n_full * per_iter + tid; v < nvec; v += kTokThreads) {
+    const int64_t e0 = v * VEC;
+    const u32x4 raw = stream_load16(pv + e0);
+    float x[VEC], y[VEC];
+    Stream16<T>::unpack(raw, y);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) x[k] = tok_bwd_elem(y[k], c, lse2, gs, (idv - e0 == k) ? 1.0f : 0.0f);
+    stream_store16(gv + e0, Pack16<T>::pack(x));
   }
 }
 
@@ -410,13 +505,11 @@ extern "C" int unirl_token_logp_bwd(const void* logits, int dtype, int64_t rows,
     A.lse = lse + r0;
     A.g = g_logp + r0;
     A.grad = const_cast<void*>(offset_ptr(grad_logits, r0 * grad_row_stride, dtype_size(dtype)));
-    int64_t nbx = (V + kTokThreads * 4 - 1) / (kTokThreads * 4);
-    if (nbx > 1024) nbx = 1024;
-    dim3 grid((unsigned int)nbx, (unsigned int)nr), block(kTokThreads);
+    dim3 grid((unsigned int)nr), block(kTokThreads);
     switch (dtype) {
-      case UNIRL_F32: hipLaunchKernelGGL((token_logp_bwd_kernel<float>), grid, block, 0, st, A); break;
-      case UNIRL_BF16: hipLaunchKernelGGL((token_logp_bwd_kernel<bf16_t>), grid, block, 0, st, A); break;
-      case UNIRL_F16: hipLaunchKernelGGL((token_logp_bwd_kernel<f16_t>), grid, block, 0, st, A); break;
+      case UNIRL_F32: hipLaunchKernelGGL((token_logp_bwd_kernel<float, 4>), grid, block, 0, st, A); break;
+      case UNIRL_BF16: hipLaunchKernelGGL((token_logp_bwd_kernel<bf16_t, 4>), grid, block, 0, st, A); break;
+      case UNIRL_F16: hipLaunchKernelGGL((token_logp_bwd_kernel<f16_t, 4>), grid, block, 0, st, A); break;
     }
     const int rc = (int)hipGetLastError();
     if (rc != 0) return rc;
