@@ -92,6 +92,49 @@ int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const void* sample,
                         float* prev_out, float* mean_out, float* logp_out, int logp_sum,
                         void* workspace, size_t workspace_bytes, void* stream);
 
+/* ------------------------------------------------------------------------
+ * The same transition with strided, typed tensors, for the replay and rollout
+ * loops that keep trajectories as [B, K, ...] stacks in a 16-bit dtype
+ * (unirl/models/sd3/diffusion.py:366-406 writes `latents.to(trajectory_dtype)`
+ * into a stack; :467-497 reads `segment.latents_at(k)` = latents[:, k] and
+ * stacks log-probs [B, S'] and means `.to(trajectory_dtype)`).  Each tensor
+ * names its dtype and the element distance between consecutive samples
+ * (0 = D, densely packed), so `latents[:, k]` is read in place and prev, mean
+ * and the log-prob column are written straight into their stacks.
+ * prev_sample.ptr == NULL selects sampling; prev_sample.dtype must equal
+ * sample.dtype.  Outputs are rounded to their dtype on store (prev has already
+ * been rounded to sample.dtype, so storing it in that dtype is exact).
+ * Other fields as in unirl_sde_step_logp. */
+struct unirl_sde_tensor {
+  const void* ptr;
+  int dtype;             /* unirl_dtype */
+  int64_t sample_stride; /* elements; 0 = D */
+};
+struct unirl_sde_step_desc {
+  struct unirl_sde_tensor noise_pred, sample, prev_sample;
+  const float* noise;    /* sampling only; NULL = no noise */
+  int64_t noise_stride;
+  const float* sigma;
+  const float* sigma_next;
+  int sigma_stride;
+  const float* sigma_max_ptr;
+  float sigma_max_val;
+  double eta;
+  int kind;
+  int64_t B, D;
+  void* prev_out;        /* NULL = not wanted */
+  int prev_dtype;
+  int64_t prev_stride;
+  void* mean_out;
+  int mean_dtype;
+  int64_t mean_stride;
+  float* logp_out;       /* element b at logp_out[b * logp_stride] */
+  int64_t logp_stride;   /* 0 = 1 */
+  int logp_sum;
+};
+int unirl_sde_step_logp_ex(const struct unirl_sde_step_desc* desc /* host */, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
 /* Backward of unirl_sde_step_logp with respect to noise_pred and sample, for
  * the autograd graph the reference builds through kernels.py:225-228 and
  * :200-204 (prev_sample is detached there).  Inputs as in the forward call;

@@ -360,3 +360,76 @@ def test_wan_video_shape_bf16_replay(dev):
                      sigma_max=SIG[1].to(dev))
     assert torch.equal(got[2].cpu(), ref[2]) and torch.equal(got[0].cpu(), ref[0])
     assert_close(got[1], ref[1], BF16_RTOL, 0.0, "wan logp")
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("traj_dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(3, 4, 8, 8), (2, 5, 7), (4, 16, 16, 16)])
+def test_stage_loops_on_stacks_match_oracle(dev, kind, traj_dtype, shape):
+    """The reference's diffuse loop (latents.to(trajectory_dtype) stacked as [B,K,...],
+    unirl/models/sd3/diffusion.py:366-406) and its replay loop (latents_at views in,
+    stack(log_probs), stack(means).to(trajectory_dtype) out, :467-497), run with denoise_into on
+    views of the stacks and compared with the oracle's step-by-step eager chain."""
+    from unirl_amd import sde
+
+    st = strategy(kind)
+    B = shape[0]
+    steps = [0, 1, 2, 5]
+    g = torch.Generator().manual_seed(hash((kind, str(traj_dtype), shape)) % 997)
+    x0 = torch.randn(shape, generator=g).to(traj_dtype)
+    vs = [torch.randn(shape, generator=g).to(traj_dtype) for _ in steps]
+    ns = [torch.randn(shape, generator=g) for _ in steps]
+    rtol = FP32_RTOL if traj_dtype == torch.float32 else BF16_RTOL
+
+    # oracle: rollout, keeping every latent in the trajectory dtype
+    ref_lat, ref_lp = [x0], []
+    for j, i in enumerate(steps):
+        prev, lp, _ = osde.sde_denoise(kind, vs[j], ref_lat[-1], SIG[i], SIG[i + 1], eta=0.7, noise=ns[j],
+                                       sigma_max=SIG[1], ieee_sqrt=True)
+        ref_lat.append(prev.to(traj_dtype))
+        ref_lp.append(lp)
+    ref_stack = torch.stack(ref_lat, dim=1)
+    ref_lp = torch.stack(ref_lp, dim=1)
+
+    # device: one stack [B, K, ...] in the trajectory dtype, written slot by slot
+    K = len(steps) + 1
+    stack = torch.zeros((B, K) + tuple(shape[1:]), dtype=traj_dtype, device=dev)
+    stack[:, 0] = x0.to(dev)
+    logp = torch.full((B, len(steps)), float("nan"), device=dev)
+    for j, i in enumerate(steps):
+        ok = st.denoise_into(vs[j].to(dev), stack[:, j], SIG[i].to(dev), SIG[i + 1].to(dev), eta=0.7,
+                             sigma_max=SIG[1].to(dev), noise=ns[j].to(dev), prev_out=stack[:, j + 1],
+                             logp_out=logp[:, j])
+        assert ok
+    assert torch.equal(stack.cpu(), ref_stack), "trajectory stack differs"
+    assert_close(logp, ref_lp, rtol, 2e-6, "rollout log-probs")
+
+    # replay: fresh velocities, stored latents read in place, means and log-probs written in place
+    v2 = [torch.randn(shape, generator=g).to(traj_dtype) for _ in steps]
+    indices = torch.arange(K)
+    ref_means, ref_rlp = [], []
+    for j, i in enumerate(steps):
+        _, lp, mean = osde.sde_denoise(kind, v2[j], ref_stack[:, j], SIG[i], SIG[i + 1], eta=0.7,
+                                       prev_sample=ref_stack[:, j + 1], sigma_max=SIG[1], ieee_sqrt=True)
+        ref_means.append(mean)
+        ref_rlp.append(lp)
+    ref_means = torch.stack(ref_means, dim=1).to(traj_dtype)
+    ref_rlp = torch.stack(ref_rlp, dim=1)
+    means = torch.zeros((B, len(steps)) + tuple(shape[1:]), dtype=traj_dtype, device=dev)
+    rlp = torch.zeros((B, len(steps)), device=dev)
+    for j, i in enumerate(steps):
+        st.denoise_into(v2[j].to(dev), sde.latents_at(stack, indices, j), SIG[i].to(dev), SIG[i + 1].to(dev),
+                        eta=0.7, prev_sample=sde.latents_at(stack, indices, j + 1), sigma_max=float(SIG[1]),
+                        mean_out=means[:, j], logp_out=rlp[:, j])
+    assert torch.equal(means.cpu(), ref_means), "replayed means differ"
+    assert_close(rlp, ref_rlp, rtol, 2e-6, "replay log-probs")
+    # eta = 0: Euler step, log-prob column untouched
+    before = rlp.clone()
+    assert not st.denoise_into(v2[0].to(dev), stack[:, 0], SIG[0].to(dev), SIG[1].to(dev), eta=0.0,
+                               sigma_max=float(SIG[1]), mean_out=means[:, 0], logp_out=rlp[:, 0])
+    assert torch.equal(rlp, before)
+    with pytest.raises(KeyError):
+        sde.latents_at(stack, indices, K + 3)
+    with pytest.raises(ValueError):
+        st.denoise_into(v2[0].to(dev), stack[:, 0], SIG[0].to(dev), SIG[1].to(dev), eta=0.7,
+                        mean_out=means[:, 0].transpose(-1, -2), logp_out=rlp[:, 0])

@@ -55,6 +55,42 @@ class RatioLossParams(Structure):
     ]
 
 
+class SdeTensor(Structure):
+    """struct unirl_sde_tensor."""
+
+    _fields_ = [("ptr", c_void_p), ("dtype", c_int), ("sample_stride", c_int64)]
+
+
+class SdeStepDesc(Structure):
+    """struct unirl_sde_step_desc."""
+
+    _fields_ = [
+        ("noise_pred", SdeTensor),
+        ("sample", SdeTensor),
+        ("prev_sample", SdeTensor),
+        ("noise", c_void_p),
+        ("noise_stride", c_int64),
+        ("sigma", c_void_p),
+        ("sigma_next", c_void_p),
+        ("sigma_stride", c_int),
+        ("sigma_max_ptr", c_void_p),
+        ("sigma_max_val", c_float),
+        ("eta", c_double),
+        ("kind", c_int),
+        ("B", c_int64),
+        ("D", c_int64),
+        ("prev_out", c_void_p),
+        ("prev_dtype", c_int),
+        ("prev_stride", c_int64),
+        ("mean_out", c_void_p),
+        ("mean_dtype", c_int),
+        ("mean_stride", c_int64),
+        ("logp_out", c_void_p),
+        ("logp_stride", c_int64),
+        ("logp_sum", c_int),
+    ]
+
+
 _SIGNATURES = {
     "unirl_abi_version": (c_int, []),
     "unirl_status_string": (c_char_p, [c_int]),
@@ -66,6 +102,7 @@ _SIGNATURES = {
         [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,
          c_double, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p],
     ),
+    "unirl_sde_step_logp_ex": (c_int, [POINTER(SdeStepDesc), c_void_p, c_size_t, c_void_p]),
     "unirl_sde_step_logp_bwd": (
         c_int,
         [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,

@@ -123,13 +123,28 @@ struct SdeStepArgs {
   int want_logp;
   int logp_sum;
   int64_t D;
-  float* prev_out;
-  float* mean_out;
+  int64_t stride_v, stride_x, stride_third;  // elements between consecutive samples
+  void* prev_out;
+  void* mean_out;
+  int prev_dtype, mean_dtype;                // unirl_dtype of the two outputs
+  int64_t stride_prev, stride_mean;
   float* logp_out;
+  int64_t stride_logp;
   double* partials;        // [B][gridDim.x]
   unsigned int nblk;       // host only: grid.x
   int items;               // host only: vectors in flight per lane
 };
+
+// Store VEC floats as `dtype` (wave-uniform switch) at element index `idx` of `base`.
+template <int VEC>
+__device__ __forceinline__ void sde_store_as(void* base, int dtype, int64_t idx, const float (&o)[VEC]) {
+  if (dtype == UNIRL_F32)
+    Vec<float, VEC>::store(reinterpret_cast<float*>(base) + idx, o);
+  else if (dtype == UNIRL_BF16)
+    Vec<bf16_t, VEC>::store(reinterpret_cast<bf16_t*>(base) + idx, o);
+  else
+    Vec<f16_t, VEC>::store(reinterpret_cast<f16_t*>(base) + idx, o);
+}
 
 template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING>
 __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
@@ -144,11 +159,13 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
   const int kind = A.kind;
   const SdeCoef c = sde_coef(kind, s, sn, smax, A.sc);
 
-  const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + b * D;
-  const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + b * D;
-  const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + b * D : nullptr;
-  float* __restrict__ po = A.prev_out ? A.prev_out + b * D : nullptr;
-  float* __restrict__ mo = A.mean_out ? A.mean_out + b * D : nullptr;
+  const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + b * A.stride_v;
+  const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + b * A.stride_x;
+  const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + b * A.stride_third : nullptr;
+  void* const po = A.prev_out;
+  void* const mo = A.mean_out;
+  const int64_t po0 = b * A.stride_prev, mo0 = b * A.stride_mean;
+  const int pdt = A.prev_dtype, mdt = A.mean_dtype;
 
   const int64_t nvec = D / VEC;  // VEC == 1 or D % VEC == 0 (checked on the host)
   const int64_t stride = (int64_t)gridDim.x * kSdeThreads;
@@ -180,8 +197,8 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
           const float d = sde_elem<TX, SAMPLING>(kind, c, v[it][k], x[it][k], t[it][k], mean[k], prev[k]);
           acc = fmaf(d, d, acc);
         }
-        if (po) Vec<float, VEC>::store(po + i * VEC, prev);
-        if (mo) Vec<float, VEC>::store(mo + i * VEC, mean);
+        if (po) sde_store_as<VEC>(po, pdt, po0 + i * VEC, prev);
+        if (mo) sde_store_as<VEC>(mo, mdt, mo0 + i * VEC, mean);
       }
     }
   }
@@ -191,7 +208,7 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
   const double part = block_sum<double>((double)acc, lds);
   if (threadIdx.x != 0) return;
   if (gridDim.x == 1) {
-    A.logp_out[b] = sde_finish_logp(kind, c, part, (double)D, A.logp_sum);
+    A.logp_out[b * A.stride_logp] = sde_finish_logp(kind, c, part, (double)D, A.logp_sum);
   } else {
     A.partials[b * gridDim.x + blockIdx.x] = part;  // summed by sde_step_finalize_kernel
   }
@@ -207,7 +224,7 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepA
   const float sn = A.sigma_next[b * A.sigma_stride];
   const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
   const SdeCoef c = sde_coef(A.kind, s, sn, smax, A.sc);
-  A.logp_out[b] = sde_finish_logp(A.kind, c, q, (double)A.D, A.logp_sum);
+  A.logp_out[b * A.stride_logp] = sde_finish_logp(A.kind, c, q, (double)A.D, A.logp_sum);
 }
 
 // ---------------------------------------------------------------------------
@@ -560,30 +577,48 @@ static int launch_rollout_x(const SdeRolloutArgs& A, int dtype_x, int64_t B, int
 
 using namespace unirl;
 
-extern "C" int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const void* sample, int dtype_x,
-                                   const void* prev_sample, const float* noise, const float* sigma,
-                                   const float* sigma_next, int sigma_stride, const float* sigma_max_ptr,
-                                   float sigma_max_val, double eta, int kind, int64_t B, int64_t D,
-                                   float* prev_out, float* mean_out, float* logp_out, int logp_sum,
-                                   void* workspace, size_t workspace_bytes, void* stream) {
+extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* workspace, size_t workspace_bytes,
+                                      void* stream) {
+  if (!d) return UNIRL_E_NULL;
+  const int dtype_v = d->noise_pred.dtype, dtype_x = d->sample.dtype;
+  const int64_t B = d->B, D = d->D;
   if (!dtype_ok(dtype_v) || !dtype_ok(dtype_x)) return UNIRL_E_DTYPE;
-  if (kind < UNIRL_SDE_FLOW || kind > UNIRL_SDE_CPS) return UNIRL_E_DTYPE;
-  if (B < 0 || D <= 0 || (sigma_stride != 0 && sigma_stride != 1)) return UNIRL_E_SHAPE;
+  if (d->kind < UNIRL_SDE_FLOW || d->kind > UNIRL_SDE_CPS) return UNIRL_E_DTYPE;
+  if ((d->prev_out && !dtype_ok(d->prev_dtype)) || (d->mean_out && !dtype_ok(d->mean_dtype))) return UNIRL_E_DTYPE;
+  if (B < 0 || D <= 0 || (d->sigma_stride != 0 && d->sigma_stride != 1)) return UNIRL_E_SHAPE;
+  // sample strides: 0 means densely packed; inputs may overlap or repeat (any stride >= 0 is
+  // readable), outputs must not alias across samples
+  const int64_t stride_v = d->noise_pred.sample_stride ? d->noise_pred.sample_stride : D;
+  const int64_t stride_x = d->sample.sample_stride ? d->sample.sample_stride : D;
+  const int64_t stride_p = d->prev_sample.sample_stride ? d->prev_sample.sample_stride : D;
+  const int64_t stride_n = d->noise_stride ? d->noise_stride : D;
+  const int64_t stride_po = d->prev_stride ? d->prev_stride : D;
+  const int64_t stride_mo = d->mean_stride ? d->mean_stride : D;
+  const int64_t stride_lp = d->logp_stride ? d->logp_stride : 1;
+  if (stride_v < 0 || stride_x < 0 || stride_p < 0 || stride_n < 0 || stride_po < D || stride_mo < D || stride_lp < 1)
+    return UNIRL_E_SHAPE;
   if (B == 0) return UNIRL_OK;
-  if (!noise_pred || !sample || !sigma || !sigma_next) return UNIRL_E_NULL;
+  const void* noise_pred = d->noise_pred.ptr;
+  const void* sample = d->sample.ptr;
+  const void* prev_sample = d->prev_sample.ptr;
+  if (!noise_pred || !sample || !d->sigma || !d->sigma_next) return UNIRL_E_NULL;
   const bool sampling = (prev_sample == nullptr);
-  const bool want_logp = (logp_out != nullptr) && !(eta < 1e-7);
+  if (!sampling && d->prev_sample.dtype != dtype_x) return UNIRL_E_DTYPE;
+  const bool want_logp = (d->logp_out != nullptr) && !(d->eta < 1e-7);
   if (want_logp && (!workspace || workspace_bytes < kWorkspaceBytes)) return UNIRL_E_WORKSPACE;
   const size_t sv = dtype_size(dtype_v), sx = dtype_size(dtype_x);
+  const size_t spo = d->prev_out ? dtype_size(d->prev_dtype) : 4, smo = d->mean_out ? dtype_size(d->mean_dtype) : 4;
   if (!aligned_to(noise_pred, sv) || !aligned_to(sample, sx) || !aligned_to(prev_sample, sx) ||
-      !aligned_to(noise, 4) || !aligned_to(prev_out, 4) || !aligned_to(mean_out, 4))
+      !aligned_to(d->noise, 4) || !aligned_to(d->prev_out, spo) || !aligned_to(d->mean_out, smo) ||
+      !aligned_to(d->logp_out, 4))
     return UNIRL_E_ALIGN;
 
   // 4-element vectors need every per-sample base to keep the vector alignment.
   int vec = 4;
   if (D % 4 != 0 || !aligned_to(noise_pred, 4 * sv) || !aligned_to(sample, 4 * sx) ||
-      !aligned_to(prev_sample, 4 * sx) || !aligned_to(noise, 16) || !aligned_to(prev_out, 16) ||
-      !aligned_to(mean_out, 16))
+      !aligned_to(prev_sample, 4 * sx) || !aligned_to(d->noise, 16) || !aligned_to(d->prev_out, 4 * spo) ||
+      !aligned_to(d->mean_out, 4 * smo) || stride_v % 4 || stride_x % 4 || (!sampling && stride_p % 4) ||
+      (sampling && d->noise && stride_n % 4) || (d->prev_out && stride_po % 4) || (d->mean_out && stride_mo % 4))
     vec = 1;
 
   const int items = (vec == 4) ? (int)tune_int("UNIRL_SDE_ITEMS", 4) : 2;
@@ -593,24 +628,31 @@ extern "C" int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const vo
 
   for (int64_t b0 = 0; b0 < B; b0 += per_launch) {
     const int64_t nb = (B - b0 < per_launch) ? (B - b0) : per_launch;
-    const int64_t off = b0 * D;
     SdeStepArgs A;
-    A.v = offset_ptr(noise_pred, off, sv);
-    A.x = offset_ptr(sample, off, sx);
-    A.third = sampling ? (const void*)offset_f32(noise, off) : offset_ptr(prev_sample, off, sx);
-    A.sigma = sigma + b0 * sigma_stride;
-    A.sigma_next = sigma_next + b0 * sigma_stride;
-    A.sigma_max_ptr = sigma_max_ptr;
-    A.sigma_max_val = sigma_max_val;
-    A.sigma_stride = sigma_stride;
-    A.sc = make_scalars(eta);
-    A.kind = kind;
+    A.v = offset_ptr(noise_pred, b0 * stride_v, sv);
+    A.x = offset_ptr(sample, b0 * stride_x, sx);
+    A.third = sampling ? (const void*)offset_f32(d->noise, b0 * stride_n) : offset_ptr(prev_sample, b0 * stride_p, sx);
+    A.stride_v = stride_v;
+    A.stride_x = stride_x;
+    A.stride_third = sampling ? stride_n : stride_p;
+    A.sigma = d->sigma + b0 * d->sigma_stride;
+    A.sigma_next = d->sigma_next + b0 * d->sigma_stride;
+    A.sigma_max_ptr = d->sigma_max_ptr;
+    A.sigma_max_val = d->sigma_max_val;
+    A.sigma_stride = d->sigma_stride;
+    A.sc = make_scalars(d->eta);
+    A.kind = d->kind;
     A.want_logp = want_logp ? 1 : 0;
-    A.logp_sum = logp_sum;
+    A.logp_sum = d->logp_sum;
     A.D = D;
-    A.prev_out = offset_f32(prev_out, off);
-    A.mean_out = offset_f32(mean_out, off);
-    A.logp_out = offset_f32(logp_out, b0);
+    A.prev_out = const_cast<void*>(offset_ptr(d->prev_out, b0 * stride_po, spo));
+    A.mean_out = const_cast<void*>(offset_ptr(d->mean_out, b0 * stride_mo, smo));
+    A.prev_dtype = d->prev_dtype;
+    A.mean_dtype = d->mean_dtype;
+    A.stride_prev = stride_po;
+    A.stride_mean = stride_mo;
+    A.logp_out = offset_f32(d->logp_out, b0 * stride_lp);
+    A.stride_logp = stride_lp;
     A.partials = ws_partials(workspace);
     A.nblk = nblk;
     A.items = items;
@@ -630,6 +672,35 @@ extern "C" int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const vo
     }
   }
   return UNIRL_OK;
+}
+
+extern "C" int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const void* sample, int dtype_x,
+                                   const void* prev_sample, const float* noise, const float* sigma,
+                                   const float* sigma_next, int sigma_stride, const float* sigma_max_ptr,
+                                   float sigma_max_val, double eta, int kind, int64_t B, int64_t D,
+                                   float* prev_out, float* mean_out, float* logp_out, int logp_sum,
+                                   void* workspace, size_t workspace_bytes, void* stream) {
+  unirl_sde_step_desc d = {};
+  d.noise_pred = {noise_pred, dtype_v, 0};
+  d.sample = {sample, dtype_x, 0};
+  d.prev_sample = {prev_sample, dtype_x, 0};
+  d.noise = noise;
+  d.sigma = sigma;
+  d.sigma_next = sigma_next;
+  d.sigma_stride = sigma_stride;
+  d.sigma_max_ptr = sigma_max_ptr;
+  d.sigma_max_val = sigma_max_val;
+  d.eta = eta;
+  d.kind = kind;
+  d.B = B;
+  d.D = D;
+  d.prev_out = prev_out;
+  d.prev_dtype = UNIRL_F32;
+  d.mean_out = mean_out;
+  d.mean_dtype = UNIRL_F32;
+  d.logp_out = logp_out;
+  d.logp_sum = logp_sum;
+  return unirl_sde_step_logp_ex(&d, workspace, workspace_bytes, stream);
 }
 
 extern "C" int unirl_sde_step_logp_bwd(const void* noise_pred, int dtype_v, const void* sample, int dtype_x,

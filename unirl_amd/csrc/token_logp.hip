@@ -222,10 +222,10 @@ struct TokArgs {
 };
 
 // One pass over the row; returns the workgroup's merged state in thread 0.
-template <typename T, int UNROLL, bool SAFE>
+template <typename T, int UNROLL, int TPB, bool SAFE>
 __device__ __forceinline__ TokState tok_scan_row(const T* __restrict__ p, int64_t V, float c, float (*lds)[5]) {
   constexpr int VEC = Stream16<T>::N;
-  constexpr int NW = kTokThreads / kWave;
+  constexpr int NW = TPB / kWave;
   constexpr int CHUNK = UNROLL * VEC;
 
   // peel to a 16-byte boundary
@@ -248,7 +248,7 @@ __device__ __forceinline__ TokState tok_scan_row(const T* __restrict__ p, int64_
   }
 
   const T* __restrict__ pv = p + head;
-  const int64_t per_iter = (int64_t)kTokThreads * UNROLL;
+  const int64_t per_iter = (int64_t)TPB * UNROLL;
   const int64_t n_full = nvec / per_iter;
   // Unguarded body: UNROLL vectors per lane, the lanes of a wavefront on consecutive 16-byte
   // words.  The next chunk's loads are issued before the current chunk is consumed.
@@ -256,11 +256,11 @@ __device__ __forceinline__ TokState tok_scan_row(const T* __restrict__ p, int64_
     const T* __restrict__ q = pv + (int64_t)threadIdx.x * VEC;
     u32x4 cur[UNROLL], nxt[UNROLL];
 #pragma unroll
-    for (int u = 0; u < UNROLL; ++u) cur[u] = stream_load16(q + (int64_t)u * kTokThreads * VEC);
+    for (int u = 0; u < UNROLL; ++u) cur[u] = stream_load16(q + (int64_t)u * TPB * VEC);
     for (int64_t it = 1; it < n_full; ++it) {  // every pass but the last prefetches unconditionally
       q += per_iter * VEC;
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u) nxt[u] = stream_load16(q + (int64_t)u * kTokThreads * VEC);
+      for (int u = 0; u < UNROLL; ++u) nxt[u] = stream_load16(q + (int64_t)u * TPB * VEC);
       float x[CHUNK];
 #pragma unroll
       for (int u = 0; u < UNROLL; ++u) Stream16<T>::unpack(cur[u], x + u * VEC);
@@ -274,7 +274,7 @@ __device__ __forceinline__ TokState tok_scan_row(const T* __restrict__ p, int64_
     tok_update<CHUNK, SAFE>(ref, acc, x, true, c);
   }
   // remainder: fewer than UNROLL vectors per lane; trip count is workgroup-uniform
-  for (int64_t i0 = n_full * per_iter; i0 < nvec; i0 += kTokThreads) {
+  for (int64_t i0 = n_full * per_iter; i0 < nvec; i0 += TPB) {
     const int64_t i = i0 + threadIdx.x;
     const bool on = i < nvec;
     float x[VEC];
@@ -307,9 +307,9 @@ __device__ __forceinline__ TokState tok_scan_row(const T* __restrict__ p, int64_
   return st;
 }
 
-template <typename T, int UNROLL>
-__global__ __launch_bounds__(kTokThreads) void token_logp_entropy_kernel(TokArgs A) {
-  __shared__ float lds[kTokThreads / kWave][5];
+template <typename T, int UNROLL, int TPB>
+__global__ __launch_bounds__(TPB) void token_logp_entropy_kernel(TokArgs A) {
+  __shared__ float lds[TPB / kWave][5];
   __shared__ int redo;
 
   const int64_t row = blockIdx.x;
@@ -317,10 +317,10 @@ __global__ __launch_bounds__(kTokThreads) void token_logp_entropy_kernel(TokArgs
   const int64_t V = A.V;
   const float c = A.c;
 
-  TokState st = tok_scan_row<T, UNROLL, false>(p, V, c, lds);
+  TokState st = tok_scan_row<T, UNROLL, TPB, false>(p, V, c, lds);
   if (threadIdx.x == 0) redo = !(fabsf(st.s) <= FLT_MAX) || !(fabsf(st.t) <= FLT_MAX);  // inf or NaN
   __syncthreads();
-  if (redo) st = tok_scan_row<T, 1, true>(p, V, c, lds);  // -inf (or NaN) logits in this row
+  if (redo) st = tok_scan_row<T, 1, TPB, true>(p, V, c, lds);  // -inf (or NaN) logits in this row
   if (threadIdx.x != 0) return;
 
   // sum = cnt*2^r0 + s relative to the reference r;  ln sum = r0 ln2 + ln cnt + log1p(s 2^-r0 / cnt)
@@ -430,19 +430,27 @@ __global__ __launch_bounds__(kTokThreads) void token_logp_bwd_kernel(TokBwdArgs 
   }
 }
 
+template <typename T, int TPB>
+static int launch_tok_tpb(const TokArgs& A, hipStream_t st, int unroll) {
+  dim3 grid((unsigned int)A.rows), block(TPB);
+  if (unroll >= 8)
+    hipLaunchKernelGGL((token_logp_entropy_kernel<T, 8, TPB>), grid, block, 0, st, A);
+  else if (unroll >= 4)
+    hipLaunchKernelGGL((token_logp_entropy_kernel<T, 4, TPB>), grid, block, 0, st, A);
+  else if (unroll >= 2)
+    hipLaunchKernelGGL((token_logp_entropy_kernel<T, 2, TPB>), grid, block, 0, st, A);
+  else
+    hipLaunchKernelGGL((token_logp_entropy_kernel<T, 1, TPB>), grid, block, 0, st, A);
+  return (int)hipGetLastError();
+}
+
 template <typename T>
 static int launch_tok(const TokArgs& A, hipStream_t st) {
   const int unroll = (int)tune_int("UNIRL_TOK_UNROLL", 4);
-  dim3 grid((unsigned int)A.rows), block(kTokThreads);
-  if (unroll >= 8)
-    hipLaunchKernelGGL((token_logp_entropy_kernel<T, 8>), grid, block, 0, st, A);
-  else if (unroll >= 4)
-    hipLaunchKernelGGL((token_logp_entropy_kernel<T, 4>), grid, block, 0, st, A);
-  else if (unroll >= 2)
-    hipLaunchKernelGGL((token_logp_entropy_kernel<T, 2>), grid, block, 0, st, A);
-  else
-    hipLaunchKernelGGL((token_logp_entropy_kernel<T, 1>), grid, block, 0, st, A);
-  return (int)hipGetLastError();
+  const int tpb = (int)tune_int("UNIRL_TOK_THREADS", 256);
+  if (tpb >= 1024) return launch_tok_tpb<T, 1024>(A, st, unroll);
+  if (tpb >= 512) return launch_tok_tpb<T, 512>(A, st, unroll);
+  return launch_tok_tpb<T, 256>(A, st, unroll);
 }
 
 }  // namespace unirl

@@ -118,6 +118,125 @@ def sde_step_logp(
     return prev_out, logp_out, mean_out
 
 
+def _per_sample_view(t: torch.Tensor, name: str, *, writable: bool = False) -> Tuple[torch.Tensor, int]:
+    """``(tensor, elements between consecutive samples)`` for a ``[B, ...]`` tensor whose samples
+    are each one contiguous block, e.g. ``stack[:, k]`` of a ``[B, K, ...]`` stack.  Inputs of any
+    other layout are copied; outputs must already have it."""
+    N.require_device(t, name)
+    B = t.shape[0]
+    D = t.numel() // B if B else 0
+    inner_ok = B == 0 or t[0].is_contiguous()
+    if inner_ok and (B <= 1 or t.stride(0) >= (D if writable else 0)):
+        return t, (t.stride(0) if B > 1 else D)
+    if writable:
+        raise ValueError(f"{name}: each sample must be one contiguous, non-overlapping block; got strides {t.stride()}")
+    t = t.contiguous()
+    return t, D
+
+
+def sde_step_logp_into(
+    noise_pred: torch.Tensor,
+    sample: torch.Tensor,
+    sigma: torch.Tensor,
+    sigma_next: torch.Tensor,
+    *,
+    kind: str = "flow",
+    eta: float = 1.0,
+    prev_sample: Optional[torch.Tensor] = None,
+    noise: Optional[torch.Tensor] = None,
+    sigma_max: Union[float, torch.Tensor] = 0.99,
+    prev_out: Optional[torch.Tensor] = None,
+    mean_out: Optional[torch.Tensor] = None,
+    logp_out: Optional[torch.Tensor] = None,
+    logp_sum: bool = False,
+) -> None:
+    """One fused SDE transition that reads strided ``[B, ...]`` views in place and writes into
+    caller-owned views (``unirl_sde_step_logp_ex``), no gradient.
+
+    ``sample`` / ``prev_sample`` may be ``stack[:, k]`` slices of a ``[B, K, ...]`` trajectory in
+    fp32, bf16 or fp16; ``prev_out`` / ``mean_out`` may be slices of such stacks in any of the
+    three dtypes (values are rounded to nearest-even on store); ``logp_out`` is a fp32 ``[B]``
+    view, e.g. ``log_probs[:, j]``.  ``logp_out`` is left untouched when ``eta < 1e-7``.
+    """
+    if sample.dim() < 2:
+        raise ValueError(f"sample needs a batch dimension and at least one more; got {tuple(sample.shape)}")
+    if noise_pred.shape != sample.shape:
+        raise ValueError(f"noise_pred {tuple(noise_pred.shape)} != sample {tuple(sample.shape)}")
+    device = sample.device
+    B = sample.shape[0]
+    D = sample.numel() // B if B else 0
+
+    def as_input(t, name):
+        t = t.detach()
+        if t.dtype not in N._DTYPE_CODE:
+            t = t.float()
+        return _per_sample_view(t, name)
+
+    v, sv = as_input(noise_pred, "noise_pred")
+    x, sx = as_input(sample, "sample")
+    pin, sp = None, 0
+    if prev_sample is not None:
+        if prev_sample.shape != sample.shape:
+            raise ValueError(f"prev_sample {tuple(prev_sample.shape)} != sample {tuple(sample.shape)}")
+        pin = prev_sample.detach()
+        if pin.dtype != x.dtype:
+            pin = pin.to(x.dtype)  # the reference's round trip through the input dtype
+        pin, sp = _per_sample_view(pin, "prev_sample")
+    nz, sn = None, 0
+    if noise is not None and prev_sample is None:
+        if noise.shape != sample.shape:
+            raise ValueError(f"noise {tuple(noise.shape)} != sample {tuple(sample.shape)}")
+        nz, sn = _per_sample_view(noise.detach().float(), "noise")
+
+    def as_output(t, name, shape):
+        if t is None:
+            return None, 0
+        if tuple(t.shape) != tuple(shape):
+            raise ValueError(f"{name} {tuple(t.shape)} != {tuple(shape)}")
+        if t.dtype not in N._DTYPE_CODE:
+            raise TypeError(f"{name}: unsupported dtype {t.dtype}")
+        if t.device != device:
+            raise ValueError(f"{name} lives on {t.device}, the inputs on {device}")
+        return _per_sample_view(t, name, writable=True)
+
+    po, spo = as_output(prev_out, "prev_out", sample.shape)
+    mo, smo = as_output(mean_out, "mean_out", sample.shape)
+    lp, slp = None, 0
+    if logp_out is not None:
+        N.require_device(logp_out, "logp_out")
+        if tuple(logp_out.shape) != (B,) or logp_out.dtype != torch.float32:
+            raise ValueError(f"logp_out must be float32 [{B}]; got {logp_out.dtype} {tuple(logp_out.shape)}")
+        lp, slp = logp_out, (logp_out.stride(0) if B > 1 else 1)
+        if B > 1 and slp < 1:
+            raise ValueError("logp_out must not alias across samples")
+    sig, stride = _sigma_arg(sigma, B, device, "sigma")
+    sig_n, stride_n = _sigma_arg(sigma_next, B, device, "sigma_next")
+    if stride != stride_n:
+        if stride == 0:
+            sig, stride = sig.expand(B).contiguous(), 1
+        else:
+            sig_n = sig_n.expand(B).contiguous()
+    smax_t, smax_v = _sigma_max_arg(sigma_max, device)
+    if B == 0 or D == 0:
+        return
+
+    d = N.SdeStepDesc()
+    d.noise_pred = N.SdeTensor(N.ptr(v), N.dtype_code(v.dtype), sv)
+    d.sample = N.SdeTensor(N.ptr(x), N.dtype_code(x.dtype), sx)
+    d.prev_sample = N.SdeTensor(N.ptr(pin), N.dtype_code(x.dtype), sp)
+    d.noise, d.noise_stride = N.ptr(nz), sn
+    d.sigma, d.sigma_next, d.sigma_stride = N.ptr(sig), N.ptr(sig_n), stride
+    d.sigma_max_ptr, d.sigma_max_val = N.ptr(smax_t), smax_v
+    d.eta, d.kind, d.B, d.D = float(eta), SDE_KINDS[kind], B, D
+    d.prev_out, d.prev_dtype, d.prev_stride = N.ptr(po), (N.dtype_code(po.dtype) if po is not None else 0), spo
+    d.mean_out, d.mean_dtype, d.mean_stride = N.ptr(mo), (N.dtype_code(mo.dtype) if mo is not None else 0), smo
+    d.logp_out, d.logp_stride, d.logp_sum = N.ptr(lp), slp, int(bool(logp_sum))
+    ws, ws_bytes = N.workspace(device)
+    with torch.cuda.device(device):
+        rc = N.lib().unirl_sde_step_logp_ex(ctypes.byref(d), N.ptr(ws), ws_bytes, N.current_stream(device))
+    N.check(rc, "unirl_sde_step_logp_ex")
+
+
 def sde_step_logp_bwd(
     noise_pred: torch.Tensor,
     sample: torch.Tensor,

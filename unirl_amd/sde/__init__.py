@@ -7,6 +7,7 @@ from .kernels import (
     FlowSDEStrategy,
     SDEStrategy,
     StepStrategy,
+    latents_at,
     sde_rollout,
 )
 from .runtime import calculate_dynamic_mu, get_sigma_schedule
@@ -20,5 +21,6 @@ __all__ = [
     "StepStrategy",
     "calculate_dynamic_mu",
     "get_sigma_schedule",
+    "latents_at",
     "sde_rollout",
 ]

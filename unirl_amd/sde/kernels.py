@@ -146,6 +146,61 @@ class StepStrategy(ABC):
         return prev, logp, mean
 
 
+    def denoise_into(
+        self,
+        noise_pred: torch.Tensor,
+        sample: torch.Tensor,
+        sigma: torch.Tensor,
+        sigma_next: torch.Tensor,
+        *,
+        eta: float = 1.0,
+        prev_sample: Optional[torch.Tensor] = None,
+        sigma_max: SigmaMax = 0.99,
+        noise: Optional[torch.Tensor] = None,
+        prev_out: Optional[torch.Tensor] = None,
+        mean_out: Optional[torch.Tensor] = None,
+        logp_out: Optional[torch.Tensor] = None,
+    ) -> bool:
+        """``denoise`` for the stage loops that keep trajectories as ``[B, K, ...]`` stacks
+        (``unirl/models/sd3/diffusion.py:366-406`` and ``:467-497``), without autograd.
+
+        ``sample`` / ``prev_sample`` may be ``latents[:, k]`` views (read in place);
+        ``prev_out`` / ``mean_out`` may be views into fp32 / bf16 / fp16 stacks and
+        ``logp_out`` a column ``log_probs[:, j]`` -- the kernel writes them directly, so the
+        loop needs no ``.to(trajectory_dtype)``, ``clone`` or ``torch.stack`` copies.  Storing
+        ``prev`` in ``sample.dtype`` is exact (it has been rounded to that dtype already);
+        storing the mean in a 16-bit dtype rounds once, like ``stack(...).to(dtype)``.
+        Returns ``False`` when ``eta < 1e-7`` (no log-prob; ``logp_out`` untouched).
+        """
+        if self._kind is None:
+            raise NotImplementedError(f"{type(self).__name__} has no fused kernel")
+        if not sample.is_cuda:
+            raise RuntimeError(
+                f"{type(self).__name__}.denoise_into: sample lives on {sample.device}; the fused SDE kernel "
+                "runs on a HIP device only and there is no CPU fallback"
+            )
+        if prev_sample is None and noise is None and float(eta) != 0.0:
+            noise = torch.randn(sample.shape, device=sample.device, dtype=torch.float32)
+        ops.sde_step_logp_into(
+            noise_pred, sample, sigma, sigma_next, kind=self._kind, eta=float(eta), prev_sample=prev_sample,
+            noise=noise, sigma_max=sigma_max, prev_out=prev_out, mean_out=mean_out, logp_out=logp_out,
+        )
+        return not (eta < 1e-7)
+
+
+def latents_at(latents: Optional[torch.Tensor], indices: Optional[torch.Tensor], step_idx: int) -> torch.Tensor:
+    """``latents[:, k]`` (a view) for the storage slot ``k`` with ``indices[k] == step_idx`` --
+    ``LatentSegment.latents_at`` (``unirl/types/segments/latent.py:82-97``) as a free function."""
+    if indices is None or latents is None:
+        raise RuntimeError("latents_at: missing indices or latents")
+    stored = [int(i) for i in indices.tolist()]
+    try:
+        k = stored.index(int(step_idx))
+    except ValueError:
+        raise KeyError(f"latents_at: step_idx={step_idx} not in stored indices={stored}") from None
+    return latents[:, k]
+
+
 class SDEStrategy(StepStrategy, ABC):
     """Stochastic strategies: a transition mean, a noise scale and a Gaussian log-prob."""
 
@@ -296,5 +351,6 @@ __all__ = [
     "SDEStrategy",
     "STRATEGIES",
     "StepStrategy",
+    "latents_at",
     "sde_rollout",
 ]
