@@ -411,7 +411,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": "f32",
         "data": "synthetic",
         "config": {
             "workload": f"token log-prob + entropy, logits bf16 [{args.rows},{args.vocab}] ~N(0,2) with 1% spiked "

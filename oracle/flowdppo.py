@@ -67,7 +67,10 @@ def sigma_t(sigmas: torch.Tensor, target_steps: List[int], eta: float, add_kl_co
 
 def gather_sde_field(tensor, sde_indices, target_steps, field_name="field"):
     if tensor is None or sde_indices is None:
-        raise ValueError(f"gather_sde_field: {field_name} or sde_indices is None")
+        raise ValueError(
+            f"gather_sde_field: {field_name} or sde_indices is None "
+            "(ensure prepare_segment ran before compute_loss_and_backward)."
+        )
     target_t = torch.tensor(target_steps, dtype=sde_indices.dtype)
     order = sde_indices.argsort()
     sorted_idx = sde_indices[order]
@@ -75,7 +78,9 @@ def gather_sde_field(tensor, sde_indices, target_steps, field_name="field"):
     pos = torch.searchsorted(sorted_idx, target_t).clamp(max=sorted_idx.shape[0] - 1)
     if (sorted_idx[pos] != target_t).any():
         bad = [int(t) for t, p in zip(target_steps, pos) if sorted_idx[p] != t]
-        raise ValueError(f"gather_sde_field({field_name}): target steps {bad} not in sde_indices")
+        raise ValueError(
+            f"gather_sde_field({field_name}): target steps {bad} not in sde_indices={sorted_idx.tolist()}"
+        )
     return tensor[:, pos.tolist()]
 
 

@@ -1,0 +1,109 @@
+"""Writes tests/golden/reference_vectors.npz: outputs of the UniRL reference itself for the two
+functions on the path whose behaviour is control flow rather than a formula, so that closed
+forms and brute force do not pin them:
+
+  * normalize_grouped / normalize_global   (unirl/algorithms/normalizers.py:8-84) -- the
+    trim-outliers branch, empty groups, the clip, the global-std switch;
+  * gather_sde_field                        (unirl/algorithms/base.py:46-80) -- argsort +
+    searchsorted + clamp + validation message.
+
+Only runs where the reference tree is mounted (/root/reference).  normalizers.py imports nothing
+but torch at module level, so it is loaded from its file.  base.py cannot be imported (its
+package pulls in ray, which is not installed); gather_sde_field is a pure function of torch
+tensors, so its definition alone is compiled out of the file's syntax tree and executed with
+torch in scope.  Nothing of the reference is written to the output: the file holds the inputs
+drawn here and the arrays (or the error text) the reference returned.
+
+Run:  python tests/golden/make_reference_vectors.py
+"""
+from __future__ import annotations
+
+import ast
+import importlib.util
+import json
+from pathlib import Path
+from typing import Dict, List, Optional
+
+import numpy as np
+import torch
+
+REF = Path("/root/reference/unirl")
+OUT = Path(__file__).with_name("reference_vectors.npz")
+
+
+def load_file_module(path: Path, name: str):
+    spec = importlib.util.spec_from_file_location(name, path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod
+
+
+def load_function(path: Path, func: str):
+    tree = ast.parse(path.read_text())
+    node = next(n for n in tree.body if isinstance(n, ast.FunctionDef) and n.name == func)
+    scope = {"torch": torch, "Optional": Optional, "List": List, "Dict": Dict}
+    exec(compile(ast.Module(body=[node], type_ignores=[]), str(path), "exec"), scope)
+    return scope[func]
+
+
+def main() -> None:
+    out: Dict[str, np.ndarray] = {}
+    g = torch.Generator().manual_seed(20240611)
+
+    # ---- normalizers -------------------------------------------------------
+    norm = load_file_module(REF / "algorithms" / "normalizers.py", "_ref_normalizers")
+    rewards = torch.randn(24, generator=g) * 2.0 + 0.5
+    rewards[5] = 9.0   # outliers for the trimmed statistics
+    rewards[17] = -7.0
+    groups = [
+        [0, 1, 2, 3, 4, 5, 6, 7],          # 8 members
+        [8, 9, 10],                         # 3 members (trim_size rounds to 0 at ratio 0.25)
+        [],                                 # empty: skipped
+        [11, 12],                           # 2 members: never trimmed
+        [13],                               # singleton: std() is NaN
+        [23, 14, 22, 15, 21, 16, 20, 17, 19, 18],  # 10 members, unordered
+    ]
+    out["ng_rewards"] = rewards.numpy()
+    out["ng_groups"] = np.frombuffer(json.dumps(groups).encode(), dtype=np.uint8)
+    cases = []
+    for ci, (trim, glob, clip) in enumerate(
+        [(0.0, False, None), (0.0, True, None), (0.0, False, 1.0), (0.125, False, None), (0.25, False, None),
+         (0.25, True, 1.5), (0.4, False, None), (0.5, False, None), (0.1, False, 0.5)]
+    ):
+        res = norm.normalize_grouped(rewards.clone(), groups, epsilon=1e-8, clip_max=clip,
+                                     trim_outliers_ratio=trim, use_global_std=glob)
+        out[f"ng_case{ci}_out"] = res.numpy()
+        cases.append({"trim": trim, "use_global_std": glob, "clip_max": clip})
+    out["ng_cases"] = np.frombuffer(json.dumps(cases).encode(), dtype=np.uint8)
+    out["nglobal_out"] = norm.normalize_global(rewards.clone(), epsilon=1e-8).numpy()
+    out["nglobal_clip_out"] = norm.normalize_global(rewards.clone(), epsilon=1e-6, clip_max=0.75).numpy()
+
+    # ---- gather_sde_field --------------------------------------------------
+    gather = load_function(REF / "algorithms" / "base.py", "gather_sde_field")
+    t = torch.randn(3, 6, 2, 5, generator=g)
+    sde_indices = torch.tensor([7, 2, 9, 0, 4, 13])
+    out["gs_tensor"] = t.numpy()
+    out["gs_indices"] = sde_indices.numpy()
+    gcases = []
+    for gi, target in enumerate([[2, 9], [0, 4, 7, 13], [9], [4, 4, 0], [13, 0], [7, 2, 9, 0, 4, 13]]):
+        out[f"gs_case{gi}_out"] = gather(t, sde_indices, target, field_name="sde_means").numpy()
+        gcases.append({"target": target})
+    for target in ([2, 3], [14], [-1, 0], [5, 6, 7]):
+        try:
+            gather(t, sde_indices, target, field_name="sde_logp")
+            gcases.append({"target": target, "error": None})
+        except ValueError as e:
+            gcases.append({"target": target, "error": str(e)})
+    for a, b in ((None, sde_indices), (t, None)):
+        try:
+            gather(a, b, [2], field_name="sde_logp")
+        except ValueError as e:
+            gcases.append({"target": None, "none_arg": 0 if a is None else 1, "error": str(e)})
+    out["gs_cases"] = np.frombuffer(json.dumps(gcases).encode(), dtype=np.uint8)
+
+    np.savez_compressed(OUT, **out)
+    print(f"wrote {OUT} ({OUT.stat().st_size} bytes, {len(out)} arrays)")
+
+
+if __name__ == "__main__":
+    main()

@@ -92,6 +92,12 @@ struct Elem<f16_t> {
   static __device__ __forceinline__ float round_trip(float v) { return f16_bits_to_f32(f32_to_f16_bits(v)); }
 };
 
+// torch.maximum / torch.minimum / torch.clamp propagate NaN; fmaxf / fminf drop it.
+__device__ __forceinline__ float nan_max(float a, float b) { return (a != a) ? a : ((b != b) ? b : fmaxf(a, b)); }
+__device__ __forceinline__ float nan_min(float a, float b) { return (a != a) ? a : ((b != b) ? b : fminf(a, b)); }
+__device__ __forceinline__ float nan_clamp(float v, float lo, float hi) { return (v != v) ? v : fminf(fmaxf(v, lo), hi); }
+__device__ __forceinline__ float quiet_nan() { return __uint_as_float(0x7fc00000u); }
+
 // Streaming (non-temporal) 8/16-byte accesses for data that is touched exactly once.
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));

@@ -232,11 +232,14 @@ __global__ __launch_bounds__(kKlThreads) void flowdppo_loss_kernel(DppoArgs A) {
   const float nf = (float)A.n;
   M[0] = (float)(tot[D_SR] / N);
   M[1] = (float)sqrt(var);
-  M[2] = rmin;
-  M[3] = rmax;
+  // min()/max() of the reference return NaN when any element is NaN; ratios and KL values are
+  // >= 0, so their sums are NaN exactly then
+  const bool r_nan = tot[D_SR] != tot[D_SR], kl_nan = tot[D_KL] != tot[D_KL];
+  M[2] = r_nan ? quiet_nan() : rmin;
+  M[3] = r_nan ? quiet_nan() : rmax;
   M[4] = (float)(tot[D_LD2] / N);
   M[5] = (float)(tot[D_KL] / N);
-  M[6] = klmax;
+  M[6] = kl_nan ? quiet_nan() : klmax;
   M[7] = (float)tot[D_NKL] / nf;
   M[8] = (float)tot[D_POS] / nf;
   M[9] = (float)tot[D_NEG] / nf;

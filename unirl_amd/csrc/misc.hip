@@ -209,7 +209,7 @@ __global__ __launch_bounds__(kAdvThreads) void normalize_grouped_kernel(NormArgs
     const float mean_f = (float)mean;
     for (int64_t a = lo; a < hi; ++a) {
       float v = (A.r[A.members[a]] - mean_f) / scale;
-      if (A.has_clip) v = fminf(fmaxf(v, -A.clip_max), A.clip_max);
+      if (A.has_clip) v = nan_clamp(v, -A.clip_max, A.clip_max);  // torch.clamp keeps NaN
       A.out[A.members[a]] = v;
     }
   }

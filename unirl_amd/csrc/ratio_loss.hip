@@ -77,9 +77,9 @@ __device__ __forceinline__ TokVals ratio_token(float nw, float od, float A, cons
     o.r = expf(o.ld);
     const float nA = -A;
     const float u = nA * o.r;
-    const float rc = fminf(fmaxf(o.r, C.clamp_lo), C.clamp_hi);
+    const float rc = nan_clamp(o.r, C.clamp_lo, C.clamp_hi);
     const float c = nA * rc;
-    o.loss = fmaxf(u, c);
+    o.loss = nan_max(u, c);
     o.hi = (o.r - 1.0f) > C.eps_hi;
     o.lo = (1.0f - o.r) > C.eps_lo;
     o.kterm = 0.5f * (o.ld * o.ld);
@@ -88,7 +88,7 @@ __device__ __forceinline__ TokVals ratio_token(float nw, float od, float A, cons
     const float dc = inside ? c : 0.0f;
     o.dloss = (u > c) ? u : ((u < c) ? dc : 0.5f * (u + dc));
   } else {
-    o.ld = fminf(fmaxf(o.d0, -20.0f), 20.0f);
+    o.ld = nan_clamp(o.d0, -20.0f, 20.0f);
     o.r = expf(o.ld);
     const float mu = expf(od);
     const float rd = o.r - 1.0f;
@@ -343,15 +343,17 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
   M[UNIRL_M_LOSS] = (float)loss;
   M[UNIRL_M_RATIO_MEAN] = (float)(sr / N);
   M[UNIRL_M_RATIO_STD] = (float)sqrt(var);
-  M[UNIRL_M_RATIO_MIN] = (float)lds_fin[P_RMIN];
-  M[UNIRL_M_RATIO_MAX] = (float)lds_fin[P_RMAX];
+  // min()/max() of the reference return NaN when any ratio is NaN; the ratios are >= 0, so their
+  // sum is NaN exactly then (likewise the absolute differences below)
+  M[UNIRL_M_RATIO_MIN] = (sr != sr) ? quiet_nan() : (float)lds_fin[P_RMIN];
+  M[UNIRL_M_RATIO_MAX] = (sr != sr) ? quiet_nan() : (float)lds_fin[P_RMAX];
   M[UNIRL_M_CLIP_FRACTION] = (float)lds_fin[P_CANY] / (float)N;
   M[UNIRL_M_CLIPFRAC_HI] = (float)lds_fin[P_CHI] / (float)N;
   M[UNIRL_M_CLIPFRAC_LO] = (float)lds_fin[P_CLO] / (float)N;
   M[UNIRL_M_APPROX_KL] = (float)(lds_fin[P_KL] / N);
   M[UNIRL_M_PENALTY_MEAN] = (float)(lds_fin[P_PEN] / N);
   M[UNIRL_M_ABSDIFF_MEAN] = (float)(lds_fin[P_ABS] / N);
-  M[UNIRL_M_ABSDIFF_MAX] = (float)lds_fin[P_AMAX];
+  M[UNIRL_M_ABSDIFF_MAX] = (lds_fin[P_ABS] != lds_fin[P_ABS]) ? quiet_nan() : (float)lds_fin[P_AMAX];
   M[UNIRL_M_NUM_TOKENS] = (float)N;
   M[13] = M[14] = M[15] = 0.0f;
 }

@@ -323,6 +323,24 @@ __global__ __launch_bounds__(TPB) void token_logp_entropy_kernel(TokArgs A) {
   if (redo) st = tok_scan_row<T, 1, TPB, true>(p, V, c, lds);  // -inf (or NaN) logits in this row
   if (threadIdx.x != 0) return;
 
+  if (st.m == INFINITY) {
+    // a +inf logit: logsumexp is +inf, so a finite logit has log-prob -inf and the +inf logit
+    // itself inf - inf = NaN; softmax is 0/NaN, so the entropy is NaN.  A NaN anywhere in the row
+    // (st.s is NaN then) makes everything NaN.
+    const bool has_nan = st.s != st.s;
+    if (A.lse) A.lse[row] = has_nan ? quiet_nan() : INFINITY;
+    if (A.ent) A.ent[row] = quiet_nan();
+    if (A.logp) {
+      const int64_t id = A.ids[row];
+      float out = quiet_nan();
+      if (!has_nan && id >= 0 && id < V) {
+        const float x_id = Elem<T>::load(p + id);
+        if (x_id < INFINITY) out = -INFINITY;  // false for +inf and NaN
+      }
+      A.logp[row] = out;
+    }
+    return;
+  }
   // sum = cnt*2^r0 + s relative to the reference r;  ln sum = r0 ln2 + ln cnt + log1p(s 2^-r0 / cnt)
   const double r0 = (double)fmaf(st.m, c, -st.r);
   const double cnt = (double)st.cnt;
