@@ -346,6 +346,18 @@ int unirl_normalize_grouped(const float* rewards, int64_t n, const int64_t* memb
 int unirl_gather_steps(const void* src, int64_t B, int64_t S, int64_t inner_bytes,
                        const int64_t* positions, int64_t n_pos, void* out, void* stream);
 
+/* ------------------------------------------------------------------------
+ * out[b, :] = cast(src[group_of[b], :]) -- the device half of the x_T noise
+ * recipe (unirl/sde/noise.py:72-97, :178-187): the reference draws one fp32
+ * CPU tensor per noise group, stacks one copy per SAMPLE on the host, and
+ * uploads and casts the whole batch.  Here only the U unique draws cross PCIe
+ * (src f32 [U, D]); this kernel replicates them to the B samples and applies
+ * the final cast (round to nearest even) in the same pass.  group_of is a
+ * device int64 [B] with values in [0, U).
+ * ---------------------------------------------------------------------- */
+int unirl_expand_groups(const float* src, int64_t U, int64_t D, const int64_t* group_of, int64_t B,
+                        void* out, int out_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

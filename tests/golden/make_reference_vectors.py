@@ -1,14 +1,17 @@
-"""Writes tests/golden/reference_vectors.npz: outputs of the UniRL reference itself for the two
-functions on the path whose behaviour is control flow rather than a formula, so that closed
+"""Writes tests/golden/reference_vectors.npz: outputs of the UniRL reference itself for the three
+pieces of the path whose behaviour is control flow or a library recipe rather than a formula, so that closed
 forms and brute force do not pin them:
 
   * normalize_grouped / normalize_global   (unirl/algorithms/normalizers.py:8-84) -- the
     trim-outliers branch, empty groups, the clip, the global-std switch;
   * gather_sde_field                        (unirl/algorithms/base.py:46-80) -- argsort +
-    searchsorted + clamp + validation message.
+    searchsorted + clamp + validation message;
+  * the x_T noise recipe                    (unirl/sde/noise.py:26-187) -- blake2b seed derivation,
+    one seeded CPU generator per noise group, sharing inside a group, cast as the last step.
 
-Only runs where the reference tree is mounted (/root/reference).  normalizers.py imports nothing
-but torch at module level, so it is loaded from its file.  base.py cannot be imported (its
+Only runs where the reference tree is mounted (/root/reference).  normalizers.py and noise.py
+import nothing but torch and the standard library at module level, so they are loaded from their
+files.  base.py cannot be imported (its
 package pulls in ray, which is not installed); gather_sde_field is a pure function of torch
 tensors, so its definition alone is compiled out of the file's syntax tree and executed with
 torch in scope.  Nothing of the reference is written to the output: the file holds the inputs
@@ -100,6 +103,21 @@ def main() -> None:
         except ValueError as e:
             gcases.append({"target": None, "none_arg": 0 if a is None else 1, "error": str(e)})
     out["gs_cases"] = np.frombuffer(json.dumps(gcases).encode(), dtype=np.uint8)
+
+    # ---- x_T noise recipe ----------------------------------------------------
+    noise = load_file_module(REF / "sde" / "noise.py", "_ref_noise")
+    gids = ["p0", "p0", "p1", "p0", "p2", "7", "p1"]
+    out["nz_gids"] = np.frombuffer(json.dumps(gids).encode(), dtype=np.uint8)
+    out["nz_seeds"] = np.array([noise._derive_group_seed(1234, g) for g in gids], dtype=np.int64)
+    out["nz_seed_big"] = np.array([noise._derive_group_seed((1 << 62) + 5, "prompt-000017")], dtype=np.int64)
+    for tag, shape in (("a", (4, 8, 8)), ("b", (3,)), ("c", (2, 3, 5, 7))):
+        x = noise.regen_initial_noise(gids, 1234, shape, torch.device("cpu"), torch.float32)
+        out[f"nz_{tag}_f32"] = x.numpy()
+        xb = noise.regen_initial_noise(gids, 1234, shape, torch.device("cpu"), torch.bfloat16)
+        out[f"nz_{tag}_bf16_bits"] = xb.view(torch.int16).numpy()
+    out["nz_latents_same"] = noise.generate_latents(
+        4, (2, 9), torch.device("cpu"), torch.float32, init_same_noise=True, samples_per_prompt=2,
+        noise_group_ids=["g0", "g0", "g1", "g1"], base_seed=99).numpy()
 
     np.savez_compressed(OUT, **out)
     print(f"wrote {OUT} ({OUT.stat().st_size} bytes, {len(out)} arrays)")

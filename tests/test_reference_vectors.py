@@ -99,3 +99,60 @@ def test_kernel_normalize_global_and_gather(dev):
     tb = t.to(torch.bfloat16)
     got = gather_sde_field(tb, idx, [9, 0], field_name="sde_means")
     assert torch.equal(got.cpu(), tb.cpu()[:, [2, 3]])
+
+
+# ---------------------------------------------------------------- x_T noise recipe (unirl/sde/noise.py)
+NZ_GIDS = meta("nz_gids")
+NZ_SHAPES = {"a": (4, 8, 8), "b": (3,), "c": (2, 3, 5, 7)}
+
+
+def test_noise_seed_derivation_and_host_recipe():
+    from unirl_amd.sde import noise
+
+    assert [noise._derive_group_seed(1234, g) for g in NZ_GIDS] == R["nz_seeds"].tolist()
+    assert noise._derive_group_seed((1 << 62) + 5, "prompt-000017") == int(R["nz_seed_big"][0])
+    cpu = torch.device("cpu")
+    for tag, shape in NZ_SHAPES.items():
+        x = noise.regen_initial_noise(NZ_GIDS, 1234, shape, cpu, torch.float32)
+        assert torch.equal(x, torch.from_numpy(R[f"nz_{tag}_f32"]))
+        xb = noise.regen_initial_noise(NZ_GIDS, 1234, shape, cpu, torch.bfloat16)
+        assert torch.equal(xb.view(torch.int16), torch.from_numpy(R[f"nz_{tag}_bf16_bits"]))
+    same = noise.generate_latents(4, (2, 9), cpu, torch.float32, init_same_noise=True, samples_per_prompt=2,
+                                  noise_group_ids=["g0", "g0", "g1", "g1"], base_seed=99)
+    assert torch.equal(same, torch.from_numpy(R["nz_latents_same"]))
+    assert noise.generate_latents(3, (2, 2), cpu).shape == (3, 2, 2)
+    with pytest.raises(ValueError, match="requires explicit noise_group_ids aligned to batch_size"):
+        noise.generate_shared_noise(3, (2,), cpu, noise_group_ids=["a", "b"])
+    with pytest.raises(ValueError, match="noise_group_ids_len=None"):
+        noise.generate_shared_noise(3, (2,), cpu, noise_group_ids=None)
+    with pytest.raises(AssertionError):
+        noise.generate_latents(2, (2,), cpu, init_same_noise=True)
+
+
+@pytest.mark.gpu
+def test_noise_recipe_on_device_is_byte_identical(dev):
+    from unirl_amd.sde import noise
+
+    for _ in range(2):  # the second pass reuses the pinned staging buffer
+        for tag, shape in NZ_SHAPES.items():
+            ref = torch.from_numpy(R[f"nz_{tag}_f32"])
+            x = noise.regen_initial_noise(NZ_GIDS, 1234, shape, dev, torch.float32)
+            assert x.is_cuda and x.dtype == torch.float32 and torch.equal(x.cpu(), ref)
+            xb = noise.regen_initial_noise(NZ_GIDS, 1234, shape, dev, torch.bfloat16)
+            assert torch.equal(xb.cpu().view(torch.int16), torch.from_numpy(R[f"nz_{tag}_bf16_bits"]))
+            xh = noise.regen_initial_noise(NZ_GIDS, 1234, shape, dev, torch.float16)
+            assert torch.equal(xh.cpu(), ref.to(torch.float16))
+    # a realistic batch: 64 samples in 4 groups of SD3-sized latents; samples of a group are equal
+    gids = [f"prompt-{i // 16}" for i in range(64)]
+    x = noise.regen_initial_noise(gids, 7, (16, 64, 64), dev, torch.bfloat16)
+    assert x.shape == (64, 16, 64, 64)
+    assert torch.equal(x[0], x[15]) and torch.equal(x[16], x[31]) and not torch.equal(x[0], x[16])
+    g = torch.Generator().manual_seed(noise._derive_group_seed(7, "prompt-2"))
+    assert torch.equal(x[40].cpu(), torch.randn(16, 64, 64, generator=g).to(torch.bfloat16))
+    # device-side draws (no recipe): groups still share, shapes and dtypes as asked
+    y = noise.generate_shared_noise(4, (8, 8), dev, torch.float32, ["a", "b", "a", "c"], base_seed=3)
+    assert y.is_cuda and torch.equal(y[0], y[2]) and not torch.equal(y[0], y[1])
+    y2 = noise.generate_shared_noise(4, (8, 8), dev, torch.float32, ["a", "b", "a", "c"], base_seed=3)
+    assert torch.equal(y, y2)
+    assert noise.generate_shared_noise(2, (4,), dev, torch.bfloat16, ["a", "a"]).dtype == torch.bfloat16
+    assert noise.regen_initial_noise([], 1, (4, 4), dev).shape == (0, 4, 4)

@@ -159,6 +159,7 @@ _SIGNATURES = {
         [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_float, c_float, c_int, c_int, c_float, c_void_p,
          c_void_p],
     ),
+    "unirl_expand_groups": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_int, c_void_p]),
     "unirl_gather_steps": (
         c_int,
         [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p, c_void_p],

@@ -215,6 +215,45 @@ __global__ __launch_bounds__(kAdvThreads) void normalize_grouped_kernel(NormArgs
   }
 }
 
+// out[b, :] = cast(src[group_of[b], :]): the batch of initial latents from one fp32 draw per
+// noise group (unirl/sde/noise.py:78-97 stacks the shared draws; :187 casts as the last step).
+struct ExpandArgs {
+  const float* src;         // [U, D]
+  const int64_t* group_of;  // [B], values in [0, U)
+  int64_t U, D;
+  void* out;                // [B, D]
+  int dtype;
+};
+
+template <typename TO, int VEC>
+__global__ __launch_bounds__(kGatherThreads) void expand_groups_kernel(ExpandArgs A) {
+  const int64_t b = blockIdx.y;
+  int64_t u = A.group_of[b];
+  u = u < 0 ? 0 : (u >= A.U ? A.U - 1 : u);  // validated by the caller; never index outside src
+  const float* __restrict__ s = A.src + u * A.D;
+  TO* __restrict__ o = reinterpret_cast<TO*>(A.out) + b * A.D;
+  const int64_t nvec = A.D / VEC;
+  const int64_t stride = (int64_t)gridDim.x * kGatherThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kGatherThreads + threadIdx.x; i < nvec; i += stride) {
+    float v[VEC];
+    Vec<float, VEC>::load(s + i * VEC, v);
+    Vec<TO, VEC>::store(o + i * VEC, v);
+  }
+}
+
+template <typename TO>
+static int launch_expand(const ExpandArgs& A, int64_t B, int vec, hipStream_t st) {
+  int64_t nbx = (A.D / vec + kGatherThreads * 4 - 1) / (kGatherThreads * 4);
+  if (nbx > 1024) nbx = 1024;
+  if (nbx < 1) nbx = 1;
+  dim3 grid((unsigned int)nbx, (unsigned int)B), block(kGatherThreads);
+  if (vec == 4)
+    hipLaunchKernelGGL((expand_groups_kernel<TO, 4>), grid, block, 0, st, A);
+  else
+    hipLaunchKernelGGL((expand_groups_kernel<TO, 1>), grid, block, 0, st, A);
+  return (int)hipGetLastError();
+}
+
 }  // namespace unirl
 
 using namespace unirl;
@@ -331,4 +370,36 @@ extern "C" int unirl_normalize_grouped(const float* rewards, int64_t n, const in
   A.out = out;
   hipLaunchKernelGGL(normalize_grouped_kernel, dim3(1), dim3(kAdvThreads), 0, (hipStream_t)stream, A);
   return (int)hipGetLastError();
+}
+
+extern "C" int unirl_expand_groups(const float* src, int64_t U, int64_t D, const int64_t* group_of, int64_t B,
+                                   void* out, int out_dtype, void* stream) {
+  if (!dtype_ok(out_dtype)) return UNIRL_E_DTYPE;
+  if (U < 0 || D < 0 || B < 0) return UNIRL_E_SHAPE;
+  if (B == 0 || D == 0) return UNIRL_OK;
+  if (U == 0) return UNIRL_E_SHAPE;
+  if (!src || !group_of || !out) return UNIRL_E_NULL;
+  const size_t so = dtype_size(out_dtype);
+  if (!aligned_to(src, 4) || !aligned_to(group_of, 8) || !aligned_to(out, so)) return UNIRL_E_ALIGN;
+  const int vec = (D % 4 == 0 && aligned_to(src, 16) && aligned_to(out, 4 * so)) ? 4 : 1;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t per_launch = 32768;  // grid.y limit is 65535
+  for (int64_t b0 = 0; b0 < B; b0 += per_launch) {
+    const int64_t nb = (B - b0 < per_launch) ? (B - b0) : per_launch;
+    ExpandArgs A;
+    A.src = src;
+    A.group_of = group_of + b0;
+    A.U = U;
+    A.D = D;
+    A.out = reinterpret_cast<char*>(out) + b0 * D * (int64_t)so;
+    A.dtype = out_dtype;
+    int rc = UNIRL_E_DTYPE;
+    switch (out_dtype) {
+      case UNIRL_F32: rc = launch_expand<float>(A, nb, vec, st); break;
+      case UNIRL_BF16: rc = launch_expand<bf16_t>(A, nb, vec, st); break;
+      case UNIRL_F16: rc = launch_expand<f16_t>(A, nb, vec, st); break;
+    }
+    if (rc != 0) return rc;
+  }
+  return UNIRL_OK;
 }

@@ -828,6 +828,29 @@ def gather_steps(tensor: torch.Tensor, positions: Sequence[int]) -> torch.Tensor
     return out
 
 
+def expand_groups(unique: torch.Tensor, group_of: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    """``out[b] = unique[group_of[b]].to(dtype)`` for fp32 ``unique [U, ...]`` and int64 ``group_of [B]``
+    (values in ``[0, U)``, checked by the caller), as one kernel."""
+    N.require_device(unique, "unique")
+    if unique.dtype != torch.float32:
+        raise TypeError(f"unique must be float32; got {unique.dtype}")
+    src = unique if unique.is_contiguous() else unique.contiguous()
+    idx = group_of.detach().to(device=src.device, dtype=torch.int64).reshape(-1).contiguous()
+    U, B = src.shape[0], idx.numel()
+    D = src.numel() // U if U else 0
+    out = torch.empty((B,) + tuple(src.shape[1:]), dtype=dtype, device=src.device)
+    if B == 0 or D == 0:
+        return out
+    if U == 0:
+        raise ValueError("no noise groups to expand")
+    with torch.cuda.device(src.device):
+        rc = N.lib().unirl_expand_groups(
+            N.ptr(src), U, D, N.ptr(idx), B, N.ptr(out), N.dtype_code(dtype), N.current_stream(src.device)
+        )
+    N.check(rc, "unirl_expand_groups")
+    return out
+
+
 METRIC_SLOTS: Dict[str, int] = {
     "loss": N.M_LOSS,
     "ratio_mean": N.M_RATIO_MEAN,

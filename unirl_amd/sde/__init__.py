@@ -10,6 +10,7 @@ from .kernels import (
     latents_at,
     sde_rollout,
 )
+from .noise import generate_latents, generate_shared_noise, regen_initial_noise
 from .runtime import calculate_dynamic_mu, get_sigma_schedule
 
 __all__ = [
@@ -20,7 +21,10 @@ __all__ = [
     "STRATEGIES",
     "StepStrategy",
     "calculate_dynamic_mu",
+    "generate_latents",
+    "generate_shared_noise",
     "get_sigma_schedule",
     "latents_at",
+    "regen_initial_noise",
     "sde_rollout",
 ]
