@@ -143,7 +143,7 @@ def make_shapes(torch, dev):
 
     shapes.append(dict(
         name="sde_step_logp", config=1, shape="fp32 [8,16,128,128], step 10/28, shift 3, eta 0.7, sampling",
-        bytes=bytes1, elements=numel, run=run1, sets=ns,
+        bytes=bytes1, read_bytes=3 * numel * 4, write_bytes=2 * numel * 4, elements=numel, run=run1, sets=ns,
         cpu=lambda: osde.sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7, noise=host1[2],
                                      sigma_max=sig[1]),
         cpu_bytes=bytes1,
@@ -171,7 +171,8 @@ def make_shapes(torch, dev):
         shapes.append(dict(
             name=f"ratio_loss_{kind}", config=3,
             shape=f"fp32 [256,8192] padded, {n_valid} valid tokens, 16x16 groups, token-mean",
-            bytes=bytes3_valid, bytes_padded=bytes3_padded, elements=n_valid,
+            bytes=bytes3_valid, bytes_padded=bytes3_padded, read_bytes=bytes3_valid, write_bytes=0,
+            elements=n_valid,
             run=(lambda i, k=kind: plans[k][i % ns3].forward(False)), sets=ns3,
             cpu=(lambda k=kind, o=okw: olos.token_loss(k, newp, oldp, adv, lengths, **o)), cpu_bytes=bytes3_valid,
         ))
@@ -195,7 +196,7 @@ def make_shapes(torch, dev):
 
     shapes.append(dict(
         name="gaussian_kl_mask", config=4, shape="bf16 [2,16,21,60,104] old/new means, threshold 0.01",
-        bytes=bytes4, elements=old_m.numel(), run=run4, sets=ns4,
+        bytes=bytes4, read_bytes=bytes4, write_bytes=0, elements=old_m.numel(), run=run4, sets=ns4,
         cpu=lambda: ofd.kl_per_sample(new_m, old_m, sig_t.reshape(1, 1, 1, 1, 1, 1)) < 0.01, cpu_bytes=bytes4,
     ))
 
@@ -213,10 +214,27 @@ def make_shapes(torch, dev):
 
     shapes.append(dict(
         name="sde_rollout_logp", config=5, shape="fp32 [16,4096,64], 10 steps from step 0, eta 0.7",
-        bytes=bytes5, elements=10 * x0.numel(), run=run5, sets=1,
+        bytes=bytes5, read_bytes=21 * x0.numel() * 4, write_bytes=x0.numel() * 4, elements=10 * x0.numel(),
+        run=run5, sets=1,
         cpu=lambda: osde.sde_rollout("flow", x0, vs, nz, sig, 0.7), cpu_bytes=bytes5, cpu_reps=3,
     ))
     return shapes
+
+
+def make_floor(torch, dev, read_bytes: int, write_bytes: int, n_sets: int, tail_launch: bool):
+    """The launch floor of a shape: a kernel that only moves the shape's bytes (same read / write
+    split, rotating buffers), plus the minimal dependent second launch of a two-launch reduction."""
+    from unirl_amd import ops
+
+    rb, wb = (read_bytes + 15) // 16 * 16, (write_bytes + 15) // 16 * 16
+    srcs = [torch.ones(max(rb, 16), dtype=torch.uint8, device=dev) for _ in range(n_sets)]
+    dsts = [torch.empty(max(wb, 16), dtype=torch.uint8, device=dev) for _ in range(n_sets)]
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+    def run(i):
+        ops.calib_stream(srcs[i % n_sets], rb, dsts[i % n_sets], wb, sink, tail_launch=tail_launch)
+
+    return run
 
 
 def make_headline(torch, dev, rows: int, vocab: int):
@@ -380,13 +398,21 @@ def main() -> int:
             }
             if "bytes_padded" in sh:
                 row["gbps_padded_bytes"] = round(sh["bytes_padded"] / (us * 1e-6) / 1e9, 1)
+            try:  # what a kernel that only moves these bytes costs in the same harness
+                floor_run = make_floor(torch, dev, sh["read_bytes"], sh["write_bytes"], sh["sets"], True)
+                floor_us = time_in_graph(torch, floor_run, sh["sets"])
+                row["floor_us"] = round(floor_us, 2)
+                row["frac_of_floor"] = round(floor_us / us, 4)
+                del floor_run
+            except Exception as exc:
+                log(f"{sh['name']}: floor measurement failed ({type(exc).__name__}: {exc})")
             if not args.skip_cpu:
                 cms = time_cpu(sh["cpu"], reps=sh.get("cpu_reps", 5), warmup=1)
                 row["cpu_ms"] = round(cms, 2)
                 row["cpu_gbps"] = round(sh["cpu_bytes"] / (cms * 1e-3) / 1e9, 3)
                 row["cpu_cores"] = torch.get_num_threads()
             log(f"{sh['name']}: {us:.2f} us/launch, {gbps:.0f} GB/s = {gbps / HBM_PEAK_GBPS:.1%} of peak, "
-                f"wrapper {lat:.0f} us")
+                f"floor {row.get('floor_us', float('nan')):.2f} us, wrapper {lat:.0f} us")
             shapes_out.append(row)
 
     # HBM bytes per launch from hardware counters, when a committed counter summary covers this workload

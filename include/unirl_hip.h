@@ -67,6 +67,16 @@ int unirl_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
  * counters read for this kernel calibrate the ones read for the kernels below. */
 int unirl_calib_copy(const void* src, void* dst, size_t bytes, void* stream);
 
+/* Measurement aid, no counterpart in the reference: the launch floor of a
+ * streaming kernel.  One kernel reads `read_bytes` from src and writes
+ * `write_bytes` to dst (multiples of 16, 16-byte aligned; the two streams are
+ * independent and no arithmetic is done), followed, when tail_launch != 0, by
+ * a one-wavefront kernel -- the shape of a fused kernel plus its finalize
+ * launch.  Timing it for the byte counts of a fused kernel gives the time no
+ * kernel of that traffic can beat on the device.  sink: 16 writable bytes. */
+int unirl_calib_stream(const void* src, size_t read_bytes, void* dst, size_t write_bytes,
+                       int tail_launch, void* sink, void* stream);
+
 /* ------------------------------------------------------------------------
  * One SDE transition + per-sample Gaussian log-prob.
  * Replaces StepStrategy.denoise -> SDEStrategy.step -> _finalize_logp

@@ -19,6 +19,38 @@ __global__ __launch_bounds__(256) void calib_copy_kernel(const u32x4* __restrict
     stream_store16(dst + i, stream_load16(src + i));
 }
 
+// Launch-floor yardstick: reads `n_read` and writes `n_write` 16-byte vectors with no arithmetic
+// and no dependence between the two streams, four vectors in flight per lane like the fused
+// kernels.  `sink` only keeps the loads alive.
+__global__ __launch_bounds__(256) void calib_stream_kernel(const u32x4* __restrict__ src, size_t n_read,
+                                                           u32x4* __restrict__ dst, size_t n_write,
+                                                           unsigned int* sink) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  const size_t n = n_read > n_write ? n_read : n_write;
+  u32x4 acc = {0u, 0u, 0u, 0u};
+  const u32x4 fill = {0x3f800000u, 0x3f800000u, 0x3f800000u, 0x3f800000u};
+  for (size_t i0 = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i0 < n; i0 += 4 * stride) {
+    u32x4 v[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const size_t i = i0 + k * stride;
+      v[k] = (i < n_read) ? stream_load16(src + i) : acc;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const size_t i = i0 + k * stride;
+      acc ^= v[k];
+      if (i < n_write) stream_store16(dst + i, fill);
+    }
+  }
+  if ((acc.x ^ acc.y ^ acc.z ^ acc.w) == 0x9e3779b9u) sink[0] = acc.x;  // practically never taken
+}
+
+// The dependent second launch of a two-launch reduction, reduced to its minimum: one wavefront, one store.
+__global__ __launch_bounds__(64) void calib_tail_kernel(unsigned int* sink) {
+  if (threadIdx.x == 0) sink[1] = 1u;
+}
+
 }  // namespace unirl
 
 using namespace unirl;
@@ -60,4 +92,29 @@ extern "C" int unirl_calib_copy(const void* src, void* dst, size_t bytes, void* 
   hipLaunchKernelGGL(calib_copy_kernel, dim3(8192), dim3(256), 0, (hipStream_t)stream,
                      reinterpret_cast<const u32x4*>(src), reinterpret_cast<u32x4*>(dst), bytes / 16);
   return (int)hipGetLastError();
+}
+
+extern "C" int unirl_calib_stream(const void* src, size_t read_bytes, void* dst, size_t write_bytes,
+                                  int tail_launch, void* sink, void* stream) {
+  if (!sink) return UNIRL_E_NULL;
+  if ((read_bytes && !src) || (write_bytes && !dst)) return UNIRL_E_NULL;
+  if (read_bytes % 16 != 0 || write_bytes % 16 != 0) return UNIRL_E_SHAPE;
+  if (!aligned_to(src, 16) || !aligned_to(dst, 16) || !aligned_to(sink, 4)) return UNIRL_E_ALIGN;
+  const size_t n_read = read_bytes / 16, n_write = write_bytes / 16;
+  const size_t n = n_read > n_write ? n_read : n_write;
+  hipStream_t st = (hipStream_t)stream;
+  if (n > 0) {
+    size_t blocks = (n + 256 * 4 - 1) / (256 * 4);
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(calib_stream_kernel, dim3((unsigned int)blocks), dim3(256), 0, st,
+                       reinterpret_cast<const u32x4*>(src), n_read, reinterpret_cast<u32x4*>(dst), n_write,
+                       reinterpret_cast<unsigned int*>(sink));
+    const int rc = (int)hipGetLastError();
+    if (rc != 0) return rc;
+  }
+  if (tail_launch) {
+    hipLaunchKernelGGL(calib_tail_kernel, dim3(1), dim3(64), 0, st, reinterpret_cast<unsigned int*>(sink));
+    return (int)hipGetLastError();
+  }
+  return UNIRL_OK;
 }

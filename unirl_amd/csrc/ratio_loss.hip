@@ -9,9 +9,10 @@
 // the three aggregation modes (grpo.py:148-155, drpo.py:323-330) are weighted
 // global sums:  token-mean = sum/N,  seq-mean-token-sum-norm = sum/(n_seq*h),
 // seq-mean-token-mean = sum_tok(loss/len_seq)/n_seq.
-// Sums of the ratio and its square run in fp64 per lane (the unbiased std of
-// ~1e6 values near 1 needs it); the other sums run fp32 per lane over a handful
-// of tokens and fp64 from the wavefront up, in a fixed order.
+// The ratio's mean and unbiased std come from the shifted moments sum(r-1) and
+// sum((r-1)^2): r-1 is exact in fp32 for r in [0.5, 2], so the variance of ~1e6
+// ratios near 1 keeps full accuracy.  Sums run fp32 per lane over at most a few
+// dozen tokens and fp64 from there up, in a fixed order.
 //
 // HBM traffic: 8 bytes read per valid token (+4 with a mask, +4 with per-token
 // advantages), +4 written when loss_per_elem is requested.
@@ -40,6 +41,7 @@ struct RatioConsts {
   float eps_lo, eps_hi;      // (float)clip_low, (float)clip_high
   float drpo_eps;            // (float)epsilon
   float drpo_two_eps;        // (float)(2.0 * epsilon)
+  float inv_two_eps;         // 1 / drpo_two_eps, correctly rounded
   float horizon;
 };
 
@@ -63,18 +65,54 @@ struct RatioArgs {
   float* grad_new;
 };
 
+// exp(x) for fp32 within ~1.5 ulp in eight instructions: 2^(x*log2(e)) on the hardware exp2,
+// with the rounding error of the product (carried in a second float) applied as a first-order
+// correction.  +inf above ln(FLT_MAX), 0 below the denormal range, NaN for NaN.
+__device__ __forceinline__ float exp_f32(float x) {
+  constexpr float kL2eHi = 1.44269502162933349609375f;  // log2(e) rounded to fp32
+  constexpr float kL2eLo = 1.925963033500011e-8f;       // log2(e) - kL2eHi
+  const float t = x * kL2eHi;
+  float lo = fmaf(x, kL2eHi, -t);
+  lo = fmaf(x, kL2eLo, lo);
+  const float e = __builtin_amdgcn_exp2f(t);
+  float r = fmaf(e, lo * 0.693147182f, e);
+  r = (x > 88.72283172607422f) ? INFINITY : r;  // e is +inf from here on and inf*lo + inf could be NaN
+  r = (x < -104.0f) ? 0.0f : r;                 // t and lo overflow for x = -inf
+  return r;
+}
+
+// x / c for a loop-invariant c with inv_c = 1/c: quotient estimate, exact remainder, one
+// correction -- the core of the IEEE division sequence without its range scaling (c is a
+// user constant of ordinary magnitude).  Correctly rounded away from overflow and underflow.
+__device__ __forceinline__ float div_by_const(float x, float c, float inv_c) {
+  const float q = x * inv_c;
+  const float rem = fmaf(-q, c, x);
+  const float q1 = fmaf(rem, inv_c, q);
+  return (q1 == q1) ? q1 : q;  // inf/NaN operands: keep the plain product's result
+}
+
+// 1 / x for x > 0 from the hardware reciprocal and one Newton step (within 1 ulp).
+__device__ __forceinline__ float recip_pos(float x) {
+  const float r0 = __builtin_amdgcn_rcpf(x);
+  const float e = fmaf(-x, r0, 1.0f);
+  const float r1 = fmaf(e, r0, r0);
+  return (r1 == r1) ? r1 : r0;  // x = inf or denormal: the step yields NaN, the estimate is exact enough
+}
+
 struct TokVals {
   float r, d0, ld, loss, pen, kterm, dloss;
   bool hi, lo;
 };
 
+// Everything about one token, backward factor included (the forward kernels use the leaner
+// accumulate_token below, which repeats the same arithmetic).
 template <int KIND>
 __device__ __forceinline__ TokVals ratio_token(float nw, float od, float A, const RatioConsts& C) {
   TokVals o;
   o.d0 = nw - od;
   if (KIND == UNIRL_LOSS_GRPO) {
     o.ld = o.d0;
-    o.r = expf(o.ld);
+    o.r = exp_f32(o.ld);
     const float nA = -A;
     const float u = nA * o.r;
     const float rc = nan_clamp(o.r, C.clamp_lo, C.clamp_hi);
@@ -89,8 +127,8 @@ __device__ __forceinline__ TokVals ratio_token(float nw, float od, float A, cons
     o.dloss = (u > c) ? u : ((u < c) ? dc : 0.5f * (u + dc));
   } else {
     o.ld = nan_clamp(o.d0, -20.0f, 20.0f);
-    o.r = expf(o.ld);
-    const float mu = expf(od);
+    o.r = exp_f32(o.ld);
+    const float mu = exp_f32(od);
     const float rd = o.r - 1.0f;
     const float w = C.mu_weighted ? mu : 1.0f;
     o.pen = ((fabsf(A) * w) * (rd * rd)) / C.drpo_two_eps;
@@ -111,12 +149,82 @@ __device__ __forceinline__ double combine(int v, double x, double y) {
   return (v == P_RMIN) ? fmin(x, y) : ((v == P_RMAX || v == P_AMAX) ? fmax(x, y) : x + y);
 }
 
+// Per-lane accumulators.  The six sums are fp32 and are flushed into fp64 totals after every
+// pass (at most ITEMS*VEC tokens), so their rounding does not grow with the input.  The extrema
+// are kept as bit patterns: ratios and |new-old| are >= 0 (or NaN), where unsigned integer order
+// is float order, so each update is one integer min / max.
 struct Acc {
-  double sr = 0.0, sr2 = 0.0;
-  float loss = 0.0f, kl = 0.0f, pen = 0.0f, ab = 0.0f;
-  float rmin = INFINITY, rmax = -INFINITY, amax = -INFINITY;
+  float s1 = 0.0f, s2 = 0.0f;  // sums of (r-1) and (r-1)^2
+  float loss = 0.0f;
+  float kl = 0.0f;             // GRPO: sum of ld^2 (halved at the end); DRPO: sum of (r-1) - ld
+  float pen = 0.0f, ab = 0.0f;
+  double t_s1 = 0.0, t_s2 = 0.0, t_loss = 0.0, t_kl = 0.0, t_pen = 0.0, t_ab = 0.0;
+  unsigned int rmin = 0x7f800000u, rmax = 0u, amax = 0u;
   unsigned int cnt = 0, chi = 0, clo = 0, cany = 0;
+
+  __device__ __forceinline__ void flush() {
+    t_s1 += (double)s1;
+    t_s2 += (double)s2;
+    t_loss += (double)loss;
+    t_kl += (double)kl;
+    t_pen += (double)pen;
+    t_ab += (double)ab;
+    s1 = s2 = loss = kl = pen = ab = 0.0f;
+  }
 };
+
+// One token into the accumulators; returns its loss.  `lw` = loss_mask * aggregation weight.
+// The arithmetic is the reference's, op for op; two rewrites are exact:
+//   maximum(u, c) = (c > u) ? c : u   -- u is NaN whenever c is (c = -A*clamp(r), u = -A*r), so
+//                                        NaN reaches the result as in torch.maximum;
+//   1 - r = -(r - 1)                  -- rounding is symmetric, so the lower clip test reuses r-1.
+template <int KIND>
+__device__ __forceinline__ float accumulate_token(float nw, float od, float A, float lw, const RatioConsts& C,
+                                                  Acc& acc) {
+  const float d0 = nw - od;
+  float r, loss;
+  bool hi, lo;
+  if (KIND == UNIRL_LOSS_GRPO) {
+    r = exp_f32(d0);
+    const float nA = -A;
+    const float u = nA * r;
+    const float c = nA * fminf(fmaxf(r, C.clamp_lo), C.clamp_hi);
+    loss = (c > u) ? c : u;
+    const float d = r - 1.0f;
+    hi = d > C.eps_hi;
+    lo = -d > C.eps_lo;
+    acc.s1 += d;
+    acc.s2 = fmaf(d, d, acc.s2);
+    acc.kl = fmaf(d0, d0, acc.kl);
+  } else {
+    const float ld = (d0 != d0) ? d0 : fminf(fmaxf(d0, -20.0f), 20.0f);  // torch.clamp keeps NaN
+    r = exp_f32(ld);
+    const float mu = exp_f32(od);
+    const float d = r - 1.0f;
+    const float w = C.mu_weighted ? mu : 1.0f;
+    const float pen = div_by_const((fabsf(A) * w) * (d * d), C.drpo_two_eps, C.inv_two_eps);
+    loss = (-A) * r + pen;
+    float aeps = C.drpo_eps;
+    if (C.mu_weighted) aeps = (mu > 0.0f) ? recip_pos(mu) * C.drpo_eps : INFINITY;
+    hi = r > (1.0f + aeps);
+    lo = r < (1.0f - aeps);
+    acc.s1 += d;
+    acc.s2 = fmaf(d, d, acc.s2);
+    acc.kl += d - ld;
+    acc.pen += pen;
+  }
+  acc.loss += loss * lw;
+  const float a0 = fabsf(d0);
+  acc.ab += a0;
+  const unsigned int rb = __float_as_uint(r), ab = __float_as_uint(a0);
+  acc.rmin = rb < acc.rmin ? rb : acc.rmin;
+  acc.rmax = rb > acc.rmax ? rb : acc.rmax;
+  acc.amax = ab > acc.amax ? ab : acc.amax;
+  acc.chi += hi ? 1u : 0u;
+  acc.clo += lo ? 1u : 0u;
+  acc.cany += (hi || lo) ? 1u : 0u;
+  return loss;
+}
 
 // sequence lookup for the packed layout: largest s with cu[s] <= tok
 __device__ __forceinline__ int64_t find_seq(const int64_t* cu, int64_t n_seq, int64_t tok) {
@@ -142,47 +250,84 @@ struct SeqCtx {
 };
 
 // One loaded vector of VEC tokens starting at row-relative index t0; tokens at or past `count`
-// are padding.  Accumulates into acc and leaves the per-token loss in out[].
-template <int KIND, int VEC>
+// are padding.  mk[] holds 1 when there is no loss mask.  Accumulates into acc and leaves the
+// per-token loss in out[].  Whole vectors outside the packed layout take a path without
+// per-token bounds or sequence checks.
+template <int KIND, int VEC, bool PACKED>
 __device__ __forceinline__ void ratio_vec_fwd(const RatioArgs& A, const RatioConsts& C, int64_t t0, int64_t count,
                                               const float (&nw)[VEC], const float (&od)[VEC],
                                               const float (&ad)[VEC], const float (&mk)[VEC], SeqCtx& sq,
                                               Acc& acc, float (&out)[VEC]) {
+  if (!PACKED && t0 + VEC <= count) {
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      const float a = C.adv_per_token ? ad[k] : sq.adv;
+      out[k] = accumulate_token<KIND>(nw[k], od[k], a, mk[k] * sq.w, C, acc);
+    }
+    acc.cnt += VEC;
+    return;
+  }
 #pragma unroll
   for (int k = 0; k < VEC; ++k) {
     const int64_t t = t0 + k;
     out[k] = 0.0f;
     if (t < count) {
-      if (A.layout == LAYOUT_PACKED && t >= sq.cur_end) {
+      if (PACKED && t >= sq.cur_end) {
         const int64_t s = find_seq(A.seq, A.n_seq, t);
         sq.cur_end = A.seq[s + 1];
         sq.w = seq_weight(C, sq.cur_end - A.seq[s]);
         if (!C.adv_per_token) sq.adv = A.adv[s];
       }
       const float a = C.adv_per_token ? ad[k] : sq.adv;
-      const TokVals v = ratio_token<KIND>(nw[k], od[k], a, C);
-      out[k] = v.loss;
-      float lm = v.loss;
-      if (A.mask) lm = lm * mk[k];
-      acc.sr += (double)v.r;
-      acc.sr2 = fma((double)v.r, (double)v.r, acc.sr2);
-      acc.loss += lm * sq.w;
-      acc.kl += v.kterm;
-      acc.pen += v.pen;
-      const float ad0 = fabsf(v.d0);
-      acc.ab += ad0;
-      acc.rmin = fminf(acc.rmin, v.r);
-      acc.rmax = fmaxf(acc.rmax, v.r);
-      acc.amax = fmaxf(acc.amax, ad0);
+      out[k] = accumulate_token<KIND>(nw[k], od[k], a, mk[k] * sq.w, C, acc);
       acc.cnt += 1u;
-      acc.chi += v.hi ? 1u : 0u;
-      acc.clo += v.lo ? 1u : 0u;
-      acc.cany += (v.hi || v.lo) ? 1u : 0u;
     }
   }
 }
 
-template <int KIND, int VEC>
+// Workgroup partial vector -> A.partials[workgroup].  Every thread must call.
+__device__ __forceinline__ void store_block_partials(const RatioArgs& A, Acc& acc, double (*lds_v)[kRlVals]) {
+  constexpr int NW = kRlThreads / kWave;
+  acc.flush();
+  double vals[kRlVals];
+  vals[P_SR] = wave_sum(acc.t_s1);
+  vals[P_SR2] = wave_sum(acc.t_s2);
+  vals[P_LOSS] = wave_sum(acc.t_loss);
+  vals[P_KL] = wave_sum(acc.t_kl);
+  vals[P_PEN] = wave_sum(acc.t_pen);
+  vals[P_ABS] = wave_sum(acc.t_ab);
+  vals[P_CNT] = (double)wave_sum(acc.cnt);
+  vals[P_CHI] = (double)wave_sum(acc.chi);
+  vals[P_CLO] = (double)wave_sum(acc.clo);
+  vals[P_CANY] = (double)wave_sum(acc.cany);
+  // NaN patterns drop out of the float min / max here; the finalize kernel restores NaN from the sums
+  vals[P_RMIN] = (double)wave_min(__uint_as_float(acc.rmin));
+  vals[P_RMAX] = (double)wave_max(acc.cnt ? __uint_as_float(acc.rmax) : -INFINITY);
+  vals[P_AMAX] = (double)wave_max(acc.cnt ? __uint_as_float(acc.amax) : -INFINITY);
+  vals[13] = vals[14] = vals[15] = 0.0;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wid = threadIdx.x / kWave;
+  if (lane == 0) {
+#pragma unroll
+    for (int v = 0; v < kRlVals; ++v) lds_v[wid][v] = vals[v];
+  }
+  __syncthreads();
+  const unsigned int blk = blockIdx.y * gridDim.x + blockIdx.x;
+  if (threadIdx.x < kRlVals) {
+    const int v = threadIdx.x;
+    double x = lds_v[0][v];
+    for (int w = 1; w < NW; ++w) x = combine(v, x, lds_v[w][v]);
+    A.partials[(int64_t)blk * kRlVals + v] = x;  // reduced by ratio_loss_finalize_kernel
+  }
+}
+
+template <int VEC>
+__device__ __forceinline__ void fill_ones(float (&m)[VEC]) {
+#pragma unroll
+  for (int k = 0; k < VEC; ++k) m[k] = 1.0f;
+}
+
+template <int KIND, int VEC, bool PACKED>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A) {
   constexpr int NW = kRlThreads / kWave;
   constexpr int ITEMS = (VEC == 4) ? 4 : 2;  // vectors in flight per lane
@@ -217,6 +362,7 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
 #pragma unroll
       for (int it = 0; it < ITEMS; ++it) {
         const int64_t i = i0 + it * stride;
+        fill_ones(mk[it]);
         if (i < nload) {
           Vec<float, VEC>::load(A.nw + base + i * VEC, nw[it]);
           Vec<float, VEC>::load(A.od + base + i * VEC, od[it]);
@@ -229,10 +375,11 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
         const int64_t i = i0 + it * stride;
         if (i < nload) {
           float out[VEC];
-          ratio_vec_fwd<KIND, VEC>(A, C, i * VEC, count, nw[it], od[it], ad[it], mk[it], sq, acc, out);
+          ratio_vec_fwd<KIND, VEC, PACKED>(A, C, i * VEC, count, nw[it], od[it], ad[it], mk[it], sq, acc, out);
           if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + base + i * VEC, out);
         }
       }
+      acc.flush();
     }
     // a row whose length is not a multiple of VEC ends in one vector that cannot be loaded whole
     if (nvec > nvec_full && first == nvec_full % stride) {
@@ -244,52 +391,22 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
         nw[k] = ok ? A.nw[base + t0 + k] : 0.0f;
         od[k] = ok ? A.od[base + t0 + k] : 0.0f;
         ad[k] = (ok && C.adv_per_token) ? A.adv[base + t0 + k] : 0.0f;
-        mk[k] = (ok && A.mask) ? A.mask[base + t0 + k] : 0.0f;
+        mk[k] = (ok && A.mask) ? A.mask[base + t0 + k] : 1.0f;
       }
-      ratio_vec_fwd<KIND, VEC>(A, C, t0, count, nw, od, ad, mk, sq, acc, out);
+      ratio_vec_fwd<KIND, VEC, PACKED>(A, C, t0, count, nw, od, ad, mk, sq, acc, out);
       if (A.loss_elem) {
 #pragma unroll
         for (int k = 0; k < VEC; ++k)
           if (t0 + k < row_end) A.loss_elem[base + t0 + k] = out[k];
       }
+      acc.flush();
     }
     // padded layout: zero the loss of the slots past the sequence end
     if (A.loss_elem && padded) {
       for (int64_t t = nvec * VEC + first; t < row_end; t += stride) A.loss_elem[base + t] = 0.0f;
     }
   }
-
-  // ---- workgroup partials -------------------------------------------------
-  double vals[kRlVals];
-  vals[P_SR] = wave_sum(acc.sr);
-  vals[P_SR2] = wave_sum(acc.sr2);
-  // 64 lanes x a handful of tokens: an fp32 shuffle tree keeps full accuracy at half the shuffles
-  vals[P_LOSS] = (double)wave_sum(acc.loss);
-  vals[P_KL] = (double)wave_sum(acc.kl);
-  vals[P_PEN] = (double)wave_sum(acc.pen);
-  vals[P_ABS] = (double)wave_sum(acc.ab);
-  vals[P_CNT] = (double)wave_sum(acc.cnt);
-  vals[P_CHI] = (double)wave_sum(acc.chi);
-  vals[P_CLO] = (double)wave_sum(acc.clo);
-  vals[P_CANY] = (double)wave_sum(acc.cany);
-  vals[P_RMIN] = (double)wave_min(acc.rmin);
-  vals[P_RMAX] = (double)wave_max(acc.rmax);
-  vals[P_AMAX] = (double)wave_max(acc.amax);
-  vals[13] = vals[14] = vals[15] = 0.0;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wid = threadIdx.x / kWave;
-  if (lane == 0) {
-#pragma unroll
-    for (int v = 0; v < kRlVals; ++v) lds_v[wid][v] = vals[v];
-  }
-  __syncthreads();
-  const unsigned int blk = blockIdx.y * gridDim.x + blockIdx.x;
-  if (threadIdx.x < kRlVals) {
-    const int v = threadIdx.x;
-    double x = lds_v[0][v];
-    for (int w = 1; w < NW; ++w) x = combine(v, x, lds_v[w][v]);
-    A.partials[(int64_t)blk * kRlVals + v] = x;  // reduced by ratio_loss_finalize_kernel
-  }
+  store_block_partials(A, acc, lds_v);
 }
 
 // One workgroup: fixed-order reduction of every workgroup's partial vector, then the metrics.
@@ -297,11 +414,11 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
   __shared__ double lds_fin[kRlThreads];
   const RatioConsts C = A.C;
   {
-    // thread = (value v, slice j0): 16 slices walk the workgroups' vectors, eight loads in flight each
+    // thread = (value v, slice j0): 16 slices walk the workgroups' vectors, kBatch loads in flight each
     const int v = threadIdx.x % kRlVals;
     const int j0 = threadIdx.x / kRlVals;  // 0..15
     constexpr int kSlices = kRlThreads / kRlVals;
-    constexpr int kBatch = 8;
+    constexpr int kBatch = 32;  // 512 workgroups: every partial of a thread in flight at once
     double x = (v == P_RMIN) ? (double)INFINITY : ((v == P_RMAX || v == P_AMAX) ? -(double)INFINITY : 0.0);
     const double ident = x;
     for (unsigned int j = j0; j < nblk; j += kSlices * kBatch) {
@@ -334,6 +451,7 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
     loss = (loss / (double)A.n_seq) / (double)C.horizon;
   else
     loss = loss / (double)A.n_seq;
+  // sr, sr2: sums of (r-1) and (r-1)^2
   double var = 0.0;
   if (N > 1.0) {
     var = (sr2 - sr * sr / N) / (N - 1.0);
@@ -341,7 +459,7 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
   }
   float* M = A.metrics;
   M[UNIRL_M_LOSS] = (float)loss;
-  M[UNIRL_M_RATIO_MEAN] = (float)(sr / N);
+  M[UNIRL_M_RATIO_MEAN] = (float)(1.0 + sr / N);
   M[UNIRL_M_RATIO_STD] = (float)sqrt(var);
   // min()/max() of the reference return NaN when any ratio is NaN; the ratios are >= 0, so their
   // sum is NaN exactly then (likewise the absolute differences below)
@@ -350,7 +468,8 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
   M[UNIRL_M_CLIP_FRACTION] = (float)lds_fin[P_CANY] / (float)N;
   M[UNIRL_M_CLIPFRAC_HI] = (float)lds_fin[P_CHI] / (float)N;
   M[UNIRL_M_CLIPFRAC_LO] = (float)lds_fin[P_CLO] / (float)N;
-  M[UNIRL_M_APPROX_KL] = (float)(lds_fin[P_KL] / N);
+  // GRPO accumulates ld^2; mean(0.5*ld^2) = 0.5*sum/N exactly (halving commutes with rounding)
+  M[UNIRL_M_APPROX_KL] = (float)((C.kind == UNIRL_LOSS_GRPO ? 0.5 : 1.0) * lds_fin[P_KL] / N);
   M[UNIRL_M_PENALTY_MEAN] = (float)(lds_fin[P_PEN] / N);
   M[UNIRL_M_ABSDIFF_MEAN] = (float)(lds_fin[P_ABS] / N);
   M[UNIRL_M_ABSDIFF_MAX] = (lds_fin[P_ABS] != lds_fin[P_ABS]) ? quiet_nan() : (float)lds_fin[P_AMAX];
@@ -459,6 +578,7 @@ static int fill_consts(const unirl_ratio_loss_params* p, RatioConsts& C) {
   C.eps_hi = (float)p->clip_high;
   C.drpo_eps = (float)p->drpo_epsilon;
   C.drpo_two_eps = (float)(2.0 * p->drpo_epsilon);
+  C.inv_two_eps = (float)(1.0 / (double)C.drpo_two_eps);
   C.horizon = (float)p->horizon;
   return UNIRL_OK;
 }
@@ -544,17 +664,20 @@ extern "C" int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp
   if ((int64_t)S.grid.x * S.grid.y * kRlVals > kPartialCapacity) return UNIRL_E_LIMIT;
   hipStream_t st = (hipStream_t)stream;
   dim3 block(kRlThreads);
+  const bool packed = (A.layout == LAYOUT_PACKED);
+#define UNIRL_LAUNCH_FWD(KIND, VEC)                                                                      \
+  do {                                                                                                   \
+    if (packed)                                                                                          \
+      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, true>), S.grid, block, 0, st, A);             \
+    else                                                                                                 \
+      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, false>), S.grid, block, 0, st, A);            \
+  } while (0)
   if (A.C.kind == UNIRL_LOSS_GRPO) {
-    if (S.vec == 4)
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<UNIRL_LOSS_GRPO, 4>), S.grid, block, 0, st, A);
-    else
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<UNIRL_LOSS_GRPO, 1>), S.grid, block, 0, st, A);
+    if (S.vec == 4) UNIRL_LAUNCH_FWD(UNIRL_LOSS_GRPO, 4); else UNIRL_LAUNCH_FWD(UNIRL_LOSS_GRPO, 1);
   } else {
-    if (S.vec == 4)
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<UNIRL_LOSS_DRPO, 4>), S.grid, block, 0, st, A);
-    else
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<UNIRL_LOSS_DRPO, 1>), S.grid, block, 0, st, A);
+    if (S.vec == 4) UNIRL_LAUNCH_FWD(UNIRL_LOSS_DRPO, 4); else UNIRL_LAUNCH_FWD(UNIRL_LOSS_DRPO, 1);
   }
+#undef UNIRL_LAUNCH_FWD
   const int launch_rc = (int)hipGetLastError();
   if (launch_rc != 0) return launch_rc;
   hipLaunchKernelGGL(ratio_loss_finalize_kernel, dim3(1), block, 0, st, A, S.grid.x * S.grid.y);

@@ -803,6 +803,24 @@ def calib_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
     N.check(rc, "unirl_calib_copy")
 
 
+def calib_stream(src: Optional[torch.Tensor], read_bytes: int, dst: Optional[torch.Tensor], write_bytes: int,
+                 sink: torch.Tensor, *, tail_launch: bool = False) -> None:
+    """Launch-floor yardstick: one kernel that reads ``read_bytes`` of ``src`` and writes
+    ``write_bytes`` of ``dst`` with no arithmetic, then (``tail_launch``) a one-wavefront kernel."""
+    N.require_device(sink, "sink")
+    for t, nbytes, name in ((src, read_bytes, "src"), (dst, write_bytes, "dst")):
+        if nbytes:
+            N.require_device(t, name)
+            if not t.is_contiguous() or t.numel() * t.element_size() < nbytes:
+                raise ValueError(f"{name} must be contiguous and hold at least {nbytes} bytes")
+    with torch.cuda.device(sink.device):
+        rc = N.lib().unirl_calib_stream(
+            N.ptr(src) if read_bytes else None, int(read_bytes), N.ptr(dst) if write_bytes else None,
+            int(write_bytes), int(bool(tail_launch)), N.ptr(sink), N.current_stream(sink.device),
+        )
+    N.check(rc, "unirl_calib_stream")
+
+
 def gather_steps(tensor: torch.Tensor, positions: Sequence[int]) -> torch.Tensor:
     """``tensor[:, positions]`` for a ``[B, S, ...]`` tensor, as one gather kernel."""
     N.require_device(tensor, "tensor")
