@@ -43,8 +43,8 @@ __device__ __forceinline__ float kl_den(const KlArgs& A, int64_t row) {
   return 2.0f * (s * s);
 }
 
-__device__ __forceinline__ void kl_finish(const KlArgs& A, int64_t row, double q) {
-  const float kl = (float)((q / (double)kl_den(A, row)) / (double)A.D);
+__device__ __forceinline__ void kl_finish(const KlArgs& A, int64_t row, double q, float den) {
+  const float kl = (float)((q / (double)den) / (double)A.D);
   A.kl[row] = kl;
   if (A.mask) A.mask[row] = (kl < A.threshold) ? 1 : 0;
 }
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(kKlThreads) void gaussian_kl_kernel(KlArgs A) {
   const double part = block_sum<double>((double)acc, lds);
   if (threadIdx.x != 0) return;
   if (gridDim.x == 1) {
-    kl_finish(A, row, part);
+    kl_finish(A, row, part, kl_den(A, row));
   } else {
     A.partials[row * gridDim.x + blockIdx.x] = part;  // summed by gaussian_kl_finalize_kernel
   }
@@ -91,8 +91,9 @@ __global__ __launch_bounds__(kKlThreads) void gaussian_kl_kernel(KlArgs A) {
 __global__ __launch_bounds__(kKlThreads) void gaussian_kl_finalize_kernel(KlArgs A, int64_t R, unsigned int nblk) {
   const int64_t row = (int64_t)blockIdx.x * (kKlThreads / kWave) + threadIdx.x / kWave;
   if (row >= R) return;
+  const float den = kl_den(A, row);  // issued with the partial loads, not after them
   const double q = wave_ordered_sum(A.partials + row * nblk, nblk);
-  if ((threadIdx.x & (kWave - 1)) == 0) kl_finish(A, row, q);
+  if ((threadIdx.x & (kWave - 1)) == 0) kl_finish(A, row, q, den);
 }
 
 template <typename T, int VEC>

@@ -153,11 +153,7 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
 
   const int64_t b = blockIdx.y;
   const int64_t D = A.D;
-  const float s = A.sigma[b * A.sigma_stride];
-  const float sn = A.sigma_next[b * A.sigma_stride];
-  const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
   const int kind = A.kind;
-  const SdeCoef c = sde_coef(kind, s, sn, smax, A.sc);
 
   const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + b * A.stride_v;
   const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + b * A.stride_x;
@@ -171,8 +167,8 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
   const int64_t stride = (int64_t)gridDim.x * kSdeThreads;
   float acc = 0.0f;
 
-  for (int64_t i0 = (int64_t)blockIdx.x * kSdeThreads + threadIdx.x; i0 < nvec; i0 += stride * ITEMS) {
-    float v[ITEMS][VEC], x[ITEMS][VEC], t[ITEMS][VEC];
+  float v[ITEMS][VEC], x[ITEMS][VEC], t[ITEMS][VEC];
+  auto load_pass = [&](int64_t i0) {
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
       const int64_t i = i0 + it * stride;
@@ -187,6 +183,19 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
         }
       }
     }
+  };
+
+  // The first pass of loads goes out before the coefficients are worked out: the sigma loads and
+  // the fp64 divide / sqrt / log behind the coefficients take about as long as a trip to memory,
+  // and at small sizes (one pass per lane) the two would otherwise run back to back.
+  int64_t i0 = (int64_t)blockIdx.x * kSdeThreads + threadIdx.x;
+  load_pass(i0);
+  const float s = A.sigma[b * A.sigma_stride];
+  const float sn = A.sigma_next[b * A.sigma_stride];
+  const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
+  const SdeCoef c = sde_coef(kind, s, sn, smax, A.sc);
+
+  while (i0 < nvec) {
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
       const int64_t i = i0 + it * stride;
@@ -201,6 +210,8 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
         if (mo) sde_store_as<VEC>(mo, mdt, mo0 + i * VEC, mean);
       }
     }
+    i0 += stride * ITEMS;
+    if (i0 < nvec) load_pass(i0);
   }
 
   if (!A.want_logp) return;  // uniform across the grid
@@ -218,12 +229,17 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
 __global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepArgs A, int64_t B, unsigned int nblk) {
   const int64_t b = (int64_t)blockIdx.x * (kSdeThreads / kWave) + threadIdx.x / kWave;
   if (b >= B) return;
-  const double q = wave_ordered_sum(A.partials + b * nblk, nblk);
-  if ((threadIdx.x & (kWave - 1)) != 0) return;
+  // the partial loads are issued first; the coefficients are worked out while they are in flight
+  const int lane = threadIdx.x & (kWave - 1);
+  const double* __restrict__ pp = A.partials + b * nblk;
+  double q = (lane < (int)nblk) ? pp[lane] : 0.0;
   const float s = A.sigma[b * A.sigma_stride];
   const float sn = A.sigma_next[b * A.sigma_stride];
   const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
   const SdeCoef c = sde_coef(A.kind, s, sn, smax, A.sc);
+  for (int64_t j = lane + kWave; j < nblk; j += kWave) q += pp[j];
+  q = wave_sum(q);
+  if (lane != 0) return;
   A.logp_out[b * A.stride_logp] = sde_finish_logp(A.kind, c, q, (double)A.D, A.logp_sum);
 }
 
@@ -346,6 +362,7 @@ template <typename TV, typename TX, int VEC, int ITEMS>
 __global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs A) {
   constexpr int NW = kSdeThreads / kWave;
   __shared__ double lds_q[UNIRL_MAX_ROLLOUT_STEPS][NW];
+  __shared__ SdeCoef lds_c[UNIRL_MAX_ROLLOUT_STEPS];
 
   const int64_t b = blockIdx.y;
   const int64_t D = A.D;
@@ -368,8 +385,15 @@ __global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs
     if (i < nvec) Vec<TX, VEC>::load(xp + i * VEC, x[it]);
   }
 
+  // Each step's coefficients cost an fp64 divide / sqrt / log chain (about a microsecond of one
+  // wavefront).  Lane k of the first wavefront works out step k once, while the x0 loads are in
+  // flight, and every wavefront reads them from LDS afterwards.
+  if ((int)threadIdx.x < S)
+    lds_c[threadIdx.x] = sde_coef(kind, A.sigmas[threadIdx.x], A.sigmas[threadIdx.x + 1], smax, A.sc[threadIdx.x]);
+  __syncthreads();
+
   for (int k = 0; k < S; ++k) {
-    const SdeCoef c = sde_coef(kind, A.sigmas[k], A.sigmas[k + 1], smax, A.sc[k]);
+    const SdeCoef c = lds_c[k];
     const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v[k]) + b * D;
     const float* __restrict__ np = A.n[k] ? A.n[k] + b * D : nullptr;
     float* __restrict__ tj = A.traj_out ? A.traj_out + (int64_t)k * A.BD + b * D : nullptr;
@@ -422,8 +446,7 @@ __global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs
     for (int w = 0; w < NW; ++w) q += lds_q[threadIdx.x][w];
     if (nblk == 1) {
       if (A.want_logp[threadIdx.x]) {
-        const SdeCoef c =
-            sde_coef(kind, A.sigmas[threadIdx.x], A.sigmas[threadIdx.x + 1], smax, A.sc[threadIdx.x]);
+        const SdeCoef c = lds_c[threadIdx.x];
         A.logp_out[b * S + threadIdx.x] = sde_finish_logp(kind, c, q, (double)D, A.logp_sum);
       } else {
         A.logp_out[b * S + threadIdx.x] = __uint_as_float(0x7fc00000u);
