@@ -262,7 +262,8 @@ def main() -> int:
     ap.add_argument("--cpu-rows", type=int, default=512, help="rows of the bounded CPU-baseline sample")
     ap.add_argument("--spinup", type=float, default=0.5, help="seconds of untimed launches before the warm-up")
     ap.add_argument("--traffic-probe", action="store_true",
-                    help="run 3 calibration copies of 1 GiB and 3 headline launches, then exit "
+                    help="run 3 calibration copies of 1 GiB, 3 headline launches and 3 launches of every "
+                         "other shape, then exit "
                          "(the command `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` is pointed at)")
     ap.add_argument("--skip-shapes", action="store_true", help="headline only")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
@@ -308,8 +309,15 @@ def main() -> int:
         for i in range(3):
             step(i)
         torch.cuda.synchronize()
-        print(json.dumps({"traffic_probe": {"calib_copy_bytes_each_way": 2**30,
-                                            "token_kernel_algorithmic_bytes": alg_bytes}}), flush=True)
+        probe = {"calib_copy_bytes_each_way": 2**30, "token_kernel_algorithmic_bytes": alg_bytes}
+        if not args.skip_shapes:
+            del src, dst
+            for sh in make_shapes(torch, dev):  # three launches of every other kernel, on distinct input sets
+                for i in range(3):
+                    sh["run"](i)
+                torch.cuda.synchronize()
+                probe[sh["name"] + "_algorithmic_bytes"] = sh.get("bytes_padded", sh["bytes"])
+        print(json.dumps({"traffic_probe": probe}), flush=True)
         return 0
 
     # Untimed spin-up: the device needs a few hundred milliseconds of work to reach its sustained
