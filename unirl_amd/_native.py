@@ -232,14 +232,37 @@ def current_stream(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+class on_device:
+    """``with on_device(dev):`` makes ``dev`` the current HIP device for a launch.  When it already
+    is (the usual case) nothing is switched, which saves the several microseconds a
+    ``torch.cuda.device`` context costs on a path whose kernels run for about ten."""
+
+    __slots__ = ("_ctx",)
+
+    def __init__(self, device: torch.device) -> None:
+        index = device.index
+        self._ctx = None if (index is None or index == torch.cuda.current_device()) else torch.cuda.device(index)
+
+    def __enter__(self):
+        if self._ctx is not None:
+            self._ctx.__enter__()
+        return self
+
+    def __exit__(self, *exc):
+        if self._ctx is not None:
+            return self._ctx.__exit__(*exc)
+        return False
+
+
 _workspaces: Dict[Tuple[int, int], torch.Tensor] = {}
 
 
-def workspace(device: torch.device) -> Tuple[torch.Tensor, int]:
+def workspace(device: torch.device, stream: Optional[int] = None) -> Tuple[torch.Tensor, int]:
     """Scratch for the reducing kernels (per-workgroup partial sums), one per (device, stream):
-    calls on different streams may overlap and must not share it."""
+    calls on different streams may overlap and must not share it.  ``stream`` is the raw handle
+    when the caller has already looked it up."""
     index = device.index if device.index is not None else torch.cuda.current_device()
-    key = (index, current_stream(device))
+    key = (index, current_stream(device) if stream is None else stream)
     ws = _workspaces.get(key)
     if ws is None:
         nbytes = int(lib().unirl_workspace_bytes())

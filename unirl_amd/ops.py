@@ -25,7 +25,13 @@ def _flat2(t: torch.Tensor, name: str) -> torch.Tensor:
 
 def _sigma_arg(sigma: torch.Tensor, B: int, device: torch.device, name: str) -> Tuple[torch.Tensor, int]:
     """f32 device tensor with 1 or B values, and the per-sample stride (0 or 1)."""
-    s = sigma.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    s = sigma
+    if s.dtype != torch.float32 or s.device != device or s.requires_grad:
+        s = s.detach().to(device=device, dtype=torch.float32)
+    n = s.numel()
+    if n == 1:
+        return (s if s.dim() <= 1 else s.reshape(-1)), 0
+    s = s.reshape(-1).contiguous()
     if s.numel() == 1:
         return s, 0
     if s.numel() == B:
@@ -106,13 +112,14 @@ def sde_step_logp(
         if logp_out is not None:
             logp_out.fill_(float("nan"))
         return prev_out, logp_out, mean_out
-    ws, ws_bytes = N.workspace(device)
-    with torch.cuda.device(device):
+    stream = N.current_stream(device)
+    ws, ws_bytes = N.workspace(device, stream)
+    with N.on_device(device):
         rc = N.lib().unirl_sde_step_logp(
             N.ptr(v), N.dtype_code(v.dtype), N.ptr(x), N.dtype_code(x.dtype), N.ptr(prev_in), N.ptr(nz),
             N.ptr(sig), N.ptr(sig_n), stride, N.ptr(smax_t), smax_v, float(eta), SDE_KINDS[kind], B, D,
             N.ptr(prev_out), N.ptr(mean_out), N.ptr(logp_out), int(bool(logp_sum)), N.ptr(ws), ws_bytes,
-            N.current_stream(device),
+            stream,
         )
     N.check(rc, "unirl_sde_step_logp")
     return prev_out, logp_out, mean_out
@@ -232,7 +239,7 @@ def sde_step_logp_into(
     d.mean_out, d.mean_dtype, d.mean_stride = N.ptr(mo), (N.dtype_code(mo.dtype) if mo is not None else 0), smo
     d.logp_out, d.logp_stride, d.logp_sum = N.ptr(lp), slp, int(bool(logp_sum))
     ws, ws_bytes = N.workspace(device)
-    with torch.cuda.device(device):
+    with N.on_device(device):
         rc = N.lib().unirl_sde_step_logp_ex(ctypes.byref(d), N.ptr(ws), ws_bytes, N.current_stream(device))
     N.check(rc, "unirl_sde_step_logp_ex")
 
@@ -284,7 +291,7 @@ def sde_step_logp_bwd(
     grad_x = torch.empty(x.shape, dtype=torch.float32, device=device) if need_grad_x else None
     if B == 0 or D == 0 or (grad_v is None and grad_x is None):
         return grad_v, grad_x
-    with torch.cuda.device(device):
+    with N.on_device(device):
         rc = N.lib().unirl_sde_step_logp_bwd(
             N.ptr(v), N.dtype_code(v.dtype), N.ptr(x), N.dtype_code(x.dtype), N.ptr(prev_in), N.ptr(nz),
             N.ptr(sig), N.ptr(sig_n), stride, N.ptr(smax_t), smax_v, float(eta), SDE_KINDS[kind], B, D,
@@ -365,7 +372,7 @@ def sde_rollout_logp(
     n_arr = (ctypes.c_void_p * S)(*[(t.data_ptr() if t is not None else None) for t in ns])
     e_arr = (ctypes.c_double * S)(*[float(e) for e in etas])
     ws, ws_bytes = N.workspace(device)
-    with torch.cuda.device(device):
+    with N.on_device(device):
         rc = N.lib().unirl_sde_rollout_logp(
             N.ptr(x), N.dtype_code(x.dtype), v_arr, N.dtype_code(vdtype), n_arr, N.ptr(sig), e_arr, S,
             N.ptr(smax_t), smax_v, SDE_KINDS[kind], B, D, N.ptr(x_out), N.ptr(traj), N.ptr(logp),
@@ -408,11 +415,12 @@ def gaussian_kl_mask(
     mask = torch.empty(lead, dtype=torch.bool, device=device) if want_mask else None
     if R == 0 or D == 0:
         return kl, mask
-    ws, ws_bytes = N.workspace(device)
-    with torch.cuda.device(device):
+    stream = N.current_stream(device)
+    ws, ws_bytes = N.workspace(device, stream)
+    with N.on_device(device):
         rc = N.lib().unirl_gaussian_kl_mask(
             N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, float(threshold),
-            N.ptr(kl), N.ptr(mask), N.ptr(ws), ws_bytes, N.current_stream(device),
+            N.ptr(kl), N.ptr(mask), N.ptr(ws), ws_bytes, stream,
         )
     N.check(rc, "unirl_gaussian_kl_mask")
     return kl, mask
@@ -453,7 +461,7 @@ def flowdppo_loss(
     ad, klc = f32c(advantages, "advantages"), f32c(kl, "kl")
     elem = torch.empty(shape, dtype=torch.float32, device=device)
     metrics = torch.empty(N.M_COUNT, dtype=torch.float32, device=device)
-    with torch.cuda.device(device):
+    with N.on_device(device):
         rc = N.lib().unirl_flowdppo_loss(
             N.ptr(nw), N.ptr(od), N.ptr(ad), N.ptr(klc), nw.numel(), float(threshold), N.ptr(elem),
             N.ptr(metrics), N.current_stream(device),
@@ -472,7 +480,7 @@ def expand_per_seq(values: torch.Tensor, cu_seqlens: torch.Tensor, n_tok: int) -
         raise ValueError(f"cu_seqlens needs {v.numel() + 1} entries; got {cu.numel()}")
     out = torch.empty(int(n_tok), dtype=torch.float32, device=device)
     if n_tok:
-        with torch.cuda.device(device):
+        with N.on_device(device):
             rc = N.lib().unirl_expand_per_seq(
                 N.ptr(v), N.ptr(cu), v.numel(), int(n_tok), N.ptr(out), N.current_stream(device)
             )
@@ -500,7 +508,7 @@ def gaussian_kl_elem(p: torch.Tensor, q: torch.Tensor, sigma: torch.Tensor, *, s
     out = torch.empty(pc.shape, dtype=torch.float32, device=device)
     if pc.numel() == 0:
         return out
-    with torch.cuda.device(device):
+    with N.on_device(device):
         rc = N.lib().unirl_gaussian_kl_elem(
             N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, N.ptr(out),
             N.current_stream(device),
@@ -547,7 +555,7 @@ def token_logp_entropy(
         return logp, ent, lse
     if V == 0:
         raise ValueError("empty vocabulary")
-    with torch.cuda.device(device):
+    with N.on_device(device):
         rc = N.lib().unirl_token_logp_entropy(
             N.ptr(x2), N.dtype_code(x2.dtype), rows, V, row_stride, N.ptr(idc), float(temperature),
             N.ptr(logp), N.ptr(ent), N.ptr(lse), N.current_stream(device),
@@ -576,7 +584,7 @@ def token_logp_bwd(
     gc = g_logp.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
     grad = torch.empty_like(x2)
     if rows and V:
-        with torch.cuda.device(device):
+        with N.on_device(device):
             rc = N.lib().unirl_token_logp_bwd(
                 N.ptr(x2), N.dtype_code(x2.dtype), rows, V, V, N.ptr(idc), float(temperature), N.ptr(lsec),
                 N.ptr(gc), N.ptr(grad), V, N.current_stream(device),
@@ -686,12 +694,13 @@ class RatioLossPlan:
             metrics.fill_(float("nan"))
             metrics[N.M_NUM_TOKENS] = 0.0
             return elem, metrics
-        ws, ws_bytes = N.workspace(device)
-        with torch.cuda.device(device):
+        stream = N.current_stream(device)
+        ws, ws_bytes = N.workspace(device, stream)
+        with N.on_device(device):
             rc = N.lib().unirl_ratio_loss_fwd(
                 N.ptr(self.nw), N.ptr(self.od), N.ptr(self.adv), N.ptr(self.seq), N.ptr(self.mask), self.n_seq,
                 self.seq_stride, self.n_tok, ctypes.byref(self.params), N.ptr(elem), N.ptr(metrics), N.ptr(ws),
-                ws_bytes, N.current_stream(device),
+                ws_bytes, stream,
             )
         N.check(rc, "unirl_ratio_loss_fwd")
         return elem, metrics
@@ -712,7 +721,7 @@ class RatioLossPlan:
         gs = None if g_scale is None else g_scale.detach().to(device=device, dtype=torch.float32).reshape(-1)[:1].contiguous()
         ge = None if g_elem is None else g_elem.detach().to(device=device, dtype=torch.float32).contiguous()
         nv = None if n_valid is None else n_valid.detach().reshape(-1)[:1].contiguous()
-        with torch.cuda.device(device):
+        with N.on_device(device):
             rc = N.lib().unirl_ratio_loss_bwd(
                 N.ptr(self.nw), N.ptr(self.od), N.ptr(self.adv), N.ptr(self.seq), N.ptr(self.mask), self.n_seq,
                 self.seq_stride, self.n_tok, ctypes.byref(self.params), N.ptr(gs), N.ptr(ge),
@@ -742,7 +751,7 @@ def group_advantages(
         return out
     if n_groups <= 0 or n % n_groups != 0:
         raise ValueError(f"non-uniform group sizes (n={n}, n_groups={n_groups})")
-    with torch.cuda.device(r.device):
+    with N.on_device(r.device):
         rc = N.lib().unirl_group_advantages(
             N.ptr(r), n_groups, n // n_groups, int(bool(normalize)), float(eps), int(scope == "global"),
             int(bool(use_global_std)), N.ptr(out), N.current_stream(r.device),
@@ -780,7 +789,7 @@ def normalize_grouped(
         return out
     mem_t = torch.tensor(members, dtype=torch.int64, device=device)
     off_t = torch.tensor(offsets, dtype=torch.int64, device=device)
-    with torch.cuda.device(device):
+    with N.on_device(device):
         rc = N.lib().unirl_normalize_grouped(
             N.ptr(r), n, N.ptr(mem_t), N.ptr(off_t), n_groups, float(eps), float(trim_outliers_ratio),
             int(bool(use_global_std)), int(clip_max is not None), float(clip_max or 0.0), N.ptr(out),
@@ -798,7 +807,7 @@ def calib_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
     nbytes = src.numel() * src.element_size()
     if nbytes != dst.numel() * dst.element_size() or not (src.is_contiguous() and dst.is_contiguous()):
         raise ValueError("calib_copy needs two contiguous tensors of the same byte size")
-    with torch.cuda.device(src.device):
+    with N.on_device(src.device):
         rc = N.lib().unirl_calib_copy(N.ptr(src), N.ptr(dst), nbytes, N.current_stream(src.device))
     N.check(rc, "unirl_calib_copy")
 
@@ -813,7 +822,7 @@ def calib_stream(src: Optional[torch.Tensor], read_bytes: int, dst: Optional[tor
             N.require_device(t, name)
             if not t.is_contiguous() or t.numel() * t.element_size() < nbytes:
                 raise ValueError(f"{name} must be contiguous and hold at least {nbytes} bytes")
-    with torch.cuda.device(sink.device):
+    with N.on_device(sink.device):
         rc = N.lib().unirl_calib_stream(
             N.ptr(src) if read_bytes else None, int(read_bytes), N.ptr(dst) if write_bytes else None,
             int(write_bytes), int(bool(tail_launch)), N.ptr(sink), N.current_stream(sink.device),
@@ -838,7 +847,7 @@ def gather_steps(tensor: torch.Tensor, positions: Sequence[int]) -> torch.Tensor
     if out.numel() == 0:
         return out
     pos_t = torch.tensor(pos, dtype=torch.int64, device=t.device)
-    with torch.cuda.device(t.device):
+    with N.on_device(t.device):
         rc = N.lib().unirl_gather_steps(
             N.ptr(t), B, S, inner_bytes, N.ptr(pos_t), len(pos), N.ptr(out), N.current_stream(t.device)
         )
@@ -861,7 +870,7 @@ def expand_groups(unique: torch.Tensor, group_of: torch.Tensor, dtype: torch.dty
         return out
     if U == 0:
         raise ValueError("no noise groups to expand")
-    with torch.cuda.device(src.device):
+    with N.on_device(src.device):
         rc = N.lib().unirl_expand_groups(
             N.ptr(src), U, D, N.ptr(idx), B, N.ptr(out), N.dtype_code(dtype), N.current_stream(src.device)
         )
