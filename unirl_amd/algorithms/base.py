@@ -143,11 +143,90 @@ class StageAlgorithm(ABC):
         ...
 
 
+NO_STEP = AlgorithmStepResult(loss=0.0, metrics={}, num_steps_or_tokens=0, has_backward=False)
+
+
+def bind_stage(owner: str, stage: Any, pipeline: Any, stage_attr: str) -> Any:
+    """The stage an algorithm drives: given directly, or looked up on a pipeline."""
+    if stage is not None:
+        return stage
+    if pipeline is None:
+        raise ValueError(f"{owner}: either `stage` or `pipeline` must be provided")
+    return getattr(pipeline, stage_attr)
+
+
+def parse_old_logp_source(owner: str, value: Any) -> str:
+    source = str(value).strip().lower()
+    if source not in ("rollout", "replay"):
+        raise ValueError(f"{owner}: old_logp_source must be 'rollout' or 'replay'; got {value!r}")
+    return source
+
+
+class SdeStepAlgorithm(StageAlgorithm):
+    """Shared plumbing of the diffusion algorithms that train on the SDE steps a rollout recorded
+    (FlowGRPO, FlowDPPO): which steps, how the stage is replayed on them, and how the old
+    policy's per-step quantities are frozen on the segment before the update loop.
+
+    Subclasses set ``anchor_fields``, implement ``_freeze(segment, replay_result)`` and the loss.
+    ``_needs_replay_for_anchor`` says whether ``prepare_segment`` must replay even when the
+    rollout's own log-probs are trusted (FlowDPPO: always, for the means).
+    """
+
+    supports_multi_update = True
+    _needs_replay_for_anchor = False
+    stage: Any
+    params: Any
+    conditions_cls: Optional[Type[Any]]
+    old_logp_source: str
+
+    def _setup(self, *, params, stage, pipeline, stage_attr, old_logp_source, conditions_cls) -> None:
+        owner = type(self).__name__
+        self.stage = bind_stage(owner, stage, pipeline, stage_attr)
+        self.params = params
+        self.old_logp_source = parse_old_logp_source(owner, old_logp_source)
+        self.conditions_cls = conditions_cls
+
+    def recomputes_anchor(self) -> bool:
+        return self._needs_replay_for_anchor or self.old_logp_source == "replay"
+
+    def _resolve_target_steps(self, segment: Any) -> List[int]:
+        """Every SDE step the rollout recorded; subclasses may filter."""
+        indices = segment.sde_indices
+        return [] if indices is None else [int(i) for i in indices.tolist()]
+
+    def _replay(self, conditions: Mapping[str, Any], segment: Any, steps: List[int]) -> Any:
+        return self.stage.replay(
+            typed_conditions(conditions, self.conditions_cls), segment=segment, params=self.params, step_indices=steps
+        )
+
+    def _freeze(self, segment: Any, result: Any) -> None:
+        raise NotImplementedError
+
+    def prepare_segment(self, *, conditions: Mapping[str, Any], segment: Any) -> None:
+        steps = self._resolve_target_steps(segment)
+        if not steps:
+            return
+        if self.old_logp_source == "rollout" and segment.sde_logp is None:
+            raise RuntimeError(
+                f"{type(self).__name__}.prepare_segment: old_logp_source='rollout' but the rollout engine emitted no "
+                "per-step log-probs (segment.sde_logp is None). Pin a rollout build that emits trajectory "
+                "log-probs, or set old_logp_source='replay'."
+            )
+        if not self.recomputes_anchor():
+            return
+        with torch.no_grad():
+            self._freeze(segment, self._replay(conditions, segment, steps))
+
+
 __all__ = [
     "ABSDIFF_METRICS",
     "AlgorithmStepResult",
     "BaseAlgorithmConfig",
+    "NO_STEP",
+    "SdeStepAlgorithm",
     "StageAlgorithm",
+    "bind_stage",
+    "parse_old_logp_source",
     "gather_sde_field",
     "rollout_replay_logp_absdiff",
     "typed_conditions",

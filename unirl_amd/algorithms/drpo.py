@@ -16,7 +16,14 @@ import torch
 from .. import _native as N
 from .. import ops
 from ._fused import ABSDIFF_METRICS, DRPO_METRICS, elem_loss, fused_token_loss, metric_tensors
-from .base import AlgorithmStepResult, BaseAlgorithmConfig, StageAlgorithm, typed_conditions
+from .base import (
+    NO_STEP,
+    AlgorithmStepResult,
+    BaseAlgorithmConfig,
+    StageAlgorithm,
+    parse_old_logp_source,
+    typed_conditions,
+)
 from .grpo import _DEFAULT_AR_TEMPERATURE, cu_seqlens_from_lengths
 
 
@@ -78,9 +85,7 @@ class DRPO(StageAlgorithm):
             _DEFAULT_AR_TEMPERATURE if sampling_temperature is None else sampling_temperature
         )
         self.conditions_cls = conditions_cls
-        self.old_logp_source = str(old_logp_source).strip().lower()
-        if self.old_logp_source not in ("rollout", "replay"):
-            raise ValueError(f"DRPO: old_logp_source must be 'rollout' or 'replay'; got {old_logp_source!r}")
+        self.old_logp_source = parse_old_logp_source("DRPO", old_logp_source)
         self.supports_multi_update = True
 
     def prepare_segment(self, *, conditions: Mapping[str, Any], segment: Any) -> None:
@@ -106,9 +111,9 @@ class DRPO(StageAlgorithm):
         loss_scale: float,
     ) -> AlgorithmStepResult:
         if segment.tokens is None or segment.lengths is None or segment.log_probs is None:
-            return AlgorithmStepResult(loss=0.0, metrics={}, num_steps_or_tokens=0, has_backward=False)
+            return NO_STEP
         if int(segment.tokens.shape[0]) == 0:
-            return AlgorithmStepResult(loss=0.0, metrics={}, num_steps_or_tokens=0, has_backward=False)
+            return NO_STEP
 
         new_logp = self.stage.replay(
             typed_conditions(conditions, self.conditions_cls), segment=segment, temperature=self.sampling_temperature

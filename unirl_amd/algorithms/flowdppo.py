@@ -17,7 +17,7 @@ from typing import Any, Dict, List, Mapping, Optional, Tuple, Type
 import torch
 
 from .. import ops
-from .base import AlgorithmStepResult, BaseAlgorithmConfig, StageAlgorithm, gather_sde_field, typed_conditions
+from .base import NO_STEP, AlgorithmStepResult, BaseAlgorithmConfig, SdeStepAlgorithm, gather_sde_field
 
 
 @dataclass
@@ -94,14 +94,11 @@ def _flowdppo_kl_adv_loss(
     return elem, metrics
 
 
-class FlowDPPO(StageAlgorithm):
+class FlowDPPO(SdeStepAlgorithm):
     """KL-divergence masking in place of ratio clipping for diffusion RL."""
 
-    supports_multi_update = True
     anchor_fields = ("sde_logp", "sde_means")
-
-    def recomputes_anchor(self) -> bool:
-        return True
+    _needs_replay_for_anchor = True  # the old policy's means exist only after a replay
 
     def __init__(
         self,
@@ -115,45 +112,20 @@ class FlowDPPO(StageAlgorithm):
         old_logp_source: str = "rollout",
         conditions_cls: Optional[Type[Any]] = None,
     ) -> None:
-        if stage is None and pipeline is not None:
-            stage = getattr(pipeline, stage_attr)
-        if stage is None:
-            raise ValueError("FlowDPPO: either `stage` or `pipeline` must be provided")
-        self.stage = stage
-        self.params = params
+        self._setup(params=params, stage=stage, pipeline=pipeline, stage_attr=stage_attr,
+                    old_logp_source=old_logp_source, conditions_cls=conditions_cls)
         self.kl_mask_threshold = float(kl_mask_threshold)
         self.add_kl_coefficient = bool(add_kl_coefficient)
-        self.old_logp_source = str(old_logp_source).strip().lower()
-        if self.old_logp_source not in ("rollout", "replay"):
-            raise ValueError(f"FlowDPPO: old_logp_source must be 'rollout' or 'replay'; got {old_logp_source!r}")
-        self.conditions_cls = conditions_cls
 
-    def prepare_segment(self, *, conditions: Mapping[str, Any], segment: Any) -> None:
-        """Freeze the old policy's means (always) and log-probs (``'replay'``) on the segment.
-        They stay on the device they were computed on."""
-        if segment.sde_indices is None:
-            return
-        target_steps = self._resolve_target_steps(segment)
-        if not target_steps:
-            return
-        if self.old_logp_source == "rollout" and segment.sde_logp is None:
-            raise RuntimeError(
-                "FlowDPPO.prepare_segment: old_logp_source='rollout' but the rollout engine emitted no "
-                "per-step log-probs (segment.sde_logp is None). Pin a rollout build that emits trajectory "
-                "log-probs, or set old_logp_source='replay'."
-            )
-        with torch.no_grad():
-            result = self.stage.replay(
-                typed_conditions(conditions, self.conditions_cls), segment=segment, params=self.params,
-                step_indices=target_steps,
-            )
-        if self.old_logp_source == "replay":
-            segment.sde_logp = result.log_probs.detach()
+    def _freeze(self, segment: Any, result: Any) -> None:
+        """Old means always, old log-probs only under ``'replay'``; both stay on the device."""
         if result.prev_sample_means is None:
             raise RuntimeError(
                 "FlowDPPO.prepare_segment: stage.replay() returned prev_sample_means=None. Ensure the "
                 "stage's replay method produces means (required for KL-ADV masking)."
             )
+        if self.old_logp_source == "replay":
+            segment.sde_logp = result.log_probs.detach()
         segment.sde_means = result.prev_sample_means.detach()
 
     def compute_loss_and_backward(
@@ -165,13 +137,11 @@ class FlowDPPO(StageAlgorithm):
         training_progress: float,
         loss_scale: float,
     ) -> AlgorithmStepResult:
-        target_steps = self._resolve_target_steps(segment)
-        if not target_steps:
-            return AlgorithmStepResult(loss=0.0, metrics={}, num_steps_or_tokens=0, has_backward=False)
-        replay = self.stage.replay(
-            typed_conditions(conditions, self.conditions_cls), segment=segment, params=self.params,
-            step_indices=target_steps,
-        )
+        del training_progress
+        steps = self._resolve_target_steps(segment)
+        if not steps:
+            return NO_STEP
+        replay = self._replay(conditions, segment, steps)
         new_logp, new_means = replay.log_probs, replay.prev_sample_means
         if new_means is None:
             raise RuntimeError(
@@ -179,40 +149,31 @@ class FlowDPPO(StageAlgorithm):
                 "Ensure the stage's replay method produces means."
             )
         device = new_logp.device
-        old_logp = gather_sde_field(segment.sde_logp, segment.sde_indices, target_steps, field_name="sde_logp").to(
-            dtype=new_logp.dtype, device=device
-        )
-        old_means = gather_sde_field(segment.sde_means, segment.sde_indices, target_steps, field_name="sde_means").to(
-            dtype=new_means.dtype, device=new_means.device
-        )
-        sigma_t = self._compute_sigma_t(segment, target_steps, device=device)
+
+        def frozen(name, like):
+            t = gather_sde_field(getattr(segment, name), segment.sde_indices, steps, field_name=name)
+            return t.to(dtype=like.dtype, device=like.device)
+
+        old_logp, old_means = frozen("sde_logp", new_logp), frozen("sde_means", new_means)
+        sigma_t = self._compute_sigma_t(segment, steps, device=device)
         adv_b = advantages.detach().to(dtype=new_logp.dtype, device=device).reshape(-1, 1).expand_as(new_logp)
 
         elem, mvec = self._loss_with_metrics(new_logp, old_logp, new_means, old_means, adv_b, sigma_t)
-        loss = elem.mean()
-        (loss * loss_scale).backward()
+        (elem.mean() * loss_scale).backward()
 
-        vals = mvec.tolist()
-        slots = ops.FLOWDPPO_METRIC_SLOTS
-        metrics: Dict[str, Any] = {
-            "policy_loss": vals[slots["loss_mean"]],
-            "kl_mask_threshold": float(self.kl_mask_threshold),
-        }
-        metrics.update({k: vals[s] for k, s in slots.items() if k != "loss_mean"})
-        return AlgorithmStepResult(
-            loss=vals[slots["loss_mean"]], metrics=metrics, num_steps_or_tokens=len(target_steps), has_backward=True
-        )
+        vals = mvec.tolist()  # the step's only device-to-host copy
+        slots = dict(ops.FLOWDPPO_METRIC_SLOTS)
+        loss_value = vals[slots.pop("loss_mean")]
+        metrics: Dict[str, Any] = {k: vals[slot] for k, slot in slots.items()}
+        metrics.update(policy_loss=loss_value, kl_mask_threshold=float(self.kl_mask_threshold))
+        return AlgorithmStepResult(loss=loss_value, metrics=metrics, num_steps_or_tokens=len(steps),
+                                   has_backward=True)
 
     def _loss_with_metrics(self, new_logp, old_logp, new_means, old_means, adv_b, sigma_t):
         kl, _ = ops.gaussian_kl_mask(
             new_means, old_means, sigma_t, self.kl_mask_threshold, reduce_from_dim=2, want_mask=False
         )
         return _MaskedRatioLossFn.apply(new_logp, old_logp, adv_b, kl, self.kl_mask_threshold)
-
-    def _resolve_target_steps(self, segment: Any) -> List[int]:
-        if segment.sde_indices is None:
-            return []
-        return [int(i) for i in segment.sde_indices.tolist()]
 
     def _compute_sigma_t(self, segment: Any, target_steps: List[int], device: torch.device) -> torch.Tensor:
         """``std_dev_t * sqrt(-dt)`` per target step, ``[1, S', 1, 1, 1]`` (ones when

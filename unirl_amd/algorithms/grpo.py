@@ -18,10 +18,12 @@ from .. import _native as N
 from .. import ops
 from ._fused import ABSDIFF_METRICS, GRPO_METRICS, fused_token_loss
 from .base import (
+    NO_STEP,
     AlgorithmStepResult,
     BaseAlgorithmConfig,
     StageAlgorithm,
     _resolve_clip_range_from_schedule,
+    bind_stage,
     typed_conditions,
 )
 
@@ -64,9 +66,7 @@ class GRPO(StageAlgorithm):
         conditions_cls: Optional[Type[Any]] = None,
         sampling_temperature: Optional[float] = None,
     ) -> None:
-        if stage is None and pipeline is None:
-            raise ValueError("GRPO: either `stage` or `pipeline` must be provided")
-        self.stage = stage if stage is not None else getattr(pipeline, stage_attr)
+        self.stage = bind_stage("GRPO", stage, pipeline, stage_attr)
         self.clip_range = float(clip_range)
         self.clip_range_high = None if clip_range_high is None else float(clip_range_high)
         self.clip_schedule = str(clip_schedule)
@@ -87,9 +87,9 @@ class GRPO(StageAlgorithm):
         loss_scale: float,
     ) -> AlgorithmStepResult:
         if segment.tokens is None or segment.lengths is None or segment.log_probs is None:
-            return AlgorithmStepResult(loss=0.0, metrics={}, num_steps_or_tokens=0, has_backward=False)
+            return NO_STEP
         if int(segment.tokens.shape[0]) == 0:
-            return AlgorithmStepResult(loss=0.0, metrics={}, num_steps_or_tokens=0, has_backward=False)
+            return NO_STEP
 
         new_logp = self.stage.replay(
             typed_conditions(conditions, self.conditions_cls), segment=segment, temperature=self.sampling_temperature
