@@ -330,7 +330,7 @@ __device__ __forceinline__ void fill_ones(float (&m)[VEC]) {
 template <int KIND, int VEC, bool PACKED>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A) {
   constexpr int NW = kRlThreads / kWave;
-  constexpr int ITEMS = (VEC == 4) ? 4 : 2;  // vectors in flight per lane
+  constexpr int ITEMS = 2;  // vectors in flight per lane
   __shared__ double lds_v[NW][kRlVals];
   const RatioConsts C = A.C;
 
@@ -428,8 +428,18 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
         const unsigned int jj = j + b * kSlices;
         y[b] = (jj < nblk) ? A.partials[(int64_t)jj * kRlVals + v] : ident;
       }
+      // one kind of operation per lane, chosen once per batch (three short divergent runs) rather
+      // than a three-way select per element
+      if (v < P_RMIN) {
 #pragma unroll
-      for (int b = 0; b < kBatch; ++b) x = combine(v, x, y[b]);
+        for (int b = 0; b < kBatch; ++b) x += y[b];
+      } else if (v == P_RMIN) {
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) x = fmin(x, y[b]);
+      } else {
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) x = fmax(x, y[b]);
+      }
     }
     lds_fin[threadIdx.x] = x;
   }
@@ -437,41 +447,51 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
   if (threadIdx.x < kRlVals) {
     const int v = threadIdx.x;
     double x = lds_fin[v];
-    for (int j = 1; j < kRlThreads / kRlVals; ++j) x = combine(v, x, lds_fin[j * kRlVals + v]);
+    if (v < P_RMIN) {
+      for (int j = 1; j < kRlThreads / kRlVals; ++j) x += lds_fin[j * kRlVals + v];
+    } else if (v == P_RMIN) {
+      for (int j = 1; j < kRlThreads / kRlVals; ++j) x = fmin(x, lds_fin[j * kRlVals + v]);
+    } else {
+      for (int j = 1; j < kRlThreads / kRlVals; ++j) x = fmax(x, lds_fin[j * kRlVals + v]);
+    }
     lds_fin[v] = x;
   }
   __syncthreads();
   if (threadIdx.x != 0) return;
   const double N = lds_fin[P_CNT];
   const double sr = lds_fin[P_SR], sr2 = lds_fin[P_SR2];
+  // One fp64 reciprocal serves every mean (this thread runs alone; an fp64 divide per metric was a
+  // third of the kernel).  x * (1/N) and x / N differ by at most an ulp of fp64, far below the
+  // fp32 result's rounding.
+  const double inv_n = 1.0 / N;
   double loss = lds_fin[P_LOSS];
   if (C.agg_mode == UNIRL_AGG_TOKEN_MEAN)
-    loss = loss / N;
+    loss = loss * inv_n;
   else if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_SUM)
-    loss = (loss / (double)A.n_seq) / (double)C.horizon;
+    loss = loss / ((double)A.n_seq * (double)C.horizon);
   else
     loss = loss / (double)A.n_seq;
   // sr, sr2: sums of (r-1) and (r-1)^2
   double var = 0.0;
   if (N > 1.0) {
-    var = (sr2 - sr * sr / N) / (N - 1.0);
+    var = (sr2 - sr * sr * inv_n) / (N - 1.0);
     if (var < 0.0) var = 0.0;
   }
   float* M = A.metrics;
   M[UNIRL_M_LOSS] = (float)loss;
-  M[UNIRL_M_RATIO_MEAN] = (float)(1.0 + sr / N);
+  M[UNIRL_M_RATIO_MEAN] = (float)(1.0 + sr * inv_n);
   M[UNIRL_M_RATIO_STD] = (float)sqrt(var);
   // min()/max() of the reference return NaN when any ratio is NaN; the ratios are >= 0, so their
   // sum is NaN exactly then (likewise the absolute differences below)
   M[UNIRL_M_RATIO_MIN] = (sr != sr) ? quiet_nan() : (float)lds_fin[P_RMIN];
   M[UNIRL_M_RATIO_MAX] = (sr != sr) ? quiet_nan() : (float)lds_fin[P_RMAX];
-  M[UNIRL_M_CLIP_FRACTION] = (float)lds_fin[P_CANY] / (float)N;
-  M[UNIRL_M_CLIPFRAC_HI] = (float)lds_fin[P_CHI] / (float)N;
-  M[UNIRL_M_CLIPFRAC_LO] = (float)lds_fin[P_CLO] / (float)N;
+  M[UNIRL_M_CLIP_FRACTION] = (float)(lds_fin[P_CANY] * inv_n);
+  M[UNIRL_M_CLIPFRAC_HI] = (float)(lds_fin[P_CHI] * inv_n);
+  M[UNIRL_M_CLIPFRAC_LO] = (float)(lds_fin[P_CLO] * inv_n);
   // GRPO accumulates ld^2; mean(0.5*ld^2) = 0.5*sum/N exactly (halving commutes with rounding)
-  M[UNIRL_M_APPROX_KL] = (float)((C.kind == UNIRL_LOSS_GRPO ? 0.5 : 1.0) * lds_fin[P_KL] / N);
-  M[UNIRL_M_PENALTY_MEAN] = (float)(lds_fin[P_PEN] / N);
-  M[UNIRL_M_ABSDIFF_MEAN] = (float)(lds_fin[P_ABS] / N);
+  M[UNIRL_M_APPROX_KL] = (float)((C.kind == UNIRL_LOSS_GRPO ? 0.5 : 1.0) * lds_fin[P_KL] * inv_n);
+  M[UNIRL_M_PENALTY_MEAN] = (float)(lds_fin[P_PEN] * inv_n);
+  M[UNIRL_M_ABSDIFF_MEAN] = (float)(lds_fin[P_ABS] * inv_n);
   M[UNIRL_M_ABSDIFF_MAX] = (lds_fin[P_ABS] != lds_fin[P_ABS]) ? quiet_nan() : (float)lds_fin[P_AMAX];
   M[UNIRL_M_NUM_TOKENS] = (float)N;
   M[13] = M[14] = M[15] = 0.0f;
@@ -597,7 +617,9 @@ static int plan(const RatioArgs& A, bool bwd, RatioShape& S) {
   if (padded && A.seq_stride % 4 != 0) vec = 1;
   const int64_t row_tok = padded ? A.seq_stride : A.n_tok;
   const int64_t nvec = (row_tok + vec - 1) / vec;
-  const int64_t cap = bwd ? 16384 : tune_int("UNIRL_RATIO_MAX_BLOCKS", 512);
+  // forward: one partial vector per workgroup is read back by a single finalize workgroup, whose
+  // time grows with their number (about 1 us per 128); 512 suits inputs of a few MB, 1024 large ones
+  const int64_t cap = bwd ? 16384 : tune_int("UNIRL_RATIO_MAX_BLOCKS", A.n_tok >= (16 << 20) ? 1024 : 512);
   int64_t rows = padded ? A.n_seq : 1;
   if (rows > cap) rows = cap;
   if (rows < 1) rows = 1;

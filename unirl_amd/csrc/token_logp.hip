@@ -317,6 +317,15 @@ __global__ __launch_bounds__(TPB) void token_logp_entropy_kernel(TokArgs A) {
   const int64_t V = A.V;
   const float c = A.c;
 
+  // The target id and its logit are fetched before the scan (two dependent trips to memory that
+  // would otherwise sit in the row's tail, after the last vector has been consumed).
+  int64_t id = -1;
+  float x_id = 0.0f;
+  if (threadIdx.x == 0 && A.logp) {
+    id = A.ids[row];
+    if (id >= 0 && id < V) x_id = Elem<T>::load(p + id);
+  }
+
   TokState st = tok_scan_row<T, UNROLL, TPB, false>(p, V, c, lds);
   if (threadIdx.x == 0) redo = !(fabsf(st.s) <= FLT_MAX) || !(fabsf(st.t) <= FLT_MAX);  // inf or NaN
   __syncthreads();
@@ -331,12 +340,8 @@ __global__ __launch_bounds__(TPB) void token_logp_entropy_kernel(TokArgs A) {
     if (A.lse) A.lse[row] = has_nan ? quiet_nan() : INFINITY;
     if (A.ent) A.ent[row] = quiet_nan();
     if (A.logp) {
-      const int64_t id = A.ids[row];
       float out = quiet_nan();
-      if (!has_nan && id >= 0 && id < V) {
-        const float x_id = Elem<T>::load(p + id);
-        if (x_id < INFINITY) out = -INFINITY;  // false for +inf and NaN
-      }
+      if (!has_nan && id >= 0 && id < V && x_id < INFINITY) out = -INFINITY;  // x_id: false for +inf and NaN
       A.logp[row] = out;
     }
     return;
@@ -351,10 +356,9 @@ __global__ __launch_bounds__(TPB) void token_logp_entropy_kernel(TokArgs A) {
   if (A.lse) A.lse[row] = (float)(kLn2 * (double)st.r + ln_sum);
   if (A.ent) A.ent[row] = (float)(ln_sum - kLn2 * t_all / sum);
   if (A.logp) {
-    const int64_t id = A.ids[row];
     float out = __uint_as_float(0x7fc00000u);
     if (id >= 0 && id < V) {
-      const double a_id = (double)Elem<T>::load(p + id) * (double)c - (double)st.r;
+      const double a_id = (double)x_id * (double)c - (double)st.r;
       out = (float)(kLn2 * a_id - ln_sum);
     }
     A.logp[row] = out;
