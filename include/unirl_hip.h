@@ -215,6 +215,14 @@ int unirl_flowdppo_loss(const float* new_logp, const float* old_logp, const floa
 int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, const float* sigma,
                            int64_t n_sigma, int64_t R, int64_t D, float* out, void* stream);
 
+/* Its backward, for callers that differentiate _gaussian_kl_div (the reference's function is
+ * plain torch and therefore differentiable; its own loss detaches the result).  g_out f32 [R,D];
+ * grad_p / grad_q in the means' dtype, either may be NULL.  Follows autograd's chain through
+ * the 16-bit subtraction and square (flowdppo.py:51). */
+int unirl_gaussian_kl_elem_bwd(const void* p, const void* q, int dtype, const float* sigma,
+                               int64_t n_sigma, int64_t R, int64_t D, const float* g_out,
+                               void* grad_p, void* grad_q, void* stream);
+
 /* ------------------------------------------------------------------------
  * Token log-prob and entropy over the vocabulary.  Replaces _logp_chunk
  * (unirl/models/qwen3/ar.py:82-85) and the log_softmax(...).gather sites

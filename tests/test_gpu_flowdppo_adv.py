@@ -225,3 +225,32 @@ def test_normalize_grouped_matches_oracle(dev):
                  "global clipped")
     with pytest.raises(IndexError):
         normalize_grouped(r.to(dev), [[0, 40]])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_gaussian_kl_div_is_differentiable(dev, dtype):
+    """The reference's _gaussian_kl_div is plain torch; a caller may differentiate it."""
+    from unirl_amd.algorithms import _gaussian_kl_div
+
+    g = torch.Generator().manual_seed(21)
+    p = torch.randn(3, 4, 4, 8, 8, generator=g).to(dtype)
+    q = (p.float() + 0.1 * torch.randn(p.shape, generator=g)).to(dtype)
+    s = torch.tensor([0.3, 0.25, 0.2, 0.15]).view(1, 4, 1, 1, 1)
+    w = torch.randn(p.shape, generator=g)
+    pr, qr = p.clone().requires_grad_(True), q.clone().requires_grad_(True)
+    (ofd.gaussian_kl(pr, qr, s) * w).sum().backward()
+    pd, qd = p.to(dev).requires_grad_(True), q.to(dev).requires_grad_(True)
+    out = _gaussian_kl_div(pd, qd, s.to(dev))
+    assert out.dtype == torch.float32 and out.requires_grad
+    (out * w.to(dev)).sum().backward()
+    rtol = FP32_RTOL if dtype == torch.float32 else 8e-3  # two 16-bit roundings in the chain
+    scale = float(pr.grad.float().abs().max())
+    assert pd.grad.dtype == dtype and qd.grad.dtype == dtype
+    assert_close(pd.grad, pr.grad, rtol, rtol * scale * 1e-2, "grad p")
+    assert_close(qd.grad, qr.grad, rtol, rtol * scale * 1e-2, "grad q")
+    # only one side needs a gradient
+    pd2 = p.to(dev).requires_grad_(True)
+    _gaussian_kl_div(pd2, q.to(dev), s.to(dev)).sum().backward()
+    pr2 = p.clone().requires_grad_(True)
+    ofd.gaussian_kl(pr2, q, s).sum().backward()
+    assert_close(pd2.grad, pr2.grad, rtol, rtol * float(pr2.grad.float().abs().max()) * 1e-2, "grad p only")

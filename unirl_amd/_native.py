@@ -132,6 +132,10 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p],
     ),
+    "unirl_gaussian_kl_elem_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
     "unirl_token_logp_entropy": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p],

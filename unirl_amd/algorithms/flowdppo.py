@@ -45,11 +45,38 @@ def _sigma_axis(p: torch.Tensor, sigma: torch.Tensor) -> Optional[int]:
     return axes[0]
 
 
+class _KlElemFn(torch.autograd.Function):
+    """Element-wise KL with gradients to both means (sigma is treated as a constant)."""
+
+    @staticmethod
+    def forward(ctx, p, q, sigma, sigma_dim):
+        ctx.save_for_backward(p.detach(), q.detach(), sigma.detach())
+        ctx.sigma_dim = sigma_dim
+        ctx.dtypes = (p.dtype, q.dtype)
+        return ops.gaussian_kl_elem(p, q, sigma, sigma_dim=sigma_dim)
+
+    @staticmethod
+    def backward(ctx, g_out):
+        p, q, sigma = ctx.saved_tensors
+        gp, gq = ops.gaussian_kl_elem_bwd(
+            p, q, sigma, g_out, sigma_dim=ctx.sigma_dim, need_p=ctx.needs_input_grad[0],
+            need_q=ctx.needs_input_grad[1],
+        )
+        if gp is not None:
+            gp = gp.reshape(p.shape).to(ctx.dtypes[0])
+        if gq is not None:
+            gq = gq.reshape(q.shape).to(ctx.dtypes[1])
+        return gp, gq, None, None
+
+
 def _gaussian_kl_div(p: torch.Tensor, q: torch.Tensor, sigma: torch.Tensor) -> torch.Tensor:
     """Per-element ``(p - q)^2 / (2 sigma^2)`` (fp32; 16-bit inputs subtract and square in
-    their own dtype first, as torch's type promotion does)."""
+    their own dtype first, as torch's type promotion does).  Differentiable w.r.t. ``p`` and ``q``."""
     axis = _sigma_axis(p, sigma)
-    return ops.gaussian_kl_elem(p, q, sigma, sigma_dim=1 if axis is None else axis)
+    sigma_dim = 1 if axis is None else axis
+    if torch.is_grad_enabled() and (p.requires_grad or q.requires_grad):
+        return _KlElemFn.apply(p, q, sigma, sigma_dim)
+    return ops.gaussian_kl_elem(p, q, sigma, sigma_dim=sigma_dim)
 
 
 class _MaskedRatioLossFn(torch.autograd.Function):

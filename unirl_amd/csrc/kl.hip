@@ -116,6 +116,53 @@ __global__ __launch_bounds__(kKlThreads) void gaussian_kl_elem_kernel(KlArgs A) 
   }
 }
 
+// Backward of the element-wise form through autograd's own chain: out = sq / den (f32),
+// sq = d*d and d = p - q in the means' dtype.  The incoming f32 gradient is divided by den and
+// rounded to that dtype, multiplied by 2d there, and reaches p as is and q negated.
+template <typename T, int VEC>
+__global__ __launch_bounds__(kKlThreads) void gaussian_kl_elem_bwd_kernel(KlArgs A, const float* g, void* grad_p,
+                                                                          void* grad_q) {
+  const int64_t row = blockIdx.y;
+  const int64_t D = A.D;
+  const T* __restrict__ pp = reinterpret_cast<const T*>(A.p) + row * D;
+  const T* __restrict__ qp = reinterpret_cast<const T*>(A.q) + row * D;
+  const float* __restrict__ gp = g + row * D;
+  T* __restrict__ op = grad_p ? reinterpret_cast<T*>(grad_p) + row * D : nullptr;
+  T* __restrict__ oq = grad_q ? reinterpret_cast<T*>(grad_q) + row * D : nullptr;
+  const float den = kl_den(A, row);
+  const int64_t nvec = D / VEC;
+  const int64_t stride = (int64_t)gridDim.x * kKlThreads;
+  for (int64_t i = (int64_t)blockIdx.x * kKlThreads + threadIdx.x; i < nvec; i += stride) {
+    float a[VEC], b[VEC], gg[VEC], o[VEC], n[VEC];
+    Vec<T, VEC>::load(pp + i * VEC, a);
+    Vec<T, VEC>::load(qp + i * VEC, b);
+    Vec<float, VEC>::load(gp + i * VEC, gg);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      const float d = Elem<T>::round_trip(a[k] - b[k]);
+      const float gs = Elem<T>::round_trip(gg[k] / den);
+      o[k] = Elem<T>::round_trip(gs * (2.0f * d));
+      n[k] = -o[k];
+    }
+    if (op) Vec<T, VEC>::store(op + i * VEC, o);
+    if (oq) Vec<T, VEC>::store(oq + i * VEC, n);
+  }
+}
+
+template <typename T>
+static int launch_kl_elem_bwd(const KlArgs& A, int64_t R, int vec, const float* g, void* gp, void* gq,
+                              hipStream_t st) {
+  int64_t nblk = (A.D / vec + kKlThreads - 1) / kKlThreads;
+  if (nblk > 2048) nblk = 2048;
+  if (nblk < 1) nblk = 1;
+  dim3 grid((unsigned int)nblk, (unsigned int)R), block(kKlThreads);
+  if (vec == 4)
+    hipLaunchKernelGGL((gaussian_kl_elem_bwd_kernel<T, 4>), grid, block, 0, st, A, g, gp, gq);
+  else
+    hipLaunchKernelGGL((gaussian_kl_elem_bwd_kernel<T, 1>), grid, block, 0, st, A, g, gp, gq);
+  return (int)hipGetLastError();
+}
+
 static unsigned int kl_blocks_per_row(int64_t nvec, int items, int64_t R) {
   const int64_t per_pass = (int64_t)kKlThreads * items;
   int64_t nblk = (nvec + per_pass - 1) / per_pass;
@@ -289,7 +336,7 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
   int vec = 4;
   if (D % 4 != 0 || !aligned_to(p, 4 * sz) || !aligned_to(q, 4 * sz)) vec = 1;
   if (sz == 2 && D % 8 == 0 && aligned_to(p, 16) && aligned_to(q, 16)) vec = 8;
-  const int items = (vec >= 4) ? (int)tune_int("UNIRL_KL_ITEMS", 1) : 2;
+  const int items = (vec >= 4) ? (int)tune_int("UNIRL_KL_ITEMS", 2) : 2;
   const unsigned int nblk = kl_blocks_per_row(D / vec, items, R);
   int64_t per_launch = kPartialCapacity / nblk;
   if (per_launch > 32768) per_launch = 32768;
@@ -357,6 +404,46 @@ extern "C" int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, c
       case UNIRL_F32: rc = launch_kl_elem<float>(A, nr, vec, st); break;
       case UNIRL_BF16: rc = launch_kl_elem<bf16_t>(A, nr, vec, st); break;
       case UNIRL_F16: rc = launch_kl_elem<f16_t>(A, nr, vec, st); break;
+    }
+    if (rc != 0) return rc;
+  }
+  return UNIRL_OK;
+}
+
+extern "C" int unirl_gaussian_kl_elem_bwd(const void* p, const void* q, int dtype, const float* sigma,
+                                          int64_t n_sigma, int64_t R, int64_t D, const float* g_out, void* grad_p,
+                                          void* grad_q, void* stream) {
+  if (!dtype_ok(dtype)) return UNIRL_E_DTYPE;
+  if (R < 0 || D <= 0 || n_sigma <= 0) return UNIRL_E_SHAPE;
+  if (R == 0 || (!grad_p && !grad_q)) return UNIRL_OK;
+  if (!p || !q || !sigma || !g_out) return UNIRL_E_NULL;
+  const size_t sz = dtype_size(dtype);
+  if (!aligned_to(p, sz) || !aligned_to(q, sz) || !aligned_to(g_out, 4) || !aligned_to(grad_p, sz) ||
+      !aligned_to(grad_q, sz))
+    return UNIRL_E_ALIGN;
+  int vec = 4;
+  if (D % 4 != 0 || !aligned_to(p, 4 * sz) || !aligned_to(q, 4 * sz) || !aligned_to(g_out, 16) ||
+      !aligned_to(grad_p, 4 * sz) || !aligned_to(grad_q, 4 * sz))
+    vec = 1;
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t per_launch = 32768;
+  for (int64_t r0 = 0; r0 < R; r0 += per_launch) {
+    const int64_t nr = (R - r0 < per_launch) ? (R - r0) : per_launch;
+    KlArgs A = {};
+    A.p = offset_ptr(p, r0 * D, sz);
+    A.q = offset_ptr(q, r0 * D, sz);
+    A.sigma = sigma;
+    A.n_sigma = n_sigma;
+    A.row0 = r0;
+    A.D = D;
+    const float* g = g_out + r0 * D;
+    void* gp = const_cast<void*>(offset_ptr(grad_p, r0 * D, sz));
+    void* gq = const_cast<void*>(offset_ptr(grad_q, r0 * D, sz));
+    int rc = UNIRL_E_DTYPE;
+    switch (dtype) {
+      case UNIRL_F32: rc = launch_kl_elem_bwd<float>(A, nr, vec, g, gp, gq, st); break;
+      case UNIRL_BF16: rc = launch_kl_elem_bwd<bf16_t>(A, nr, vec, g, gp, gq, st); break;
+      case UNIRL_F16: rc = launch_kl_elem_bwd<f16_t>(A, nr, vec, g, gp, gq, st); break;
     }
     if (rc != 0) return rc;
   }

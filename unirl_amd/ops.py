@@ -517,6 +517,35 @@ def gaussian_kl_elem(p: torch.Tensor, q: torch.Tensor, sigma: torch.Tensor, *, s
     return out
 
 
+def gaussian_kl_elem_bwd(
+    p: torch.Tensor, q: torch.Tensor, sigma: torch.Tensor, g_out: torch.Tensor, *, sigma_dim: int = 1,
+    need_p: bool = True, need_q: bool = True,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Gradients of :func:`gaussian_kl_elem` w.r.t. ``p`` and ``q`` (in their dtype)."""
+    device = p.device
+    pc = _flat2(p.detach(), "p")
+    qc = _flat2(q.detach(), "q").to(pc.dtype)
+    if pc.dtype not in N._DTYPE_CODE:
+        pc, qc = pc.float(), qc.float()
+    sig = sigma.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    if sig.numel() == 1:
+        R, D = 1, pc.numel()
+    else:
+        R = int(math.prod(pc.shape[: sigma_dim + 1]))
+        D = pc.numel() // R if R else 0
+    g = g_out.detach().to(device=device, dtype=torch.float32).contiguous()
+    gp = torch.empty_like(pc) if need_p else None
+    gq = torch.empty_like(pc) if need_q else None
+    if pc.numel() and (need_p or need_q):
+        with N.on_device(device):
+            rc = N.lib().unirl_gaussian_kl_elem_bwd(
+                N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, N.ptr(g), N.ptr(gp),
+                N.ptr(gq), N.current_stream(device),
+            )
+        N.check(rc, "unirl_gaussian_kl_elem_bwd")
+    return gp, gq
+
+
 def token_logp_entropy(
     logits: torch.Tensor,
     ids: Optional[torch.Tensor],
