@@ -292,10 +292,12 @@ __device__ __forceinline__ void store_block_partials(const RatioArgs& A, Acc& ac
   double vals[kRlVals];
   vals[P_SR] = wave_sum(acc.t_s1);
   vals[P_SR2] = wave_sum(acc.t_s2);
-  vals[P_LOSS] = wave_sum(acc.t_loss);
-  vals[P_KL] = wave_sum(acc.t_kl);
-  vals[P_PEN] = wave_sum(acc.t_pen);
-  vals[P_ABS] = wave_sum(acc.t_ab);
+  // a lane's total of these four is a handful of fp32 terms: rounding it to fp32 loses nothing the
+  // 1e-5 budget can see, and an fp32 DPP tree costs half the moves of an fp64 one
+  vals[P_LOSS] = (double)wave_sum((float)acc.t_loss);
+  vals[P_KL] = (double)wave_sum((float)acc.t_kl);
+  vals[P_PEN] = (double)wave_sum((float)acc.t_pen);
+  vals[P_ABS] = (double)wave_sum((float)acc.t_ab);
   vals[P_CNT] = (double)wave_sum(acc.cnt);
   vals[P_CHI] = (double)wave_sum(acc.chi);
   vals[P_CLO] = (double)wave_sum(acc.clo);
