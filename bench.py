@@ -149,6 +149,26 @@ def make_shapes(torch, dev):
         cpu_bytes=bytes1,
     ))
 
+    # the same step in replay mode: the stored next latent is given, mean and log-prob come back
+    prev_host = osde.sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7, noise=host1[2],
+                                 sigma_max=sig[1])[0]
+    prev1 = [prev_host.to(dev) + 0.0 * k for k in range(ns)]
+    bytes1r = 5 * numel * 4
+
+    def run1r(i):
+        x, v, _ = sets1[i % ns]
+        return ops.sde_step_logp(v, x, s10, s11, kind="flow", eta=0.7, prev_sample=prev1[i % ns], sigma_max=smax,
+                                 want_prev=False)
+
+    shapes.append(dict(
+        name="sde_step_logp_replay", config=1,
+        shape="fp32 [8,16,128,128], step 10/28, replay of a stored transition (4 reads, 1 write)",
+        bytes=bytes1r, read_bytes=4 * numel * 4, write_bytes=numel * 4, elements=numel, run=run1r, sets=ns,
+        cpu=lambda: osde.sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7,
+                                     prev_sample=prev_host, sigma_max=sig[1]),
+        cpu_bytes=bytes1r,
+    ))
+
     # -- config 3: GRPO / DRPO token loss, fp32 [256, 8192], lengths U[512, 8192] -----------------
     g = torch.Generator().manual_seed(1003)
     old = -8 * torch.rand(256, 8192, generator=g)

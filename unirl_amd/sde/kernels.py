@@ -129,6 +129,11 @@ class StepStrategy(ABC):
             # the reference draws with generator=None on noise_pred's device, in fp32
             noise = torch.randn(sample.shape, device=sample.device, dtype=torch.float32)
         needs_grad = torch.is_grad_enabled() and (noise_pred.requires_grad or sample.requires_grad)
+        # fp32 replay: the reference's .float() / .to(float32) round trip is the identity, so the
+        # caller's own tensor is handed back and the kernel need not write a copy of it
+        reuse_prev = (
+            prev_sample is not None and prev_sample.dtype == torch.float32 and sample.dtype == torch.float32
+        )
         if needs_grad:
             prev, logp, mean = _SdeStepFn.apply(
                 noise_pred, sample, prev_sample, noise, sigma, sigma_next, sigma_max, float(eta), kind
@@ -138,10 +143,9 @@ class StepStrategy(ABC):
         else:
             prev, logp, mean = ops.sde_step_logp(
                 noise_pred, sample, sigma, sigma_next, kind=kind, eta=float(eta), prev_sample=prev_sample,
-                noise=noise, sigma_max=sigma_max,
+                noise=noise, sigma_max=sigma_max, want_prev=not reuse_prev,
             )
-        if prev_sample is not None and prev_sample.dtype == torch.float32 and sample.dtype == torch.float32:
-            # the reference's .float() / .to(float32) are no-ops here: hand the caller's tensor back
+        if reuse_prev:
             prev = prev_sample
         return prev, logp, mean
 
