@@ -1,0 +1,150 @@
+"""Seeded random shapes, dtypes, strides and lengths against the oracle: the tails, alignments and
+layout switches that hand-picked shapes may miss.  Every case is small; each test draws a few dozen."""
+
+import random
+
+import pytest
+import torch
+
+from oracle import flowdppo as ofd
+from oracle import losses as olos
+from oracle import schedule as osch
+from oracle import sde as osde
+from oracle import token_logp as otok
+from tests._util import BF16_RTOL, FP32_RTOL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+SIG = osch.sigma_schedule(28, 3.0)
+DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+
+
+def rand_shape(rng, max_elems=6000):
+    nd = rng.choice((2, 3, 4, 5))
+    while True:
+        shape = tuple(rng.randint(1, 9) if i else rng.randint(1, 5) for i in range(nd - 1)) + (rng.randint(1, 67),)
+        n = 1
+        for s in shape[1:]:
+            n *= s
+        if n <= max_elems:
+            return shape
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_sde_step_random(dev, seed):
+    from unirl_amd import sde
+
+    rng = random.Random(1000 + seed)
+    for _ in range(6):
+        shape, kind = rand_shape(rng), rng.choice(("flow", "dance", "cps"))
+        dtype, vdtype = rng.choice(DTYPES), rng.choice(DTYPES)
+        i, eta = rng.randint(0, 27), rng.choice((0.3, 0.7, 1.0))
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        x = torch.randn(shape, generator=g).to(dtype)
+        v = torch.randn(shape, generator=g).to(vdtype)
+        n = torch.randn(shape, generator=g)
+        what = f"{kind} {shape} {dtype}/{vdtype} step {i} eta {eta}"
+        ref_prev, ref_lp, ref_mean = osde.sde_denoise(kind, v, x, SIG[i], SIG[i + 1], eta=eta, noise=n,
+                                                      sigma_max=SIG[1], ieee_sqrt=True)
+        st = sde.STRATEGIES[kind]()
+        prev, lp, mean = st.denoise(v.to(dev), x.to(dev), SIG[i].to(dev), SIG[i + 1].to(dev), eta=eta,
+                                    sigma_max=SIG[1].to(dev), noise=n.to(dev))
+        assert torch.equal(mean.cpu(), ref_mean) and torch.equal(prev.cpu(), ref_prev), what
+        rtol = FP32_RTOL if dtype == torch.float32 and vdtype == torch.float32 else BF16_RTOL
+        assert_close(lp, ref_lp, rtol, 2e-6, what)
+        # replay from a stack slice with an odd sample stride
+        K = rng.randint(2, 4)
+        stack = torch.zeros((shape[0], K) + shape[1:], dtype=dtype, device=dev)
+        stack[:, 0], stack[:, K - 1] = x.to(dev), ref_prev.to(dtype).to(dev)
+        _, r_lp, r_mean = osde.sde_denoise(kind, v, x, SIG[i], SIG[i + 1], eta=eta, prev_sample=ref_prev.to(dtype),
+                                           sigma_max=SIG[1], ieee_sqrt=True)
+        means = torch.zeros((shape[0], 3) + shape[1:], dtype=dtype, device=dev)
+        lps = torch.zeros(shape[0], 3, device=dev)
+        st.denoise_into(v.to(dev), stack[:, 0], SIG[i].to(dev), SIG[i + 1].to(dev), eta=eta,
+                        prev_sample=stack[:, K - 1], sigma_max=float(SIG[1]), mean_out=means[:, 1], logp_out=lps[:, 2])
+        assert torch.equal(means[:, 1].cpu(), r_mean.to(dtype)), what + " (stack replay)"
+        assert_close(lps[:, 2], r_lp, rtol, 2e-6, what + " (stack replay)")
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_token_logp_random(dev, seed):
+    from unirl_amd import models
+
+    rng = random.Random(2000 + seed)
+    for _ in range(8):
+        rows, V = rng.randint(1, 9), rng.choice((1, 2, 7, 8, 9, 63, 64, 65, 255, 1023, 2049, 4100, 33001))
+        dtype, T = rng.choice(DTYPES), rng.choice((1.0, 0.7, 1.3, 0.0))
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        pad = rng.randint(0, 9)
+        big = (3 * torch.randn(rows, V + pad, generator=g)).to(dtype)
+        x = big[:, pad:] if rng.random() < 0.5 else big[:, :V]  # row views: odd strides, odd base alignment
+        ids = torch.randint(0, V, (rows,), generator=g)
+        what = f"[{rows},{V}] {dtype} T={T} pad={pad}"
+        ref_lp = otok.token_logp(x, ids, T)
+        ref_ent = otok.token_entropy(x, T)
+        xd = big.to(dev)[:, pad:] if x.data_ptr() != big.data_ptr() else big.to(dev)[:, :V]
+        lp, ent = models.token_logp_entropy(xd, ids.to(dev), T)
+        assert_close(lp, ref_lp, 2e-5, 2e-6, what + " logp")
+        assert_close(ent, ref_ent, 2e-5, 2e-6, what + " entropy")
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_ratio_loss_random(dev, seed):
+    from unirl_amd.algorithms import fused_token_loss
+
+    rng = random.Random(3000 + seed)
+    for _ in range(6):
+        n_seq, max_len = rng.randint(1, 40), rng.choice((1, 3, 4, 8, 31, 64, 100, 257, 1024))
+        kind = rng.choice(("grpo", "drpo"))
+        mode = rng.choice(("token-mean", "seq-mean-token-sum-norm") + (("seq-mean-token-mean",) if kind == "grpo" else ()))
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        old = -8 * torch.rand(n_seq, max_len, generator=g)
+        new = old + rng.choice((0.01, 0.05, 0.5)) * torch.randn(n_seq, max_len, generator=g)
+        lengths = torch.randint(0 if mode != "seq-mean-token-mean" else 1, max_len + 1, (n_seq,), generator=g)
+        if int(lengths.sum()) == 0:
+            lengths[0] = max_len
+        adv = torch.randn(n_seq, generator=g)
+        what = f"{kind} {mode} [{n_seq},{max_len}]"
+        newp, oldp = olos.pack_padded(new, lengths), olos.pack_padded(old, lengths)
+        kw = dict(clip_range=0.2, clip_range_high=0.28, epsilon=5.0)
+        npk = newp.clone().requires_grad_(True)
+        ref_loss, _ = olos.token_loss(kind, npk, oldp, adv, lengths, mode=mode, horizon=max_len, **kw)
+        ref_loss.backward()
+        scale = float(olos.token_loss(kind, newp, oldp, adv, lengths, mode="token-mean", **kw)[0].abs()) + float(adv.abs().mean())
+        nd = new.to(dev).requires_grad_(True)
+        loss, _ = fused_token_loss(kind, nd, old.to(dev), adv.to(dev), lengths=lengths.to(dev), loss_agg_mode=mode,
+                                   horizon=max_len, clip_range=0.2, clip_range_high=0.28, drpo_epsilon=5.0)
+        loss.backward()
+        assert_close(loss, ref_loss, 2e-5, 4e-6 * scale, what + " padded")
+        gmax = float(npk.grad.abs().max())
+        assert_close(olos.pack_padded(nd.grad.cpu(), lengths), npk.grad, 2e-5, 2e-6 * gmax, what + " padded grad")
+        cu = torch.cat([torch.zeros(1, dtype=torch.int64), lengths.cumsum(0)])
+        nd2 = newp.to(dev).requires_grad_(True)
+        loss2, _ = fused_token_loss(kind, nd2, oldp.to(dev), adv.to(dev), cu_seqlens=cu.to(dev), loss_agg_mode=mode,
+                                    horizon=max_len, clip_range=0.2, clip_range_high=0.28, drpo_epsilon=5.0)
+        loss2.backward()
+        assert_close(loss2, ref_loss, 2e-5, 4e-6 * scale, what + " packed")
+        assert_close(nd2.grad, npk.grad, 2e-5, 2e-6 * gmax, what + " packed grad")
+
+
+@pytest.mark.parametrize("seed", range(3))
+def test_kl_mask_random(dev, seed):
+    from unirl_amd import ops
+
+    rng = random.Random(4000 + seed)
+    for _ in range(8):
+        B, S = rng.randint(1, 4), rng.randint(1, 5)
+        inner = rand_shape(rng, 3000)[1:]
+        dtype = rng.choice(DTYPES)
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        base = torch.randn((B, S) + inner, generator=g)
+        p = (base + 0.02 * torch.randn(base.shape, generator=g)).to(dtype)
+        q = (base + 0.02 * torch.randn(base.shape, generator=g)).to(dtype)
+        sig = (0.1 + torch.rand(S, generator=g)).view((1, S) + (1,) * len(inner)) if rng.random() < 0.7 else torch.tensor([0.4])  # 1-dim: a 0-dim sigma would keep torch's result in 16 bits
+        ref = ofd.kl_per_sample(p, q, sig)
+        thr = float(ref.median()) if ref.numel() > 1 else 0.01
+        kl, mask = ops.gaussian_kl_mask(p.to(dev), q.to(dev), sig.to(dev), thr)
+        rtol = FP32_RTOL if dtype == torch.float32 else BF16_RTOL
+        assert_close(kl, ref, rtol, 1e-9, f"kl {tuple(base.shape)} {dtype}")
+        near = (ref - thr).abs() <= 4 * torch.finfo(torch.float32).eps * abs(thr) + rtol * abs(thr) * (dtype != torch.float32)
+        assert torch.equal(mask.cpu()[~near], (ref < thr)[~near])

@@ -71,7 +71,9 @@ class _KlElemFn(torch.autograd.Function):
 
 def _gaussian_kl_div(p: torch.Tensor, q: torch.Tensor, sigma: torch.Tensor) -> torch.Tensor:
     """Per-element ``(p - q)^2 / (2 sigma^2)`` (fp32; 16-bit inputs subtract and square in
-    their own dtype first, as torch's type promotion does).  Differentiable w.r.t. ``p`` and ``q``."""
+    their own dtype first, as torch's type promotion does).  Differentiable w.r.t. ``p`` and ``q``.
+    The result is always fp32: with a 0-dim ``sigma`` eager torch would keep a 16-bit result
+    (0-dim tensors do not promote); the reference always passes ``[1, S', 1, 1, 1]``."""
     axis = _sigma_axis(p, sigma)
     sigma_dim = 1 if axis is None else axis
     if torch.is_grad_enabled() and (p.requires_grad or q.requires_grad):
