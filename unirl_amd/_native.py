@@ -270,6 +270,12 @@ def workspace(device: torch.device, stream: Optional[int] = None) -> Tuple[torch
     ws = _workspaces.get(key)
     if ws is None:
         nbytes = int(lib().unirl_workspace_bytes())
+        if torch.cuda.is_current_stream_capturing():
+            # First use of this stream happens inside a graph capture: the allocation belongs to
+            # the graph's private pool and dies with the graph, so it must not be cached.  (The
+            # workspace needs no initialisation, and the pool keeps it valid for every replay.)
+            ws = torch.empty(nbytes, dtype=torch.uint8, device=torch.device("cuda", index))
+            return ws, nbytes
         ws = torch.zeros(nbytes, dtype=torch.uint8, device=torch.device("cuda", index))
         _workspaces[key] = ws
     return ws, ws.numel()
