@@ -13,7 +13,7 @@ which are absent).  The formula functions are pinned by what the mathematics
 fixes (``tests/test_oracle_*``) and by an independent numpy float64 restatement
 (``tests/golden/vectors.npz``); the control-flow functions are pinned by outputs
 of the reference itself, produced by loading the two self-contained reference
-files and one extracted function (``tests/golden/reference_vectors.npz``):
+files and two extracted definitions (``tests/golden/reference_vectors.npz``):
 
   sigma_schedule            closed form, end points, shift=1, six known answers
   sde_step / sde_denoise    scipy.stats.norm.logpdf, torch.distributions.Normal,
@@ -25,15 +25,15 @@ files and one extracted function (``tests/golden/reference_vectors.npz``):
                             float64, brute force over a grid around the clip edges
   gaussian_kl / flowdppo    torch.distributions.kl_divergence, exact power-of-two
                             cases, the mask truth table
-  compute_advantages        numpy mean/var closed forms, degenerate groups
+  compute_advantages        reference-run vectors (all switches, root track,
+                            singleton groups), numpy mean/var closed forms
   normalize_grouped/global  reference-run vectors (trimmed statistics, empty and
                             singleton groups, clip, global std)
   gather_sde_field          reference-run vectors (values and error text),
                             dictionary lookup
 
-Parity unpinned: the wording of compute_advantages' two validation errors (the
-reference method cannot run without ray), and the entropy, which the reference
-does not compute anywhere (defined as lse - sum softmax*lf, 0*log 0 = 0).
+Parity unpinned: the entropy, which the reference does not compute anywhere
+(defined as lse - sum softmax*lf, 0*log 0 = 0).
 
 Reference line numbers are cited per function (paths relative to the reference
 tree).

@@ -1,4 +1,4 @@
-"""Writes tests/golden/reference_vectors.npz: outputs of the UniRL reference itself for the three
+"""Writes tests/golden/reference_vectors.npz: outputs of the UniRL reference itself for the four
 pieces of the path whose behaviour is control flow or a library recipe rather than a formula, so that closed
 forms and brute force do not pin them:
 
@@ -7,7 +7,9 @@ forms and brute force do not pin them:
   * gather_sde_field                        (unirl/algorithms/base.py:46-80) -- argsort +
     searchsorted + clamp + validation message;
   * the x_T noise recipe                    (unirl/sde/noise.py:26-187) -- blake2b seed derivation,
-    one seeded CPU generator per noise group, sharing inside a group, cast as the last step.
+    one seeded CPU generator per noise group, sharing inside a group, cast as the last step;
+  * RolloutTrack.compute_advantages         (unirl/types/rollout_resp.py:220-333) -- the scope /
+    normalize / use_global_std switches, root tracks, and the text of the validation errors.
 
 Only runs where the reference tree is mounted (/root/reference).  normalizers.py and noise.py
 import nothing but torch and the standard library at module level, so they are loaded from their
@@ -47,6 +49,34 @@ def load_function(path: Path, func: str):
     scope = {"torch": torch, "Optional": Optional, "List": List, "Dict": Dict}
     exec(compile(ast.Module(body=[node], type_ignores=[]), str(path), "exec"), scope)
     return scope[func]
+
+
+def load_compute_advantages():
+    """RolloutTrack.compute_advantages (unirl/types/rollout_resp.py:220-333) as a function of
+    (track, ...): the method's definition and the module helper _track_with_field are compiled
+    out of the syntax tree.  The module's other helper, _hydrate_tensor_meta, fetches tensors
+    from Ray workers; for a plain torch.Tensor it returns its argument unchanged, which is the
+    only behaviour this script needs, so an identity takes its place."""
+    import dataclasses
+    from typing import Any
+
+    path = REF / "types" / "rollout_resp.py"
+    tree = ast.parse(path.read_text())
+    cls = next(n for n in tree.body if isinstance(n, ast.ClassDef) and n.name == "RolloutTrack")
+    method = next(n for n in cls.body if isinstance(n, ast.FunctionDef) and n.name == "compute_advantages")
+    helper = next(n for n in tree.body if isinstance(n, ast.FunctionDef) and n.name == "_track_with_field")
+    scope = {"torch": torch, "Any": Any, "Dict": Dict, "List": List, "Optional": Optional, "TR": Any,
+             "dc_fields": dataclasses.fields, "_hydrate_tensor_meta": lambda value: value}
+    exec(compile(ast.Module(body=[helper, method], type_ignores=[]), str(path), "exec"), scope)
+
+    @dataclasses.dataclass
+    class Track:  # the four fields the method touches
+        sample_ids: list
+        parent_ids: Optional[list]
+        rewards: Optional[torch.Tensor] = None
+        advantages: Optional[torch.Tensor] = None
+
+    return scope["compute_advantages"], Track
 
 
 def main() -> None:
@@ -118,6 +148,34 @@ def main() -> None:
     out["nz_latents_same"] = noise.generate_latents(
         4, (2, 9), torch.device("cpu"), torch.float32, init_same_noise=True, samples_per_prompt=2,
         noise_group_ids=["g0", "g0", "g1", "g1"], base_seed=99).numpy()
+
+    # ---- RolloutTrack.compute_advantages ------------------------------------
+    compute_advantages, Track = load_compute_advantages()
+    rew = (torch.rand(24, generator=g) < 0.5).float() + 0.25 * torch.randn(24, generator=g)
+    rew[8:12] = 1.0  # an all-equal group
+    pids = [f"p{i // 4}" for i in range(24)]
+    out["ca_rewards"] = rew.numpy()
+    out["ca_parent_ids"] = np.frombuffer(json.dumps(pids).encode(), dtype=np.uint8)
+    ca_cases = []
+    for ci, kw in enumerate([{}, {"normalize": False}, {"use_global_std": True}, {"scope": "global"},
+                             {"scope": "global", "normalize": False}, {"eps": 1e-4}]):
+        t = compute_advantages(Track([str(i) for i in range(24)], pids, rew.clone()), **kw)
+        out[f"ca_case{ci}_out"] = t.advantages.numpy()
+        ca_cases.append(kw)
+    out["ca_cases"] = np.frombuffer(json.dumps(ca_cases).encode(), dtype=np.uint8)
+    out["ca_root_out"] = compute_advantages(Track([str(i) for i in range(24)], None, rew.clone())).advantages.numpy()
+    one = compute_advantages(Track(["a", "b", "c"], ["x", "y", "z"], torch.tensor([1.0, 2.0, 3.0])))
+    out["ca_singletons_out"] = one.advantages.numpy()
+    ca_errors = {}
+    for name, ids, r in (("interleaved", ["a", "b", "a", "b", "a", "b"], torch.arange(6.0)),
+                         ("nonuniform", ["a", "a", "a", "b", "b"], torch.arange(5.0)),
+                         ("no_rewards", ["a"], None)):
+        try:
+            compute_advantages(Track([str(i) for i in range(len(ids))], ids, r))
+            ca_errors[name] = None
+        except ValueError as e:
+            ca_errors[name] = str(e)
+    out["ca_errors"] = np.frombuffer(json.dumps(ca_errors).encode(), dtype=np.uint8)
 
     np.savez_compressed(OUT, **out)
     print(f"wrote {OUT} ({OUT.stat().st_size} bytes, {len(out)} arrays)")

@@ -156,3 +156,46 @@ def test_noise_recipe_on_device_is_byte_identical(dev):
     assert torch.equal(y, y2)
     assert noise.generate_shared_noise(2, (4,), dev, torch.bfloat16, ["a", "a"]).dtype == torch.bfloat16
     assert noise.regen_initial_noise([], 1, (4, 4), dev).shape == (0, 4, 4)
+
+
+# ---------------------------------------------------------------- RolloutTrack.compute_advantages
+CA_CASES = meta("ca_cases")
+CA_PIDS = meta("ca_parent_ids")
+CA_ERRORS = meta("ca_errors")
+
+
+@pytest.mark.parametrize("ci", range(len(CA_CASES)))
+def test_oracle_compute_advantages(ci):
+    got = oadv.compute_advantages(torch.from_numpy(R["ca_rewards"]), CA_PIDS, **CA_CASES[ci])
+    check(got, f"ca_case{ci}_out", rtol=1e-6, atol=1e-7)
+
+
+def test_compute_advantages_host_rules_and_error_text():
+    from unirl_amd.types import RolloutTrack, compute_advantages
+
+    r = torch.from_numpy(R["ca_rewards"])
+    check(compute_advantages(r, None), "ca_root_out", rtol=0, atol=0)  # root track: zeros, no kernel
+    check(oadv.compute_advantages(r, None), "ca_root_out", rtol=0, atol=0)
+    cases = {"interleaved": (["a", "b", "a", "b", "a", "b"], torch.arange(6.0)),
+             "nonuniform": (["a", "a", "a", "b", "b"], torch.arange(5.0))}
+    for name, (ids, rew) in cases.items():
+        with pytest.raises(ValueError) as e:
+            compute_advantages(rew, ids)
+        assert str(e.value) == CA_ERRORS[name]
+    with pytest.raises(ValueError) as e:
+        RolloutTrack(sample_ids=["a"], parent_ids=["a"]).compute_advantages()
+    assert str(e.value) == CA_ERRORS["no_rewards"]
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("ci", range(len(CA_CASES)))
+def test_kernel_compute_advantages(dev, ci):
+    from unirl_amd.types import RolloutTrack, compute_advantages
+
+    r = torch.from_numpy(R["ca_rewards"]).to(dev)
+    check(compute_advantages(r, CA_PIDS, **CA_CASES[ci]), f"ca_case{ci}_out")
+    track = RolloutTrack(sample_ids=[str(i) for i in range(24)], parent_ids=CA_PIDS, rewards=r)
+    check(track.compute_advantages(**CA_CASES[ci]).advantages, f"ca_case{ci}_out")
+    if ci == 0:
+        one = compute_advantages(torch.tensor([1.0, 2.0, 3.0], device=dev), ["x", "y", "z"])
+        check(one, "ca_singletons_out", rtol=0, atol=0)
