@@ -258,6 +258,15 @@ __device__ __forceinline__ double dpp_f64_or_zero(double v) {
   return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
 }
 
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_f64_or_self(double v) {
+  const long long b = __double_as_longlong(v);
+  const int l = (int)(unsigned int)b, h = (int)(unsigned int)((unsigned long long)b >> 32);
+  const unsigned int lo = (unsigned int)__builtin_amdgcn_update_dpp(l, l, CTRL, ROW_MASK, 0xf, false);
+  const unsigned int hi = (unsigned int)__builtin_amdgcn_update_dpp(h, h, CTRL, ROW_MASK, 0xf, false);
+  return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
 __device__ __forceinline__ float op_add(float a, float b) { return a + b; }
 __device__ __forceinline__ double op_add(double a, double b) { return a + b; }
 __device__ __forceinline__ unsigned int op_add(unsigned int a, unsigned int b) { return a + b; }
@@ -275,6 +284,23 @@ __device__ __forceinline__ double last_lane(double v) {
   const unsigned int lo = (unsigned int)__builtin_amdgcn_readlane((int)(unsigned int)b, kWave - 1);
   const unsigned int hi = (unsigned int)__builtin_amdgcn_readlane((int)(unsigned int)((unsigned long long)b >> 32), kWave - 1);
   return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
+// Reductions over each 16-lane row of a wavefront (four row shifts); the result is in the
+// row's last lane only.
+__device__ __forceinline__ double row_sum_last(double v) {
+  v += dpp_f64_or_zero<0x111, 0xf>(v);
+  v += dpp_f64_or_zero<0x112, 0xf>(v);
+  v += dpp_f64_or_zero<0x114, 0xf>(v);
+  v += dpp_f64_or_zero<0x118, 0xf>(v);
+  return v;
+}
+__device__ __forceinline__ double row_max_last(double v) {
+  v = fmax(v, dpp_f64_or_self<0x111, 0xf>(v));
+  v = fmax(v, dpp_f64_or_self<0x112, 0xf>(v));
+  v = fmax(v, dpp_f64_or_self<0x114, 0xf>(v));
+  v = fmax(v, dpp_f64_or_self<0x118, 0xf>(v));
+  return v;
 }
 
 // Wave-uniform results.

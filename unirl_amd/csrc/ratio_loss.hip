@@ -27,10 +27,16 @@ constexpr int kRlVals = 16;  // partial values per workgroup
 
 enum { LAYOUT_FLAT = 0, LAYOUT_PADDED = 1, LAYOUT_PACKED = 2 };
 
-// slots of the per-workgroup partial vector
+// Slots of the per-workgroup partial vector.  Slots below kFirstMax are sums, the rest maxima
+// (the ratio minimum travels negated); the reductions handle four consecutive slots per
+// wavefront, so this order keeps the two kinds in different wavefronts.  10, 11, 15 are unused.
 enum {
-  P_SR = 0, P_SR2, P_LOSS, P_KL, P_PEN, P_ABS, P_CNT, P_CHI, P_CLO, P_CANY, P_RMIN, P_RMAX, P_AMAX
+  P_SR = 0, P_SR2, P_LOSS, P_KL, P_PEN, P_ABS, P_CNT, P_CHI, P_CLO, P_CANY,
+  P_NRMIN = 12, P_RMAX = 13, P_AMAX = 14
 };
+constexpr int kFirstMax = 12;
+constexpr int kRlParts = 16;  // threads that share one slot in the reductions below
+static_assert(kRlParts * 16 == 256, "reductions assume 256 threads = 16 slots x 16 parts");
 
 struct RatioConsts {
   int kind;
@@ -65,20 +71,25 @@ struct RatioArgs {
   float* grad_new;
 };
 
-// exp(x) for fp32 within ~1.5 ulp in eight instructions: 2^(x*log2(e)) on the hardware exp2,
-// with the rounding error of the product (carried in a second float) applied as a first-order
-// correction.  +inf above ln(FLT_MAX), 0 below the denormal range, NaN for NaN.
-__device__ __forceinline__ float exp_f32(float x) {
+// exp(x) for fp32 within ~1.5 ulp: 2^(x*log2(e)) on the hardware exp2, with the rounding error
+// of the product (carried in a second float) applied as a first-order correction.
+// exp_f32_core is valid for |x| < 88.7 and NaN (callers that clamp x use it directly);
+// exp_f32 falls back to the bare 2^t outside that range, which is exactly +inf above
+// ln(FLT_MAX), 0 for -inf, and a denormal within 1e-5 relative in between.
+__device__ __forceinline__ float exp_f32_core(float x, float& e_out) {
   constexpr float kL2eHi = 1.44269502162933349609375f;  // log2(e) rounded to fp32
   constexpr float kL2eLo = 1.925963033500011e-8f;       // log2(e) - kL2eHi
   const float t = x * kL2eHi;
   float lo = fmaf(x, kL2eHi, -t);
   lo = fmaf(x, kL2eLo, lo);
   const float e = __builtin_amdgcn_exp2f(t);
-  float r = fmaf(e, lo * 0.693147182f, e);
-  r = (x > 88.72283172607422f) ? INFINITY : r;  // e is +inf from here on and inf*lo + inf could be NaN
-  r = (x < -104.0f) ? 0.0f : r;                 // t and lo overflow for x = -inf
-  return r;
+  e_out = e;
+  return fmaf(e, lo * 0.693147182f, e);
+}
+__device__ __forceinline__ float exp_f32(float x) {
+  float e;
+  const float r = exp_f32_core(x, e);
+  return (fabsf(x) < 88.72283172607422f) ? r : e;  // inf * lo and inf - inf would give NaN out there
 }
 
 // x / c for a loop-invariant c with inv_c = 1/c: quotient estimate, exact remainder, one
@@ -144,28 +155,26 @@ __device__ __forceinline__ TokVals ratio_token(float nw, float od, float A, cons
   return o;
 }
 
-// min for the ratio minimum, max for the two maxima, sum for everything else
-__device__ __forceinline__ double combine(int v, double x, double y) {
-  return (v == P_RMIN) ? fmin(x, y) : ((v == P_RMAX || v == P_AMAX) ? fmax(x, y) : x + y);
-}
-
 // Per-lane accumulators.  The six sums are fp32 and are flushed into fp64 totals after every
-// pass (at most ITEMS*VEC tokens), so their rounding does not grow with the input.  The extrema
-// are kept as bit patterns: ratios and |new-old| are >= 0 (or NaN), where unsigned integer order
-// is float order, so each update is one integer min / max.
+// pass (at most ITEMS*VEC tokens), so their rounding does not grow with the input.  The ratio
+// extrema are kept as bit patterns: ratios are >= 0 (or NaN), where unsigned integer order is
+// float order, so each update is one integer min / max.
 struct Acc {
   float s1 = 0.0f, s2 = 0.0f;  // sums of (r-1) and (r-1)^2
   float loss = 0.0f;
   float kl = 0.0f;             // GRPO: sum of ld^2 (halved at the end); DRPO: sum of (r-1) - ld
   float pen = 0.0f, ab = 0.0f;
   double t_s1 = 0.0, t_s2 = 0.0, t_loss = 0.0, t_kl = 0.0, t_pen = 0.0, t_ab = 0.0;
-  unsigned int rmin = 0x7f800000u, rmax = 0u, amax = 0u;
-  unsigned int cnt = 0, chi = 0, clo = 0, cany = 0;
+  unsigned int rmin = 0x7f800000u, rmax = 0u;
+  float amax = 0.0f;
+  unsigned int cnt = 0;
+  unsigned int chi = 0, clo = 0, cany = 0;  // clip counts of the guarded path (see WaveCounts)
 
-  __device__ __forceinline__ void flush() {
+  // `w`: aggregation weight shared by every token of the pass (1 when the tokens carry their own)
+  __device__ __forceinline__ void flush(double w) {
     t_s1 += (double)s1;
     t_s2 += (double)s2;
-    t_loss += (double)loss;
+    t_loss = fma((double)loss, w, t_loss);  // the product is exact in fp64
     t_kl += (double)kl;
     t_pen += (double)pen;
     t_ab += (double)ab;
@@ -173,22 +182,38 @@ struct Acc {
   }
 };
 
-// One token into the accumulators; returns its loss.  `lw` = loss_mask * aggregation weight.
+// Clip counters of one wavefront.  A comparison result is a lane mask, so counting it is one
+// scalar population count: the counters cost the vector unit nothing beyond the compare.  Only
+// for code the whole wavefront runs together (a pass over 64 whole vectors); lanes that sit
+// behind a lane-dependent branch count in Acc instead.
+struct WaveCounts {
+  unsigned int hi = 0, lo = 0, any = 0;
+  __device__ __forceinline__ void add(bool h, bool l) {
+    const unsigned long long mh = __builtin_amdgcn_ballot_w64(h), ml = __builtin_amdgcn_ballot_w64(l);
+    hi += (unsigned int)__builtin_popcountll(mh);
+    lo += (unsigned int)__builtin_popcountll(ml);
+    any += (unsigned int)__builtin_popcountll(mh | ml);
+  }
+};
+
+// One token into the accumulators; returns its loss and its two clip flags.  `lw` multiplies the
+// loss inside the sum (loss mask, and the aggregation weight where it changes inside a pass).
 // The arithmetic is the reference's, op for op; two rewrites are exact:
 //   maximum(u, c) = (c > u) ? c : u   -- u is NaN whenever c is (c = -A*clamp(r), u = -A*r), so
 //                                        NaN reaches the result as in torch.maximum;
 //   1 - r = -(r - 1)                  -- rounding is symmetric, so the lower clip test reuses r-1.
 template <int KIND>
 __device__ __forceinline__ float accumulate_token(float nw, float od, float A, float lw, const RatioConsts& C,
-                                                  Acc& acc) {
+                                                  Acc& acc, bool& hi, bool& lo) {
   const float d0 = nw - od;
   float r, loss;
-  bool hi, lo;
   if (KIND == UNIRL_LOSS_GRPO) {
     r = exp_f32(d0);
     const float nA = -A;
     const float u = nA * r;
-    const float c = nA * fminf(fmaxf(r, C.clamp_lo), C.clamp_hi);
+    // clamp as a median of three (fill_consts keeps clamp_lo <= clamp_hi); like fmin(fmax()) it
+    // drops a NaN ratio, which the select below then restores from u
+    const float c = nA * __builtin_amdgcn_fmed3f(r, C.clamp_lo, C.clamp_hi);
     loss = (c > u) ? c : u;
     const float d = r - 1.0f;
     hi = d > C.eps_hi;
@@ -198,7 +223,8 @@ __device__ __forceinline__ float accumulate_token(float nw, float od, float A, f
     acc.kl = fmaf(d0, d0, acc.kl);
   } else {
     const float ld = (d0 != d0) ? d0 : fminf(fmaxf(d0, -20.0f), 20.0f);  // torch.clamp keeps NaN
-    r = exp_f32(ld);
+    float e;
+    r = exp_f32_core(ld, e);  // |ld| <= 20
     const float mu = exp_f32(od);
     const float d = r - 1.0f;
     const float w = C.mu_weighted ? mu : 1.0f;
@@ -216,13 +242,10 @@ __device__ __forceinline__ float accumulate_token(float nw, float od, float A, f
   acc.loss += loss * lw;
   const float a0 = fabsf(d0);
   acc.ab += a0;
-  const unsigned int rb = __float_as_uint(r), ab = __float_as_uint(a0);
+  acc.amax = fmaxf(acc.amax, a0);  // a NaN drops out here; the finalize kernel restores it from the sum
+  const unsigned int rb = __float_as_uint(r);
   acc.rmin = rb < acc.rmin ? rb : acc.rmin;
   acc.rmax = rb > acc.rmax ? rb : acc.rmax;
-  acc.amax = ab > acc.amax ? ab : acc.amax;
-  acc.chi += hi ? 1u : 0u;
-  acc.clo += lo ? 1u : 0u;
-  acc.cany += (hi || lo) ? 1u : 0u;
   return loss;
 }
 
@@ -250,19 +273,25 @@ struct SeqCtx {
 };
 
 // One loaded vector of VEC tokens starting at row-relative index t0; tokens at or past `count`
-// are padding.  mk[] holds 1 when there is no loss mask.  Accumulates into acc and leaves the
-// per-token loss in out[].  Whole vectors outside the packed layout take a path without
-// per-token bounds or sequence checks.
+// are padding.  mk[] holds 1 when there is no loss mask.  Accumulates into acc, leaves the
+// per-token loss in out[] and the clip flags in hi[] / lo[] (false for padding).  Whole vectors
+// outside the packed layout take a path without per-token bounds or sequence checks.  Outside
+// the packed layout the aggregation weight is the same for the whole pass and is applied by
+// Acc::flush; in the packed layout it rides on every token.
 template <int KIND, int VEC, bool PACKED>
 __device__ __forceinline__ void ratio_vec_fwd(const RatioArgs& A, const RatioConsts& C, int64_t t0, int64_t count,
                                               const float (&nw)[VEC], const float (&od)[VEC],
-                                              const float (&ad)[VEC], const float (&mk)[VEC], SeqCtx& sq,
-                                              Acc& acc, float (&out)[VEC]) {
+                                              const float (&ad)[VEC], const float (&mk)[VEC], bool adv_tok,
+                                              SeqCtx& sq, Acc& acc, float (&out)[VEC]) {
   if (!PACKED && t0 + VEC <= count) {
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
-      const float a = C.adv_per_token ? ad[k] : sq.adv;
-      out[k] = accumulate_token<KIND>(nw[k], od[k], a, mk[k] * sq.w, C, acc);
+      const float a = adv_tok ? ad[k] : sq.adv;
+      bool hi, lo;
+      out[k] = accumulate_token<KIND>(nw[k], od[k], a, mk[k], C, acc, hi, lo);
+      acc.chi += hi ? 1u : 0u;
+      acc.clo += lo ? 1u : 0u;
+      acc.cany += (hi || lo) ? 1u : 0u;
     }
     acc.cnt += VEC;
     return;
@@ -276,51 +305,80 @@ __device__ __forceinline__ void ratio_vec_fwd(const RatioArgs& A, const RatioCon
         const int64_t s = find_seq(A.seq, A.n_seq, t);
         sq.cur_end = A.seq[s + 1];
         sq.w = seq_weight(C, sq.cur_end - A.seq[s]);
-        if (!C.adv_per_token) sq.adv = A.adv[s];
+        if (!adv_tok) sq.adv = A.adv[s];
       }
-      const float a = C.adv_per_token ? ad[k] : sq.adv;
-      out[k] = accumulate_token<KIND>(nw[k], od[k], a, mk[k] * sq.w, C, acc);
+      const float a = adv_tok ? ad[k] : sq.adv;
+      bool hi, lo;
+      out[k] = accumulate_token<KIND>(nw[k], od[k], a, PACKED ? mk[k] * sq.w : mk[k], C, acc, hi, lo);
+      acc.chi += hi ? 1u : 0u;
+      acc.clo += lo ? 1u : 0u;
+      acc.cany += (hi || lo) ? 1u : 0u;
       acc.cnt += 1u;
     }
   }
 }
 
-// Workgroup partial vector -> A.partials[workgroup].  Every thread must call.
-__device__ __forceinline__ void store_block_partials(const RatioArgs& A, Acc& acc, double (*lds_v)[kRlVals]) {
-  constexpr int NW = kRlThreads / kWave;
-  acc.flush();
-  double vals[kRlVals];
-  vals[P_SR] = wave_sum(acc.t_s1);
-  vals[P_SR2] = wave_sum(acc.t_s2);
-  // a lane's total of these four is a handful of fp32 terms: rounding it to fp32 loses nothing the
-  // 1e-5 budget can see, and an fp32 DPP tree costs half the moves of an fp64 one
-  vals[P_LOSS] = (double)wave_sum((float)acc.t_loss);
-  vals[P_KL] = (double)wave_sum((float)acc.t_kl);
-  vals[P_PEN] = (double)wave_sum((float)acc.t_pen);
-  vals[P_ABS] = (double)wave_sum((float)acc.t_ab);
-  vals[P_CNT] = (double)wave_sum(acc.cnt);
-  vals[P_CHI] = (double)wave_sum(acc.chi);
-  vals[P_CLO] = (double)wave_sum(acc.clo);
-  vals[P_CANY] = (double)wave_sum(acc.cany);
-  // NaN patterns drop out of the float min / max here; the finalize kernel restores NaN from the sums
-  vals[P_RMIN] = (double)wave_min(__uint_as_float(acc.rmin));
-  vals[P_RMAX] = (double)wave_max(acc.cnt ? __uint_as_float(acc.rmax) : -INFINITY);
-  vals[P_AMAX] = (double)wave_max(acc.cnt ? __uint_as_float(acc.amax) : -INFINITY);
-  vals[13] = vals[14] = vals[15] = 0.0;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wid = threadIdx.x / kWave;
-  if (lane == 0) {
+// The same for a vector that is whole and valid in all 64 lanes (outside the packed layout): no
+// bounds checks, and the clip flags are counted per wavefront.
+template <int KIND, int VEC>
+__device__ __forceinline__ void ratio_vec_wave(const RatioConsts& C, const float (&nw)[VEC],
+                                               const float (&od)[VEC], const float (&ad)[VEC],
+                                               const float (&mk)[VEC], bool adv_tok, const SeqCtx& sq, Acc& acc,
+                                               WaveCounts& wc, float (&out)[VEC]) {
 #pragma unroll
-    for (int v = 0; v < kRlVals; ++v) lds_v[wid][v] = vals[v];
+  for (int k = 0; k < VEC; ++k) {
+    const float a = adv_tok ? ad[k] : sq.adv;
+    bool hi, lo;
+    out[k] = accumulate_token<KIND>(nw[k], od[k], a, mk[k], C, acc, hi, lo);
+    wc.add(hi, lo);
   }
+  acc.cnt += VEC;
+}
+
+__device__ __forceinline__ bool slot_used(int v) { return v <= P_CANY || (v >= P_NRMIN && v <= P_AMAX); }
+
+// Workgroup partial vector -> A.partials[workgroup].  Every thread must call.
+// Through LDS rather than thirteen wavefront reductions: every thread stores its values as
+// [slot][thread] (consecutive lanes, consecutive words), then thread (slot, part) = (tid / 16,
+// tid % 16) combines the sixteen entries part, part + 16, ... of its slot and four row shifts
+// finish each 16-lane row.  Fixed order, one barrier.
+__device__ __forceinline__ void store_block_partials(const RatioArgs& A, Acc& acc, const WaveCounts& wc,
+                                                     double (*lds_v)[kRlThreads]) {
+  const int t = threadIdx.x;
+  const bool lead = (t & (kWave - 1)) == 0;  // carries the wavefront's own counters
+  lds_v[P_SR][t] = acc.t_s1;
+  lds_v[P_SR2][t] = acc.t_s2;
+  lds_v[P_LOSS][t] = acc.t_loss;
+  lds_v[P_KL][t] = acc.t_kl;
+  lds_v[P_PEN][t] = acc.t_pen;
+  lds_v[P_ABS][t] = acc.t_ab;
+  lds_v[P_CNT][t] = (double)acc.cnt;
+  lds_v[P_CHI][t] = (double)(acc.chi + (lead ? wc.hi : 0u));
+  lds_v[P_CLO][t] = (double)(acc.clo + (lead ? wc.lo : 0u));
+  lds_v[P_CANY][t] = (double)(acc.cany + (lead ? wc.any : 0u));
+  // NaN ratios drop out of the maxima below; the finalize kernel restores NaN from the sums
+  lds_v[P_NRMIN][t] = -(double)__uint_as_float(acc.rmin);
+  lds_v[P_RMAX][t] = acc.cnt ? (double)__uint_as_float(acc.rmax) : -(double)INFINITY;
+  lds_v[P_AMAX][t] = acc.cnt ? (double)acc.amax : -(double)INFINITY;
   __syncthreads();
-  const unsigned int blk = blockIdx.y * gridDim.x + blockIdx.x;
-  if (threadIdx.x < kRlVals) {
-    const int v = threadIdx.x;
-    double x = lds_v[0][v];
-    for (int w = 1; w < NW; ++w) x = combine(v, x, lds_v[w][v]);
-    A.partials[(int64_t)blk * kRlVals + v] = x;  // reduced by ratio_loss_finalize_kernel
+  const int v = t / kRlParts, part = t % kRlParts;
+  double x = 0.0;
+  if (slot_used(v)) {
+    double y[kRlThreads / kRlParts];
+#pragma unroll
+    for (int j = 0; j < kRlThreads / kRlParts; ++j) y[j] = lds_v[v][j * kRlParts + part];
+    x = y[0];
+    if (v < kFirstMax) {
+#pragma unroll
+      for (int j = 1; j < kRlThreads / kRlParts; ++j) x += y[j];
+    } else {
+#pragma unroll
+      for (int j = 1; j < kRlThreads / kRlParts; ++j) x = fmax(x, y[j]);
+    }
   }
+  x = (v < kFirstMax) ? row_sum_last(x) : row_max_last(x);
+  const unsigned int blk = blockIdx.y * gridDim.x + blockIdx.x;
+  if (part == kRlParts - 1) A.partials[(int64_t)blk * kRlVals + v] = x;  // reduced by ratio_loss_finalize_kernel
 }
 
 template <int VEC>
@@ -329,19 +387,33 @@ __device__ __forceinline__ void fill_ones(float (&m)[VEC]) {
   for (int k = 0; k < VEC; ++k) m[k] = 1.0f;
 }
 
-template <int KIND, int VEC, bool PACKED>
+#ifndef UNIRL_RATIO_ITEMS
+#define UNIRL_RATIO_ITEMS 2
+#endif
+
+// FLAGS >= 0 fixes at compile time whether a loss mask (bit 0) and per-token advantages (bit 1)
+// are read, which keeps the loads of a pass straight-line code (all of them in flight before the
+// first use); FLAGS < 0 reads both switches at run time.
+template <int KIND, int VEC, bool PACKED, int FLAGS>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A) {
-  constexpr int NW = kRlThreads / kWave;
-  constexpr int ITEMS = 2;  // vectors in flight per lane
-  __shared__ double lds_v[NW][kRlVals];
+  constexpr int ITEMS = UNIRL_RATIO_ITEMS;  // vectors in flight per lane
+  __shared__ double lds_v[kRlVals][kRlThreads];
   const RatioConsts C = A.C;
+  const bool has_mask = (FLAGS < 0) ? (A.mask != nullptr) : ((FLAGS & 1) != 0);
+  const bool adv_tok = (FLAGS < 0) ? (C.adv_per_token != 0) : ((FLAGS & 2) != 0);
 
   Acc acc;
+  WaveCounts wc;
   SeqCtx sq;
   const bool padded = (A.layout == LAYOUT_PADDED);
   const int64_t n_rows = padded ? A.n_seq : 1;
   const int64_t stride = (int64_t)gridDim.x * kRlThreads;
-  const int64_t first = (int64_t)blockIdx.x * kRlThreads + threadIdx.x;
+  // The pass loop runs on a wave-uniform index (every lane makes the same trips; lanes past the
+  // end idle inside a pass), which keeps the wave together where the clip flags are counted.
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave_first =
+      (int64_t)blockIdx.x * kRlThreads + (__builtin_amdgcn_readfirstlane((int)threadIdx.x) & ~(kWave - 1));
+  const int64_t first = wave_first + lane;
 
   for (int64_t r = blockIdx.y; r < n_rows; r += gridDim.y) {
     // tokens [base, base+count) are valid; whole vectors may be loaded up to base+row_end
@@ -352,38 +424,47 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
       base = r * A.seq_stride;
       count = len;
       row_end = A.seq_stride;
-      if (!C.adv_per_token) sq.adv = A.adv[r];
+      if (!adv_tok) sq.adv = A.adv[r];
       sq.w = (len > 0) ? seq_weight(C, len) : 1.0f;
     }
+    const double pass_w = PACKED ? 1.0 : (double)sq.w;
     const int64_t nvec = (count + VEC - 1) / VEC;  // vectors holding a valid token
     const int64_t nvec_full = row_end / VEC;       // vectors that can be loaded whole
     const int64_t nload = nvec < nvec_full ? nvec : nvec_full;
 
-    for (int64_t i0 = first; i0 < nload; i0 += stride * ITEMS) {
+    for (int64_t w0 = wave_first; w0 < nload; w0 += stride * ITEMS) {
       float nw[ITEMS][VEC], od[ITEMS][VEC], ad[ITEMS][VEC], mk[ITEMS][VEC];
+      // Every item loads: past the end the index falls back to the row's last loadable vector
+      // (in flight for another lane anyway) and the values go unused, so no load waits behind a
+      // branch and all of a pass are in flight together.
 #pragma unroll
       for (int it = 0; it < ITEMS; ++it) {
-        const int64_t i = i0 + it * stride;
-        fill_ones(mk[it]);
-        if (i < nload) {
-          Vec<float, VEC>::load(A.nw + base + i * VEC, nw[it]);
-          Vec<float, VEC>::load(A.od + base + i * VEC, od[it]);
-          if (C.adv_per_token) Vec<float, VEC>::load(A.adv + base + i * VEC, ad[it]);
-          if (A.mask) Vec<float, VEC>::load(A.mask + base + i * VEC, mk[it]);
-        }
+        const int64_t i = w0 + lane + it * stride;
+        const int64_t ic = (i < nload) ? i : nload - 1;
+        Vec<float, VEC>::load(A.nw + base + ic * VEC, nw[it]);
+        Vec<float, VEC>::load(A.od + base + ic * VEC, od[it]);
+        if (adv_tok) Vec<float, VEC>::load(A.adv + base + ic * VEC, ad[it]);
+        if (has_mask) Vec<float, VEC>::load(A.mask + base + ic * VEC, mk[it]);
+        else fill_ones(mk[it]);
       }
 #pragma unroll
       for (int it = 0; it < ITEMS; ++it) {
-        const int64_t i = i0 + it * stride;
-        if (i < nload) {
-          float out[VEC];
-          ratio_vec_fwd<KIND, VEC, PACKED>(A, C, i * VEC, count, nw[it], od[it], ad[it], mk[it], sq, acc, out);
+        const int64_t wv = w0 + it * stride;  // the wavefront's first vector of this item
+        const int64_t i = wv + lane;
+        float out[VEC];
+        if (!PACKED && (wv + kWave) * VEC <= count) {
+          ratio_vec_wave<KIND, VEC>(C, nw[it], od[it], ad[it], mk[it], adv_tok, sq, acc, wc, out);
+          if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + base + i * VEC, out);
+        } else if (i < nload) {
+          ratio_vec_fwd<KIND, VEC, PACKED>(A, C, i * VEC, count, nw[it], od[it], ad[it], mk[it], adv_tok, sq, acc,
+                                           out);
           if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + base + i * VEC, out);
         }
       }
-      acc.flush();
+      acc.flush(pass_w);
     }
-    // a row whose length is not a multiple of VEC ends in one vector that cannot be loaded whole
+    // a row whose length is not a multiple of VEC ends in one vector that cannot be loaded whole;
+    // one lane of the grid takes it token by token
     if (nvec > nvec_full && first == nvec_full % stride) {
       const int64_t t0 = nvec_full * VEC;
       float nw[VEC], od[VEC], ad[VEC], mk[VEC], out[VEC];
@@ -392,37 +473,40 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
         const bool ok = (t0 + k) < count;
         nw[k] = ok ? A.nw[base + t0 + k] : 0.0f;
         od[k] = ok ? A.od[base + t0 + k] : 0.0f;
-        ad[k] = (ok && C.adv_per_token) ? A.adv[base + t0 + k] : 0.0f;
-        mk[k] = (ok && A.mask) ? A.mask[base + t0 + k] : 1.0f;
+        ad[k] = (ok && adv_tok) ? A.adv[base + t0 + k] : 0.0f;
+        mk[k] = (ok && has_mask) ? A.mask[base + t0 + k] : 1.0f;
       }
-      ratio_vec_fwd<KIND, VEC, PACKED>(A, C, t0, count, nw, od, ad, mk, sq, acc, out);
+      ratio_vec_fwd<KIND, VEC, PACKED>(A, C, t0, count, nw, od, ad, mk, adv_tok, sq, acc, out);
       if (A.loss_elem) {
 #pragma unroll
         for (int k = 0; k < VEC; ++k)
           if (t0 + k < row_end) A.loss_elem[base + t0 + k] = out[k];
       }
-      acc.flush();
+      acc.flush(pass_w);
     }
     // padded layout: zero the loss of the slots past the sequence end
     if (A.loss_elem && padded) {
       for (int64_t t = nvec * VEC + first; t < row_end; t += stride) A.loss_elem[base + t] = 0.0f;
     }
   }
-  store_block_partials(A, acc, lds_v);
+  store_block_partials(A, acc, wc, lds_v);
 }
 
 // One workgroup: fixed-order reduction of every workgroup's partial vector, then the metrics.
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioArgs A, unsigned int nblk) {
-  __shared__ double lds_fin[kRlThreads];
+  __shared__ double lds_t[kRlThreads];
+  __shared__ double lds_tot[kRlVals];
   const RatioConsts C = A.C;
+  const int t = threadIdx.x;
   {
-    // thread = (value v, slice j0): 16 slices walk the workgroups' vectors, kBatch loads in flight each
-    const int v = threadIdx.x % kRlVals;
-    const int j0 = threadIdx.x / kRlVals;  // 0..15
+    // thread = (slot v, slice j0): 16 slices walk the workgroups' vectors (a wavefront reads four
+    // whole vectors per load), kBatch loads in flight each
+    const int v = t % kRlVals;
+    const int j0 = t / kRlVals;  // 0..15
     constexpr int kSlices = kRlThreads / kRlVals;
     constexpr int kBatch = 32;  // 512 workgroups: every partial of a thread in flight at once
-    double x = (v == P_RMIN) ? (double)INFINITY : ((v == P_RMAX || v == P_AMAX) ? -(double)INFINITY : 0.0);
-    const double ident = x;
+    const double ident = (v < kFirstMax) ? 0.0 : -(double)INFINITY;
+    double x = ident;
     for (unsigned int j = j0; j < nblk; j += kSlices * kBatch) {
       double y[kBatch];
 #pragma unroll
@@ -430,73 +514,71 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
         const unsigned int jj = j + b * kSlices;
         y[b] = (jj < nblk) ? A.partials[(int64_t)jj * kRlVals + v] : ident;
       }
-      // one kind of operation per lane, chosen once per batch (three short divergent runs) rather
-      // than a three-way select per element
-      if (v < P_RMIN) {
+      // one kind of operation per lane, chosen once per batch rather than per element
+      if (v < kFirstMax) {
 #pragma unroll
         for (int b = 0; b < kBatch; ++b) x += y[b];
-      } else if (v == P_RMIN) {
-#pragma unroll
-        for (int b = 0; b < kBatch; ++b) x = fmin(x, y[b]);
       } else {
 #pragma unroll
         for (int b = 0; b < kBatch; ++b) x = fmax(x, y[b]);
       }
     }
-    lds_fin[threadIdx.x] = x;
+    lds_t[v * kSlices + j0] = x;  // transposed: the sixteen slices of a slot side by side
   }
   __syncthreads();
-  if (threadIdx.x < kRlVals) {
-    const int v = threadIdx.x;
-    double x = lds_fin[v];
-    if (v < P_RMIN) {
-      for (int j = 1; j < kRlThreads / kRlVals; ++j) x += lds_fin[j * kRlVals + v];
-    } else if (v == P_RMIN) {
-      for (int j = 1; j < kRlThreads / kRlVals; ++j) x = fmin(x, lds_fin[j * kRlVals + v]);
-    } else {
-      for (int j = 1; j < kRlThreads / kRlVals; ++j) x = fmax(x, lds_fin[j * kRlVals + v]);
-    }
-    lds_fin[v] = x;
+  {
+    // thread = (slot, slice) again, now with a slot's slices in one 16-lane row
+    const int v = t / kRlParts;
+    double z = lds_t[t];
+    z = (v < kFirstMax) ? row_sum_last(z) : row_max_last(z);
+    if (t % kRlParts == kRlParts - 1) lds_tot[v] = z;
   }
   __syncthreads();
-  if (threadIdx.x != 0) return;
-  const double N = lds_fin[P_CNT];
-  const double sr = lds_fin[P_SR], sr2 = lds_fin[P_SR2];
-  // One fp64 reciprocal serves every mean (this thread runs alone; an fp64 divide per metric was a
-  // third of the kernel).  x * (1/N) and x / N differ by at most an ulp of fp64, far below the
-  // fp32 result's rounding.
+  if (t >= kRlVals) return;
+  // Lane v turns slot v into its metric; the lanes run the same straight-line code.
+  const int v = t;
+  const double N = lds_tot[P_CNT], sr = lds_tot[P_SR], sr2 = lds_tot[P_SR2], sab = lds_tot[P_ABS];
+  const double x = lds_tot[v];
+  // One fp64 reciprocal serves every mean: x * (1/N) and x / N differ by at most an ulp of fp64,
+  // far below the fp32 result's rounding.
   const double inv_n = 1.0 / N;
-  double loss = lds_fin[P_LOSS];
-  if (C.agg_mode == UNIRL_AGG_TOKEN_MEAN)
-    loss = loss * inv_n;
-  else if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_SUM)
-    loss = loss / ((double)A.n_seq * (double)C.horizon);
-  else
-    loss = loss / (double)A.n_seq;
+  double loss_scale = inv_n;
+  if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_SUM)
+    loss_scale = 1.0 / ((double)A.n_seq * (double)C.horizon);
+  else if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_MEAN)
+    loss_scale = 1.0 / (double)A.n_seq;
   // sr, sr2: sums of (r-1) and (r-1)^2
   double var = 0.0;
   if (N > 1.0) {
     var = (sr2 - sr * sr * inv_n) / (N - 1.0);
     if (var < 0.0) var = 0.0;
   }
-  float* M = A.metrics;
-  M[UNIRL_M_LOSS] = (float)loss;
-  M[UNIRL_M_RATIO_MEAN] = (float)(1.0 + sr * inv_n);
-  M[UNIRL_M_RATIO_STD] = (float)sqrt(var);
-  // min()/max() of the reference return NaN when any ratio is NaN; the ratios are >= 0, so their
-  // sum is NaN exactly then (likewise the absolute differences below)
-  M[UNIRL_M_RATIO_MIN] = (sr != sr) ? quiet_nan() : (float)lds_fin[P_RMIN];
-  M[UNIRL_M_RATIO_MAX] = (sr != sr) ? quiet_nan() : (float)lds_fin[P_RMAX];
-  M[UNIRL_M_CLIP_FRACTION] = (float)(lds_fin[P_CANY] * inv_n);
-  M[UNIRL_M_CLIPFRAC_HI] = (float)(lds_fin[P_CHI] * inv_n);
-  M[UNIRL_M_CLIPFRAC_LO] = (float)(lds_fin[P_CLO] * inv_n);
+  const double sd = sqrt(var);
+  double y = x * inv_n;  // the means: penalty, |new-old|, the three clip fractions
+  if (v == P_SR) y = 1.0 + y;
   // GRPO accumulates ld^2; mean(0.5*ld^2) = 0.5*sum/N exactly (halving commutes with rounding)
-  M[UNIRL_M_APPROX_KL] = (float)((C.kind == UNIRL_LOSS_GRPO ? 0.5 : 1.0) * lds_fin[P_KL] * inv_n);
-  M[UNIRL_M_PENALTY_MEAN] = (float)(lds_fin[P_PEN] * inv_n);
-  M[UNIRL_M_ABSDIFF_MEAN] = (float)(lds_fin[P_ABS] * inv_n);
-  M[UNIRL_M_ABSDIFF_MAX] = (lds_fin[P_ABS] != lds_fin[P_ABS]) ? quiet_nan() : (float)lds_fin[P_AMAX];
-  M[UNIRL_M_NUM_TOKENS] = (float)N;
-  M[13] = M[14] = M[15] = 0.0f;
+  if (v == P_KL && C.kind == UNIRL_LOSS_GRPO) y = 0.5 * y;
+  if (v == P_LOSS) y = x * loss_scale;
+  if (v == P_SR2) y = sd;
+  if (v == P_CNT) y = x;
+  // min()/max() of the reference return NaN when any ratio is NaN; the ratios are >= 0, so their
+  // sum is NaN exactly then (likewise the absolute differences)
+  if (v == P_NRMIN) y = (sr != sr) ? (double)quiet_nan() : -x;
+  if (v == P_RMAX) y = (sr != sr) ? (double)quiet_nan() : x;
+  if (v == P_AMAX) y = (sab != sab) ? (double)quiet_nan() : x;
+  if (!slot_used(v)) y = 0.0;
+  // metric index of each slot, four bits per slot
+  constexpr unsigned long long kMetricOf =
+      ((unsigned long long)UNIRL_M_RATIO_MEAN << (4 * P_SR)) | ((unsigned long long)UNIRL_M_RATIO_STD << (4 * P_SR2)) |
+      ((unsigned long long)UNIRL_M_LOSS << (4 * P_LOSS)) | ((unsigned long long)UNIRL_M_APPROX_KL << (4 * P_KL)) |
+      ((unsigned long long)UNIRL_M_PENALTY_MEAN << (4 * P_PEN)) |
+      ((unsigned long long)UNIRL_M_ABSDIFF_MEAN << (4 * P_ABS)) |
+      ((unsigned long long)UNIRL_M_NUM_TOKENS << (4 * P_CNT)) | ((unsigned long long)UNIRL_M_CLIPFRAC_HI << (4 * P_CHI)) |
+      ((unsigned long long)UNIRL_M_CLIPFRAC_LO << (4 * P_CLO)) |
+      ((unsigned long long)UNIRL_M_CLIP_FRACTION << (4 * P_CANY)) | (13ull << (4 * 10)) | (14ull << (4 * 11)) |
+      ((unsigned long long)UNIRL_M_RATIO_MIN << (4 * P_NRMIN)) | ((unsigned long long)UNIRL_M_RATIO_MAX << (4 * P_RMAX)) |
+      ((unsigned long long)UNIRL_M_ABSDIFF_MAX << (4 * P_AMAX)) | (15ull << (4 * 15));
+  A.metrics[(kMetricOf >> (4 * v)) & 15u] = (float)y;
 }
 
 template <int KIND, int VEC>
@@ -596,6 +678,9 @@ static int fill_consts(const unirl_ratio_loss_params* p, RatioConsts& C) {
   C.adv_per_token = p->adv_per_token;
   C.clamp_lo = (float)(1.0 - p->clip_low);
   C.clamp_hi = (float)(1.0 + p->clip_high);
+  // torch.clamp(min > max) returns max everywhere; a collapsed interval gives the kernel's
+  // median-of-three the same result
+  if (C.clamp_lo > C.clamp_hi) C.clamp_lo = C.clamp_hi;
   C.eps_lo = (float)p->clip_low;
   C.eps_hi = (float)p->clip_high;
   C.drpo_eps = (float)p->drpo_epsilon;
@@ -689,21 +774,32 @@ extern "C" int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp
   hipStream_t st = (hipStream_t)stream;
   dim3 block(kRlThreads);
   const bool packed = (A.layout == LAYOUT_PACKED);
-#define UNIRL_LAUNCH_FWD(KIND, VEC)                                                                      \
+  // 16-byte vectors: mask / per-token-advantage switches compiled in; scalar tokens: read at run time
+  const int flags = (A.mask ? 1 : 0) | (A.C.adv_per_token ? 2 : 0);
+#define UNIRL_LAUNCH_FWD3(KIND, VEC, FLAGS)                                                              \
   do {                                                                                                   \
     if (packed)                                                                                          \
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, true>), S.grid, block, 0, st, A);             \
+      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, true, FLAGS>), S.grid, block, 0, st, A);      \
     else                                                                                                 \
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, false>), S.grid, block, 0, st, A);            \
+      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, false, FLAGS>), S.grid, block, 0, st, A);     \
   } while (0)
-  if (A.C.kind == UNIRL_LOSS_GRPO) {
-    if (S.vec == 4) UNIRL_LAUNCH_FWD(UNIRL_LOSS_GRPO, 4); else UNIRL_LAUNCH_FWD(UNIRL_LOSS_GRPO, 1);
-  } else {
-    if (S.vec == 4) UNIRL_LAUNCH_FWD(UNIRL_LOSS_DRPO, 4); else UNIRL_LAUNCH_FWD(UNIRL_LOSS_DRPO, 1);
+#define UNIRL_LAUNCH_FWD(KIND)                                                                           \
+  do {                                                                                                   \
+    if (S.vec != 4) UNIRL_LAUNCH_FWD3(KIND, 1, -1);                                                      \
+    else if (flags == 0) UNIRL_LAUNCH_FWD3(KIND, 4, 0);                                                  \
+    else if (flags == 1) UNIRL_LAUNCH_FWD3(KIND, 4, 1);                                                  \
+    else if (flags == 2) UNIRL_LAUNCH_FWD3(KIND, 4, 2);                                                  \
+    else UNIRL_LAUNCH_FWD3(KIND, 4, 3);                                                                  \
+  } while (0)
+  const int64_t dbg = tune_int("UNIRL_DBG_ONLY", 0);
+  if (dbg != 2) {
+  if (A.C.kind == UNIRL_LOSS_GRPO) UNIRL_LAUNCH_FWD(UNIRL_LOSS_GRPO); else UNIRL_LAUNCH_FWD(UNIRL_LOSS_DRPO);
   }
+#undef UNIRL_LAUNCH_FWD3
 #undef UNIRL_LAUNCH_FWD
   const int launch_rc = (int)hipGetLastError();
   if (launch_rc != 0) return launch_rc;
+  if (dbg == 1) return 0;
   hipLaunchKernelGGL(ratio_loss_finalize_kernel, dim3(1), block, 0, st, A, S.grid.x * S.grid.y);
   return (int)hipGetLastError();
 }
