@@ -271,6 +271,7 @@ __device__ __forceinline__ float op_add(float a, float b) { return a + b; }
 __device__ __forceinline__ double op_add(double a, double b) { return a + b; }
 __device__ __forceinline__ unsigned int op_add(unsigned int a, unsigned int b) { return a + b; }
 __device__ __forceinline__ float op_max(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ double op_max(double a, double b) { return fmax(a, b); }
 __device__ __forceinline__ float op_min(float a, float b) { return fminf(a, b); }
 
 __device__ __forceinline__ float last_lane(float v) {
@@ -318,6 +319,10 @@ __device__ __forceinline__ unsigned int wave_sum(unsigned int v) {
 }
 __device__ __forceinline__ float wave_max(float v) {
   UNIRL_DPP_REDUCE(v, op_max, dpp_f32_or_self)
+  return last_lane(v);
+}
+__device__ __forceinline__ double wave_max(double v) {
+  UNIRL_DPP_REDUCE(v, op_max, dpp_f64_or_self)
   return last_lane(v);
 }
 __device__ __forceinline__ float wave_min(float v) {

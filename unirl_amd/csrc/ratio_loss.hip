@@ -388,7 +388,7 @@ __device__ __forceinline__ void fill_ones(float (&m)[VEC]) {
 }
 
 #ifndef UNIRL_RATIO_ITEMS
-#define UNIRL_RATIO_ITEMS 2
+#define UNIRL_RATIO_ITEMS 2  // 4 measured slower on large inputs (registers), equal on small ones
 #endif
 
 // FLAGS >= 0 fixes at compile time whether a loss mask (bit 0) and per-token advantages (bit 1)
@@ -492,19 +492,23 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
   store_block_partials(A, acc, wc, lds_v);
 }
 
-// One workgroup: fixed-order reduction of every workgroup's partial vector, then the metrics.
-__global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioArgs A, unsigned int nblk) {
-  __shared__ double lds_t[kRlThreads];
+// One workgroup of T threads (256, or 1024 when there are more than 512 partial vectors, so that
+// every load of a thread is still in flight at once): fixed-order reduction of every
+// workgroup's partial vector, then the metrics.
+template <int T>
+__global__ __launch_bounds__(T) void ratio_loss_finalize_kernel(RatioArgs A, unsigned int nblk) {
+  constexpr int kSlices = T / kRlVals;  // 16 or 64
+  static_assert(kSlices == kRlParts || kSlices == kWave, "a slot's slices fill a 16-lane row or a wavefront");
+  __shared__ double lds_t[T];
   __shared__ double lds_tot[kRlVals];
   const RatioConsts C = A.C;
   const int t = threadIdx.x;
   {
-    // thread = (slot v, slice j0): 16 slices walk the workgroups' vectors (a wavefront reads four
-    // whole vectors per load), kBatch loads in flight each
+    // thread = (slot v, slice j0): the slices walk the workgroups' vectors (a wavefront reads
+    // four whole vectors per load), kBatch loads in flight each
     const int v = t % kRlVals;
-    const int j0 = t / kRlVals;  // 0..15
-    constexpr int kSlices = kRlThreads / kRlVals;
-    constexpr int kBatch = 32;  // 512 workgroups: every partial of a thread in flight at once
+    const int j0 = t / kRlVals;
+    constexpr int kBatch = 32;
     const double ident = (v < kFirstMax) ? 0.0 : -(double)INFINITY;
     double x = ident;
     for (unsigned int j = j0; j < nblk; j += kSlices * kBatch) {
@@ -523,15 +527,20 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_finalize_kernel(RatioAr
         for (int b = 0; b < kBatch; ++b) x = fmax(x, y[b]);
       }
     }
-    lds_t[v * kSlices + j0] = x;  // transposed: the sixteen slices of a slot side by side
+    lds_t[v * kSlices + j0] = x;  // transposed: the slices of a slot side by side
   }
   __syncthreads();
   {
-    // thread = (slot, slice) again, now with a slot's slices in one 16-lane row
-    const int v = t / kRlParts;
+    // thread = (slot, slice) again, now with a slot's slices in one 16-lane row / one wavefront
+    const int v = t / kSlices;
     double z = lds_t[t];
-    z = (v < kFirstMax) ? row_sum_last(z) : row_max_last(z);
-    if (t % kRlParts == kRlParts - 1) lds_tot[v] = z;
+    if (kSlices == kRlParts) {
+      z = (v < kFirstMax) ? row_sum_last(z) : row_max_last(z);
+      if (t % kRlParts == kRlParts - 1) lds_tot[v] = z;
+    } else {
+      z = (v < kFirstMax) ? wave_sum(z) : wave_max(z);
+      if (t % kWave == 0) lds_tot[v] = z;
+    }
   }
   __syncthreads();
   if (t >= kRlVals) return;
@@ -704,9 +713,10 @@ static int plan(const RatioArgs& A, bool bwd, RatioShape& S) {
   if (padded && A.seq_stride % 4 != 0) vec = 1;
   const int64_t row_tok = padded ? A.seq_stride : A.n_tok;
   const int64_t nvec = (row_tok + vec - 1) / vec;
-  // forward: one partial vector per workgroup is read back by a single finalize workgroup, whose
-  // time grows with their number (about 1 us per 128); 512 suits inputs of a few MB, 1024 large ones
-  const int64_t cap = bwd ? 16384 : tune_int("UNIRL_RATIO_MAX_BLOCKS", A.n_tok >= (16 << 20) ? 1024 : 512);
+  // forward: one partial vector per workgroup is read back by a single finalize workgroup, which
+  // one compute unit's memory pipeline feeds (about 1 us per 512 vectors); 512 workgroups suit
+  // inputs of a few MB, 1024 large ones
+  const int64_t cap = bwd ? 16384 : tune_int("UNIRL_RATIO_MAX_BLOCKS", A.n_tok >= (8 << 20) ? 1024 : 512);
   int64_t rows = padded ? A.n_seq : 1;
   if (rows > cap) rows = cap;
   if (rows < 1) rows = 1;
@@ -800,7 +810,11 @@ extern "C" int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp
   const int launch_rc = (int)hipGetLastError();
   if (launch_rc != 0) return launch_rc;
   if (dbg == 1) return 0;
-  hipLaunchKernelGGL(ratio_loss_finalize_kernel, dim3(1), block, 0, st, A, S.grid.x * S.grid.y);
+  const unsigned int nblk = S.grid.x * S.grid.y;
+  if (nblk <= 512)
+    hipLaunchKernelGGL(ratio_loss_finalize_kernel<256>, dim3(1), dim3(256), 0, st, A, nblk);
+  else
+    hipLaunchKernelGGL(ratio_loss_finalize_kernel<1024>, dim3(1), dim3(1024), 0, st, A, nblk);
   return (int)hipGetLastError();
 }
 
