@@ -196,6 +196,22 @@ def make_shapes(torch, dev):
             run=(lambda i, k=kind: plans[k][i % ns3].forward(False)), sets=ns3,
             cpu=(lambda k=kind, o=okw: olos.token_loss(k, newp, oldp, adv, lengths, **o)), cpu_bytes=bytes3_valid,
         ))
+    # the whole training micro-step: loss, metrics and the gradient w.r.t. new_logp in one pass
+    # (the gradient tensor has the padded shape; the padding is written as zeros)
+    bytes3_step = bytes3_valid + new.numel() * 4
+
+    def cpu_step(k, o):
+        leaf = newp.clone().requires_grad_(True)
+        olos.token_loss(k, leaf, oldp, adv, lengths, **o)[0].backward()
+
+    for kind, okw in (("grpo", dict(clip_range=0.2, clip_range_high=0.28)), ("drpo", dict(epsilon=5.0))):
+        shapes.append(dict(
+            name=f"ratio_step_{kind}", config=3,
+            shape=f"fp32 [256,8192] padded, {n_valid} valid tokens: loss + metrics + grad_new in one pass",
+            bytes=bytes3_step, read_bytes=bytes3_valid, write_bytes=new.numel() * 4, elements=n_valid,
+            run=(lambda i, k=kind: plans[k][i % ns3].forward_backward(1.0)), sets=ns3,
+            cpu=(lambda k=kind, o=okw: cpu_step(k, o)), cpu_bytes=bytes3_step,
+        ))
 
     # -- config 4: Flow-DPPO KL mask, WAN bf16 [2,16,21,60,104] -----------------------------------
     g = torch.Generator().manual_seed(1004)

@@ -324,6 +324,22 @@ int unirl_ratio_loss_bwd(const float* new_logp, const float* old_logp, const flo
                                                  of the forward; token-mean only */,
                          float* grad_new, void* stream);
 
+/* Forward and backward of one training micro-step in a single pass over new / old:
+ * the metrics of unirl_ratio_loss_fwd plus grad_new = loss_scale * w_tok * dloss/dnew,
+ * i.e. what `(loss * loss_scale).backward()` leaves in new_logp.grad
+ * (unirl/algorithms/grpo.py:134-160, drpo.py:310-334, flowgrpo.py:174-193).
+ * n_valid: the token-mean denominator in the padded layout (every token inside
+ * the lengths, masked or not) when the host knows it; < 0 lets the kernel sum
+ * the lengths.  Ignored in the other layouts (n_tok).  Padded slots past a
+ * sequence's length receive 0. */
+int unirl_ratio_loss_fwd_bwd(const float* new_logp, const float* old_logp, const float* advantages,
+                             const int64_t* lengths, const float* loss_mask, int64_t n_seq,
+                             int64_t seq_stride, int64_t n_tok,
+                             const struct unirl_ratio_loss_params* params /* host */,
+                             float loss_scale, int64_t n_valid, float* grad_new,
+                             float* metrics /* [UNIRL_M_COUNT] f32 */, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
 /* out[t] = vals[r] for every token t of sequence r (packed layout, cu_seqlens
  * int64 [n_seq+1]): GRPO._expand_advantages_to_tokens
  * (unirl/algorithms/grpo.py:187-198) as one kernel. */

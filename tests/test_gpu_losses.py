@@ -310,3 +310,86 @@ def test_config3_shape(dev):
         check_metrics(kind, {k: vals[s] for k, s in slots.items()}, ref_m, n_tok)
         assert_close(olos.pack_padded(nd.grad.cpu(), lengths), npk.grad, 1e-5, 1e-6 * float(npk.grad.abs().max()),
                      "config-3 grad")
+
+
+@pytest.mark.parametrize("kind", ["grpo", "drpo"])
+@pytest.mark.parametrize("mode", MODES)
+@pytest.mark.parametrize("shape", [(16, 512), (7, 37), (3, 1000), (40, 2048)])
+@pytest.mark.parametrize("with_mask", [False, True])
+def test_one_pass_loss_and_gradient(dev, kind, mode, shape, with_mask):
+    """The one-pass training step: metrics of the forward, and in new_logp.grad what
+    (loss * loss_scale).backward() of the oracle leaves there -- padded layout with device and host
+    lengths, packed layout, with and without a loss mask."""
+    from unirl_amd import _native as N
+    from unirl_amd.algorithms._fused import ABSDIFF_METRICS, DRPO_METRICS, GRPO_METRICS, fused_token_loss_backward
+
+    if kind == "drpo" and mode == "seq-mean-token-mean":
+        pytest.skip("the reference's DRPO has no seq-mean-token-mean mode")
+    if kind == "grpo" and with_mask:
+        pytest.skip("the reference's GRPO takes no loss mask")
+    loss_scale = 0.37
+    new, old, lengths, adv = batch(*shape, seed=11 + sum(shape))
+    newp, oldp = olos.pack_padded(new, lengths), olos.pack_padded(old, lengths)
+    g = torch.Generator().manual_seed(5)
+    maskp = (torch.rand(newp.shape, generator=g) < 0.7).float() if with_mask else None
+    kw = dict(clip_range=0.2, clip_range_high=0.28, epsilon=5.0)
+    npk = newp.clone().requires_grad_(True)
+    ref_loss, ref_m = olos.token_loss(kind, npk, oldp, adv, lengths, mode=mode, horizon=shape[1], loss_mask=maskp, **kw)
+    (ref_loss * loss_scale).backward()
+    elem_abs = float(olos.token_loss(kind, newp, oldp, adv, lengths, mode="token-mean", **kw)[0].abs()) + float(adv.abs().mean())
+    slots = dict(GRPO_METRICS if kind == "grpo" else DRPO_METRICS, **ABSDIFF_METRICS)
+    gtol = 1e-6 * float(npk.grad.abs().max())
+    common = dict(loss_scale=loss_scale, loss_agg_mode=mode, horizon=shape[1], clip_range=0.2, clip_range_high=0.28,
+                  drpo_epsilon=5.0)
+    mask2d = None
+    if with_mask:
+        mask2d = torch.zeros(shape)
+        col = torch.arange(shape[1])[None, :] < lengths[:, None]
+        mask2d[col] = maskp
+
+    for where in ("device", "host"):  # lengths on the host let the wrapper pass the token count
+        nd = new.to(dev).requires_grad_(True)
+        twice = nd * 1.0  # a non-leaf: the gradient must flow on through the graph
+        mvec = fused_token_loss_backward(
+            kind, twice, old.to(dev), adv.to(dev), lengths=lengths.to(dev) if where == "device" else lengths,
+            loss_mask=None if mask2d is None else mask2d.to(dev), **common)
+        vals = mvec.tolist()
+        assert_close(torch.tensor(vals[N.M_LOSS]), ref_loss, FP32_RTOL, loss_atol(elem_abs), f"{kind} {mode} loss")
+        assert vals[N.M_NUM_TOKENS] == float(lengths.sum())
+        check_metrics(kind, {k: vals[s] for k, s in slots.items()}, ref_m, int(lengths.sum()))
+        assert_close(olos.pack_padded(nd.grad.cpu(), lengths), npk.grad, 1e-5, gtol, f"padded grad ({where} lengths)")
+        pad = torch.arange(shape[1])[None, :] >= lengths[:, None]
+        assert float(nd.grad.cpu()[pad].abs().sum()) == 0.0
+
+    cu = torch.cat([torch.zeros(1, dtype=torch.int64), lengths.cumsum(0)])
+    nd2 = newp.to(dev).requires_grad_(True)
+    mvec2 = fused_token_loss_backward(kind, nd2, oldp.to(dev), adv.to(dev), cu_seqlens=cu.to(dev),
+                                      loss_mask=None if maskp is None else maskp.to(dev), **common)
+    assert_close(torch.tensor(mvec2.tolist()[N.M_LOSS]), ref_loss, FP32_RTOL, loss_atol(elem_abs), "packed loss")
+    assert_close(nd2.grad, npk.grad, 1e-5, gtol, "packed grad")
+
+
+def test_one_pass_matches_two_launch_backward_bitwise(dev):
+    """Same expressions as the stand-alone backward kernel: identical bits, ties and clamps included."""
+    from unirl_amd import _native as N
+    from unirl_amd.ops import RatioLossPlan
+
+    new, old, lengths, adv = batch(32, 777, seed=3, scale=0.3)
+    new[0, :5] = old[0, :5] + math.log(1.28)  # on / next to the clip edge
+    new[1, :5] = old[1, :5] + 25.0            # past DRPO's clamp
+    for code, kw in ((N.LOSS_GRPO, dict(clip_low=0.2, clip_high=0.28)), (N.LOSS_DRPO, dict(drpo_epsilon=5.0))):
+        plan = RatioLossPlan(new.to(dev), old.to(dev), adv.to(dev), kind=code, lengths=lengths.to(dev), **kw)
+        _, m = plan.forward(False)
+        scale = torch.tensor([0.37], device=dev)
+        g2 = plan.backward(g_scale=scale, g_elem=None, aggregate=True, n_valid=m[N.M_NUM_TOKENS : N.M_NUM_TOKENS + 1])
+        g1, m1 = plan.forward_backward(0.37)
+        assert torch.equal(g1, g2)
+        assert torch.equal(m1[:13], m[:13])
+
+
+def test_one_pass_without_graph_runs_forward_only(dev):
+    from unirl_amd.algorithms._fused import fused_token_loss_backward
+
+    new, old, lengths, adv = batch(4, 64, seed=9)
+    m = fused_token_loss_backward("grpo", new.to(dev), old.to(dev), adv.to(dev), lengths=lengths.to(dev), loss_scale=1.0)
+    assert m.shape == (16,) and bool(torch.isfinite(m[:13]).all())

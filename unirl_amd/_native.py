@@ -155,6 +155,11 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, POINTER(RatioLossParams),
          c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
     ),
+    "unirl_ratio_loss_fwd_bwd": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, POINTER(RatioLossParams),
+         c_float, c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    ),
     "unirl_group_advantages": (
         c_int,
         [c_void_p, c_int64, c_int64, c_int, c_float, c_int, c_int, c_void_p, c_void_p],

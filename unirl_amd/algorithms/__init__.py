@@ -1,6 +1,6 @@
 """Loss math of the RL algorithms: GRPO / DRPO (token level), FlowGRPO / FlowDPPO (diffusion)."""
 
-from ._fused import fused_token_loss
+from ._fused import fused_token_loss, fused_token_loss_backward
 from .base import (
     AlgorithmStepResult,
     StageAlgorithm,
@@ -28,6 +28,7 @@ __all__ = [
     "GRPOConfig",
     "StageAlgorithm",
     "fused_token_loss",
+    "fused_token_loss_backward",
     "gather_sde_field",
     "normalize_global",
     "normalize_grouped",

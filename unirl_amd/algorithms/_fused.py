@@ -61,6 +61,43 @@ def scalar_loss(new_logp: torch.Tensor, plan: RatioLossPlan) -> Tuple[torch.Tens
     return metrics[N.M_LOSS].clone(), metrics
 
 
+def fused_token_loss_backward(
+    kind: str,
+    new_logp: torch.Tensor,
+    old_logp: torch.Tensor,
+    advantages: torch.Tensor,
+    *,
+    loss_scale: float,
+    lengths: Optional[torch.Tensor] = None,
+    cu_seqlens: Optional[torch.Tensor] = None,
+    loss_mask: Optional[torch.Tensor] = None,
+    loss_agg_mode: str = "token-mean",
+    horizon: int = 8192,
+    clip_range: float = 0.2,
+    clip_range_high: Optional[float] = None,
+    drpo_epsilon: float = 12.5,
+    mu_weighted: bool = True,
+) -> torch.Tensor:
+    """``(loss * loss_scale).backward()`` of :func:`fused_token_loss` without building the loss
+    in autograd: one kernel reads ``new_logp`` / ``old_logp`` once, reduces the loss and every
+    metric and writes the gradient, which is then pushed into ``new_logp``'s graph.  Returns the
+    ``[16]`` metrics vector (``M_LOSS`` holds the unscaled loss).  Without a graph behind
+    ``new_logp`` only the forward runs."""
+    code = {"grpo": N.LOSS_GRPO, "drpo": N.LOSS_DRPO}[kind]
+    plan = RatioLossPlan(
+        new_logp, old_logp, advantages, kind=code, lengths=lengths, cu_seqlens=cu_seqlens, loss_mask=loss_mask,
+        agg_mode=loss_agg_mode, clip_low=clip_range, clip_high=clip_range_high, drpo_epsilon=drpo_epsilon,
+        mu_weighted=mu_weighted, horizon=horizon,
+    )
+    if not (torch.is_grad_enabled() and new_logp.requires_grad):
+        return plan.forward(want_elem=False)[1]
+    grad, metrics = plan.forward_backward(float(loss_scale))
+    if grad.dtype != new_logp.dtype:
+        grad = grad.to(new_logp.dtype)
+    new_logp.backward(grad)
+    return metrics
+
+
 GRPO_METRICS: Dict[str, int] = {
     "ratio_mean": N.M_RATIO_MEAN,
     "ratio_std": N.M_RATIO_STD,

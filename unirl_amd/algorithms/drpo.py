@@ -15,7 +15,7 @@ import torch
 
 from .. import _native as N
 from .. import ops
-from ._fused import ABSDIFF_METRICS, DRPO_METRICS, elem_loss, fused_token_loss, metric_tensors
+from ._fused import ABSDIFF_METRICS, DRPO_METRICS, elem_loss, fused_token_loss_backward, metric_tensors
 from .base import (
     NO_STEP,
     AlgorithmStepResult,
@@ -124,13 +124,13 @@ class DRPO(StageAlgorithm):
                 f"GRPO advantage expansion: advantages batch={bs} != lengths={int(segment.lengths.shape[0])}"
             )
         mode = "seq-mean-token-sum-norm" if self.loss_agg_mode == "seq-mean-token-sum-norm" else "token-mean"
-        loss, mvec = fused_token_loss(
-            "drpo", new_logp, segment.log_probs, advantages,
+        # loss, metrics and `(loss * loss_scale).backward()` in one pass over the tokens
+        mvec = fused_token_loss_backward(
+            "drpo", new_logp, segment.log_probs, advantages, loss_scale=loss_scale,
             cu_seqlens=cu_seqlens_from_lengths(segment.lengths, new_logp.device),
             loss_mask=getattr(segment, "loss_mask", None), loss_agg_mode=mode, horizon=self.horizon,
             drpo_epsilon=self.drpo_epsilon, mu_weighted=self.penalty_mu_weighted,
         )
-        (loss * loss_scale).backward()
 
         vals = mvec.tolist()
         metrics: Dict[str, Any] = {"policy_loss": vals[N.M_LOSS], "drpo_epsilon": self.drpo_epsilon}

@@ -10,7 +10,7 @@ from typing import Any, Dict, Mapping, Optional, Type
 import torch
 
 from .. import _native as N
-from ._fused import GRPO_METRICS, fused_token_loss
+from ._fused import GRPO_METRICS, fused_token_loss_backward
 from .base import (
     NO_STEP,
     AlgorithmStepResult,
@@ -72,10 +72,9 @@ class FlowGRPO(SdeStepAlgorithm):
         eps = _resolve_clip_range_from_schedule(self.clip_range, self.clip_schedule, training_progress)
         # every step of sample b shares advantages[b]: the padded layout with S' tokens per row
         rows, n_steps = new_logp.shape
-        full = torch.full((rows,), n_steps, dtype=torch.int64, device=new_logp.device)
-        loss, mvec = fused_token_loss("grpo", new_logp, old_logp, advantages.detach().reshape(-1), lengths=full,
-                                      clip_range=eps)
-        (loss * loss_scale).backward()
+        full = torch.full((rows,), n_steps, dtype=torch.int64)  # host lengths: the token count is known
+        mvec = fused_token_loss_backward("grpo", new_logp, old_logp, advantages.detach().reshape(-1),
+                                         loss_scale=loss_scale, lengths=full, clip_range=eps)
         vals = mvec.tolist()  # the step's only device-to-host copy
         metrics: Dict[str, Any] = {k: vals[slot] for k, slot in GRPO_METRICS.items()}
         metrics.update(policy_loss=vals[N.M_LOSS], clip_range=float(eps))

@@ -2,9 +2,10 @@
 
 ``stage.replay`` still owns the teacher-forced forward; everything after it --
 advantage expansion (:172-198), the clipped ratio (base.py:115-157), the
-aggregation mode (:148-155), the drift gauge and all metric reductions -- is one
-forward kernel and, for ``.backward()``, one backward kernel.  The metrics reach
-the host with a single device-to-host copy instead of one ``.item()`` each.
+aggregation mode (:148-155), the drift gauge, all metric reductions and the
+gradient that ``(loss * loss_scale).backward()`` sends into ``new_logp`` -- is one
+kernel that reads the tokens once.  The metrics reach the host with a single
+device-to-host copy instead of one ``.item()`` each.
 """
 
 from __future__ import annotations
@@ -16,7 +17,7 @@ import torch
 
 from .. import _native as N
 from .. import ops
-from ._fused import ABSDIFF_METRICS, GRPO_METRICS, fused_token_loss
+from ._fused import ABSDIFF_METRICS, GRPO_METRICS, fused_token_loss_backward
 from .base import (
     NO_STEP,
     AlgorithmStepResult,
@@ -108,12 +109,12 @@ class GRPO(StageAlgorithm):
         mode = self.loss_agg_mode
         if mode not in ("seq-mean-token-sum-norm", "seq-mean-token-mean"):
             mode = "token-mean"
-        loss, mvec = fused_token_loss(
-            "grpo", new_logp, segment.log_probs, advantages,
+        # loss, metrics and `(loss * loss_scale).backward()` in one pass over the tokens
+        mvec = fused_token_loss_backward(
+            "grpo", new_logp, segment.log_probs, advantages, loss_scale=loss_scale,
             cu_seqlens=cu_seqlens_from_lengths(segment.lengths, new_logp.device), loss_agg_mode=mode,
             horizon=self.horizon, clip_range=clip_range, clip_range_high=clip_high,
         )
-        (loss * loss_scale).backward()
 
         vals = mvec.tolist()  # the step's only device-to-host copy
         metrics: Dict[str, Any] = {"policy_loss": vals[N.M_LOSS], "clip_range": float(clip_range)}

@@ -69,6 +69,9 @@ struct RatioArgs {
   const float* n_valid;  // device scalar: valid-token count from the forward
   int aggregate;
   float* grad_new;
+  // fused forward + backward only
+  float loss_scale;      // gradient arriving at the aggregated loss
+  int64_t n_valid_host;  // token-mean denominator when the host knows it, else < 0
 };
 
 // exp(x) for fp32 within ~1.5 ulp: 2^(x*log2(e)) on the hardware exp2, with the rounding error
@@ -202,11 +205,14 @@ struct WaveCounts {
 //   maximum(u, c) = (c > u) ? c : u   -- u is NaN whenever c is (c = -A*clamp(r), u = -A*r), so
 //                                        NaN reaches the result as in torch.maximum;
 //   1 - r = -(r - 1)                  -- rounding is symmetric, so the lower clip test reuses r-1.
-template <int KIND>
+// With GRAD the derivative of the token's loss with respect to new_logp is left in `dl` (the
+// expressions of ratio_token, which the stand-alone backward kernel uses).
+template <int KIND, bool GRAD>
 __device__ __forceinline__ float accumulate_token(float nw, float od, float A, float lw, const RatioConsts& C,
-                                                  Acc& acc, bool& hi, bool& lo) {
+                                                  Acc& acc, bool& hi, bool& lo, float& dl) {
   const float d0 = nw - od;
   float r, loss;
+  dl = 0.0f;
   if (KIND == UNIRL_LOSS_GRPO) {
     r = exp_f32(d0);
     const float nA = -A;
@@ -221,6 +227,11 @@ __device__ __forceinline__ float accumulate_token(float nw, float od, float A, f
     acc.s1 += d;
     acc.s2 = fmaf(d, d, acc.s2);
     acc.kl = fmaf(d0, d0, acc.kl);
+    if (GRAD) {
+      const bool inside = (r >= C.clamp_lo) && (r <= C.clamp_hi);
+      const float dc = inside ? c : 0.0f;
+      dl = (u > c) ? u : ((u < c) ? dc : 0.5f * (u + dc));
+    }
   } else {
     const float ld = (d0 != d0) ? d0 : fminf(fmaxf(d0, -20.0f), 20.0f);  // torch.clamp keeps NaN
     float e;
@@ -238,6 +249,10 @@ __device__ __forceinline__ float accumulate_token(float nw, float od, float A, f
     acc.s2 = fmaf(d, d, acc.s2);
     acc.kl += d - ld;
     acc.pen += pen;
+    if (GRAD) {
+      const bool clamped = (d0 < -20.0f) || (d0 > 20.0f);
+      dl = clamped ? 0.0f : ((-A) + (fabsf(A) * w) * d / C.drpo_eps) * r;
+    }
   }
   acc.loss += loss * lw;
   const float a0 = fabsf(d0);
@@ -278,17 +293,21 @@ struct SeqCtx {
 // outside the packed layout take a path without per-token bounds or sequence checks.  Outside
 // the packed layout the aggregation weight is the same for the whole pass and is applied by
 // Acc::flush; in the packed layout it rides on every token.
-template <int KIND, int VEC, bool PACKED>
+template <int KIND, int VEC, bool PACKED, bool GRAD>
 __device__ __forceinline__ void ratio_vec_fwd(const RatioArgs& A, const RatioConsts& C, int64_t t0, int64_t count,
                                               const float (&nw)[VEC], const float (&od)[VEC],
                                               const float (&ad)[VEC], const float (&mk)[VEC], bool adv_tok,
-                                              SeqCtx& sq, Acc& acc, float (&out)[VEC]) {
+                                              float gfac, SeqCtx& sq, Acc& acc, float (&out)[VEC],
+                                              float (&gr)[VEC]) {
   if (!PACKED && t0 + VEC <= count) {
+    const float grow = gfac * sq.w;
 #pragma unroll
     for (int k = 0; k < VEC; ++k) {
       const float a = adv_tok ? ad[k] : sq.adv;
       bool hi, lo;
-      out[k] = accumulate_token<KIND>(nw[k], od[k], a, mk[k], C, acc, hi, lo);
+      float dl;
+      out[k] = accumulate_token<KIND, GRAD>(nw[k], od[k], a, mk[k], C, acc, hi, lo, dl);
+      gr[k] = (grow * mk[k]) * dl;
       acc.chi += hi ? 1u : 0u;
       acc.clo += lo ? 1u : 0u;
       acc.cany += (hi || lo) ? 1u : 0u;
@@ -300,6 +319,7 @@ __device__ __forceinline__ void ratio_vec_fwd(const RatioArgs& A, const RatioCon
   for (int k = 0; k < VEC; ++k) {
     const int64_t t = t0 + k;
     out[k] = 0.0f;
+    gr[k] = 0.0f;
     if (t < count) {
       if (PACKED && t >= sq.cur_end) {
         const int64_t s = find_seq(A.seq, A.n_seq, t);
@@ -309,7 +329,9 @@ __device__ __forceinline__ void ratio_vec_fwd(const RatioArgs& A, const RatioCon
       }
       const float a = adv_tok ? ad[k] : sq.adv;
       bool hi, lo;
-      out[k] = accumulate_token<KIND>(nw[k], od[k], a, PACKED ? mk[k] * sq.w : mk[k], C, acc, hi, lo);
+      float dl;
+      out[k] = accumulate_token<KIND, GRAD>(nw[k], od[k], a, PACKED ? mk[k] * sq.w : mk[k], C, acc, hi, lo, dl);
+      gr[k] = ((gfac * sq.w) * mk[k]) * dl;
       acc.chi += hi ? 1u : 0u;
       acc.clo += lo ? 1u : 0u;
       acc.cany += (hi || lo) ? 1u : 0u;
@@ -320,16 +342,19 @@ __device__ __forceinline__ void ratio_vec_fwd(const RatioArgs& A, const RatioCon
 
 // The same for a vector that is whole and valid in all 64 lanes (outside the packed layout): no
 // bounds checks, and the clip flags are counted per wavefront.
-template <int KIND, int VEC>
+template <int KIND, int VEC, bool GRAD>
 __device__ __forceinline__ void ratio_vec_wave(const RatioConsts& C, const float (&nw)[VEC],
                                                const float (&od)[VEC], const float (&ad)[VEC],
-                                               const float (&mk)[VEC], bool adv_tok, const SeqCtx& sq, Acc& acc,
-                                               WaveCounts& wc, float (&out)[VEC]) {
+                                               const float (&mk)[VEC], bool adv_tok, float gfac, const SeqCtx& sq,
+                                               Acc& acc, WaveCounts& wc, float (&out)[VEC], float (&gr)[VEC]) {
+  const float grow = gfac * sq.w;
 #pragma unroll
   for (int k = 0; k < VEC; ++k) {
     const float a = adv_tok ? ad[k] : sq.adv;
     bool hi, lo;
-    out[k] = accumulate_token<KIND>(nw[k], od[k], a, mk[k], C, acc, hi, lo);
+    float dl;
+    out[k] = accumulate_token<KIND, GRAD>(nw[k], od[k], a, mk[k], C, acc, hi, lo, dl);
+    gr[k] = (grow * mk[k]) * dl;
     wc.add(hi, lo);
   }
   acc.cnt += VEC;
@@ -394,13 +419,39 @@ __device__ __forceinline__ void fill_ones(float (&m)[VEC]) {
 // FLAGS >= 0 fixes at compile time whether a loss mask (bit 0) and per-token advantages (bit 1)
 // are read, which keeps the loads of a pass straight-line code (all of them in flight before the
 // first use); FLAGS < 0 reads both switches at run time.
-template <int KIND, int VEC, bool PACKED, int FLAGS>
+// With GRAD the kernel also writes grad_new = loss_scale * w_tok * dloss/dnew (the aggregation
+// weights of ratio_loss_bwd_kernel with aggregate set), so a training step reads new / old once.
+template <int KIND, int VEC, bool PACKED, int FLAGS, bool GRAD>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A) {
   constexpr int ITEMS = UNIRL_RATIO_ITEMS;  // vectors in flight per lane
   __shared__ double lds_v[kRlVals][kRlThreads];
   const RatioConsts C = A.C;
   const bool has_mask = (FLAGS < 0) ? (A.mask != nullptr) : ((FLAGS & 1) != 0);
   const bool adv_tok = (FLAGS < 0) ? (C.adv_per_token != 0) : ((FLAGS & 2) != 0);
+
+  // global factor of the gradient; the token-mean denominator is the number of valid tokens,
+  // which is the sum of the (clamped) lengths when the host did not pass it
+  float gfac = 0.0f;
+  if (GRAD) {
+    if (C.agg_mode == UNIRL_AGG_TOKEN_MEAN) {
+      double nv = (double)A.n_valid_host;
+      if (A.n_valid_host < 0) {
+        double s = 0.0;  // exact: lengths are far below 2^53
+        for (int64_t i = threadIdx.x; i < A.n_seq; i += kRlThreads) {
+          int64_t len = A.seq[i];
+          len = len < 0 ? 0 : (len > A.seq_stride ? A.seq_stride : len);
+          s += (double)len;
+        }
+        nv = block_sum(s, &lds_v[0][0]);
+        __syncthreads();  // lds_v is reused below
+      }
+      gfac = A.loss_scale / (float)nv;
+    } else if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_SUM) {
+      gfac = (A.loss_scale / (float)A.n_seq) / C.horizon;
+    } else {
+      gfac = A.loss_scale / (float)A.n_seq;
+    }
+  }
 
   Acc acc;
   WaveCounts wc;
@@ -451,14 +502,16 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
       for (int it = 0; it < ITEMS; ++it) {
         const int64_t wv = w0 + it * stride;  // the wavefront's first vector of this item
         const int64_t i = wv + lane;
-        float out[VEC];
+        float out[VEC], gr[VEC];
         if (!PACKED && (wv + kWave) * VEC <= count) {
-          ratio_vec_wave<KIND, VEC>(C, nw[it], od[it], ad[it], mk[it], adv_tok, sq, acc, wc, out);
+          ratio_vec_wave<KIND, VEC, GRAD>(C, nw[it], od[it], ad[it], mk[it], adv_tok, gfac, sq, acc, wc, out, gr);
           if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + base + i * VEC, out);
+          if (GRAD) Vec<float, VEC>::store(A.grad_new + base + i * VEC, gr);
         } else if (i < nload) {
-          ratio_vec_fwd<KIND, VEC, PACKED>(A, C, i * VEC, count, nw[it], od[it], ad[it], mk[it], adv_tok, sq, acc,
-                                           out);
+          ratio_vec_fwd<KIND, VEC, PACKED, GRAD>(A, C, i * VEC, count, nw[it], od[it], ad[it], mk[it], adv_tok, gfac,
+                                                 sq, acc, out, gr);
           if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + base + i * VEC, out);
+          if (GRAD) Vec<float, VEC>::store(A.grad_new + base + i * VEC, gr);
         }
       }
       acc.flush(pass_w);
@@ -467,7 +520,7 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
     // one lane of the grid takes it token by token
     if (nvec > nvec_full && first == nvec_full % stride) {
       const int64_t t0 = nvec_full * VEC;
-      float nw[VEC], od[VEC], ad[VEC], mk[VEC], out[VEC];
+      float nw[VEC], od[VEC], ad[VEC], mk[VEC], out[VEC], gr[VEC];
 #pragma unroll
       for (int k = 0; k < VEC; ++k) {
         const bool ok = (t0 + k) < count;
@@ -476,17 +529,22 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
         ad[k] = (ok && adv_tok) ? A.adv[base + t0 + k] : 0.0f;
         mk[k] = (ok && has_mask) ? A.mask[base + t0 + k] : 1.0f;
       }
-      ratio_vec_fwd<KIND, VEC, PACKED>(A, C, t0, count, nw, od, ad, mk, adv_tok, sq, acc, out);
-      if (A.loss_elem) {
+      ratio_vec_fwd<KIND, VEC, PACKED, GRAD>(A, C, t0, count, nw, od, ad, mk, adv_tok, gfac, sq, acc, out, gr);
 #pragma unroll
-        for (int k = 0; k < VEC; ++k)
-          if (t0 + k < row_end) A.loss_elem[base + t0 + k] = out[k];
+      for (int k = 0; k < VEC; ++k) {
+        if (t0 + k < row_end) {
+          if (A.loss_elem) A.loss_elem[base + t0 + k] = out[k];
+          if (GRAD) A.grad_new[base + t0 + k] = gr[k];
+        }
       }
       acc.flush(pass_w);
     }
-    // padded layout: zero the loss of the slots past the sequence end
-    if (A.loss_elem && padded) {
-      for (int64_t t = nvec * VEC + first; t < row_end; t += stride) A.loss_elem[base + t] = 0.0f;
+    // padded layout: zero the loss (and the gradient) of the slots past the sequence end
+    if ((A.loss_elem || GRAD) && padded) {
+      for (int64_t t = nvec * VEC + first; t < row_end; t += stride) {
+        if (A.loss_elem) A.loss_elem[base + t] = 0.0f;
+        if (GRAD) A.grad_new[base + t] = 0.0f;
+      }
     }
   }
   store_block_partials(A, acc, wc, lds_v);
@@ -764,6 +822,49 @@ static int check_common(const float* new_logp, const float* old_logp, const floa
   return UNIRL_OK;
 }
 
+// Forward kernel (+ gradient when A.grad_new is set) and its finalize launch.
+static int launch_forward(RatioArgs& A, hipStream_t st) {
+  RatioShape S;
+  plan(A, false, S);
+  if ((int64_t)S.grid.x * S.grid.y * kRlVals > kPartialCapacity) return UNIRL_E_LIMIT;
+  dim3 block(kRlThreads);
+  const bool packed = (A.layout == LAYOUT_PACKED);
+  const bool grad = (A.grad_new != nullptr);
+  // 16-byte vectors: mask / per-token-advantage switches compiled in; scalar tokens: read at run time
+  const int flags = (A.mask ? 1 : 0) | (A.C.adv_per_token ? 2 : 0);
+#define UNIRL_LAUNCH_FWD4(KIND, VEC, PACKED, FLAGS)                                                            \
+  do {                                                                                                         \
+    if (grad)                                                                                                  \
+      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, PACKED, FLAGS, true>), S.grid, block, 0, st, A);    \
+    else                                                                                                       \
+      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, PACKED, FLAGS, false>), S.grid, block, 0, st, A);   \
+  } while (0)
+#define UNIRL_LAUNCH_FWD3(KIND, VEC, FLAGS)                                                                    \
+  do {                                                                                                         \
+    if (packed) UNIRL_LAUNCH_FWD4(KIND, VEC, true, FLAGS); else UNIRL_LAUNCH_FWD4(KIND, VEC, false, FLAGS);    \
+  } while (0)
+#define UNIRL_LAUNCH_FWD(KIND)                                                                                 \
+  do {                                                                                                         \
+    if (S.vec != 4) UNIRL_LAUNCH_FWD3(KIND, 1, -1);                                                            \
+    else if (flags == 0) UNIRL_LAUNCH_FWD3(KIND, 4, 0);                                                        \
+    else if (flags == 1) UNIRL_LAUNCH_FWD3(KIND, 4, 1);                                                        \
+    else if (flags == 2) UNIRL_LAUNCH_FWD3(KIND, 4, 2);                                                        \
+    else UNIRL_LAUNCH_FWD3(KIND, 4, 3);                                                                        \
+  } while (0)
+  if (A.C.kind == UNIRL_LOSS_GRPO) UNIRL_LAUNCH_FWD(UNIRL_LOSS_GRPO); else UNIRL_LAUNCH_FWD(UNIRL_LOSS_DRPO);
+#undef UNIRL_LAUNCH_FWD4
+#undef UNIRL_LAUNCH_FWD3
+#undef UNIRL_LAUNCH_FWD
+  const int launch_rc = (int)hipGetLastError();
+  if (launch_rc != 0) return launch_rc;
+  const unsigned int nblk = S.grid.x * S.grid.y;
+  if (nblk <= 512)
+    hipLaunchKernelGGL(ratio_loss_finalize_kernel<256>, dim3(1), dim3(256), 0, st, A, nblk);
+  else
+    hipLaunchKernelGGL(ratio_loss_finalize_kernel<1024>, dim3(1), dim3(1024), 0, st, A, nblk);
+  return (int)hipGetLastError();
+}
+
 extern "C" int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp, const float* advantages,
                                     const int64_t* lengths, const float* loss_mask, int64_t n_seq,
                                     int64_t seq_stride, int64_t n_tok, const unirl_ratio_loss_params* params,
@@ -778,44 +879,30 @@ extern "C" int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp
   A.loss_elem = loss_per_elem;
   A.metrics = metrics;
   A.partials = ws_partials(workspace);
-  RatioShape S;
-  plan(A, false, S);
-  if ((int64_t)S.grid.x * S.grid.y * kRlVals > kPartialCapacity) return UNIRL_E_LIMIT;
-  hipStream_t st = (hipStream_t)stream;
-  dim3 block(kRlThreads);
-  const bool packed = (A.layout == LAYOUT_PACKED);
-  // 16-byte vectors: mask / per-token-advantage switches compiled in; scalar tokens: read at run time
-  const int flags = (A.mask ? 1 : 0) | (A.C.adv_per_token ? 2 : 0);
-#define UNIRL_LAUNCH_FWD3(KIND, VEC, FLAGS)                                                              \
-  do {                                                                                                   \
-    if (packed)                                                                                          \
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, true, FLAGS>), S.grid, block, 0, st, A);      \
-    else                                                                                                 \
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, false, FLAGS>), S.grid, block, 0, st, A);     \
-  } while (0)
-#define UNIRL_LAUNCH_FWD(KIND)                                                                           \
-  do {                                                                                                   \
-    if (S.vec != 4) UNIRL_LAUNCH_FWD3(KIND, 1, -1);                                                      \
-    else if (flags == 0) UNIRL_LAUNCH_FWD3(KIND, 4, 0);                                                  \
-    else if (flags == 1) UNIRL_LAUNCH_FWD3(KIND, 4, 1);                                                  \
-    else if (flags == 2) UNIRL_LAUNCH_FWD3(KIND, 4, 2);                                                  \
-    else UNIRL_LAUNCH_FWD3(KIND, 4, 3);                                                                  \
-  } while (0)
-  const int64_t dbg = tune_int("UNIRL_DBG_ONLY", 0);
-  if (dbg != 2) {
-  if (A.C.kind == UNIRL_LOSS_GRPO) UNIRL_LAUNCH_FWD(UNIRL_LOSS_GRPO); else UNIRL_LAUNCH_FWD(UNIRL_LOSS_DRPO);
-  }
-#undef UNIRL_LAUNCH_FWD3
-#undef UNIRL_LAUNCH_FWD
-  const int launch_rc = (int)hipGetLastError();
-  if (launch_rc != 0) return launch_rc;
-  if (dbg == 1) return 0;
-  const unsigned int nblk = S.grid.x * S.grid.y;
-  if (nblk <= 512)
-    hipLaunchKernelGGL(ratio_loss_finalize_kernel<256>, dim3(1), dim3(256), 0, st, A, nblk);
-  else
-    hipLaunchKernelGGL(ratio_loss_finalize_kernel<1024>, dim3(1), dim3(1024), 0, st, A, nblk);
-  return (int)hipGetLastError();
+  return launch_forward(A, (hipStream_t)stream);
+}
+
+extern "C" int unirl_ratio_loss_fwd_bwd(const float* new_logp, const float* old_logp, const float* advantages,
+                                        const int64_t* lengths, const float* loss_mask, int64_t n_seq,
+                                        int64_t seq_stride, int64_t n_tok, const unirl_ratio_loss_params* params,
+                                        float loss_scale, int64_t n_valid, float* grad_new, float* metrics,
+                                        void* workspace, size_t workspace_bytes, void* stream) {
+  RatioArgs A = {};
+  const int rc = check_common(new_logp, old_logp, advantages, lengths, n_seq, seq_stride, n_tok, params, A);
+  if (rc != 0) return rc;
+  if (!metrics || !grad_new) return UNIRL_E_NULL;
+  if (!aligned_to(grad_new, 4)) return UNIRL_E_ALIGN;
+  if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
+  if (n_tok == 0) return UNIRL_OK;
+  A.mask = loss_mask;
+  A.metrics = metrics;
+  A.partials = ws_partials(workspace);
+  A.grad_new = grad_new;
+  A.loss_scale = loss_scale;
+  // the token-mean denominator counts every valid token (masked ones too): all tokens outside
+  // the padded layout; in the padded layout the caller's count, or the kernel sums the lengths
+  A.n_valid_host = (A.layout == LAYOUT_PADDED) ? n_valid : n_tok;
+  return launch_forward(A, (hipStream_t)stream);
 }
 
 extern "C" int unirl_ratio_loss_bwd(const float* new_logp, const float* old_logp, const float* advantages,

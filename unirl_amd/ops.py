@@ -680,12 +680,15 @@ class RatioLossPlan:
         self.seq = None
         self.n_seq = 0
         self.seq_stride = 0
+        self.n_valid_host = -1  # padded layout: valid-token count when known without a device sync
         if lengths is not None and cu_seqlens is not None:
             raise ValueError("pass lengths (padded layout) or cu_seqlens (packed layout), not both")
         if lengths is not None:
             if new_logp.dim() != 2:
                 raise ValueError("the padded layout needs [n_seq, max_len] log-probs")
             self.n_seq, self.seq_stride = self.shape
+            if lengths.device.type == "cpu":  # the token count is free on the host
+                self.n_valid_host = int(lengths.detach().reshape(-1).clamp(0, self.seq_stride).sum())
             self.seq = lengths.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
             if self.seq.numel() != self.n_seq:
                 raise ValueError(f"lengths has {self.seq.numel()} entries for {self.n_seq} sequences")
@@ -733,6 +736,27 @@ class RatioLossPlan:
             )
         N.check(rc, "unirl_ratio_loss_fwd")
         return elem, metrics
+
+    def forward_backward(self, loss_scale: float) -> Tuple[torch.Tensor, torch.Tensor]:
+        """One pass for a whole training micro-step: ``(grad_new f32, metrics [16] f32)`` with
+        ``grad_new`` = what ``(loss * loss_scale).backward()`` leaves in ``new_logp.grad``."""
+        device = self.device
+        metrics = torch.empty(N.M_COUNT, dtype=torch.float32, device=device)
+        grad = torch.empty(self.shape, dtype=torch.float32, device=device)
+        if self.n_tok == 0:
+            metrics.fill_(float("nan"))
+            metrics[N.M_NUM_TOKENS] = 0.0
+            return grad, metrics
+        stream = N.current_stream(device)
+        ws, ws_bytes = N.workspace(device, stream)
+        with N.on_device(device):
+            rc = N.lib().unirl_ratio_loss_fwd_bwd(
+                N.ptr(self.nw), N.ptr(self.od), N.ptr(self.adv), N.ptr(self.seq), N.ptr(self.mask), self.n_seq,
+                self.seq_stride, self.n_tok, ctypes.byref(self.params), float(loss_scale), int(self.n_valid_host),
+                N.ptr(grad), N.ptr(metrics), N.ptr(ws), ws_bytes, stream,
+            )
+        N.check(rc, "unirl_ratio_loss_fwd_bwd")
+        return grad, metrics
 
     def backward(
         self,
