@@ -153,7 +153,7 @@ def make_shapes(torch, dev):
     prev_host = osde.sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7, noise=host1[2],
                                  sigma_max=sig[1])[0]
     prev1 = [prev_host.to(dev) + 0.0 * k for k in range(ns)]
-    bytes1r = 5 * numel * 4
+    bytes1r = 4 * numel * 4  # reads noise_pred, sample, prev_sample; writes the mean
 
     def run1r(i):
         x, v, _ = sets1[i % ns]
@@ -162,8 +162,8 @@ def make_shapes(torch, dev):
 
     shapes.append(dict(
         name="sde_step_logp_replay", config=1,
-        shape="fp32 [8,16,128,128], step 10/28, replay of a stored transition (4 reads, 1 write)",
-        bytes=bytes1r, read_bytes=4 * numel * 4, write_bytes=numel * 4, elements=numel, run=run1r, sets=ns,
+        shape="fp32 [8,16,128,128], step 10/28, replay of a stored transition (3 reads, 1 write)",
+        bytes=bytes1r, read_bytes=3 * numel * 4, write_bytes=numel * 4, elements=numel, run=run1r, sets=ns,
         cpu=lambda: osde.sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7,
                                      prev_sample=prev_host, sigma_max=sig[1]),
         cpu_bytes=bytes1r,
