@@ -189,3 +189,62 @@ def test_config2_full_shape(dev):
     # determinism
     lp2, ent2 = models.token_logp_entropy(x, ids, 1.0)
     assert torch.equal(lp, lp2) and torch.equal(ent, ent2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_chunked_replay_recomputes_logits_in_backward(dev, dtype):
+    """Training path of the chunked replay: the chunk's logits are dropped after the forward and
+    rebuilt in the backward (the reference's per-chunk checkpoint).  Gradients of the hidden states
+    and of the head's weight and bias against autograd through the reference's chunk function."""
+    from unirl_amd import models
+
+    g = torch.Generator().manual_seed(11)
+    B, T_max, H, V, T = 3, 150, 32, 1000, 0.7
+    hidden = torch.randn(B, T_max, H, generator=g)
+    toks = torch.randint(0, V, (B, T_max), generator=g)
+    upstream = torch.randn(B, T_max, generator=g)
+    head = torch.nn.Linear(H, V)
+    with torch.no_grad():
+        head.weight.copy_(0.2 * torch.randn(V, H, generator=g))
+        head.bias.copy_(0.1 * torch.randn(V, generator=g))
+
+    # reference chunk function (qwen3/ar.py:82-85) on the CPU, fp32
+    h_ref = hidden.clone().requires_grad_(True)
+    lf = head(h_ref).float() / T
+    ref = lf.gather(-1, toks.unsqueeze(-1)).squeeze(-1) - torch.logsumexp(lf, dim=-1)
+    (ref * upstream).sum().backward()
+    ref_grads = (h_ref.grad.clone(), head.weight.grad.clone(), head.bias.grad.clone())
+    head.zero_grad()
+
+    def run(keep):
+        hd = torch.nn.Linear(H, V).to(dev).to(dtype)
+        with torch.no_grad():
+            hd.weight.copy_(head.weight.to(dtype))
+            hd.bias.copy_(head.bias.to(dtype))
+        h = hidden.to(dev).to(dtype).requires_grad_(True)
+        out = models.chunked_replay_logp(hd, h, toks.to(dev), temperature=T, chunk=64, keep_logits=keep)
+        (out * upstream.to(dev)).sum().backward()
+        return out.detach().cpu(), (h.grad.float().cpu(), hd.weight.grad.float().cpu(), hd.bias.grad.float().cpu())
+
+    out_r, grads_r = run(False)
+    out_k, grads_k = run(True)
+    # dropping the logits changes nothing: same kernels on the same recomputed values
+    assert torch.equal(out_r, out_k)
+    for a, b in zip(grads_r, grads_k):
+        assert torch.equal(a, b)
+    if dtype == torch.float32:
+        assert_close(out_r, ref.detach(), 1e-5, 2e-5, "log-probs")  # the GEMMs differ in summation order
+        for name, a, b in zip(("hidden", "weight", "bias"), grads_r, ref_grads):
+            assert_close(a, b, 1e-4, 1e-5 * float(b.abs().max()), f"{name} grad")
+    else:
+        for name, a, b in zip(("hidden", "weight", "bias"), grads_r, ref_grads):
+            assert_close(a, b, 5e-2, 2e-2 * float(b.abs().max()), f"{name} grad (bf16 head)")
+
+    # hidden states without grad, head parameters with: still the recomputing path, same result
+    hd = torch.nn.Linear(H, V).to(dev)
+    with torch.no_grad():
+        hd.weight.copy_(head.weight)
+        hd.bias.copy_(head.bias)
+    out = models.chunked_replay_logp(hd, hidden.to(dev), toks.to(dev), temperature=T, chunk=64)
+    (out * upstream.to(dev)).sum().backward()
+    assert_close(hd.weight.grad.cpu(), ref_grads[1], 1e-4, 1e-5 * float(ref_grads[1].abs().max()), "weight grad only")

@@ -41,6 +41,50 @@ class _TokenLogpFn(torch.autograd.Function):
         return ops.token_logp_bwd(logits, tokens, ctx.temperature, lse, g_logp), None, None
 
 
+class _RecomputedChunkFn(torch.autograd.Function):
+    """Log-probs of one chunk whose ``[B, chunk, V]`` logits are not kept for the backward.
+
+    The reference wraps each chunk in ``torch.utils.checkpoint`` (``qwen3/ar.py:93-96``): the
+    backward runs ``lm_head`` again and then the whole log-softmax forward and backward.  Here
+    the forward keeps the per-token log-sum-exp (4 bytes a token), so the backward runs
+    ``lm_head`` again and goes straight to the gradient kernel -- the recomputed logits are
+    read once instead of twice -- and, for a plain ``nn.Linear`` head, the gradient overwrites
+    the logits buffer.
+    """
+
+    @staticmethod
+    def forward(ctx, hidden: torch.Tensor, tokens: torch.Tensor, lm_head, temperature: float, *params):
+        del params  # listed only so autograd sees the head's parameters as inputs of this node
+        ctx.autocast = (torch.is_autocast_enabled("cuda"), torch.get_autocast_dtype("cuda"))
+        with torch.no_grad():
+            logits = lm_head(hidden)
+            logp, _, lse = ops.token_logp_entropy(
+                logits, tokens, temperature, want_logp=True, want_entropy=False, want_lse=True
+            )
+        ctx.save_for_backward(hidden, tokens, lse)
+        ctx.lm_head, ctx.temperature = lm_head, temperature
+        return logp
+
+    @staticmethod
+    def backward(ctx, g_logp):
+        hidden, tokens, lse = ctx.saved_tensors
+        enabled, dtype = ctx.autocast
+        h = hidden.detach().requires_grad_(hidden.requires_grad)
+        with torch.enable_grad(), torch.autocast("cuda", dtype=dtype, enabled=enabled):
+            logits = ctx.lm_head(h)
+        plain = isinstance(ctx.lm_head, torch.nn.Linear) and logits.is_contiguous()
+        d_logits = ops.token_logp_bwd(
+            logits.detach(), tokens, ctx.temperature, lse, g_logp, in_place=plain and logits.dtype in _KERNEL_DTYPES
+        )
+        # parameter gradients accumulate into .grad here, as under a re-entrant checkpoint
+        torch.autograd.backward(logits, d_logits)
+        n_params = len(ctx.needs_input_grad) - 4
+        return (h.grad, None, None, None) + (None,) * n_params
+
+
+_KERNEL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+
+
 def token_logp(logits: torch.Tensor, tokens: torch.Tensor, temperature: float = 1.0) -> torch.Tensor:
     """fp32 ``log_softmax(logits.float() / T)[..., tokens]`` with shape ``logits.shape[:-1]``.
 
@@ -83,21 +127,36 @@ def chunked_replay_logp(
     response_tokens: torch.Tensor,
     temperature: float = 1.0,
     chunk: Optional[int] = None,
+    keep_logits: bool = False,
 ) -> torch.Tensor:
     """Padded ``[B, T_max]`` fp32 log-probs of ``response_tokens`` under ``lm_head(resp_hidden)``.
 
     Same chunking rule as the reference (``chunk = max(64, 2048 // B)``), so the
     ``[B, chunk, V]`` logits block -- the only large transient -- stays bounded; each
-    block is consumed by the fused kernel in the dtype ``lm_head`` produced.
+    block is consumed by the fused kernel in the dtype ``lm_head`` produced.  Under autograd
+    the logits of a chunk are dropped and recomputed in the backward, like the reference's
+    per-chunk checkpoint (``keep_logits=True`` keeps them instead: no second ``lm_head``
+    pass, ``B * T_max * V`` elements of memory).  The recomputing path is taken when
+    ``resp_hidden`` or a parameter of an ``nn.Module`` head requires grad; a bare callable whose
+    captured weights alone require grad keeps its logits.
     """
     bsz, t_max = int(resp_hidden.size(0)), int(response_tokens.size(1))
     if t_max == 0:
         return resp_hidden.new_zeros((bsz, 0), dtype=torch.float32)
     step = int(chunk) if chunk is not None else max(64, 2048 // max(1, bsz))
+    T = float(temperature) if float(temperature) > 0.0 else 1.0
+    params = tuple(lm_head.parameters()) if isinstance(lm_head, torch.nn.Module) else ()
+    recompute = (
+        not keep_logits and torch.is_grad_enabled()
+        and (resp_hidden.requires_grad or any(p.requires_grad for p in params))
+    )
     parts: List[torch.Tensor] = []
     for s in range(0, t_max, step):
-        logits = lm_head(resp_hidden[:, s : s + step, :])
-        parts.append(token_logp(logits, response_tokens[:, s : s + step], temperature))
+        h, tok = resp_hidden[:, s : s + step, :], response_tokens[:, s : s + step]
+        if recompute:
+            parts.append(_RecomputedChunkFn.apply(h, tok, lm_head, T, *params))
+        else:
+            parts.append(token_logp(lm_head(h), tok, temperature))
     return torch.cat(parts, dim=1)
 
 

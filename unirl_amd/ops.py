@@ -594,9 +594,14 @@ def token_logp_entropy(
 
 
 def token_logp_bwd(
-    logits: torch.Tensor, ids: torch.Tensor, temperature: float, lse: torch.Tensor, g_logp: torch.Tensor
+    logits: torch.Tensor, ids: torch.Tensor, temperature: float, lse: torch.Tensor, g_logp: torch.Tensor,
+    *, in_place: bool = False,
 ) -> torch.Tensor:
-    """``d logp / d logits`` contracted with ``g_logp``, in the dtype of ``logits``."""
+    """``d logp / d logits`` contracted with ``g_logp``, in the dtype of ``logits``.
+
+    ``in_place`` overwrites ``logits`` with its gradient (every element is read and written by
+    the same lane, so no second ``[rows, V]`` buffer is needed); it needs contiguous logits in a
+    dtype the kernel reads directly."""
     N.require_device(logits, "logits")
     device = logits.device
     V = logits.shape[-1]
@@ -611,7 +616,12 @@ def token_logp_bwd(
     idc = ids.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
     lsec = lse.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
     gc = g_logp.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
-    grad = torch.empty_like(x2)
+    if in_place:
+        if x2.data_ptr() != logits.data_ptr() or x2.dtype != orig_dtype:
+            raise ValueError("token_logp_bwd(in_place=True) needs contiguous bf16 / fp16 / fp32 logits")
+        grad = x2
+    else:
+        grad = torch.empty_like(x2)
     if rows and V:
         with N.on_device(device):
             rc = N.lib().unirl_token_logp_bwd(
