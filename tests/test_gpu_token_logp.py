@@ -121,6 +121,13 @@ def test_backward_matches_autograd_of_oracle(dev, dtype, T):
     assert xg.grad.dtype == dtype and xg.grad.shape == x.shape
     tol = 1e-5 if dtype == torch.float32 else 1e-2
     assert_close(xg.grad.float(), xr.grad.float(), tol, tol * float(xr.grad.float().abs().max()) * 0.1, "grad")
+    # log-prob with the entropy beside it: one pass, same gradient, entropy detached
+    xe = x.to(dev).requires_grad_(True)
+    lp, ent = models.token_logp_entropy(xe, ids.to(dev), T)
+    assert not ent.requires_grad and lp.requires_grad
+    (lp * g.to(dev)).sum().backward()
+    assert torch.equal(xe.grad, xg.grad)
+    assert torch.equal(ent, models.token_entropy(x.to(dev), T))
 
 
 def test_chunked_replay_matches_reference_chunk_loop(dev):

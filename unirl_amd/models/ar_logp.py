@@ -26,19 +26,24 @@ from .. import ops
 
 
 class _TokenLogpFn(torch.autograd.Function):
+    """Log-prob (differentiable) and, on request, entropy (detached) from one pass over the logits."""
+
     @staticmethod
-    def forward(ctx, logits: torch.Tensor, tokens: torch.Tensor, temperature: float):
-        logp, _, lse = ops.token_logp_entropy(
-            logits, tokens, temperature, want_logp=True, want_entropy=False, want_lse=True
+    def forward(ctx, logits: torch.Tensor, tokens: torch.Tensor, temperature: float, want_entropy: bool):
+        logp, ent, lse = ops.token_logp_entropy(
+            logits, tokens, temperature, want_logp=True, want_entropy=want_entropy, want_lse=True
         )
         ctx.save_for_backward(logits, tokens, lse)
         ctx.temperature = temperature
-        return logp
+        if not want_entropy:
+            return logp
+        ctx.mark_non_differentiable(ent)
+        return logp, ent
 
     @staticmethod
-    def backward(ctx, g_logp):
+    def backward(ctx, g_logp, *_g_entropy):
         logits, tokens, lse = ctx.saved_tensors
-        return ops.token_logp_bwd(logits, tokens, ctx.temperature, lse, g_logp), None, None
+        return ops.token_logp_bwd(logits, tokens, ctx.temperature, lse, g_logp), None, None, None
 
 
 class _RecomputedChunkFn(torch.autograd.Function):
@@ -93,7 +98,7 @@ def token_logp(logits: torch.Tensor, tokens: torch.Tensor, temperature: float = 
     """
     T = float(temperature) if float(temperature) > 0.0 else 1.0
     if torch.is_grad_enabled() and logits.requires_grad:
-        return _TokenLogpFn.apply(logits, tokens, T)
+        return _TokenLogpFn.apply(logits, tokens, T, False)
     logp, _, _ = ops.token_logp_entropy(logits, tokens, T, want_logp=True, want_entropy=False)
     return logp
 
@@ -107,9 +112,7 @@ def token_logp_entropy(
     """
     T = float(temperature) if float(temperature) > 0.0 else 1.0
     if torch.is_grad_enabled() and logits.requires_grad:
-        logp = _TokenLogpFn.apply(logits, tokens, T)
-        _, ent, _ = ops.token_logp_entropy(logits, None, T, want_logp=False, want_entropy=True)
-        return logp, ent
+        return _TokenLogpFn.apply(logits, tokens, T, True)
     logp, ent, _ = ops.token_logp_entropy(logits, tokens, T, want_logp=True, want_entropy=True)
     return logp, ent
 
