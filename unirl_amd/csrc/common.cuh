@@ -137,6 +137,34 @@ struct Vec<float, 4> {
     stream_store16(p, v);
   }
 };
+// eight floats: two 16-byte accesses (the pointer needs 16-byte alignment only)
+template <>
+struct Vec<float, 8> {
+  static __device__ __forceinline__ void load(const float* p, float (&o)[8]) {
+    const u32x4 a = stream_load16(p), b = stream_load16(p + 4);
+    o[0] = __uint_as_float(a.x);
+    o[1] = __uint_as_float(a.y);
+    o[2] = __uint_as_float(a.z);
+    o[3] = __uint_as_float(a.w);
+    o[4] = __uint_as_float(b.x);
+    o[5] = __uint_as_float(b.y);
+    o[6] = __uint_as_float(b.z);
+    o[7] = __uint_as_float(b.w);
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&o)[8]) {
+    u32x4 a, b;
+    a.x = __float_as_uint(o[0]);
+    a.y = __float_as_uint(o[1]);
+    a.z = __float_as_uint(o[2]);
+    a.w = __float_as_uint(o[3]);
+    b.x = __float_as_uint(o[4]);
+    b.y = __float_as_uint(o[5]);
+    b.z = __float_as_uint(o[6]);
+    b.w = __float_as_uint(o[7]);
+    stream_store16(p, a);
+    stream_store16(p + 4, b);
+  }
+};
 template <>
 struct Vec<float, 1> {
   static __device__ __forceinline__ void load(const float* p, float (&o)[1]) { o[0] = *p; }
@@ -171,6 +199,14 @@ struct Vec<bf16_t, 8> {
     o[5] = __uint_as_float(v.z & 0xffff0000u);
     o[6] = __uint_as_float(v.w << 16);
     o[7] = __uint_as_float(v.w & 0xffff0000u);
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&o)[8]) {
+    u32x4 v;
+    v.x = f32x2_to_bf16x2_bits(o[0], o[1]);
+    v.y = f32x2_to_bf16x2_bits(o[2], o[3]);
+    v.z = f32x2_to_bf16x2_bits(o[4], o[5]);
+    v.w = f32x2_to_bf16x2_bits(o[6], o[7]);
+    stream_store16(p, v);
   }
 };
 template <>
@@ -207,6 +243,14 @@ struct Vec<f16_t, 8> {
     o[5] = f16_bits_to_f32(v.z >> 16);
     o[6] = f16_bits_to_f32(v.w & 0xffffu);
     o[7] = f16_bits_to_f32(v.w >> 16);
+  }
+  static __device__ __forceinline__ void store(f16_t* p, const float (&o)[8]) {
+    u32x4 v;
+    v.x = f32_to_f16_bits(o[0]) | (f32_to_f16_bits(o[1]) << 16);
+    v.y = f32_to_f16_bits(o[2]) | (f32_to_f16_bits(o[3]) << 16);
+    v.z = f32_to_f16_bits(o[4]) | (f32_to_f16_bits(o[5]) << 16);
+    v.w = f32_to_f16_bits(o[6]) | (f32_to_f16_bits(o[7]) << 16);
+    stream_store16(p, v);
   }
 };
 template <>

@@ -511,7 +511,13 @@ template <typename TV, typename TX, bool SAMPLING>
 static int launch_step(const SdeStepArgs& A, int64_t B, int vec, hipStream_t st) {
   const int items = A.items;
   dim3 grid(A.nblk, (unsigned int)B), block(kSdeThreads);
-  if (vec == 4) {
+  if (vec == 8) {
+    // sixteen-byte accesses on the 16-bit operands; only built where there is one
+    if constexpr (sizeof(TV) == 2 || sizeof(TX) == 2)
+      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 8, 2, SAMPLING>), grid, block, 0, st, A);
+    else
+      return UNIRL_E_DTYPE;
+  } else if (vec == 4) {
     if (items >= 4)
       hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 4, SAMPLING>), grid, block, 0, st, A);
     else if (items >= 2)
@@ -644,7 +650,28 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
       (sampling && d->noise && stride_n % 4) || (d->prev_out && stride_po % 4) || (d->mean_out && stride_mo % 4))
     vec = 1;
 
-  const int items = (vec == 4) ? (int)tune_int("UNIRL_SDE_ITEMS", 4) : 2;
+  // 16-bit operands: eight elements per lane make their accesses sixteen bytes too, while an
+  // fp32 operand then takes two accesses that each cover only half of every cache line, which
+  // costs more than it gains once fp32 traffic dominates (sampling with fp32 noise and outputs:
+  // 55 -> 61 us at [8, 2M]; replay of bf16 tensors: 45 -> 38 us).  So: eight when the 16-bit
+  // tensors carry at least as many bytes as the fp32 ones, and every base and sample stride of a
+  // 16-bit tensor sits on a 16-byte boundary.
+  if (vec == 4 && (sv == 2 || sx == 2) && tune_int("UNIRL_SDE_VEC8", 1) == 1) {
+    size_t narrow = 0, wide = 0;
+    bool ok = (D % 8 == 0);
+    auto visit = [&](const void* p, size_t es, int64_t stride) {
+      if (!p) return;
+      (es == 2 ? narrow : wide) += es;
+      ok = ok && aligned_to(p, 16) && (es == 4 || stride % 8 == 0);
+    };
+    visit(noise_pred, sv, stride_v);
+    visit(sample, sx, stride_x);
+    if (sampling) visit(d->noise, 4, stride_n); else visit(prev_sample, sx, stride_p);
+    visit(d->prev_out, spo, stride_po);
+    visit(d->mean_out, smo, stride_mo);
+    if (ok && narrow >= wide) vec = 8;
+  }
+  const int items = (vec == 8) ? 2 : (vec == 4) ? (int)tune_int("UNIRL_SDE_ITEMS", 4) : 2;
   const unsigned int nblk = sde_blocks_per_sample(D / vec, items, B);
   const int64_t per_launch = sde_samples_per_launch(B, nblk);
   hipStream_t st = (hipStream_t)stream;
