@@ -149,14 +149,17 @@ int unirl_sde_step_logp_ex(const struct unirl_sde_step_desc* desc /* host */, vo
  * the autograd graph the reference builds through kernels.py:225-228 and
  * :200-204 (prev_sample is detached there).  Inputs as in the forward call;
  * g_logp [B] f32 (NULL = 0), g_mean [B,D] f32 (NULL = 0), g_prev [B,D] f32
- * (sampling only, NULL = 0).  Outputs grad_v / grad_x are f32 [B,D], either
- * may be NULL. */
+ * (sampling only, NULL = 0).  Outputs grad_v / grad_x are [B,D] in the dtype
+ * given for each (autograd hands a gradient back in its input's dtype, so a
+ * bf16 noise_pred takes a bf16 gradient without a cast pass); either may be
+ * NULL. */
 int unirl_sde_step_logp_bwd(const void* noise_pred, int dtype_v, const void* sample, int dtype_x,
                             const void* prev_sample, const float* noise, const float* sigma,
                             const float* sigma_next, int sigma_stride, const float* sigma_max_ptr,
                             float sigma_max_val, double eta, int kind, int64_t B, int64_t D,
                             const float* g_logp, const float* g_mean, const float* g_prev,
-                            int logp_sum, float* grad_v, float* grad_x, void* stream);
+                            int logp_sum, void* grad_v, int dtype_gv, void* grad_x, int dtype_gx,
+                            void* stream);
 
 /* ------------------------------------------------------------------------
  * S chained SDE transitions with the latent held in registers: the loop of

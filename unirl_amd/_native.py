@@ -107,7 +107,8 @@ _SIGNATURES = {
     "unirl_sde_step_logp_bwd": (
         c_int,
         [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,
-         c_double, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p],
+         c_double, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int, c_void_p, c_int,
+         c_void_p],
     ),
     "unirl_sde_rollout_logp": (
         c_int,

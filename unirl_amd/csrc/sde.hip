@@ -267,8 +267,9 @@ struct SdeBwdArgs {
   const float* g_logp;
   const float* g_mean;
   const float* g_prev;
-  float* grad_v;
-  float* grad_x;
+  void* grad_v;
+  void* grad_x;
+  int dtype_gv, dtype_gx;  // unirl_dtype of the two outputs
 };
 
 template <typename TV, typename TX, int VEC, bool SAMPLING>
@@ -287,8 +288,9 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_bwd_kernel(SdeBwdArgs A)
   const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + b * D : nullptr;
   const float* __restrict__ gm = A.g_mean ? A.g_mean + b * D : nullptr;
   const float* __restrict__ gp = A.g_prev ? A.g_prev + b * D : nullptr;
-  float* __restrict__ gv = A.grad_v ? A.grad_v + b * D : nullptr;
-  float* __restrict__ gx = A.grad_x ? A.grad_x + b * D : nullptr;
+  void* const gv = A.grad_v;
+  void* const gx = A.grad_x;
+  const int dgv = A.dtype_gv, dgx = A.dtype_gx;
 
   float dmean_dv, dmean_dx, k_lp;
   const float glp = A.g_logp ? A.g_logp[b] : 0.0f;
@@ -328,8 +330,8 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_bwd_kernel(SdeBwdArgs A)
       ov[k] = g * dmean_dv;
       ox[k] = g * dmean_dx;
     }
-    if (gv) Vec<float, VEC>::store(gv + i * VEC, ov);
-    if (gx) Vec<float, VEC>::store(gx + i * VEC, ox);
+    if (gv) sde_store_as<VEC>(gv, dgv, b * D + i * VEC, ov);
+    if (gx) sde_store_as<VEC>(gx, dgx, b * D + i * VEC, ox);
   }
 }
 
@@ -550,10 +552,16 @@ static int launch_bwd(const SdeBwdArgs& A, int64_t B, int vec, hipStream_t st) {
   const int64_t nvec = A.D / vec;
   const unsigned int nblk = sde_blocks_per_sample(nvec, 1, B);
   dim3 grid(nblk, (unsigned int)B), block(kSdeThreads);
-  if (vec == 4)
+  if (vec == 8) {
+    if constexpr (sizeof(TV) == 2 || sizeof(TX) == 2)
+      hipLaunchKernelGGL((sde_step_bwd_kernel<TV, TX, 8, SAMPLING>), grid, block, 0, st, A);
+    else
+      return UNIRL_E_DTYPE;
+  } else if (vec == 4) {
     hipLaunchKernelGGL((sde_step_bwd_kernel<TV, TX, 4, SAMPLING>), grid, block, 0, st, A);
-  else
+  } else {
     hipLaunchKernelGGL((sde_step_bwd_kernel<TV, TX, 1, SAMPLING>), grid, block, 0, st, A);
+  }
   return (int)hipGetLastError();
 }
 
@@ -758,8 +766,10 @@ extern "C" int unirl_sde_step_logp_bwd(const void* noise_pred, int dtype_v, cons
                                        const float* sigma_next, int sigma_stride, const float* sigma_max_ptr,
                                        float sigma_max_val, double eta, int kind, int64_t B, int64_t D,
                                        const float* g_logp, const float* g_mean, const float* g_prev,
-                                       int logp_sum, float* grad_v, float* grad_x, void* stream) {
+                                       int logp_sum, void* grad_v, int dtype_gv, void* grad_x, int dtype_gx,
+                                       void* stream) {
   if (!dtype_ok(dtype_v) || !dtype_ok(dtype_x)) return UNIRL_E_DTYPE;
+  if ((grad_v && !dtype_ok(dtype_gv)) || (grad_x && !dtype_ok(dtype_gx))) return UNIRL_E_DTYPE;
   if (kind < UNIRL_SDE_FLOW || kind > UNIRL_SDE_CPS) return UNIRL_E_DTYPE;
   if (B < 0 || D <= 0 || (sigma_stride != 0 && sigma_stride != 1)) return UNIRL_E_SHAPE;
   if (B == 0) return UNIRL_OK;
@@ -767,15 +777,35 @@ extern "C" int unirl_sde_step_logp_bwd(const void* noise_pred, int dtype_v, cons
   if (!grad_v && !grad_x) return UNIRL_OK;
   const bool sampling = (prev_sample == nullptr);
   const size_t sv = dtype_size(dtype_v), sx = dtype_size(dtype_x);
+  const size_t sgv = grad_v ? dtype_size(dtype_gv) : 4, sgx = grad_x ? dtype_size(dtype_gx) : 4;
   if (!aligned_to(noise_pred, sv) || !aligned_to(sample, sx) || !aligned_to(prev_sample, sx) ||
-      !aligned_to(noise, 4) || !aligned_to(g_mean, 4) || !aligned_to(g_prev, 4) || !aligned_to(grad_v, 4) ||
-      !aligned_to(grad_x, 4))
+      !aligned_to(noise, 4) || !aligned_to(g_mean, 4) || !aligned_to(g_prev, 4) || !aligned_to(grad_v, sgv) ||
+      !aligned_to(grad_x, sgx))
     return UNIRL_E_ALIGN;
   int vec = 4;
   if (D % 4 != 0 || !aligned_to(noise_pred, 4 * sv) || !aligned_to(sample, 4 * sx) ||
       !aligned_to(prev_sample, 4 * sx) || !aligned_to(noise, 16) || !aligned_to(g_mean, 16) ||
-      !aligned_to(g_prev, 16) || !aligned_to(grad_v, 16) || !aligned_to(grad_x, 16))
+      !aligned_to(g_prev, 16) || !aligned_to(grad_v, 4 * sgv) || !aligned_to(grad_x, 4 * sgx))
     vec = 1;
+  // eight elements per lane when the 16-bit tensors carry at least as many bytes as the fp32
+  // ones (same rule and reason as in the forward step)
+  if (vec == 4 && (sv == 2 || sx == 2) && D % 8 == 0 && tune_int("UNIRL_SDE_VEC8", 1) == 1) {
+    size_t narrow = 0, wide = 0;
+    bool ok = true;
+    auto visit = [&](const void* p, size_t es) {
+      if (!p) return;
+      (es == 2 ? narrow : wide) += es;
+      ok = ok && aligned_to(p, 16);
+    };
+    visit(noise_pred, sv);
+    visit(sample, sx);
+    if (sampling) visit(noise, 4); else visit(prev_sample, sx);
+    visit(g_mean, 4);
+    if (sampling) visit(g_prev, 4);
+    visit(grad_v, sgv);
+    visit(grad_x, sgx);
+    if (ok && narrow >= wide) vec = 8;
+  }
   hipStream_t st = (hipStream_t)stream;
   const int64_t per_launch = 32768;  // grid.y limit is 65535
   for (int64_t b0 = 0; b0 < B; b0 += per_launch) {
@@ -797,8 +827,10 @@ extern "C" int unirl_sde_step_logp_bwd(const void* noise_pred, int dtype_v, cons
     A.g_logp = (eta < 1e-7) ? nullptr : offset_f32(g_logp, b0);
     A.g_mean = offset_f32(g_mean, off);
     A.g_prev = offset_f32(g_prev, off);
-    A.grad_v = offset_f32(grad_v, off);
-    A.grad_x = offset_f32(grad_x, off);
+    A.grad_v = const_cast<void*>(offset_ptr(grad_v, off, sgv));
+    A.grad_x = const_cast<void*>(offset_ptr(grad_x, off, sgx));
+    A.dtype_gv = dtype_gv;
+    A.dtype_gx = dtype_gx;
     int rc = UNIRL_E_DTYPE;
     switch (dtype_v) {
       case UNIRL_F32: rc = launch_bwd_x<float>(A, dtype_x, nb, vec, sampling, st); break;

@@ -262,7 +262,8 @@ def sde_step_logp_bwd(
     need_grad_x: bool,
     logp_sum: bool = False,
 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
-    """Gradients of :func:`sde_step_logp` w.r.t. ``noise_pred`` and ``sample`` (f32)."""
+    """Gradients of :func:`sde_step_logp` w.r.t. ``noise_pred`` and ``sample``, each written by the
+    kernel in its tensor's own dtype (fp32 for dtypes the kernel does not read directly)."""
     device = sample.device
     v = _flat2(noise_pred.detach(), "noise_pred")
     x = _flat2(sample.detach(), "sample")
@@ -287,16 +288,18 @@ def sde_step_logp_bwd(
         return None if t is None else t.detach().to(device=device, dtype=torch.float32).contiguous()
 
     gl, gm, gp = f32c(g_logp), f32c(g_mean), f32c(g_prev)
-    grad_v = torch.empty(x.shape, dtype=torch.float32, device=device) if need_grad_v else None
-    grad_x = torch.empty(x.shape, dtype=torch.float32, device=device) if need_grad_x else None
+    grad_v = torch.empty(x.shape, dtype=v.dtype, device=device) if need_grad_v else None
+    grad_x = torch.empty(x.shape, dtype=x.dtype, device=device) if need_grad_x else None
     if B == 0 or D == 0 or (grad_v is None and grad_x is None):
         return grad_v, grad_x
+    if gl is None and gm is None and gp is None:  # nothing flows back
+        return (None if grad_v is None else grad_v.zero_()), (None if grad_x is None else grad_x.zero_())
     with N.on_device(device):
         rc = N.lib().unirl_sde_step_logp_bwd(
             N.ptr(v), N.dtype_code(v.dtype), N.ptr(x), N.dtype_code(x.dtype), N.ptr(prev_in), N.ptr(nz),
             N.ptr(sig), N.ptr(sig_n), stride, N.ptr(smax_t), smax_v, float(eta), SDE_KINDS[kind], B, D,
-            N.ptr(gl), N.ptr(gm), N.ptr(gp), int(bool(logp_sum)), N.ptr(grad_v), N.ptr(grad_x),
-            N.current_stream(device),
+            N.ptr(gl), N.ptr(gm), N.ptr(gp), int(bool(logp_sum)), N.ptr(grad_v), N.dtype_code(v.dtype),
+            N.ptr(grad_x), N.dtype_code(x.dtype), N.current_stream(device),
         )
     N.check(rc, "unirl_sde_step_logp_bwd")
     return grad_v, grad_x

@@ -41,6 +41,7 @@ class _SdeStepFn(torch.autograd.Function):
             noise_pred, sample, sigma, sigma_next, kind=kind, eta=eta, prev_sample=prev_sample, noise=noise,
             sigma_max=sigma_max,
         )
+        ctx.set_materialize_grads(False)  # an unused output hands back None, not a zero tensor to read
         ctx.kind, ctx.eta = kind, eta
         ctx.sampling = prev_sample is None
         ctx.has_logp = logp is not None
@@ -57,6 +58,8 @@ class _SdeStepFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g_prev, g_logp, g_mean):
         v, x, prev_sample, noise, sigma, sigma_next = ctx.saved
+        if g_prev is None and g_logp is None and g_mean is None:
+            return (None,) * 9
         grad_v, grad_x = ops.sde_step_logp_bwd(
             v, x, sigma, sigma_next, kind=ctx.kind, eta=ctx.eta, prev_sample=prev_sample, noise=noise,
             sigma_max=ctx.sigma_max, g_logp=g_logp if ctx.has_logp else None, g_mean=g_mean,
