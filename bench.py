@@ -236,6 +236,27 @@ def make_shapes(torch, dev):
         cpu=lambda: ofd.kl_per_sample(new_m, old_m, sig_t.reshape(1, 1, 1, 1, 1, 1)) < 0.01, cpu_bytes=bytes4,
     ))
 
+    # the loss step of Flow-DPPO around that kernel: KL, masks, loss, metrics and the gradient
+    new_lp = 1e-3 * torch.randn(2, 1, generator=g)
+    old_lp = new_lp + 2e-4 * torch.randn(2, 1, generator=g)
+    adv4 = torch.tensor([[1.0], [-1.0]])
+    lp_d = (new_lp.to(dev), old_lp.to(dev), adv4.to(dev))
+
+    def run4s(i):
+        p, q = sets4[i % ns4]
+        return ops.flowdppo_step(lp_d[0], lp_d[1], p, q, lp_d[2], sig_t_d, 0.01, loss_scale=1.0)
+
+    def cpu4s():
+        leaf = new_lp.clone().requires_grad_(True)
+        ofd.flowdppo_loss(leaf, old_lp, new_m, old_m, adv4, sig_t.reshape(1, 1, 1, 1, 1, 1), 0.01)[0].mean().backward()
+
+    shapes.append(dict(
+        name="flowdppo_step", config=4,
+        shape="bf16 [2,1,16,21,60,104] means + [2,1] log-probs: KL, masks, loss, 12 metrics, grad_new",
+        bytes=bytes4, read_bytes=bytes4, write_bytes=0, elements=old_m.numel(), run=run4s, sets=ns4,
+        cpu=cpu4s, cpu_bytes=bytes4,
+    ))
+
     # -- config 5: 10-step rollout, Qwen-Image packed latents fp32 [16,4096,64] -------------------
     g = torch.Generator().manual_seed(1005)
     shp5 = (16, 4096, 64)

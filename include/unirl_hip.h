@@ -214,6 +214,21 @@ int unirl_flowdppo_loss(const float* new_logp, const float* old_logp, const floa
                         const float* kl, int64_t n, float threshold, float* loss_elem,
                         float* metrics, void* stream);
 
+/* unirl_gaussian_kl_mask and unirl_flowdppo_loss as one call of two launches for
+ * the loss step of FlowDPPO.compute_loss_and_backward (flowdppo.py:309-320):
+ * the streaming KL kernel, then one workgroup that adds its partials row by
+ * row and runs the [B,S'] problem on the result.  R = B*S' rows of D elements
+ * in p / q; new_logp, old_logp, advantages, kl_out, loss_elem are f32 [R].
+ * grad_new (NULL or f32 [R]) receives loss_scale * loss_elem / R, the gradient
+ * `(loss_elem.mean() * loss_scale).backward()` leaves in new_logp.  Limit:
+ * R <= 4096 (UNIRL_E_LIMIT beyond; use the two entry points above). */
+int unirl_flowdppo_step(const void* p, const void* q, int dtype, const float* sigma,
+                        int64_t n_sigma, int64_t R, int64_t D, const float* new_logp,
+                        const float* old_logp, const float* advantages, float threshold,
+                        float loss_scale, float* kl_out, float* loss_elem, float* grad_new,
+                        float* metrics /* [16] f32, as unirl_flowdppo_loss */, void* workspace,
+                        size_t workspace_bytes, void* stream);
+
 /* Element-wise form of the same quantity (flowdppo.py:51), f32 output [R,D]. */
 int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, const float* sigma,
                            int64_t n_sigma, int64_t R, int64_t D, float* out, void* stream);

@@ -113,6 +113,43 @@ def test_flowdppo_loss_matches_oracle(dev):
         assert 0.0 < float(m["masked_fraction"]) < 1.0
 
 
+@pytest.mark.parametrize("shape", [(8, 3, 4, 16, 16), (2, 1, 16, 21, 60, 104), (5, 7, 37), (64, 12, 8, 8)])
+def test_flowdppo_step_two_launches(dev, shape):
+    """The fused loss step (KL kernel + one finishing workgroup) against the oracle: KL, loss,
+    metrics, and the gradient of (loss.mean() * loss_scale); and bit for bit against the
+    separate entry points."""
+    from unirl_amd import ops
+
+    g = torch.Generator().manual_seed(sum(shape))
+    B, S = shape[:2]
+    loss_scale = 0.37
+    for dtype in (torch.bfloat16, torch.float32):
+        new_means, old_means = means(shape, 3, dtype, pert=0.02)
+        old_means[::2] = new_means[::2]
+        new_logp = 1e-3 * torch.randn(B, S, generator=g)
+        old_logp = new_logp + 2e-4 * torch.randn(B, S, generator=g)
+        adv = torch.randn(B, 1, generator=g).expand(B, S).clone()
+        steps = sorted(torch.randperm(14, generator=g)[:S].tolist())
+        sig_t = ofd.sigma_t(SIG, steps, 0.7).reshape(1, S, *([1] * (len(shape) - 2)))  # one per step
+        nr = new_logp.clone().requires_grad_(True)
+        ref_elem, ref_m = ofd.flowdppo_loss(nr, old_logp, new_means, old_means, adv, sig_t, 1e-3)
+        (ref_elem.mean() * loss_scale).backward()
+        dv = [t.to(dev) for t in (new_logp, old_logp, new_means, old_means, adv, sig_t)]
+        kl, elem, mvec, grad = ops.flowdppo_step(*dv, 1e-3, loss_scale=loss_scale)
+        assert_close(elem, ref_elem, FP32_RTOL, 1e-8, "loss")
+        assert_close(grad, nr.grad, FP32_RTOL, 1e-9, "grad")
+        vals = mvec.tolist()
+        for k, slot in ops.FLOWDPPO_METRIC_SLOTS.items():
+            if k != "loss_mean":
+                assert abs(vals[slot] - float(ref_m[k])) <= 1e-5 * abs(float(ref_m[k])) + 1e-7, (k, vals[slot], float(ref_m[k]))
+        # the separate entry points give the same bits
+        kl2, _ = ops.gaussian_kl_mask(dv[2], dv[3], dv[5], 1e-3, reduce_from_dim=2, want_mask=False)
+        elem2, mvec2 = ops.flowdppo_loss(dv[0], dv[1], dv[4], kl2, 1e-3)
+        assert torch.equal(kl, kl2) and torch.equal(elem, elem2) and torch.equal(mvec[:13], mvec2[:13])
+        _, _, _, none = ops.flowdppo_step(*dv, 1e-3)
+        assert none is None
+
+
 def test_flowdppo_truth_table(dev):
     from unirl_amd.algorithms import _flowdppo_kl_adv_loss
 

@@ -125,6 +125,11 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_float, c_void_p, c_void_p, c_void_p],
     ),
+    "unirl_flowdppo_step": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_float,
+         c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    ),
     "unirl_expand_per_seq": (
         c_int,
         [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p],

@@ -187,8 +187,18 @@ class FlowDPPO(SdeStepAlgorithm):
         sigma_t = self._compute_sigma_t(segment, steps, device=device)
         adv_b = advantages.detach().to(dtype=new_logp.dtype, device=device).reshape(-1, 1).expand_as(new_logp)
 
-        elem, mvec = self._loss_with_metrics(new_logp, old_logp, new_means, old_means, adv_b, sigma_t)
-        (elem.mean() * loss_scale).backward()
+        if new_logp.dim() == 2 and 0 < new_logp.numel() <= ops.FLOWDPPO_STEP_MAX_ROWS:
+            # KL, masks, loss, metrics and `(elem.mean() * loss_scale).backward()` in two launches
+            need_grad = torch.is_grad_enabled() and new_logp.requires_grad
+            _, _, mvec, grad = ops.flowdppo_step(
+                new_logp, old_logp, new_means, old_means, adv_b, sigma_t, self.kl_mask_threshold,
+                loss_scale=loss_scale if need_grad else None,
+            )
+            if need_grad:
+                new_logp.backward(grad if grad.dtype == new_logp.dtype else grad.to(new_logp.dtype))
+        else:
+            elem, mvec = self._loss_with_metrics(new_logp, old_logp, new_means, old_means, adv_b, sigma_t)
+            (elem.mean() * loss_scale).backward()
 
         vals = mvec.tolist()  # the step's only device-to-host copy
         slots = dict(ops.FLOWDPPO_METRIC_SLOTS)

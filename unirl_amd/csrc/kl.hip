@@ -30,6 +30,7 @@ struct KlArgs {
   uint8_t* mask;
   float* elem_out;
   double* partials;
+  int always_partials;  // store workgroup partials even when one workgroup covers a row
 };
 
 template <typename T>
@@ -80,7 +81,7 @@ __global__ __launch_bounds__(kKlThreads) void gaussian_kl_kernel(KlArgs A) {
   }
   const double part = block_sum<double>((double)acc, lds);
   if (threadIdx.x != 0) return;
-  if (gridDim.x == 1) {
+  if (gridDim.x == 1 && !A.always_partials) {
     kl_finish(A, row, part, kl_den(A, row));
   } else {
     A.partials[row * gridDim.x + blockIdx.x] = part;  // summed by gaussian_kl_finalize_kernel
@@ -228,73 +229,129 @@ struct DppoArgs {
   float threshold;
   float* loss_elem;
   float* metrics;
+  float* grad_new;  // NULL, or receives grad_scale * loss_elem (the gradient of grad_scale * n * mean)
+  float grad_scale;
 };
 
 enum { D_SR = 0, D_SR2, D_LD2, D_KL, D_LOSS, D_NKL, D_POS, D_NEG, D_RM, D_SUMS, D_RMIN = D_SUMS, D_RMAX, D_KLMAX, D_VALS };
 
-__global__ __launch_bounds__(kKlThreads) void flowdppo_loss_kernel(DppoArgs A) {
-  __shared__ double lds[kKlThreads / kWave];
-  __shared__ float ldsf[kKlThreads / kWave];
+struct DppoAcc {
   double acc[D_SUMS];
-#pragma unroll
-  for (int v = 0; v < D_SUMS; ++v) acc[v] = 0.0;
   float rmin = INFINITY, rmax = -INFINITY, klmax = -INFINITY;
-  for (int64_t i = threadIdx.x; i < A.n; i += kKlThreads) {
-    const float ld = A.nw[i] - A.od[i];
-    const float r = expf(ld);
-    const float a = A.adv[i];
-    const float kl = A.kl[i];
-    const bool low_kl = kl < A.threshold;
-    const bool pos = !low_kl && (r > 1.0f) && (a > 0.0f);
-    const bool neg = !low_kl && (r < 1.0f) && (a < 0.0f);
-    const bool rm = pos || neg;
-    const float loss = rm ? 0.0f : (-a) * r;
-    A.loss_elem[i] = loss;
-    acc[D_SR] += (double)r;
-    acc[D_SR2] += (double)r * (double)r;
-    acc[D_LD2] += (double)(0.5f * (ld * ld));
-    acc[D_KL] += (double)kl;
-    acc[D_LOSS] += (double)loss;
-    acc[D_NKL] += low_kl ? 0.0 : 1.0;
-    acc[D_POS] += pos ? 1.0 : 0.0;
-    acc[D_NEG] += neg ? 1.0 : 0.0;
-    acc[D_RM] += rm ? 1.0 : 0.0;
-    rmin = fminf(rmin, r);
-    rmax = fmaxf(rmax, r);
-    klmax = fmaxf(klmax, kl);
-  }
-  double tot[D_SUMS];
+  __device__ __forceinline__ DppoAcc() {
 #pragma unroll
-  for (int v = 0; v < D_SUMS; ++v) tot[v] = block_sum<double>(acc[v], lds);
-  rmin = block_min(rmin, ldsf);
-  rmax = block_max(rmax, ldsf);
-  klmax = block_max(klmax, ldsf);
-  if (threadIdx.x != 0) return;
+    for (int v = 0; v < D_SUMS; ++v) acc[v] = 0.0;
+  }
+};
+
+// Element i of the [B,S'] problem: ratio, the two removal masks, the kept loss (and its gradient).
+__device__ __forceinline__ void dppo_elem(const DppoArgs& A, int64_t i, float kl, DppoAcc& s) {
+  const float ld = A.nw[i] - A.od[i];
+  const float r = expf(ld);
+  const float a = A.adv[i];
+  const bool low_kl = kl < A.threshold;
+  const bool pos = !low_kl && (r > 1.0f) && (a > 0.0f);
+  const bool neg = !low_kl && (r < 1.0f) && (a < 0.0f);
+  const bool rm = pos || neg;
+  const float loss = rm ? 0.0f : (-a) * r;
+  A.loss_elem[i] = loss;
+  if (A.grad_new) A.grad_new[i] = A.grad_scale * loss;  // d(-a*exp(new-old))/dnew = the loss itself
+  s.acc[D_SR] += (double)r;
+  s.acc[D_SR2] += (double)r * (double)r;
+  s.acc[D_LD2] += (double)(0.5f * (ld * ld));
+  s.acc[D_KL] += (double)kl;
+  s.acc[D_LOSS] += (double)loss;
+  s.acc[D_NKL] += low_kl ? 0.0 : 1.0;
+  s.acc[D_POS] += pos ? 1.0 : 0.0;
+  s.acc[D_NEG] += neg ? 1.0 : 0.0;
+  s.acc[D_RM] += rm ? 1.0 : 0.0;
+  s.rmin = fminf(s.rmin, r);
+  s.rmax = fmaxf(s.rmax, r);
+  s.klmax = fmaxf(s.klmax, kl);
+}
+
+// The twelve metrics from the totals; one thread.
+__device__ __forceinline__ void dppo_metrics(const DppoArgs& A, const double (&tot)[D_SUMS], float rmin, float rmax,
+                                             float klmax) {
   const double N = (double)A.n;
+  // one reciprocal for every mean (x * (1/N) and x / N agree to an ulp of fp64, far below fp32)
+  const double inv_n = 1.0 / N;
   double var = 0.0;
   if (A.n > 1) {
-    var = (tot[D_SR2] - tot[D_SR] * tot[D_SR] / N) / (N - 1.0);
+    var = (tot[D_SR2] - tot[D_SR] * tot[D_SR] * inv_n) / (N - 1.0);
     if (var < 0.0) var = 0.0;
   }
   float* M = A.metrics;
-  const float nf = (float)A.n;
-  M[0] = (float)(tot[D_SR] / N);
+  M[0] = (float)(tot[D_SR] * inv_n);
   M[1] = (float)sqrt(var);
   // min()/max() of the reference return NaN when any element is NaN; ratios and KL values are
   // >= 0, so their sums are NaN exactly then
   const bool r_nan = tot[D_SR] != tot[D_SR], kl_nan = tot[D_KL] != tot[D_KL];
   M[2] = r_nan ? quiet_nan() : rmin;
   M[3] = r_nan ? quiet_nan() : rmax;
-  M[4] = (float)(tot[D_LD2] / N);
-  M[5] = (float)(tot[D_KL] / N);
+  M[4] = (float)(tot[D_LD2] * inv_n);
+  M[5] = (float)(tot[D_KL] * inv_n);
   M[6] = kl_nan ? quiet_nan() : klmax;
-  M[7] = (float)tot[D_NKL] / nf;
-  M[8] = (float)tot[D_POS] / nf;
-  M[9] = (float)tot[D_NEG] / nf;
-  M[10] = (float)tot[D_RM] / nf;
-  M[11] = (float)(N - tot[D_RM]) / nf;
-  M[12] = (float)(tot[D_LOSS] / N);
+  M[7] = (float)(tot[D_NKL] * inv_n);
+  M[8] = (float)(tot[D_POS] * inv_n);
+  M[9] = (float)(tot[D_NEG] * inv_n);
+  M[10] = (float)(tot[D_RM] * inv_n);
+  M[11] = (float)((N - tot[D_RM]) * inv_n);
+  M[12] = (float)(tot[D_LOSS] * inv_n);
   M[13] = M[14] = M[15] = 0.0f;
+}
+
+// The whole [B,S'] problem on one wavefront (it is a few dozen elements): no barriers, the
+// reductions are DPP only.  `kl` points at global or LDS memory.  Every lane must call.
+__device__ __forceinline__ void dppo_on_one_wave(const DppoArgs& A, const float* kl) {
+  const int lane = threadIdx.x & (kWave - 1);
+  DppoAcc s;
+  for (int64_t i = lane; i < A.n; i += kWave) dppo_elem(A, i, kl[i], s);
+  double tot[D_SUMS];
+#pragma unroll
+  for (int v = 0; v < D_SUMS; ++v) tot[v] = wave_sum(s.acc[v]);
+  const float rmin = wave_min(s.rmin), rmax = wave_max(s.rmax), klmax = wave_max(s.klmax);
+  if (lane == 0) dppo_metrics(A, tot, rmin, rmax, klmax);
+}
+
+// Launched with one wavefront for up to kDppoWaveMax elements, with a workgroup beyond.
+constexpr int64_t kDppoWaveMax = 4096;
+
+__global__ __launch_bounds__(kKlThreads) void flowdppo_loss_kernel(DppoArgs A) {
+  if (blockDim.x == kWave) {
+    dppo_on_one_wave(A, A.kl);
+    return;
+  }
+  __shared__ double lds[kKlThreads / kWave];
+  __shared__ float ldsf[kKlThreads / kWave];
+  DppoAcc s;
+  for (int64_t i = threadIdx.x; i < A.n; i += kKlThreads) dppo_elem(A, i, A.kl[i], s);
+  double tot[D_SUMS];
+#pragma unroll
+  for (int v = 0; v < D_SUMS; ++v) tot[v] = block_sum<double>(s.acc[v], lds);
+  const float rmin = block_min(s.rmin, ldsf), rmax = block_max(s.rmax, ldsf), klmax = block_max(s.klmax, ldsf);
+  if (threadIdx.x == 0) dppo_metrics(A, tot, rmin, rmax, klmax);
+}
+
+// KL finalize and the KL-ADV loss in one launch: the wavefronts of one workgroup add the
+// streaming kernel's partials row by row (fixed order), leave the per-row KL in LDS, and the
+// first wavefront runs the [B,S'] problem on it.  R <= kDppoWaveMax.
+__global__ __launch_bounds__(kKlThreads) void flowdppo_finish_kernel(KlArgs K, DppoArgs A, unsigned int nblk) {
+  __shared__ float lds_kl[kDppoWaveMax];
+  const int wave = threadIdx.x / kWave;
+  const int64_t R = A.n;
+  for (int64_t row = wave; row < R; row += kKlThreads / kWave) {
+    const float den = kl_den(K, row);  // issued with the partial loads, not after them
+    const double q = wave_ordered_sum(K.partials + row * nblk, nblk);
+    const float kl = (float)((q / (double)den) / (double)K.D);
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      K.kl[row] = kl;
+      if (K.mask) K.mask[row] = (kl < K.threshold) ? 1 : 0;
+      lds_kl[row] = kl;
+    }
+  }
+  __syncthreads();
+  if (wave == 0) dppo_on_one_wave(A, lds_kl);
 }
 
 }  // namespace unirl
@@ -319,7 +376,10 @@ extern "C" int unirl_flowdppo_loss(const float* new_logp, const float* old_logp,
   A.threshold = threshold;
   A.loss_elem = loss_elem;
   A.metrics = metrics;
-  hipLaunchKernelGGL(flowdppo_loss_kernel, dim3(1), dim3(kKlThreads), 0, (hipStream_t)stream, A);
+  A.grad_new = nullptr;
+  A.grad_scale = 0.0f;
+  hipLaunchKernelGGL(flowdppo_loss_kernel, dim3(1), dim3(n <= kDppoWaveMax ? kWave : kKlThreads), 0,
+                     (hipStream_t)stream, A);
   return (int)hipGetLastError();
 }
 
@@ -343,7 +403,7 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
   hipStream_t st = (hipStream_t)stream;
   for (int64_t r0 = 0; r0 < R; r0 += per_launch) {
     const int64_t nr = (R - r0 < per_launch) ? (R - r0) : per_launch;
-    KlArgs A;
+    KlArgs A = {};
     A.p = offset_ptr(p, r0 * D, sz);
     A.q = offset_ptr(q, r0 * D, sz);
     A.sigma = sigma;
@@ -373,6 +433,61 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
   return UNIRL_OK;
 }
 
+extern "C" int unirl_flowdppo_step(const void* p, const void* q, int dtype, const float* sigma, int64_t n_sigma,
+                                   int64_t R, int64_t D, const float* new_logp, const float* old_logp,
+                                   const float* advantages, float threshold, float loss_scale, float* kl_out,
+                                   float* loss_elem, float* grad_new, float* metrics, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  if (!dtype_ok(dtype)) return UNIRL_E_DTYPE;
+  if (R <= 0 || D <= 0 || n_sigma <= 0) return UNIRL_E_SHAPE;
+  if (R > kDppoWaveMax) return UNIRL_E_LIMIT;
+  if (!p || !q || !sigma || !kl_out || !new_logp || !old_logp || !advantages || !loss_elem || !metrics)
+    return UNIRL_E_NULL;
+  if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
+  const size_t sz = dtype_size(dtype);
+  if (!aligned_to(p, sz) || !aligned_to(q, sz) || !aligned_to(new_logp, 4) || !aligned_to(old_logp, 4) ||
+      !aligned_to(advantages, 4) || !aligned_to(kl_out, 4) || !aligned_to(loss_elem, 4) ||
+      !aligned_to(grad_new, 4) || !aligned_to(metrics, 4))
+    return UNIRL_E_ALIGN;
+  int vec = 4;
+  if (D % 4 != 0 || !aligned_to(p, 4 * sz) || !aligned_to(q, 4 * sz)) vec = 1;
+  if (sz == 2 && D % 8 == 0 && aligned_to(p, 16) && aligned_to(q, 16)) vec = 8;
+  const int items = (vec >= 4) ? (int)tune_int("UNIRL_KL_ITEMS", 2) : 2;
+  const unsigned int nblk = kl_blocks_per_row(D / vec, items, R);
+  if ((int64_t)nblk * R > kPartialCapacity) return UNIRL_E_LIMIT;
+  hipStream_t st = (hipStream_t)stream;
+  KlArgs K = {};
+  K.p = p;
+  K.q = q;
+  K.sigma = sigma;
+  K.n_sigma = n_sigma;
+  K.D = D;
+  K.threshold = threshold;
+  K.kl = kl_out;
+  K.partials = ws_partials(workspace);
+  K.always_partials = 1;
+  int rc = UNIRL_E_DTYPE;
+  switch (dtype) {
+    case UNIRL_F32: rc = launch_kl<float>(K, R, vec, nblk, items, st); break;
+    case UNIRL_BF16: rc = launch_kl<bf16_t>(K, R, vec, nblk, items, st); break;
+    case UNIRL_F16: rc = launch_kl<f16_t>(K, R, vec, nblk, items, st); break;
+  }
+  if (rc != 0) return rc;
+  DppoArgs A;
+  A.nw = new_logp;
+  A.od = old_logp;
+  A.adv = advantages;
+  A.kl = nullptr;  // read from LDS
+  A.n = R;
+  A.threshold = threshold;
+  A.loss_elem = loss_elem;
+  A.metrics = metrics;
+  A.grad_new = grad_new;
+  A.grad_scale = loss_scale / (float)R;  // d(loss_scale * mean(elem)) / d elem
+  hipLaunchKernelGGL(flowdppo_finish_kernel, dim3(1), dim3(kKlThreads), 0, st, K, A, nblk);
+  return (int)hipGetLastError();
+}
+
 extern "C" int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, const float* sigma, int64_t n_sigma,
                                       int64_t R, int64_t D, float* out, void* stream) {
   if (!dtype_ok(dtype)) return UNIRL_E_DTYPE;
@@ -387,7 +502,7 @@ extern "C" int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, c
   const int64_t per_launch = 32768;
   for (int64_t r0 = 0; r0 < R; r0 += per_launch) {
     const int64_t nr = (R - r0 < per_launch) ? (R - r0) : per_launch;
-    KlArgs A;
+    KlArgs A = {};
     A.p = offset_ptr(p, r0 * D, sz);
     A.q = offset_ptr(q, r0 * D, sz);
     A.sigma = sigma;

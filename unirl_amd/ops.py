@@ -473,6 +473,72 @@ def flowdppo_loss(
     return elem, metrics
 
 
+FLOWDPPO_STEP_MAX_ROWS = 4096
+
+
+def flowdppo_step(
+    new_logp: torch.Tensor,
+    old_logp: torch.Tensor,
+    new_means: torch.Tensor,
+    old_means: torch.Tensor,
+    advantages: torch.Tensor,
+    sigma_t: torch.Tensor,
+    threshold: float,
+    *,
+    loss_scale: Optional[float] = None,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    """KL over the means, KL-ADV masked loss and metrics in two launches.
+
+    ``new_logp`` / ``old_logp`` / ``advantages`` are ``[B, S']`` (advantages may broadcast), the
+    means ``[B, S', ...]``, ``sigma_t`` one value or one per step.  Returns ``(kl [B,S'],
+    loss_elem [B,S'], metrics [16], grad_new [B,S'] or None)`` in fp32; with ``loss_scale``
+    given, ``grad_new`` is what ``(loss_elem.mean() * loss_scale).backward()`` leaves in
+    ``new_logp``.  At most ``FLOWDPPO_STEP_MAX_ROWS`` rows.
+    """
+    N.require_device(new_logp, "new_logp")
+    if new_means.shape != old_means.shape:
+        raise ValueError(f"new_means {tuple(new_means.shape)} != old_means {tuple(old_means.shape)}")
+    if new_logp.dim() != 2 or tuple(new_means.shape[:2]) != tuple(new_logp.shape) or new_means.dim() < 3:
+        raise ValueError(
+            f"need log-probs [B, S'] and means [B, S', ...]; got {tuple(new_logp.shape)} and {tuple(new_means.shape)}"
+        )
+    device = new_logp.device
+    shape = tuple(new_logp.shape)
+    R = shape[0] * shape[1]
+    if R == 0 or R > FLOWDPPO_STEP_MAX_ROWS:
+        raise ValueError(f"flowdppo_step handles 1..{FLOWDPPO_STEP_MAX_ROWS} rows; got {R}")
+    pc = _flat2(new_means.detach(), "new_means")
+    qc = _flat2(old_means.detach(), "old_means").to(pc.dtype)
+    if pc.dtype not in N._DTYPE_CODE:
+        pc, qc = pc.float(), qc.float()
+    D = pc.numel() // R
+    sig = sigma_t.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    if sig.numel() not in (1, shape[1]):
+        raise ValueError(f"sigma_t must hold 1 or {shape[1]} values; got {tuple(sigma_t.shape)}")
+
+    def f32c(t):
+        t = t.detach().to(device=device, dtype=torch.float32)
+        if tuple(t.shape) != shape:
+            t = t.expand(shape)
+        return t.contiguous()
+
+    nw, od, ad = f32c(new_logp), f32c(old_logp), f32c(advantages)
+    kl = torch.empty(shape, dtype=torch.float32, device=device)
+    elem = torch.empty(shape, dtype=torch.float32, device=device)
+    grad = torch.empty(shape, dtype=torch.float32, device=device) if loss_scale is not None else None
+    metrics = torch.empty(N.M_COUNT, dtype=torch.float32, device=device)
+    stream = N.current_stream(device)
+    ws, ws_bytes = N.workspace(device, stream)
+    with N.on_device(device):
+        rc = N.lib().unirl_flowdppo_step(
+            N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, N.ptr(nw), N.ptr(od),
+            N.ptr(ad), float(threshold), float(loss_scale or 0.0), N.ptr(kl), N.ptr(elem), N.ptr(grad),
+            N.ptr(metrics), N.ptr(ws), ws_bytes, stream,
+        )
+    N.check(rc, "unirl_flowdppo_step")
+    return kl, elem, metrics, grad
+
+
 def expand_per_seq(values: torch.Tensor, cu_seqlens: torch.Tensor, n_tok: int) -> torch.Tensor:
     """``out[t] = values[r]`` for the tokens of packed sequence ``r`` (f32 ``[n_tok]``)."""
     N.require_device(values, "values")
