@@ -213,6 +213,22 @@ def make_shapes(torch, dev):
             cpu=(lambda k=kind, o=okw: cpu_step(k, o)), cpu_bytes=bytes3_step,
         ))
 
+    # the same tokens in the packed layout the AR algorithms use ([total_tokens] + cu_seqlens)
+    cu3 = torch.cat([torch.zeros(1, dtype=torch.int64), lengths.cumsum(0)]).to(dev)
+    ns3p = n_sets_for(3 * n_valid * 4)
+    sets3p = [(newp.to(dev) + 0.0 * k, oldp.to(dev) + 0.0 * k) for k in range(ns3p)]
+    pplans = {}
+    for kind, code, kw in (("grpo", N.LOSS_GRPO, dict(clip_low=0.2, clip_high=0.28)),
+                           ("drpo", N.LOSS_DRPO, dict(drpo_epsilon=5.0))):
+        pplans[kind] = [ops.RatioLossPlan(a, b, adv_d, kind=code, cu_seqlens=cu3, **kw) for a, b in sets3p]
+    for kind in ("grpo", "drpo"):
+        shapes.append(dict(
+            name=f"ratio_step_{kind}_packed", config=3,
+            shape=f"fp32 packed [{n_valid}] + cu_seqlens[257]: loss + metrics + grad_new in one pass",
+            bytes=3 * n_valid * 4, read_bytes=bytes3_valid, write_bytes=n_valid * 4, elements=n_valid,
+            run=(lambda i, k=kind: pplans[k][i % ns3p].forward_backward(1.0)), sets=ns3p,
+        ))
+
     # -- config 4: Flow-DPPO KL mask, WAN bf16 [2,16,21,60,104] -----------------------------------
     g = torch.Generator().manual_seed(1004)
     shp4 = (2, 1, 16, 21, 60, 104)
@@ -471,7 +487,7 @@ def main() -> int:
                 del floor_run
             except Exception as exc:
                 log(f"{sh['name']}: floor measurement failed ({type(exc).__name__}: {exc})")
-            if not args.skip_cpu:
+            if not args.skip_cpu and "cpu" in sh:
                 cms = time_cpu(sh["cpu"], reps=sh.get("cpu_reps", 5), warmup=1)
                 row["cpu_ms"] = round(cms, 2)
                 row["cpu_gbps"] = round(sh["cpu_bytes"] / (cms * 1e-3) / 1e9, 3)

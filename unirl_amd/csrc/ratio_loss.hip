@@ -342,7 +342,8 @@ __device__ __forceinline__ void ratio_vec_fwd(const RatioArgs& A, const RatioCon
 
 // The same for a vector that is whole and valid in all 64 lanes (outside the packed layout): no
 // bounds checks, and the clip flags are counted per wavefront.
-template <int KIND, int VEC, bool GRAD>
+// WTOK: the aggregation weight rides on every token (packed layout) instead of on the flush.
+template <int KIND, int VEC, bool GRAD, bool WTOK = false>
 __device__ __forceinline__ void ratio_vec_wave(const RatioConsts& C, const float (&nw)[VEC],
                                                const float (&od)[VEC], const float (&ad)[VEC],
                                                const float (&mk)[VEC], bool adv_tok, float gfac, const SeqCtx& sq,
@@ -353,7 +354,7 @@ __device__ __forceinline__ void ratio_vec_wave(const RatioConsts& C, const float
     const float a = adv_tok ? ad[k] : sq.adv;
     bool hi, lo;
     float dl;
-    out[k] = accumulate_token<KIND, GRAD>(nw[k], od[k], a, mk[k], C, acc, hi, lo, dl);
+    out[k] = accumulate_token<KIND, GRAD>(nw[k], od[k], a, WTOK ? mk[k] * sq.w : mk[k], C, acc, hi, lo, dl);
     gr[k] = (grow * mk[k]) * dl;
     wc.add(hi, lo);
   }
@@ -546,6 +547,208 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
         if (GRAD) A.grad_new[base + t] = 0.0f;
       }
     }
+  }
+  store_block_partials(A, acc, wc, lds_v);
+}
+
+// Largest s in [lo, n_seq) with cu(s) <= tok, found by the whole wavefront: every round 64 lanes
+// probe the bracket at equal steps and a ballot picks the step, so n_seq <= 4096 takes two
+// dependent loads where a bisection takes twelve.  Requires cu(lo) <= tok; wave-uniform result.
+template <typename CU>
+__device__ __forceinline__ int64_t wave_find_seq(const CU& cu, int64_t n_seq, int64_t tok, int64_t lo) {
+  const int lane = threadIdx.x & (kWave - 1);
+  int64_t hi = n_seq;
+  while (hi - lo > 1) {
+    const int64_t step = (hi - lo + kWave - 1) / kWave;
+    const int64_t probe = lo + lane * step;
+    const bool ok = probe < hi && cu(probe) <= tok;  // true on a prefix of the lanes (cu is sorted)
+    int k = __builtin_popcountll(__builtin_amdgcn_ballot_w64(ok)) - 1;
+    k = k < 0 ? 0 : k;
+    const int64_t nlo = lo + k * step;
+    const int64_t nhi = nlo + step;
+    lo = nlo;
+    hi = nhi < hi ? nhi : hi;
+  }
+  return lo;
+}
+
+// Packed layout ([n_tok] tokens, cu_seqlens), 16-byte vectors.  Every wavefront owns one
+// contiguous run of vectors -- the valid tokens are balanced exactly, whatever the sequence
+// lengths -- and walks it in spans of 64 vectors while it tracks the sequence under its span
+// in scalar registers.  A span inside one sequence (all but one or two per sequence) runs the
+// wave-uniform path of the padded kernel with a scalar advantage and weight; a span that holds
+// one sequence boundary picks the advantage and the weight per token from the two sequences;
+// only a span with several boundaries (sequences shorter than 256 tokens) walks lane by lane.
+// The sequence lookups read cu_seqlens from memory (a 64-way search: two dependent loads up to
+// 4096 sequences; afterwards the next sequence is one load away).  Copies of the table in LDS,
+// or in the wavefront's registers with ballot searches, were measured and are no faster: the
+// workgroup barrier, or the chain of lane reads, costs what the loads cost.
+template <int KIND, int FLAGS, bool GRAD, int ITEMS>
+__global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs A) {
+  constexpr int VEC = 4;
+  __shared__ double lds_v[kRlVals][kRlThreads];
+  const RatioConsts C = A.C;
+  const bool has_mask = (FLAGS & 1) != 0;
+  const bool adv_tok = (FLAGS & 2) != 0;
+
+  float gfac = 0.0f;
+  if (GRAD) {
+    if (C.agg_mode == UNIRL_AGG_TOKEN_MEAN)
+      gfac = A.loss_scale / (float)A.n_tok;
+    else if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_SUM)
+      gfac = (A.loss_scale / (float)A.n_seq) / C.horizon;
+    else
+      gfac = A.loss_scale / (float)A.n_seq;
+  }
+
+  Acc acc;
+  WaveCounts wc;
+  SeqCtx sq;  // per-lane state of the boundary path
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t n_waves = (int64_t)gridDim.x * (kRlThreads / kWave);
+  const int64_t wave_id =
+      (int64_t)blockIdx.x * (kRlThreads / kWave) + __builtin_amdgcn_readfirstlane((int)threadIdx.x) / kWave;
+  const int64_t count = A.n_tok;
+  const int64_t nvec_full = count / VEC;
+  // vectors per wavefront: an equal share, rounded up to whole spans.  (Dealing the spans to the
+  // wavefronts in turn instead, as the padded kernel does, needs a sequence search per span and
+  // measured 10 % slower.)
+  const int64_t per_wave = ((nvec_full + n_waves - 1) / n_waves + kWave - 1) / kWave * kWave;
+  const int64_t v0 = wave_id * per_wave;
+  const int64_t v1 = (v0 + per_wave < nvec_full) ? v0 + per_wave : nvec_full;
+
+  int64_t cur = 0, cur_end = -1;  // sequence under the current span; cur_end < 0: none yet
+  SeqCtx u;                       // its advantage and weight (wave-uniform)
+
+  float nw[ITEMS][VEC], od[ITEMS][VEC], ad[ITEMS][VEC], mk[ITEMS][VEC];
+  // every lane loads every item: past the run's end the index falls back to its last vector
+  auto load_pass = [&](int64_t w0) {
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t i = w0 + it * kWave + lane;
+      const int64_t ic = (i < v1) ? i : v1 - 1;
+      Vec<float, VEC>::load(A.nw + ic * VEC, nw[it]);
+      Vec<float, VEC>::load(A.od + ic * VEC, od[it]);
+      if (adv_tok) Vec<float, VEC>::load(A.adv + ic * VEC, ad[it]);
+      if (has_mask) Vec<float, VEC>::load(A.mask + ic * VEC, mk[it]);
+      else fill_ones(mk[it]);
+    }
+  };
+  if (v0 < v1) load_pass(v0);  // in flight while the first sequence is looked up
+
+  const int64_t n_seq = A.n_seq;
+  auto cu = [&](int64_t j) -> int64_t { return A.seq[j]; };
+  auto seq_adv = [&](int64_t j) -> float { return A.adv[j]; };
+
+  for (int64_t w0 = v0; w0 < v1; w0 += kWave * ITEMS) {
+#pragma unroll
+    for (int it = 0; it < ITEMS; ++it) {
+      const int64_t s0 = w0 + it * kWave;  // first vector of the span (wave-uniform)
+      if (s0 < v1) {
+        const int64_t tok0 = s0 * VEC;
+        if (tok0 >= cur_end) {
+          // usually the next sequence; a full search only at the start and past very short ones
+          bool found = false;
+          if (cur_end >= 0 && cur + 2 <= n_seq) {
+            const int64_t e2 = cu(cur + 2);
+            if (tok0 < e2) {
+              u.w = seq_weight(C, e2 - cur_end);
+              cur += 1;
+              cur_end = e2;
+              found = true;
+            }
+          }
+          if (!found) {
+            cur = wave_find_seq(cu, n_seq, tok0, cur_end < 0 ? 0 : cur);
+            const int64_t beg = cu(cur);
+            cur_end = cu(cur + 1);
+            u.w = seq_weight(C, cur_end - beg);
+          }
+          if (!adv_tok) u.adv = seq_adv(cur);
+        }
+        const int64_t i = s0 + lane;
+        float out[VEC], gr[VEC];
+        const bool whole = (s0 + kWave <= v1);  // all 64 lanes hold a vector of the run
+        const int64_t span_end = (s0 + kWave) * VEC;
+        // end of the next sequence, when the span runs past the current one
+        const int64_t next_end = (whole && span_end > cur_end && cur + 2 <= n_seq) ? cu(cur + 2) : -1;
+        if (whole && span_end <= cur_end) {
+          ratio_vec_wave<KIND, VEC, GRAD, true>(C, nw[it], od[it], ad[it], mk[it], adv_tok, gfac, u, acc, wc, out, gr);
+          if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + i * VEC, out);
+          if (GRAD) Vec<float, VEC>::store(A.grad_new + i * VEC, gr);
+        } else if (whole && span_end <= next_end) {
+          // exactly one sequence ends inside the span: still the wave-uniform path, with the
+          // advantage and the weight picked per token from the two sequences
+          SeqCtx nx;
+          nx.w = seq_weight(C, next_end - cur_end);
+          if (!adv_tok) nx.adv = seq_adv(cur + 1);
+          float ad2[VEC], mk2[VEC];
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) {
+            const bool second = (i * VEC + k) >= cur_end;
+            ad2[k] = adv_tok ? ad[it][k] : (second ? nx.adv : u.adv);
+            mk2[k] = mk[it][k] * (second ? nx.w : u.w);
+          }
+          SeqCtx one;  // weight 1: it is inside mk2
+          ratio_vec_wave<KIND, VEC, GRAD, false>(C, nw[it], od[it], ad2, mk2, true, gfac, one, acc, wc, out, gr);
+          cur += 1;
+          cur_end = next_end;
+          u = nx;
+          if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + i * VEC, out);
+          if (GRAD) Vec<float, VEC>::store(A.grad_new + i * VEC, gr);
+        } else if (i < v1) {
+          // a sequence ends inside the span: every lane walks on from the span's first sequence
+          int64_t ls = cur, lend = cur_end;
+          float lw = u.w, ladv = u.adv;
+#pragma unroll
+          for (int k = 0; k < VEC; ++k) {
+            const int64_t t = i * VEC + k;
+            while (t >= lend && ls + 1 < n_seq) {
+              ++ls;
+              const int64_t e = A.seq[ls + 1];
+              lw = seq_weight(C, e - lend);
+              lend = e;
+              if (!adv_tok) ladv = A.adv[ls];
+            }
+            bool hi, lo;
+            float dl;
+            out[k] = accumulate_token<KIND, GRAD>(nw[it][k], od[it][k], adv_tok ? ad[it][k] : ladv, mk[it][k] * lw, C,
+                                                  acc, hi, lo, dl);
+            gr[k] = ((gfac * lw) * mk[it][k]) * dl;
+            acc.chi += hi ? 1u : 0u;
+            acc.clo += lo ? 1u : 0u;
+            acc.cany += (hi || lo) ? 1u : 0u;
+          }
+          acc.cnt += VEC;
+          if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + i * VEC, out);
+          if (GRAD) Vec<float, VEC>::store(A.grad_new + i * VEC, gr);
+        }
+      }
+    }
+    if (w0 + kWave * ITEMS < v1) load_pass(w0 + kWave * ITEMS);
+    acc.flush(1.0);
+  }
+  // the last count % VEC tokens cannot be loaded as a vector; one lane takes them
+  if (nvec_full * VEC < count && blockIdx.x == 0 && threadIdx.x == 0) {
+    const int64_t t0 = nvec_full * VEC;
+    float nw[VEC], od[VEC], ad[VEC], mk[VEC], out[VEC], gr[VEC];
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      const bool ok = (t0 + k) < count;
+      nw[k] = ok ? A.nw[t0 + k] : 0.0f;
+      od[k] = ok ? A.od[t0 + k] : 0.0f;
+      ad[k] = (ok && adv_tok) ? A.adv[t0 + k] : 0.0f;
+      mk[k] = (ok && has_mask) ? A.mask[t0 + k] : 1.0f;
+    }
+    ratio_vec_fwd<KIND, VEC, true, GRAD>(A, C, t0, count, nw, od, ad, mk, adv_tok, gfac, sq, acc, out, gr);
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      if (t0 + k < count) {
+        if (A.loss_elem) A.loss_elem[t0 + k] = out[k];
+        if (GRAD) A.grad_new[t0 + k] = gr[k];
+      }
+    }
+    acc.flush(1.0);
   }
   store_block_partials(A, acc, wc, lds_v);
 }
@@ -832,12 +1035,26 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
   const bool grad = (A.grad_new != nullptr);
   // 16-byte vectors: mask / per-token-advantage switches compiled in; scalar tokens: read at run time
   const int flags = (A.mask ? 1 : 0) | (A.C.adv_per_token ? 2 : 0);
+  // packed layout: a wavefront's run of up to four spans goes out as a single pass of loads
+  const int64_t n_waves = (int64_t)S.grid.x * (kRlThreads / kWave);
+  const bool one_pass = ((A.n_tok / 4 + n_waves - 1) / n_waves + kWave - 1) / kWave <= 4;
 #define UNIRL_LAUNCH_FWD4(KIND, VEC, PACKED, FLAGS)                                                            \
   do {                                                                                                         \
     if (grad)                                                                                                  \
       hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, PACKED, FLAGS, true>), S.grid, block, 0, st, A);    \
     else                                                                                                       \
       hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, PACKED, FLAGS, false>), S.grid, block, 0, st, A);   \
+  } while (0)
+#define UNIRL_LAUNCH_PACKED2(KIND, FLAGS, ITEMS)                                                               \
+  do {                                                                                                         \
+    if (grad)                                                                                                  \
+      hipLaunchKernelGGL((ratio_loss_packed_kernel<KIND, FLAGS, true, ITEMS>), S.grid, block, 0, st, A);       \
+    else                                                                                                       \
+      hipLaunchKernelGGL((ratio_loss_packed_kernel<KIND, FLAGS, false, ITEMS>), S.grid, block, 0, st, A);      \
+  } while (0)
+#define UNIRL_LAUNCH_PACKED(KIND, FLAGS)                                                                       \
+  do {                                                                                                         \
+    if (one_pass) UNIRL_LAUNCH_PACKED2(KIND, FLAGS, 4); else UNIRL_LAUNCH_PACKED2(KIND, FLAGS, 2);             \
   } while (0)
 #define UNIRL_LAUNCH_FWD3(KIND, VEC, FLAGS)                                                                    \
   do {                                                                                                         \
@@ -846,13 +1063,19 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
 #define UNIRL_LAUNCH_FWD(KIND)                                                                                 \
   do {                                                                                                         \
     if (S.vec != 4) UNIRL_LAUNCH_FWD3(KIND, 1, -1);                                                            \
-    else if (flags == 0) UNIRL_LAUNCH_FWD3(KIND, 4, 0);                                                        \
-    else if (flags == 1) UNIRL_LAUNCH_FWD3(KIND, 4, 1);                                                        \
-    else if (flags == 2) UNIRL_LAUNCH_FWD3(KIND, 4, 2);                                                        \
-    else UNIRL_LAUNCH_FWD3(KIND, 4, 3);                                                                        \
+    else if (packed && flags == 0) UNIRL_LAUNCH_PACKED(KIND, 0);                                               \
+    else if (packed && flags == 1) UNIRL_LAUNCH_PACKED(KIND, 1);                                               \
+    else if (packed && flags == 2) UNIRL_LAUNCH_PACKED(KIND, 2);                                               \
+    else if (packed) UNIRL_LAUNCH_PACKED(KIND, 3);                                                             \
+    else if (flags == 0) UNIRL_LAUNCH_FWD4(KIND, 4, false, 0);                                                 \
+    else if (flags == 1) UNIRL_LAUNCH_FWD4(KIND, 4, false, 1);                                                 \
+    else if (flags == 2) UNIRL_LAUNCH_FWD4(KIND, 4, false, 2);                                                 \
+    else UNIRL_LAUNCH_FWD4(KIND, 4, false, 3);                                                                 \
   } while (0)
   if (A.C.kind == UNIRL_LOSS_GRPO) UNIRL_LAUNCH_FWD(UNIRL_LOSS_GRPO); else UNIRL_LAUNCH_FWD(UNIRL_LOSS_DRPO);
 #undef UNIRL_LAUNCH_FWD4
+#undef UNIRL_LAUNCH_PACKED
+#undef UNIRL_LAUNCH_PACKED2
 #undef UNIRL_LAUNCH_FWD3
 #undef UNIRL_LAUNCH_FWD
   const int launch_rc = (int)hipGetLastError();
