@@ -393,3 +393,48 @@ def test_one_pass_without_graph_runs_forward_only(dev):
     new, old, lengths, adv = batch(4, 64, seed=9)
     m = fused_token_loss_backward("grpo", new.to(dev), old.to(dev), adv.to(dev), lengths=lengths.to(dev), loss_scale=1.0)
     assert m.shape == (16,) and bool(torch.isfinite(m[:13]).all())
+
+
+@pytest.mark.parametrize("kind", ["grpo", "drpo"])
+@pytest.mark.parametrize("case", ["many_short", "mixed", "one", "edges"])
+def test_packed_layout_sequence_tracking(dev, kind, case):
+    """The packed kernel follows the sequences span by span: thousands of sequences shorter than a
+    span (several boundaries per span, more than 4096 sequences: a three-round search), long and
+    short ones mixed, a single sequence, boundaries exactly on span and vector edges, empty
+    sequences, a token count that is no multiple of four -- loss, metrics and the one-pass
+    gradient against the oracle in every aggregation mode."""
+    from unirl_amd import _native as N
+    from unirl_amd.algorithms._fused import fused_token_loss_backward
+
+    g = torch.Generator().manual_seed({"many_short": 1, "mixed": 2, "one": 3, "edges": 4}[case])
+    if case == "many_short":
+        lengths = torch.randint(0, 41, (5000,), generator=g)
+    elif case == "mixed":
+        lengths = torch.cat([torch.randint(1000, 5000, (6,), generator=g), torch.randint(0, 300, (60,), generator=g)])
+        lengths = lengths[torch.randperm(lengths.numel(), generator=g)]
+    elif case == "one":
+        lengths = torch.tensor([70001])
+    else:
+        lengths = torch.tensor([256, 256, 512, 0, 0, 252, 4, 1, 3, 1024, 255, 257, 768, 2])
+    n_seq, T = lengths.numel(), int(lengths.sum())
+    old = -8 * torch.rand(T, generator=g)
+    new = old + 0.05 * torch.randn(T, generator=g)
+    adv = torch.randn(n_seq, generator=g)
+    cu = torch.cat([torch.zeros(1, dtype=torch.int64), lengths.cumsum(0)])
+    kw = dict(clip_range=0.2, clip_range_high=0.28, epsilon=5.0)
+    for mode in MODES:
+        if kind == "drpo" and mode == "seq-mean-token-mean":
+            continue
+        leaf = new.clone().requires_grad_(True)
+        ref_loss, ref_m = olos.token_loss(kind, leaf, old, adv, lengths, mode=mode, horizon=4096, **kw)
+        (ref_loss * 0.5).backward()
+        nd = new.to(dev).requires_grad_(True)
+        mvec = fused_token_loss_backward(kind, nd, old.to(dev), adv.to(dev), cu_seqlens=cu.to(dev), loss_scale=0.5,
+                                         loss_agg_mode=mode, horizon=4096, clip_range=0.2, clip_range_high=0.28,
+                                         drpo_epsilon=5.0)
+        vals = mvec.tolist()
+        scale = float(olos.token_loss(kind, new, old, adv, lengths, mode="token-mean", **kw)[0].abs()) + float(adv.abs().mean())
+        assert_close(torch.tensor(vals[N.M_LOSS]), ref_loss, FP32_RTOL, loss_atol(scale), f"{case} {mode} loss")
+        assert vals[N.M_NUM_TOKENS] == float(T)
+        assert_close(nd.grad.cpu(), leaf.grad, 1e-5, 1e-6 * float(leaf.grad.abs().max()), f"{case} {mode} grad")
+        assert abs(vals[N.M_RATIO_MAX] - float(ref_m["ratio_max"])) <= 2e-6 * float(ref_m["ratio_max"])

@@ -1014,6 +1014,7 @@ static int check_common(const float* new_logp, const float* old_logp, const floa
     if (n_seq * seq_stride != n_tok) return UNIRL_E_SHAPE;
   } else {
     A.layout = LAYOUT_PACKED;
+    if (n_tok > 0 && n_seq < 1) return UNIRL_E_SHAPE;  // cu_seqlens holds n_seq + 1 >= 2 entries
   }
   A.nw = new_logp;
   A.od = old_logp;
