@@ -593,12 +593,14 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs
 
   float gfac = 0.0f;
   if (GRAD) {
+    // the gradient arriving at the loss: a host scalar (one-pass step) or a device scalar (backward)
+    const float ls = A.g_scale ? *A.g_scale : A.loss_scale;
     if (C.agg_mode == UNIRL_AGG_TOKEN_MEAN)
-      gfac = A.loss_scale / (float)A.n_tok;
+      gfac = ls / (float)A.n_tok;
     else if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_SUM)
-      gfac = (A.loss_scale / (float)A.n_seq) / C.horizon;
+      gfac = (ls / (float)A.n_seq) / C.horizon;
     else
-      gfac = A.loss_scale / (float)A.n_seq;
+      gfac = ls / (float)A.n_seq;
   }
 
   Acc acc;
@@ -750,7 +752,7 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs
     }
     acc.flush(1.0);
   }
-  store_block_partials(A, acc, wc, lds_v);
+  if (A.partials) store_block_partials(A, acc, wc, lds_v);  // absent when only the gradient is wanted
 }
 
 // One workgroup of T threads (256, or 1024 when there are more than 512 partial vectors, so that
@@ -1080,7 +1082,7 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
 #undef UNIRL_LAUNCH_FWD3
 #undef UNIRL_LAUNCH_FWD
   const int launch_rc = (int)hipGetLastError();
-  if (launch_rc != 0) return launch_rc;
+  if (launch_rc != 0 || !A.metrics) return launch_rc;
   const unsigned int nblk = S.grid.x * S.grid.y;
   if (nblk <= 512)
     hipLaunchKernelGGL(ratio_loss_finalize_kernel<256>, dim3(1), dim3(256), 0, st, A, nblk);
@@ -1149,6 +1151,15 @@ extern "C" int unirl_ratio_loss_bwd(const float* new_logp, const float* old_logp
   RatioShape S;
   plan(A, true, S);
   hipStream_t st = (hipStream_t)stream;
+  // packed layout, gradient of the aggregated loss: the packed forward kernel with its gradient
+  // output and nothing else stored -- it follows the sequences span by span, where the kernel
+  // below looks each token's sequence up (37 -> 25 us on 8.8 M tokens)
+  if (A.layout == LAYOUT_PACKED && S.vec == 4 && aggregate && !g_elem) {
+    A.loss_scale = 1.0f;  // stands in for a NULL g_scale
+    A.partials = nullptr;
+    A.metrics = nullptr;
+    return launch_forward(A, st);
+  }
   dim3 block(kRlThreads);
   if (A.C.kind == UNIRL_LOSS_GRPO) {
     if (S.vec == 4)
