@@ -35,7 +35,9 @@
 extern "C" {
 #endif
 
-#define UNIRL_ABI_VERSION 1
+/* 2: typed gradient outputs in unirl_sde_step_logp_bwd; unirl_ratio_loss_fwd_bwd and
+ * unirl_flowdppo_step added. */
+#define UNIRL_ABI_VERSION 2
 
 enum unirl_dtype { UNIRL_F32 = 0, UNIRL_BF16 = 1, UNIRL_F16 = 2 };
 

@@ -91,6 +91,9 @@ class SdeStepDesc(Structure):
     ]
 
 
+# UNIRL_ABI_VERSION of include/unirl_hip.h that the signatures below describe
+ABI_VERSION = 2
+
 _SIGNATURES = {
     "unirl_abi_version": (c_int, []),
     "unirl_status_string": (c_char_p, [c_int]),
@@ -205,6 +208,13 @@ def lib() -> ctypes.CDLL:
                     "(hipcc, gfx950). unirl_amd has no CPU or eager-torch path behind its kernels."
                 )
             handle = ctypes.CDLL(str(LIB_PATH))
+            handle.unirl_abi_version.restype = c_int
+            built = handle.unirl_abi_version()
+            if built != ABI_VERSION:
+                raise RuntimeError(
+                    f"{LIB_PATH} was built for ABI version {built}, this package binds version {ABI_VERSION}: "
+                    "rebuild it with `python -m unirl_amd.build`"
+                )
             for name, (restype, argtypes) in _SIGNATURES.items():
                 fn = getattr(handle, name)
                 fn.restype = restype
