@@ -542,7 +542,16 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
     }
     // padded layout: zero the loss (and the gradient) of the slots past the sequence end
     if ((A.loss_elem || GRAD) && padded) {
-      for (int64_t t = nvec * VEC + first; t < row_end; t += stride) {
+      // whole vectors first (about half of a ragged batch is padding), then the row's last slots
+      float zero[VEC];
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) zero[k] = 0.0f;
+      for (int64_t i = nvec + first; i < nvec_full; i += stride) {
+        if (A.loss_elem) Vec<float, VEC>::store(A.loss_elem + base + i * VEC, zero);
+        if (GRAD) Vec<float, VEC>::store(A.grad_new + base + i * VEC, zero);
+      }
+      const int64_t t_tail = (nvec > nvec_full ? nvec : nvec_full) * VEC;
+      for (int64_t t = t_tail + first; t < row_end; t += stride) {
         if (A.loss_elem) A.loss_elem[base + t] = 0.0f;
         if (GRAD) A.grad_new[base + t] = 0.0f;
       }
