@@ -220,3 +220,14 @@ def test_algorithm_constructors_validate():
     assert FlowDPPO(params=None, pipeline=P()).recomputes_anchor()
     assert not FlowGRPO(params=None, pipeline=P()).recomputes_anchor()
     assert FlowGRPO(params=None, pipeline=P(), old_logp_source="replay").recomputes_anchor()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The bench measures one GPU's share of the path; asking for more exits with a message."""
+    import subprocess
+    import sys
+
+    r = subprocess.run([sys.executable, str(ROOT / "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in (r.stderr + r.stdout)
+    assert not r.stdout.strip().startswith("{")  # no result line
