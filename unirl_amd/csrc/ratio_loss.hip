@@ -14,8 +14,14 @@
 // ratios near 1 keeps full accuracy.  Sums run fp32 per lane over at most a few
 // dozen tokens and fp64 from there up, in a fixed order.
 //
+// Kernels: ratio_loss_fwd_kernel (padded [n_seq, stride] + lengths, and flat),
+// ratio_loss_packed_kernel ([n_tok] + cu_seqlens), each optionally writing the
+// gradient of the aggregated loss in the same pass (the one-pass training step),
+// ratio_loss_finalize_kernel (workgroup partials -> the 16 metrics) and
+// ratio_loss_bwd_kernel (stand-alone backward).
+//
 // HBM traffic: 8 bytes read per valid token (+4 with a mask, +4 with per-token
-// advantages), +4 written when loss_per_elem is requested.
+// advantages), +4 written per slot when loss_per_elem or grad_new is requested.
 
 #include "common.cuh"
 #include "unirl_internal.h"
@@ -72,6 +78,7 @@ struct RatioArgs {
   // fused forward + backward only
   float loss_scale;      // gradient arriving at the aggregated loss
   int64_t n_valid_host;  // token-mean denominator when the host knows it, else < 0
+  int64_t per_wave;      // packed kernel: vectors in a wavefront's run (a multiple of 64)
 };
 
 // exp(x) for fp32 within ~1.5 ulp: 2^(x*log2(e)) on the hardware exp2, with the rounding error
@@ -614,18 +621,17 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs
 
   Acc acc;
   WaveCounts wc;
-  SeqCtx sq;  // per-lane state of the boundary path
+  SeqCtx sq;  // per-lane state of the token-by-token tail
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t n_waves = (int64_t)gridDim.x * (kRlThreads / kWave);
   const int64_t wave_id =
       (int64_t)blockIdx.x * (kRlThreads / kWave) + __builtin_amdgcn_readfirstlane((int)threadIdx.x) / kWave;
   const int64_t count = A.n_tok;
   const int64_t nvec_full = count / VEC;
-  // vectors per wavefront: an equal share, rounded up to whole spans.  (Dealing the spans to the
-  // wavefronts in turn instead, as the padded kernel does, needs a sequence search per span and
-  // measured 10 % slower.)
-  const int64_t per_wave = ((nvec_full + n_waves - 1) / n_waves + kWave - 1) / kWave * kWave;
-  const int64_t v0 = wave_id * per_wave;
+  // The wavefront's run: A.per_wave vectors, an equal share rounded up to whole spans (the host
+  // launches just the wavefronts that have one).  Dealing the spans to the wavefronts in turn
+  // instead, as the padded kernel does, needs a sequence search per span: 10 % slower.
+  const int64_t per_wave = A.per_wave;
+  const int64_t v0 = wave_id * per_wave < nvec_full ? wave_id * per_wave : nvec_full;
   const int64_t v1 = (v0 + per_wave < nvec_full) ? v0 + per_wave : nvec_full;
 
   int64_t cur = 0, cur_end = -1;  // sequence under the current span; cur_end < 0: none yet
@@ -1047,9 +1053,22 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
   const bool grad = (A.grad_new != nullptr);
   // 16-byte vectors: mask / per-token-advantage switches compiled in; scalar tokens: read at run time
   const int flags = (A.mask ? 1 : 0) | (A.C.adv_per_token ? 2 : 0);
-  // packed layout: a wavefront's run of up to four spans goes out as a single pass of loads
-  const int64_t n_waves = (int64_t)S.grid.x * (kRlThreads / kWave);
-  const bool one_pass = ((A.n_tok / 4 + n_waves - 1) / n_waves + kWave - 1) / kWave <= 4;
+  // packed layout: every wavefront takes one contiguous run of vectors, an equal share rounded up
+  // to whole spans of 64; only the workgroups whose wavefronts have a run are launched, and a run
+  // of up to four spans goes out as a single pass of loads
+  bool one_pass = false;
+  if (packed && S.vec == 4) {
+    const int64_t waves_per_wg = kRlThreads / kWave;
+    const int64_t n_waves = (int64_t)S.grid.x * waves_per_wg;
+    const int64_t nvec = A.n_tok / 4;
+    A.per_wave = ((nvec + n_waves - 1) / n_waves + kWave - 1) / kWave * kWave;
+    if (A.per_wave < kWave) A.per_wave = kWave;
+    const int64_t active = (nvec + A.per_wave - 1) / A.per_wave;
+    int64_t nwg = (active + waves_per_wg - 1) / waves_per_wg;
+    if (nwg < 1) nwg = 1;
+    S.grid.x = (unsigned int)nwg;
+    one_pass = A.per_wave / kWave <= 4;
+  }
 #define UNIRL_LAUNCH_FWD4(KIND, VEC, PACKED, FLAGS)                                                            \
   do {                                                                                                         \
     if (grad)                                                                                                  \
