@@ -71,6 +71,28 @@ def test_row_views_strides_and_misalignment(dev):
     # transposed logits are made contiguous by the wrapper
     xt = x.t().contiguous().to(dev).t()
     assert_close(models.token_logp(xt, ids.to(dev)), otok.token_logp(x, ids), FP32_RTOL, 2e-6, "transposed")
+    # the shifted logits of a training step, [B, S, V][:, :-1], are read in place: one launch per
+    # batch entry, no flattened copy
+    x3, ids3 = logits(3 * 7, 1003, 4, torch.bfloat16)
+    x3, ids3 = x3.reshape(3, 7, 1003), ids3.reshape(3, 7)
+    x3d = x3.to(dev)
+    shifted, sh_ids = x3d[:, :-1], ids3[:, 1:]
+    assert not shifted.is_contiguous()
+    blocks = list(ops._row_blocks(shifted, 1003))
+    assert len(blocks) == 3 and all(b.data_ptr() == x3d[k].data_ptr() for k, b in enumerate(blocks))
+    lp, ent, _ = ops.token_logp_entropy(shifted, sh_ids.to(dev), 0.7)
+    assert lp.shape == (3, 6)
+    assert_close(lp, otok.token_logp(x3[:, :-1], sh_ids, 0.7), FP32_RTOL, 2e-6, "shifted logits")
+    assert_close(ent, otok.token_entropy(x3[:, :-1], 0.7), FP32_RTOL, 1e-6, "shifted logits entropy")
+    assert len(list(ops._row_blocks(x3d, 1003))) == 1 and len(list(ops._row_blocks(xd[:, 5:905], 900))) == 1
+    # and their backward, through autograd: the gradient of the slice lands in the parent
+    leaf = x3.float().requires_grad_(True)
+    w = torch.randn(3, 6, generator=torch.Generator().manual_seed(1))
+    (otok.token_logp(leaf[:, :-1], sh_ids, 0.7) * w).sum().backward()
+    leaf_d = x3.float().to(dev).requires_grad_(True)
+    (models.token_logp(leaf_d[:, :-1], sh_ids.to(dev), 0.7) * w.to(dev)).sum().backward()
+    assert_close(leaf_d.grad, leaf.grad, 1e-5, 1e-6 * float(leaf.grad.abs().max()), "grad through the shifted view")
+    assert float(leaf_d.grad[:, -1].abs().sum()) == 0.0
 
 
 def test_uniform_peaked_and_minus_inf(dev):

@@ -634,11 +634,6 @@ def token_logp_entropy(
     x = logits.detach()
     if x.dtype not in N._DTYPE_CODE:
         x = x.float()
-    x2 = x.reshape(-1, V)
-    if x2.stride(-1) != 1 or (x2.shape[0] > 1 and x2.stride(0) < V):
-        x2 = x2.contiguous()
-    rows = x2.shape[0]
-    row_stride = x2.stride(0) if rows > 1 else V
     idc = None
     if want_logp:
         if ids is None:
@@ -649,17 +644,55 @@ def token_logp_entropy(
     logp = torch.empty(lead, dtype=torch.float32, device=device) if want_logp else None
     ent = torch.empty(lead, dtype=torch.float32, device=device) if want_entropy else None
     lse = torch.empty(lead, dtype=torch.float32, device=device) if want_lse else None
-    if rows == 0:
+    n_rows = math.prod(lead)
+    if n_rows == 0:
         return logp, ent, lse
     if V == 0:
         raise ValueError("empty vocabulary")
+
+    def flat(t):
+        return None if t is None else t.reshape(-1)
+
+    stream = N.current_stream(device)
+    # One launch per block of rows that share a row stride.  `[B, S, V][:, :-1]` (the shifted
+    # logits of a training step) is B such blocks: reading it in place costs B launches, flattening
+    # it would cost a copy of the logits.
+    off = 0
     with N.on_device(device):
-        rc = N.lib().unirl_token_logp_entropy(
-            N.ptr(x2), N.dtype_code(x2.dtype), rows, V, row_stride, N.ptr(idc), float(temperature),
-            N.ptr(logp), N.ptr(ent), N.ptr(lse), N.current_stream(device),
-        )
-    N.check(rc, "unirl_token_logp_entropy")
+        for x2 in _row_blocks(x, V):
+            rows = x2.shape[0]
+            row_stride = x2.stride(0) if rows > 1 else V
+
+            def part(t):
+                return None if t is None else t[off : off + rows]
+
+            rc = N.lib().unirl_token_logp_entropy(
+                N.ptr(x2), N.dtype_code(x2.dtype), rows, V, row_stride, N.ptr(part(idc)), float(temperature),
+                N.ptr(part(flat(logp))), N.ptr(part(flat(ent))), N.ptr(part(flat(lse))), stream,
+            )
+            N.check(rc, "unirl_token_logp_entropy")
+            off += rows
     return logp, ent, lse
+
+
+def _row_blocks(x: torch.Tensor, V: int):
+    """``x [..., V]`` as a sequence of 2-D ``[rows, V]`` views, in row-major order of the leading
+    dimensions, each with unit element stride and one row stride >= V.  A tensor that is one such
+    block yields itself; a batch of them (a slice along an inner dimension) yields one per batch
+    entry; anything else is copied once."""
+    if x.stride(-1) == 1 or x.shape[-1] == 1:
+        try:
+            x2 = x.view(-1, V)
+            if x2.shape[0] <= 1 or x2.stride(0) >= V:
+                yield x2
+                return
+        except RuntimeError:
+            pass
+        if x.dim() >= 3 and x.shape[0] <= 64:
+            for b in range(x.shape[0]):
+                yield from _row_blocks(x[b], V)
+            return
+    yield x.reshape(-1, V).contiguous()
 
 
 def token_logp_bwd(
@@ -678,26 +711,29 @@ def token_logp_bwd(
     orig_dtype = x.dtype
     if x.dtype not in N._DTYPE_CODE:
         x = x.float()
-    x2 = x.reshape(-1, V)
-    if not x2.is_contiguous():
-        x2 = x2.contiguous()
-    rows = x2.shape[0]
+    n_rows = math.prod(logits.shape[:-1])
     idc = ids.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
     lsec = lse.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
     gc = g_logp.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
     if in_place:
-        if x2.data_ptr() != logits.data_ptr() or x2.dtype != orig_dtype:
+        if not x.is_contiguous() or x.dtype != orig_dtype:
             raise ValueError("token_logp_bwd(in_place=True) needs contiguous bf16 / fp16 / fp32 logits")
-        grad = x2
+        grad = x.view(-1, V)
     else:
-        grad = torch.empty_like(x2)
-    if rows and V:
+        grad = torch.empty((n_rows, V), dtype=x.dtype, device=device)
+    if n_rows and V:
+        stream = N.current_stream(device)
+        off = 0
         with N.on_device(device):
-            rc = N.lib().unirl_token_logp_bwd(
-                N.ptr(x2), N.dtype_code(x2.dtype), rows, V, V, N.ptr(idc), float(temperature), N.ptr(lsec),
-                N.ptr(gc), N.ptr(grad), V, N.current_stream(device),
-            )
-        N.check(rc, "unirl_token_logp_bwd")
+            for x2 in _row_blocks(x, V):  # sliced logits are read in place, block by block
+                rows = x2.shape[0]
+                rc = N.lib().unirl_token_logp_bwd(
+                    N.ptr(x2), N.dtype_code(x2.dtype), rows, V, x2.stride(0) if rows > 1 else V,
+                    N.ptr(idc[off : off + rows]), float(temperature), N.ptr(lsec[off : off + rows]),
+                    N.ptr(gc[off : off + rows]), N.ptr(grad[off : off + rows]), V, stream,
+                )
+                N.check(rc, "unirl_token_logp_bwd")
+                off += rows
     grad = grad.reshape(logits.shape)
     return grad if grad.dtype == orig_dtype else grad.to(orig_dtype)
 
