@@ -328,12 +328,12 @@ def make_headline(torch, dev, rows: int, vocab: int):
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--rows", type=int, default=8192, help="token rows of the headline workload")
     ap.add_argument("--vocab", type=int, default=151936)
     ap.add_argument("--cpu-rows", type=int, default=2048, help="rows of the bounded CPU-baseline sample")
-    ap.add_argument("--spinup", type=float, default=0.5, help="seconds of untimed launches before the warm-up")
+    ap.add_argument("--spinup", type=float, default=1.0, help="seconds of untimed launches before the warm-up")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="run 3 calibration copies of 1 GiB, 3 headline launches and 3 launches of every "
                          "other shape, then exit "
