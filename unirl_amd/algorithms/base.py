@@ -38,7 +38,8 @@ def gather_sde_field(
 
     ``sde_indices`` need not be sorted.  A device tensor is gathered by one copy kernel;
     a host tensor is indexed where its bytes are (the caller uploads only the gathered
-    slices, as the reference does).
+    slices, as the reference does).  When the targets are all recorded steps in recorded order
+    the tensor itself is returned (callers only read the result).
     """
     if tensor is None or sde_indices is None:
         raise ValueError(
@@ -55,6 +56,8 @@ def gather_sde_field(
             f"gather_sde_field({field_name}): target steps {missing} not in sde_indices={sorted(recorded)}"
         )
     positions = [slot_of[int(t)] for t in target_steps]
+    if positions == list(range(int(tensor.shape[1]))):
+        return tensor  # every recorded step, in recorded order: nothing to move
     if tensor.is_cuda:
         return ops.gather_steps(tensor, positions)
     return tensor[:, positions]
