@@ -9,7 +9,7 @@ and of the step gather, unirl/algorithms/base.py:61-80.
 
 from __future__ import annotations
 
-from typing import Dict, List, Tuple
+from typing import List
 
 import torch
 

@@ -18,7 +18,7 @@ in the logits' dtype, so the chunk needs no activation checkpoint of an fp32 cop
 
 from __future__ import annotations
 
-from typing import Any, Callable, List, Optional, Tuple
+from typing import Callable, List, Optional, Tuple
 
 import torch
 
