@@ -351,7 +351,8 @@ int unirl_ratio_loss_bwd(const float* new_logp, const float* old_logp, const flo
  * n_valid: the token-mean denominator in the padded layout (every token inside
  * the lengths, masked or not) when the host knows it; < 0 lets the kernel sum
  * the lengths.  Ignored in the other layouts (n_tok).  Padded slots past a
- * sequence's length receive 0. */
+ * sequence's length receive 0.  With n_tok == 0 both entry points write only the
+ * metrics (count 0, the means NaN like torch's mean of nothing). */
 int unirl_ratio_loss_fwd_bwd(const float* new_logp, const float* old_logp, const float* advantages,
                              const int64_t* lengths, const float* loss_mask, int64_t n_seq,
                              int64_t seq_stride, int64_t n_tok,

@@ -438,3 +438,32 @@ def test_packed_layout_sequence_tracking(dev, kind, case):
         assert vals[N.M_NUM_TOKENS] == float(T)
         assert_close(nd.grad.cpu(), leaf.grad, 1e-5, 1e-6 * float(leaf.grad.abs().max()), f"{case} {mode} grad")
         assert abs(vals[N.M_RATIO_MAX] - float(ref_m["ratio_max"])) <= 2e-6 * float(ref_m["ratio_max"])
+
+
+@pytest.mark.parametrize("with_grad", [False, True])
+def test_c_abi_empty_input_writes_the_metrics(dev, with_grad):
+    """n_tok == 0 through the C ABI itself (the tensor wrapper answers empty inputs on the host):
+    nothing is read, the count is 0 and the means are NaN, like ``torch.mean`` of nothing."""
+    import ctypes
+
+    from unirl_amd import _native as N
+    from unirl_amd import ops
+
+    params = ops._ratio_params(N.LOSS_GRPO, "token-mean", 0.2, 0.28, 12.5, True, 8192, True)
+    dummy = torch.zeros(4, device=dev)
+    metrics = torch.full((N.M_COUNT,), 7.0, device=dev)
+    stream = N.current_stream(dev)
+    ws, ws_bytes = N.workspace(dev, stream)
+    head = (N.ptr(dummy), N.ptr(dummy), N.ptr(dummy), None, None, 0, 0, 0, ctypes.byref(params))
+    tail = (N.ptr(metrics), N.ptr(ws), ws_bytes, stream)
+    if with_grad:
+        rc = N.lib().unirl_ratio_loss_fwd_bwd(*head, 1.0, -1, N.ptr(dummy), *tail)
+    else:
+        rc = N.lib().unirl_ratio_loss_fwd(*head, None, *tail)
+    assert rc == 0
+    torch.cuda.synchronize()
+    got = metrics.cpu()
+    assert float(got[N.M_NUM_TOKENS]) == 0.0
+    for slot in (N.M_LOSS, N.M_RATIO_MEAN, N.M_APPROX_KL, N.M_CLIP_FRACTION, N.M_ABSDIFF_MEAN):
+        assert math.isnan(float(got[slot])), slot
+    assert torch.equal(dummy.cpu(), torch.zeros(4))

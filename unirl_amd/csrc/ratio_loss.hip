@@ -1147,7 +1147,6 @@ extern "C" int unirl_ratio_loss_fwd_bwd(const float* new_logp, const float* old_
   if (!metrics || !grad_new) return UNIRL_E_NULL;
   if (!aligned_to(grad_new, 4)) return UNIRL_E_ALIGN;
   if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
-  if (n_tok == 0) return UNIRL_OK;
   A.mask = loss_mask;
   A.metrics = metrics;
   A.partials = ws_partials(workspace);

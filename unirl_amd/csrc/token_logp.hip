@@ -89,10 +89,12 @@ __device__ __forceinline__ void tok_update(TokRef& ref, TokAcc& acc, const float
   float cm = x[0];
 #pragma unroll
   for (int k = 1; k < N; ++k) cm = fmaxf(cm, x[k]);
-  const float wm = wave_max(active ? cm : -INFINITY);  // wave-uniform, DPP
-  if (__builtin_expect(wm > ref.m, 0)) {
+  // "does any lane hold a new maximum" is one compare (its lane mask is tested on the scalar
+  // unit); the DPP max-reduction runs only when it does
+  if (__builtin_expect(__builtin_amdgcn_ballot_w64(active && cm > ref.m) != 0, 0)) {
     // Wave-uniform and rare (about ln(chunks) times per row): move to the new maximum, then
     // split this chunk's exact maxima from the rest.
+    const float wm = wave_max(active ? cm : -INFINITY);
     tok_raise(ref.m, ref.r, acc, wm, c);
     if (active) {
 #pragma unroll
