@@ -14,10 +14,12 @@
 //     a_i = fma(x_i, c, -r)        one FMA; exact single rounding
 //     e_i = 2^a_i                  one v_exp_f32
 //     s  += e_i ,  t += e_i * a_i  (t <= ~0: every term has the same sign)
-// One DPP max-reduction per chunk of UNROLL vectors keeps m wave-uniform, so
-// raising the reference is a uniform, rarely taken branch (about ln(#chunks)
-// times per row; per-lane maxima would make some lane take it in almost every
-// chunk); inside that branch the elements equal to the new maximum are
+// m is wave-uniform: per chunk of UNROLL vectors every lane compares its own
+// maximum with m and the wavefront branches on the compare's lane mask, so
+// raising the reference (a DPP max-reduction, then the rescale) is a uniform,
+// rarely taken branch (about ln(#chunks) times per row; per-lane references
+// would make some lane take it in almost every chunk) and the common path pays
+// one compare per chunk for it; inside that branch the elements equal to the new maximum are
 // counted apart (cnt) so that sum = cnt*2^r0 + s keeps full relative accuracy
 // when one logit dominates (sum = 1 + tiny), r0 = fma(m, c, -r) being the exact
 // residual of the rounded reference.  With sum and t:
