@@ -467,3 +467,32 @@ def test_c_abi_empty_input_writes_the_metrics(dev, with_grad):
     for slot in (N.M_LOSS, N.M_RATIO_MEAN, N.M_APPROX_KL, N.M_CLIP_FRACTION, N.M_ABSDIFF_MEAN):
         assert math.isnan(float(got[slot])), slot
     assert torch.equal(dummy.cpu(), torch.zeros(4))
+
+
+@pytest.mark.parametrize("lengths", [[2, 1, 0], [0, 1, 2], [1, 0, 0, 3, 1, 0, 0, 2, 1, 2, 0, 2]])
+def test_packed_batch_with_as_many_tokens_as_sequences(dev, lengths):
+    """``advantages [n]`` fits both readings when a packed batch holds n tokens in n sequences:
+    it is read per sequence (what the reference's algorithms pass) unless the caller says per token."""
+    from unirl_amd.algorithms import fused_token_loss
+
+    lengths = torch.tensor(lengths)
+    n = int(lengths.numel())
+    assert int(lengths.sum()) == n
+    g = torch.Generator().manual_seed(11 + n)
+    old = -8 * torch.rand(n, generator=g)
+    new = old + 0.3 * torch.randn(n, generator=g)
+    adv = torch.randn(n, generator=g)
+    cu = torch.cat([torch.zeros(1, dtype=torch.int64), lengths.cumsum(0)])
+    kw = dict(clip_range=0.2, clip_range_high=0.28)
+    ref_seq, _ = olos.token_loss("grpo", new, old, adv, lengths, mode="token-mean", epsilon=5.0, **kw)
+    ref_tok = olos.grpo_clip_loss(new, old, adv, 0.2, 0.28)[0].mean()
+    assert abs(float(ref_seq) - float(ref_tok)) > 1e-3  # the two readings differ on these inputs
+    args = ("grpo", new.to(dev), old.to(dev), adv.to(dev))
+    got_seq, _ = fused_token_loss(*args, cu_seqlens=cu.to(dev), **kw)
+    got_seq2, _ = fused_token_loss(*args, cu_seqlens=cu.to(dev), adv_per_token=False, **kw)
+    got_tok, _ = fused_token_loss(*args, cu_seqlens=cu.to(dev), adv_per_token=True, **kw)
+    assert_close(got_seq, ref_seq, FP32_RTOL, 1e-6, "per sequence (default)")
+    assert_close(got_seq2, ref_seq, FP32_RTOL, 1e-6, "per sequence (explicit)")
+    assert_close(got_tok, ref_tok, FP32_RTOL, 1e-6, "per token (explicit)")
+    with pytest.raises(ValueError):
+        fused_token_loss(*args[:3], adv.to(dev)[:-1], cu_seqlens=cu.to(dev), adv_per_token=True, **kw)

@@ -77,6 +77,7 @@ def fused_token_loss_backward(
     clip_range_high: Optional[float] = None,
     drpo_epsilon: float = 12.5,
     mu_weighted: bool = True,
+    adv_per_token: Optional[bool] = None,
 ) -> torch.Tensor:
     """``(loss * loss_scale).backward()`` of :func:`fused_token_loss` without building the loss
     in autograd: one kernel reads ``new_logp`` / ``old_logp`` once, reduces the loss and every
@@ -87,7 +88,7 @@ def fused_token_loss_backward(
     plan = RatioLossPlan(
         new_logp, old_logp, advantages, kind=code, lengths=lengths, cu_seqlens=cu_seqlens, loss_mask=loss_mask,
         agg_mode=loss_agg_mode, clip_low=clip_range, clip_high=clip_range_high, drpo_epsilon=drpo_epsilon,
-        mu_weighted=mu_weighted, horizon=horizon,
+        mu_weighted=mu_weighted, horizon=horizon, adv_per_token=adv_per_token,
     )
     if not (torch.is_grad_enabled() and new_logp.requires_grad):
         return plan.forward(want_elem=False)[1]
@@ -145,18 +146,20 @@ def fused_token_loss(
     clip_range_high: Optional[float] = None,
     drpo_epsilon: float = 12.5,
     mu_weighted: bool = True,
+    adv_per_token: Optional[bool] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
     """Whole micro-batch loss of GRPO / DRPO in one launch.
 
     ``new_logp`` / ``old_logp`` are padded ``[n_seq, max_len]`` with ``lengths``, packed
     ``[total_tokens]`` with ``cu_seqlens``, or flat with per-token ``advantages``.
-    ``advantages`` is per sequence ``[n_seq]`` or per token.  Returns the differentiable
+    ``advantages`` is per sequence ``[n_seq]`` or per token; a packed batch with as many tokens
+    as sequences fits both, and is read per sequence unless ``adv_per_token`` is given.  Returns the differentiable
     scalar loss and the ``[16]`` metrics vector (slots: ``unirl_amd._native.M_*``).
     """
     code = {"grpo": N.LOSS_GRPO, "drpo": N.LOSS_DRPO}[kind]
     plan = RatioLossPlan(
         new_logp, old_logp, advantages, kind=code, lengths=lengths, cu_seqlens=cu_seqlens, loss_mask=loss_mask,
         agg_mode=loss_agg_mode, clip_low=clip_range, clip_high=clip_range_high, drpo_epsilon=drpo_epsilon,
-        mu_weighted=mu_weighted, horizon=horizon,
+        mu_weighted=mu_weighted, horizon=horizon, adv_per_token=adv_per_token,
     )
     return scalar_loss(new_logp, plan)

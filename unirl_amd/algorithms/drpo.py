@@ -129,7 +129,7 @@ class DRPO(StageAlgorithm):
             "drpo", new_logp, segment.log_probs, advantages, loss_scale=loss_scale,
             cu_seqlens=cu_seqlens_from_lengths(segment.lengths, new_logp.device),
             loss_mask=getattr(segment, "loss_mask", None), loss_agg_mode=mode, horizon=self.horizon,
-            drpo_epsilon=self.drpo_epsilon, mu_weighted=self.penalty_mu_weighted,
+            drpo_epsilon=self.drpo_epsilon, mu_weighted=self.penalty_mu_weighted, adv_per_token=False,
         )
 
         vals = mvec.tolist()

@@ -74,7 +74,7 @@ class FlowGRPO(SdeStepAlgorithm):
         rows, n_steps = new_logp.shape
         full = torch.full((rows,), n_steps, dtype=torch.int64)  # host lengths: the token count is known
         mvec = fused_token_loss_backward("grpo", new_logp, old_logp, advantages.detach().reshape(-1),
-                                         loss_scale=loss_scale, lengths=full, clip_range=eps)
+                                         loss_scale=loss_scale, lengths=full, clip_range=eps, adv_per_token=False)
         vals = mvec.tolist()  # the step's only device-to-host copy
         metrics: Dict[str, Any] = {k: vals[slot] for k, slot in GRPO_METRICS.items()}
         metrics.update(policy_loss=vals[N.M_LOSS], clip_range=float(eps))

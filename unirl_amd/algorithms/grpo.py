@@ -113,7 +113,7 @@ class GRPO(StageAlgorithm):
         mvec = fused_token_loss_backward(
             "grpo", new_logp, segment.log_probs, advantages, loss_scale=loss_scale,
             cu_seqlens=cu_seqlens_from_lengths(segment.lengths, new_logp.device), loss_agg_mode=mode,
-            horizon=self.horizon, clip_range=clip_range, clip_range_high=clip_high,
+            horizon=self.horizon, clip_range=clip_range, clip_range_high=clip_high, adv_per_token=False,
         )
 
         vals = mvec.tolist()  # the step's only device-to-host copy

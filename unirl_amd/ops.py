@@ -781,6 +781,7 @@ class RatioLossPlan:
         drpo_epsilon: float = 12.5,
         mu_weighted: bool = True,
         horizon: float = 8192,
+        adv_per_token: Optional[bool] = None,
     ) -> None:
         N.require_device(new_logp, "new_logp")
         if new_logp.shape != old_logp.shape:
@@ -812,11 +813,14 @@ class RatioLossPlan:
             self.n_seq = self.seq.numel() - 1
             if self.n_seq < 0:
                 raise ValueError("cu_seqlens needs n_seq + 1 entries")
-        if adv.shape == self.nw.shape or (adv.numel() == self.n_tok and self.seq is None):
-            adv_per_token = True
-        elif self.seq is not None and adv.numel() == self.n_seq:
-            adv_per_token = False
-        else:
+        # One advantage per sequence, as the reference's algorithms pass them, or one per token.
+        # A packed batch with as many tokens as sequences fits both readings: per sequence wins
+        # unless `adv_per_token` says otherwise.
+        fits_seq = self.seq is not None and adv.numel() == self.n_seq
+        fits_tok = adv.shape == self.nw.shape or (adv.numel() == self.n_tok and self.seq is None)
+        if adv_per_token is None:
+            adv_per_token = fits_tok and not fits_seq
+        if not (fits_tok if adv_per_token else fits_seq):
             raise ValueError(
                 f"advantages {tuple(advantages.shape)} match neither the tokens {self.shape} "
                 f"nor the {self.n_seq} sequences"
