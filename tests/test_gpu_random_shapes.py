@@ -30,7 +30,7 @@ def rand_shape(rng, max_elems=6000):
             return shape
 
 
-@pytest.mark.parametrize("seed", range(6))
+@pytest.mark.parametrize("seed", range(10))
 def test_sde_step_random(dev, seed):
     from unirl_amd import sde
 
@@ -66,7 +66,7 @@ def test_sde_step_random(dev, seed):
         assert_close(lps[:, 2], r_lp, rtol, 2e-6, what + " (stack replay)")
 
 
-@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("seed", range(8))
 def test_token_logp_random(dev, seed):
     from unirl_amd import models
 
@@ -88,7 +88,7 @@ def test_token_logp_random(dev, seed):
         assert_close(ent, ref_ent, 2e-5, 2e-6, what + " entropy")
 
 
-@pytest.mark.parametrize("seed", range(4))
+@pytest.mark.parametrize("seed", range(12))
 def test_ratio_loss_random(dev, seed):
     from unirl_amd.algorithms import fused_token_loss
 
@@ -127,7 +127,7 @@ def test_ratio_loss_random(dev, seed):
         assert_close(nd2.grad, npk.grad, 2e-5, 2e-6 * gmax, what + " packed grad")
 
 
-@pytest.mark.parametrize("seed", range(3))
+@pytest.mark.parametrize("seed", range(6))
 def test_kl_mask_random(dev, seed):
     from unirl_amd import ops
 
