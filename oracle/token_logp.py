@@ -2,7 +2,9 @@
 
 Log-prob follows unirl/models/qwen3/ar.py:78-85: ``lf = logits.float()/T`` (T<=0
 means 1), ``lf[tok] - logsumexp(lf)``.  The reference computes no entropy; it is
-defined here as ``H = logsumexp(lf) - sum softmax(lf)*lf``.
+defined here as ``H = logsumexp(lf) - sum softmax(lf)*lf`` with ``0 * log 0 = 0``: a logit of
+-inf (a masked token) has probability 0 and contributes nothing, the convention of
+``torch.distributions.Categorical``.
 """
 
 from __future__ import annotations
@@ -26,7 +28,8 @@ def token_entropy(logits: torch.Tensor, temperature: float = 1.0) -> torch.Tenso
     lf = (logits.float() / T).double()
     lse = torch.logsumexp(lf, dim=-1)
     p = torch.softmax(lf, dim=-1)
-    return (lse - (p * lf).sum(dim=-1)).float()
+    terms = torch.where(p == 0, torch.zeros_like(p), p * lf)  # p == 0 is False for NaN: NaN rows stay NaN
+    return (lse - terms.sum(dim=-1)).clamp_min(0.0).float()  # clamp keeps NaN
 
 
 def token_entropy_fp32(logits: torch.Tensor, temperature: float = 1.0) -> torch.Tensor:

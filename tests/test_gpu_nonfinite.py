@@ -118,6 +118,144 @@ def test_flowdppo_loss_nonfinite(dev, case):
         same(m[k], r, f"flowdppo {k} [{case}]", rtol=2e-3 if "kl_new_old" in k else 2e-5, atol=1e-6)
 
 
+def test_token_rows_where_a_nan_precedes_every_finite_logit(dev):
+    """A wavefront that has met nothing but -inf and NaN sums nothing yet; the NaN must survive
+    until the row's result (three-element rows put each element into a scan step of its own)."""
+    from unirl_amd import models
+
+    x = torch.tensor([[0.5, 1.0, -1.0], [NAN, 3.0, 1.25], [-INF, NAN, 2.0], [NAN, -INF, -INF], [-INF, 0.25, NAN]])
+    ids = torch.tensor([0, 1, 2, 0, 1])
+    for dtype in (torch.float32, torch.bfloat16):
+        xd = x.to(dtype)
+        lp, ent = models.token_logp_entropy(xd.to(dev), ids.to(dev), 0.7)
+        same(lp, otok.token_logp(xd, ids, 0.7), f"log-prob {dtype}", 2e-5, 2e-6)
+        same(ent, otok.token_entropy(xd, 0.7), f"entropy {dtype}", 2e-5, 2e-6)
+    big = torch.randn(3, 5000)
+    big[1, :700] = NAN          # the first chunks of several wavefronts hold nothing but NaN
+    big[2, :300] = -INF
+    big[2, 17] = NAN
+    ids = torch.tensor([5, 4000, 4000])
+    lp, ent = models.token_logp_entropy(big.to(dev), ids.to(dev), 1.0)
+    same(lp, otok.token_logp(big, ids), "log-prob, long rows", 2e-5, 2e-6)
+    same(ent, otok.token_entropy(big), "entropy, long rows", 2e-5, 2e-6)
+
+
+def _poison(rng, t, values):
+    t = t.clone()
+    flat = t.view(-1)
+    for _ in range(rng.randint(1, 3)):
+        flat[rng.randrange(flat.numel())] = rng.choice(values)
+    return t
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_nonfinite_injection(dev, seed):
+    """One to three NaN / +-inf / overflowing values dropped at random into otherwise ordinary
+    inputs of every kernel: NaN positions, infinities and the finite rest follow the oracle."""
+    import random
+    import warnings
+
+    from unirl_amd import models, ops, sde
+    from unirl_amd.algorithms import fused_token_loss
+    from unirl_amd.algorithms._fused import ABSDIFF_METRICS, DRPO_METRICS, GRPO_METRICS
+
+    rng = random.Random(7000 + seed)
+    sig = osch.sigma_schedule(28, 3.0)
+    for _ in range(6):
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        # token log-prob and entropy (|logits| stay small: the reference's `chosen - logsumexp`
+        # itself loses digits to cancellation at logits of 1e4)
+        rows, V = rng.randint(1, 5), rng.choice((3, 8, 65, 300, 2049))
+        dtype, T = rng.choice((torch.float32, torch.bfloat16, torch.float16)), rng.choice((1.0, 0.7))
+        x = _poison(rng, 3 * torch.randn(rows, V, generator=g), (NAN, INF, -INF, 100.0, -200.0)).to(dtype)
+        ids = torch.randint(0, V, (rows,), generator=g)
+        bad = (~torch.isfinite(x.float())).nonzero()
+        if len(bad) and rng.random() < 0.5:
+            ids[bad[0, 0]] = bad[0, 1]  # the target is the poisoned token
+        lp, ent = models.token_logp_entropy(x.to(dev), ids.to(dev), T)
+        what = f"token [{rows},{V}] {dtype} T={T}"
+        same(lp, otok.token_logp(x, ids, T), what + " log-prob", 2e-5, 2e-5)
+        same(ent, otok.token_entropy(x, T), what + " entropy", 2e-5, 2e-6)
+
+        # ratio losses, padded and packed
+        n_seq, max_len = rng.randint(1, 6), rng.choice((3, 4, 8, 31, 64, 257))
+        kind, mode = rng.choice(("grpo", "drpo")), rng.choice(("token-mean", "seq-mean-token-sum-norm"))
+        old = -8 * torch.rand(n_seq, max_len, generator=g)
+        new = old + 0.3 * torch.randn(n_seq, max_len, generator=g)
+        lengths = torch.randint(1, max_len + 1, (n_seq,), generator=g)
+        adv = torch.randn(n_seq, generator=g)
+        which = rng.choice(("new", "old", "adv"))
+        if which == "new":
+            new = _poison(rng, new, (NAN, INF, -INF, 100.0, -200.0, 0.0))
+        elif which == "old":
+            old = _poison(rng, old, (NAN, INF, -INF, 100.0, -200.0, 0.0))
+        else:
+            adv = _poison(rng, adv, (NAN, INF, -INF, 0.0))
+        newp, oldp = olos.pack_padded(new, lengths), olos.pack_padded(old, lengths)
+        ref_loss, ref_m = olos.token_loss(kind, newp, oldp, adv, lengths, mode=mode, horizon=max_len, clip_range=0.2,
+                                          clip_range_high=0.28, epsilon=5.0)
+        cu = torch.cat([torch.zeros(1, dtype=torch.int64), lengths.cumsum(0)])
+        kw = dict(loss_agg_mode=mode, horizon=max_len, clip_range=0.2, clip_range_high=0.28, drpo_epsilon=5.0,
+                  adv_per_token=False)
+        slots = dict(GRPO_METRICS if kind == "grpo" else DRPO_METRICS)
+        slots.update(ABSDIFF_METRICS)
+        for layout in ("padded", "packed"):
+            if layout == "padded":
+                loss, mvec = fused_token_loss(kind, new.to(dev), old.to(dev), adv.to(dev), lengths=lengths.to(dev), **kw)
+            else:
+                loss, mvec = fused_token_loss(kind, newp.to(dev), oldp.to(dev), adv.to(dev), cu_seqlens=cu.to(dev), **kw)
+            what = f"{kind} {mode} [{n_seq},{max_len}] {layout}, poisoned {which}"
+            same(loss, ref_loss, what + " loss", 3e-5, 1e-5)
+            got = mvec.cpu()
+            for name, slot in slots.items():
+                if name in ref_m:
+                    atol = 2.0 / newp.numel() + 1e-6 if "clip" in name else 1e-5
+                    same(got[slot], ref_m[name], f"{what} {name}", 3e-5, atol)
+
+        # Gaussian KL and mask
+        B, S, inner = rng.randint(1, 3), rng.randint(1, 3), (rng.randint(1, 9), rng.randint(1, 40))
+        dtype = rng.choice((torch.float32, torch.bfloat16, torch.float16))
+        base = torch.randn((B, S) + inner, generator=g)
+        p = base + 0.02 * torch.randn(base.shape, generator=g)
+        q = base + 0.02 * torch.randn(base.shape, generator=g)
+        if rng.random() < 0.5:
+            p = _poison(rng, p, (NAN, INF, -INF, 1e30, 60000.0))
+        else:
+            q = _poison(rng, q, (NAN, INF, -INF, 1e30, 60000.0))
+        p, q = p.to(dtype), q.to(dtype)
+        sg = (0.1 + torch.rand(S, generator=g)).view(1, S, 1, 1)
+        ref = ofd.kl_per_sample(p, q, sg)
+        kl, mask = ops.gaussian_kl_mask(p.to(dev), q.to(dev), sg.to(dev), 0.01)
+        same(kl, ref, f"kl {tuple(base.shape)} {dtype}", 2e-5 if dtype == torch.float32 else 2e-3, 1e-9)
+        sure = ~torch.isfinite(ref) | ((ref - 0.01).abs() > 1e-5)
+        assert torch.equal(mask.cpu().bool()[sure], (ref < 0.01)[sure])
+
+        # SDE transition and log-prob
+        shape, kind = (rng.randint(1, 3), rng.randint(1, 9), rng.randint(1, 40)), rng.choice(("flow", "dance", "cps"))
+        i, eta = rng.randint(0, 27), rng.choice((0.3, 0.7, 1.0))
+        xs, v, n = (torch.randn(shape, generator=g) for _ in range(3))
+        which = rng.choice("xvn")
+        vals = (NAN, INF, -INF, 100.0, 3.0e38, 0.0)
+        xs, v, n = (_poison(rng, t, vals) if name == which else t for name, t in zip("xvn", (xs, v, n)))
+        r_prev, r_lp, r_mean = osde.sde_denoise(kind, v, xs, sig[i], sig[i + 1], eta=eta, noise=n, sigma_max=sig[1],
+                                                ieee_sqrt=True)
+        prev, lp, mean = sde.STRATEGIES[kind]().denoise(v.to(dev), xs.to(dev), sig[i].to(dev), sig[i + 1].to(dev), eta=eta,
+                                                        sigma_max=sig[1].to(dev), noise=n.to(dev))
+        what = f"sde {kind} {shape} step {i} eta {eta}, poisoned {which}"
+        same(mean, r_mean, what + " mean", 1e-6, 0)
+        same(prev, r_prev, what + " prev", 1e-6, 0)
+        same(lp, r_lp, what + " log-prob", 3e-5, 2e-6)
+
+        # group-normalised advantages
+        G, b = rng.randint(1, 8), rng.randint(1, 6)
+        r = _poison(rng, torch.randn(G * b, generator=g), (NAN, INF, -INF, 1e-45))
+        akw = dict(normalize=rng.random() < 0.7, scope=rng.choice(("group", "global")), use_global_std=rng.random() < 0.3)
+        with warnings.catch_warnings():
+            warnings.simplefilter("ignore")  # torch warns about std() of a single element
+            ref = oadv.compute_advantages(r, [j // b for j in range(G * b)], **akw)
+        same(ops.group_advantages(r.to(dev), G, **akw), ref, f"advantages G={G} b={b} {akw}", 3e-5, 2e-6)
+
+
 def test_token_logp_nonfinite_rows(dev):
     from unirl_amd import models
 

@@ -67,6 +67,26 @@ def test_against_float64_brute_force():
     assert torch.equal(a, otok.token_logp(x, ids, 0.7)) and torch.equal(b, otok.token_entropy(x, 0.7))
 
 
+def test_entropy_of_masked_logits_follows_categorical():
+    """A -inf logit (a masked token) has probability 0 and adds nothing to the entropy: the value is
+    that of the remaining tokens, as ``torch.distributions.Categorical`` computes it; a row with
+    one finite logit has entropy 0; NaN and +inf logits give NaN."""
+    x, _ = _logits(6, 40, 9)
+    x[0, 3] = x[0, 17] = -math.inf
+    x[1, :] = -math.inf
+    x[1, 2] = 1.5
+    x[2, ::2] = -math.inf
+    ent = otok.token_entropy(x[:3], 0.7)
+    ref = torch.distributions.Categorical(logits=(x[:3] / 0.7).double()).entropy()
+    assert torch.allclose(ent.double(), ref, rtol=1e-6, atol=1e-9)
+    kept = x[0][torch.isfinite(x[0])]
+    assert abs(float(ent[0]) - float(otok.token_entropy(kept[None], 0.7))) < 1e-6  # the masked entries drop out
+    assert float(ent[1]) == 0.0
+    x[4, 5] = math.nan
+    x[5, 1] = math.inf
+    assert bool(torch.isnan(otok.token_entropy(x[4:])).all())
+
+
 # ---------------------------------------------------------------- GRPO clip loss
 def _logps(n, seed=0, scale=0.05, dtype=torch.float32):
     g = torch.Generator().manual_seed(seed)

@@ -66,10 +66,7 @@ __device__ __forceinline__ float tok_exp2(float a) { return __builtin_amdgcn_exp
 __device__ __forceinline__ void tok_raise(float& m, float& r, TokAcc& acc, float M, float c) {
   if (m == M) return;
   const float R = M * c;
-  if (m == -INFINITY) {
-    acc.s = 0.0f;
-    acc.t = 0.0f;
-  } else {
+  if (m != -INFINITY) {
     // the former maxima become ordinary terms: each is 2^r0 with a = r0
     const float r0 = fmaf(m, c, -r);
     const float e0 = acc.cnt * tok_exp2(r0);
@@ -79,7 +76,7 @@ __device__ __forceinline__ void tok_raise(float& m, float& r, TokAcc& acc, float
     const float f = tok_exp2(delta);
     acc.s = f * s_all;
     acc.t = f * fmaf(delta, s_all, t_all);
-  }
+  }  // else nothing has been summed yet: s and t are 0, or s carries the NaN mark of tok_update
   acc.cnt = 0.0f;
   m = M;
   r = R;
@@ -112,15 +109,23 @@ __device__ __forceinline__ void tok_update(TokRef& ref, TokAcc& acc, const float
         }
       }
     }
-  } else if (active && ref.m != -INFINITY) {
+  } else if (ref.m != -INFINITY) {
+    if (active) {
 #pragma unroll
-    for (int k = 0; k < N; ++k) {
-      float a = fmaf(x[k], c, -ref.r);
-      if (SAFE) a = (a < -FLT_MAX) ? -FLT_MAX : a;  // -inf logit: e = 0 and e*a = 0; NaN stays NaN
-      const float e = tok_exp2(a);
-      acc.s += e;
-      acc.t = fmaf(e, a, acc.t);
+      for (int k = 0; k < N; ++k) {
+        float a = fmaf(x[k], c, -ref.r);
+        if (SAFE) a = (a < -FLT_MAX) ? -FLT_MAX : a;  // -inf logit: e = 0 and e*a = 0; NaN stays NaN
+        const float e = tok_exp2(a);
+        acc.s += e;
+        acc.t = fmaf(e, a, acc.t);
+      }
     }
+  } else if (active) {
+    // The wavefront has met nothing but -inf and NaN so far, and so nothing is summed: a NaN has
+    // to be remembered by hand (the maximum above dropped it).  Rare: the start of a masked row.
+#pragma unroll
+    for (int k = 0; k < N; ++k)
+      if (x[k] != x[k]) acc.s = x[k];
   }
 }
 
@@ -358,7 +363,10 @@ __global__ __launch_bounds__(TPB) void token_logp_entropy_kernel(TokArgs A) {
   const double ln_sum = r0 * kLn2 + log(cnt) + log1p((double)st.s * exp2(-r0) / cnt);
   const double t_all = (double)st.t + e0 * r0;
   if (A.lse) A.lse[row] = (float)(kLn2 * (double)st.r + ln_sum);
-  if (A.ent) A.ent[row] = (float)(ln_sum - kLn2 * t_all / sum);
+  if (A.ent) {
+    const double h = ln_sum - kLn2 * t_all / sum;
+    A.ent[row] = (float)(h < 0.0 ? 0.0 : h);  // rounding may leave -1e-21 when one logit holds all the mass; NaN stays
+  }
   if (A.logp) {
     float out = __uint_as_float(0x7fc00000u);
     if (id >= 0 && id < V) {
