@@ -79,6 +79,53 @@ def test_grpo_micro_step(dev, mode):
     assert_close(stage.theta.grad, cpu.theta.grad, 1e-5, 1e-8, "d loss / d theta")
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_ar_micro_steps_on_random_segments(dev, seed):
+    """GRPO and DRPO micro-steps on segments of random size, among them segments with as many
+    tokens as sequences (the per-sample advantages must not be mistaken for per-token ones)."""
+    import random
+
+    from unirl_amd.algorithms import DRPO, GRPO
+
+    rng = random.Random(500 + seed)
+    for case in range(6):
+        n_seq, max_len = rng.randint(1, 14), rng.choice((1, 2, 3, 8, 60, 300))
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        lengths = torch.randint(0, max_len + 1, (n_seq,), generator=g)
+        if case == 0:  # n_tok == n_seq with unequal lengths
+            lengths = torch.zeros(n_seq, dtype=torch.int64)
+            lengths[0] = n_seq
+        if int(lengths.sum()) == 0:
+            lengths[-1] = max_len
+        n_tok = int(lengths.sum())
+        old = -6 * torch.rand(n_tok, generator=g)
+        base = old + 0.05 * torch.randn(n_tok, generator=g)
+        direction = 0.3 * torch.randn(n_tok, generator=g)
+        adv = torch.randn(n_seq, generator=g)
+        kind = rng.choice(("grpo", "drpo"))
+        mode = rng.choice(("token-mean", "seq-mean-token-sum-norm"))
+        scale = rng.choice((1.0, 0.25))
+        cpu = FakeARStage(base, direction, torch.device("cpu"))
+        new = cpu.replay(None, segment=None, temperature=1.0)
+        ref_loss, ref_m = olos.token_loss(kind, new, old, adv, lengths, mode=mode, horizon=64, clip_range=0.2,
+                                          clip_range_high=0.28, epsilon=12.5)
+        (ref_loss * scale).backward()
+        stage = FakeARStage(base, direction, dev)
+        if kind == "grpo":
+            algo = GRPO(stage=stage, clip_range=0.2, clip_range_high=0.28, loss_agg_mode=mode, horizon=64)
+        else:
+            algo = DRPO(pipeline=types.SimpleNamespace(ar=stage), loss_agg_mode=mode, horizon=64)
+        seg = text_segment(torch.zeros(n_tok, dtype=torch.int64, device=dev), lengths, old.to(dev))
+        res = algo.compute_loss_and_backward(conditions={}, segment=seg, advantages=adv.to(dev), training_progress=0.0,
+                                             loss_scale=scale)
+        what = f"{kind} {mode} lengths {lengths.tolist()}"
+        assert abs(res.loss - float(ref_loss)) <= 2e-5 * abs(float(ref_loss)) + 2e-6 * float(adv.abs().max()), what
+        for k, v in ref_m.items():
+            if k in res.metrics:
+                assert abs(res.metrics[k] - float(v)) <= 2e-5 * abs(float(v)) + 2.0 / n_tok * ("clip" in k) + 1e-6, (what, k)
+        assert_close(stage.theta.grad, cpu.theta.grad, 2e-5, 1e-7, what + ": d loss / d theta")
+
+
 def test_drpo_micro_step_with_mask_and_replay_anchor(dev):
     from unirl_amd.algorithms import DRPO
 
