@@ -71,6 +71,21 @@ def test_argument_errors_return_statuses_without_launching(built_lib):
                                   None) == -3
     assert L.unirl_group_advantages(None, 2, 2, 1, 1e-8, 0, 0, None, None) == -1
     assert L.unirl_group_advantages(None, 0, 2, 1, 1e-8, 0, 0, None, None) == 0
+    good = N.RatioLossParams(kind=N.LOSS_GRPO, agg_mode=N.AGG_TOKEN_MEAN, clip_low=0.2, clip_high=0.2, adv_per_token=1)
+    fake = ctypes.c_void_p(0x10000)
+    # the one-pass step: no gradient buffer, no workspace, a flat layout with per-sequence advantages
+    assert L.unirl_ratio_loss_fwd_bwd(fake, fake, fake, None, None, 0, 0, 8, ctypes.byref(good), 1.0, -1, None, fake,
+                                      fake, 1 << 30, None) == -1
+    assert L.unirl_ratio_loss_fwd_bwd(fake, fake, fake, None, None, 0, 0, 8, ctypes.byref(good), 1.0, -1, fake, fake,
+                                      None, 0, None) == -4
+    good.adv_per_token = 0
+    assert L.unirl_ratio_loss_fwd_bwd(fake, fake, fake, None, None, 0, 0, 8, ctypes.byref(good), 1.0, -1, fake, fake,
+                                      fake, 1 << 30, None) == -1
+    # the Flow-DPPO loss step: row limit, NULL outputs
+    assert L.unirl_flowdppo_step(fake, fake, N.BF16, fake, 1, 1 << 20, 64, fake, fake, fake, 0.01, 1.0, fake, fake,
+                                 None, fake, fake, 1 << 30, None) == -6
+    assert L.unirl_flowdppo_step(fake, fake, N.BF16, fake, 1, 4, 64, fake, fake, fake, 0.01, 1.0, fake, None, None,
+                                 fake, fake, 1 << 30, None) == -1
     # misaligned pointer
     assert L.unirl_token_logp_entropy(ctypes.c_void_p(0x1001), N.BF16, 1, 10, 10, ctypes.c_void_p(0x1000), 1.0,
                                       ctypes.c_void_p(0x2000), None, None, None) == -5
