@@ -87,10 +87,9 @@ class GRPO(StageAlgorithm):
         training_progress: float,
         loss_scale: float,
     ) -> AlgorithmStepResult:
-        if segment.tokens is None or segment.lengths is None or segment.log_probs is None:
-            return NO_STEP
-        if int(segment.tokens.shape[0]) == 0:
-            return NO_STEP
+        stored = (segment.tokens, segment.lengths, segment.log_probs)
+        if any(t is None for t in stored) or int(segment.tokens.shape[0]) == 0:
+            return NO_STEP  # nothing recorded for this stage, or an empty micro-batch
 
         new_logp = self.stage.replay(
             typed_conditions(conditions, self.conditions_cls), segment=segment, temperature=self.sampling_temperature
@@ -100,11 +99,10 @@ class GRPO(StageAlgorithm):
             raise ValueError(
                 f"GRPO advantage expansion: advantages batch={bs} != lengths={int(segment.lengths.shape[0])}"
             )
-        clip_range = _resolve_clip_range_from_schedule(self.clip_range, self.clip_schedule, training_progress)
-        clip_high = (
-            None
-            if self.clip_range_high is None
-            else _resolve_clip_range_from_schedule(self.clip_range_high, self.clip_schedule, training_progress)
+        # both epsilons follow the schedule; no upper epsilon means a symmetric clip
+        clip_range, clip_high = (
+            None if eps is None else _resolve_clip_range_from_schedule(eps, self.clip_schedule, training_progress)
+            for eps in (self.clip_range, self.clip_range_high)
         )
         mode = self.loss_agg_mode
         if mode not in ("seq-mean-token-sum-norm", "seq-mean-token-mean"):
