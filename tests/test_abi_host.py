@@ -246,3 +246,30 @@ def test_bench_refuses_more_than_one_gpu():
     assert r.returncode != 0
     assert "ONE GPU" in (r.stderr + r.stdout)
     assert not r.stdout.strip().startswith("{")  # no result line
+
+
+def test_header_is_plain_c_and_a_c_program_links(built_lib, tmp_path):
+    """The boundary is a C ABI: the header compiles as C99 (no C++ in it), and a C program linked
+    against the library alone (no torch, no Python) reads its version and a status string."""
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no C compiler on this host")
+    src = tmp_path / "abi.c"
+    src.write_text(
+        '#include <string.h>\n#include "unirl_hip.h"\n'
+        "int main(void) {\n"
+        "  if (unirl_abi_version() != UNIRL_ABI_VERSION) return 1;\n"
+        '  if (strcmp(unirl_status_string(UNIRL_OK), "ok") != 0) return 2;\n'
+        "  if (unirl_workspace_bytes() < 65536) return 3;\n"
+        "  /* argument errors come back as statuses before anything touches a device */\n"
+        "  if (unirl_token_logp_entropy(0, UNIRL_BF16, 1, 10, 10, 0, 1.0f, 0, 0, 0, 0) != UNIRL_E_NULL) return 4;\n"
+        "  return 0;\n}\n"
+    )
+    exe = tmp_path / "abi"
+    lib_dir = str(Path(built_lib).parent)
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", f"-I{HEADER.parent}", str(src),
+                    f"-L{lib_dir}", "-lunirl_hip", f"-Wl,-rpath,{lib_dir}", "-o", str(exe)], check=True)
+    assert subprocess.run([str(exe)]).returncode == 0
