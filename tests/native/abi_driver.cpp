@@ -1,0 +1,326 @@
+// A C++ program that uses the library the way a non-Python host would: hipMalloc'd buffers, the
+// C ABI of include/unirl_hip.h, nothing else (no torch, no Python).  Each entry point of the hot
+// path is called on small seeded inputs and checked against a float64 evaluation of the
+// reference's formula written out below (file:line cited per check).  Exit status 0 = all
+// checks passed; every check prints one line.  Test infrastructure, not part of the product.
+//
+// Build (tests/native/build.py):  hipcc --offload-arch=gfx950 -Iinclude abi_driver.cpp -L... -lunirl_hip
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <vector>
+
+#include "unirl_hip.h"
+
+namespace {
+
+int g_failures = 0;
+
+#define HIP_OK(call)                                                                  \
+  do {                                                                                \
+    hipError_t e_ = (call);                                                           \
+    if (e_ != hipSuccess) {                                                           \
+      std::printf("HIP error %d at %s:%d\n", (int)e_, __FILE__, __LINE__);           \
+      std::exit(2);                                                                   \
+    }                                                                                 \
+  } while (0)
+
+struct Rng {  // 64-bit LCG; uniform() in [0,1), normal() by Box-Muller
+  uint64_t s;
+  explicit Rng(uint64_t seed) : s(seed * 2862933555777941757ull + 3037000493ull) {}
+  double uniform() {
+    s = s * 6364136223846793005ull + 1442695040888963407ull;
+    return (double)(s >> 11) * (1.0 / 9007199254740992.0);
+  }
+  double normal() {
+    double u = uniform(), v = uniform();
+    if (u < 1e-300) u = 1e-300;
+    return std::sqrt(-2.0 * std::log(u)) * std::cos(6.283185307179586 * v);
+  }
+};
+
+uint16_t to_bf16(float f) {  // round to nearest even
+  uint32_t u;
+  std::memcpy(&u, &f, 4);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+float from_bf16(uint16_t h) {
+  uint32_t u = (uint32_t)h << 16;
+  float f;
+  std::memcpy(&f, &u, 4);
+  return f;
+}
+
+template <typename T>
+struct DevBuf {
+  T* p = nullptr;
+  size_t n = 0;
+  explicit DevBuf(size_t count) : n(count) { HIP_OK(hipMalloc((void**)&p, (count ? count : 1) * sizeof(T))); }
+  explicit DevBuf(const std::vector<T>& h) : DevBuf(h.size()) {
+    if (n) HIP_OK(hipMemcpy(p, h.data(), n * sizeof(T), hipMemcpyHostToDevice));
+  }
+  ~DevBuf() { (void)hipFree(p); }
+  std::vector<T> host() const {
+    std::vector<T> h(n);
+    if (n) HIP_OK(hipMemcpy(h.data(), p, n * sizeof(T), hipMemcpyDeviceToHost));
+    return h;
+  }
+  DevBuf(const DevBuf&) = delete;
+  DevBuf& operator=(const DevBuf&) = delete;
+};
+
+void expect_close(const char* what, double got, double ref, double rtol, double atol) {
+  const double err = std::fabs(got - ref);
+  if (!(err <= rtol * std::fabs(ref) + atol)) {
+    std::printf("FAIL %s: got %.9g, expected %.9g\n", what, got, ref);
+    ++g_failures;
+  }
+}
+void expect_status(const char* what, int rc) {
+  if (rc != 0) {
+    std::printf("FAIL %s: status %d (%s)\n", what, rc, unirl_status_string(rc));
+    ++g_failures;
+  }
+}
+
+// logp = lf[id] - logsumexp(lf), lf = logits.float() / T  (unirl/models/qwen3/ar.py:82-85);
+// entropy = logsumexp(lf) - sum softmax(lf) * lf.
+void check_token_logp(hipStream_t st) {
+  const int64_t rows = 7, V = 4099, stride = V + 5;
+  const float T = 0.7f;
+  Rng rng(11);
+  std::vector<uint16_t> x((size_t)rows * stride);
+  for (auto& v : x) v = to_bf16((float)(2.0 * rng.normal()));
+  x[3 * stride + 17] = to_bf16(15.0f);
+  std::vector<int64_t> ids(rows);
+  for (auto& i : ids) i = (int64_t)(rng.uniform() * V);
+  ids[3] = 17;
+  DevBuf<uint16_t> dx(x);
+  DevBuf<int64_t> dids(ids);
+  DevBuf<float> dlp(rows), dent(rows), dlse(rows);
+  expect_status("unirl_token_logp_entropy",
+                unirl_token_logp_entropy(dx.p, UNIRL_BF16, rows, V, stride, dids.p, T, dlp.p, dent.p, dlse.p, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto lp = dlp.host(), ent = dent.host(), lse = dlse.host();
+  for (int64_t r = 0; r < rows; ++r) {
+    double m = -1e300;
+    std::vector<double> lf(V);
+    for (int64_t j = 0; j < V; ++j) {
+      lf[j] = (double)(from_bf16(x[r * stride + j]) / T);  // the division is fp32 in the reference
+      m = std::fmax(m, lf[j]);
+    }
+    double s = 0.0, t = 0.0;
+    for (int64_t j = 0; j < V; ++j) {
+      const double e = std::exp(lf[j] - m);
+      s += e;
+      t += e * lf[j];
+    }
+    const double ref_lse = m + std::log(s);
+    expect_close("token lse", lse[r], ref_lse, 1e-5, 1e-6);
+    expect_close("token logp", lp[r], lf[ids[r]] - ref_lse, 1e-5, 2e-6);
+    expect_close("token entropy", ent[r], ref_lse - t / s, 1e-5, 2e-6);
+  }
+  std::printf("token log-prob + entropy: checked %lld rows\n", (long long)rows);
+}
+
+// FlowSDEStrategy.step + compute_log_prob, sampling then replay (unirl/sde/kernels.py:207-236, :193-205, :154-177).
+void check_sde_step(hipStream_t st, void* ws, size_t ws_bytes) {
+  const int64_t B = 3, D = 1000;
+  const double sigma = 0.84375006, sigma_next = 0.82258058, eta = 0.7, sigma_max = 0.98780483;
+  Rng rng(12);
+  std::vector<float> x(B * D), v(B * D), n(B * D);
+  for (int64_t i = 0; i < B * D; ++i) {
+    x[i] = (float)rng.normal();
+    v[i] = (float)rng.normal();
+    n[i] = (float)rng.normal();
+  }
+  const std::vector<float> sg = {(float)sigma}, sn = {(float)sigma_next};
+  DevBuf<float> dx(x), dv(v), dn(n), dsg(sg), dsn(sn), dprev(B * D), dmean(B * D), dlp(B), dlp2(B);
+  expect_status("unirl_sde_step_logp (sampling)",
+                unirl_sde_step_logp(dv.p, UNIRL_F32, dx.p, UNIRL_F32, nullptr, dn.p, dsg.p, dsn.p, 0, nullptr,
+                                    (float)sigma_max, eta, UNIRL_SDE_FLOW, B, D, dprev.p, dmean.p, dlp.p, 0, ws,
+                                    ws_bytes, st));
+  expect_status("unirl_sde_step_logp (replay)",
+                unirl_sde_step_logp(dv.p, UNIRL_F32, dx.p, UNIRL_F32, dprev.p, nullptr, dsg.p, dsn.p, 0, nullptr,
+                                    (float)sigma_max, eta, UNIRL_SDE_FLOW, B, D, nullptr, nullptr, dlp2.p, 0, ws,
+                                    ws_bytes, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto prev = dprev.host(), mean = dmean.host(), lp = dlp.host(), lp2 = dlp2.host();
+  const double s = (double)sg[0], s1 = (double)sn[0], dt = s1 - s;
+  const double stdv = std::sqrt(s / (1.0 - (s == 1.0 ? sigma_max : s))) * eta;
+  const double a = 1.0 + stdv * stdv / (2.0 * s) * dt, b = 1.0 + stdv * stdv * (1.0 - s) / (2.0 * s);
+  const double std_var = stdv * std::sqrt(-dt);
+  for (int64_t r = 0; r < B; ++r) {
+    double acc = 0.0;
+    for (int64_t j = 0; j < D; ++j) {
+      const int64_t i = r * D + j;
+      const double m = (double)x[i] * a + (double)v[i] * b * dt;
+      const double p = m + std_var * (double)n[i];
+      expect_close("sde mean", mean[i], m, 2e-6, 2e-6);
+      expect_close("sde prev", prev[i], p, 2e-6, 2e-6);
+      const double d = (double)prev[i] - (double)mean[i];  // the log-prob sees the stored fp32 values
+      acc += -(d * d) / (2.0 * std_var * std_var) - std::log(std_var) - 0.9189385332046727;
+    }
+    expect_close("sde log-prob (sampling)", lp[r], acc / (double)D, 2e-5, 2e-6);
+    expect_close("sde log-prob (replay)", lp2[r], acc / (double)D, 2e-5, 2e-6);
+  }
+  std::printf("sde step + log-prob: checked %lld elements, sampling and replay\n", (long long)(B * D));
+}
+
+// _gaussian_kl_div and the mean / threshold of _flowdppo_kl_adv_loss (unirl/algorithms/flowdppo.py:43-51, :92-96):
+// bf16 subtraction and square, fp32 division, mean over the row.
+void check_kl(hipStream_t st, void* ws, size_t ws_bytes) {
+  const int64_t R = 4, D = 2048;
+  Rng rng(13);
+  std::vector<uint16_t> p(R * D), q(R * D);
+  for (int64_t i = 0; i < R * D; ++i) {
+    const double base = rng.normal();
+    p[i] = to_bf16((float)(base + 0.02 * rng.normal()));
+    q[i] = to_bf16((float)(base + 0.02 * rng.normal()));
+  }
+  const std::vector<float> sig = {0.3f, 0.2f};
+  std::vector<double> ref(R);
+  for (int64_t r = 0; r < R; ++r) {
+    const double den = 2.0 * (double)(sig[r % 2] * sig[r % 2]);
+    double acc = 0.0;
+    for (int64_t j = 0; j < D; ++j) {
+      const float d = from_bf16(to_bf16(from_bf16(p[r * D + j]) - from_bf16(q[r * D + j])));
+      acc += (double)from_bf16(to_bf16(d * d)) / den;
+    }
+    ref[r] = acc / (double)D;
+  }
+  const float thr = (float)(0.5 * (ref[0] + ref[1]));
+  DevBuf<uint16_t> dp(p), dq(q);
+  DevBuf<float> dsig(sig), dkl(R);
+  DevBuf<uint8_t> dmask(R);
+  expect_status("unirl_gaussian_kl_mask", unirl_gaussian_kl_mask(dp.p, dq.p, UNIRL_BF16, dsig.p, 2, R, D, thr, dkl.p,
+                                                                 dmask.p, ws, ws_bytes, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto kl = dkl.host();
+  const auto mask = dmask.host();
+  for (int64_t r = 0; r < R; ++r) {
+    expect_close("gaussian kl", kl[r], ref[r], 1e-5, 1e-12);
+    if (std::fabs(ref[r] - thr) > 1e-5 * thr && (int)mask[r] != (ref[r] < thr ? 1 : 0)) {
+      std::printf("FAIL kl mask row %lld\n", (long long)r);
+      ++g_failures;
+    }
+  }
+  std::printf("gaussian kl + mask: checked %lld rows\n", (long long)R);
+}
+
+// _grpo_clip_loss with the token-mean aggregation on a padded batch (unirl/algorithms/base.py:133-156,
+// grpo.py:148-155), forward and the one-pass forward + backward.
+void check_grpo(hipStream_t st, void* ws, size_t ws_bytes) {
+  const int64_t n_seq = 5, L = 64;
+  const double eps_lo = 0.2, eps_hi = 0.28;
+  Rng rng(14);
+  std::vector<float> nw(n_seq * L), od(n_seq * L), adv(n_seq);
+  std::vector<int64_t> len = {64, 1, 17, 0, 40};
+  for (int64_t i = 0; i < n_seq * L; ++i) {
+    od[i] = (float)(-8.0 * rng.uniform());
+    nw[i] = od[i] + (float)(0.3 * rng.normal());
+  }
+  for (auto& a : adv) a = (float)rng.normal();
+  unirl_ratio_loss_params P;
+  std::memset(&P, 0, sizeof(P));
+  P.kind = UNIRL_LOSS_GRPO;
+  P.agg_mode = UNIRL_AGG_TOKEN_MEAN;
+  P.clip_low = (float)eps_lo;
+  P.clip_high = (float)eps_hi;
+  P.horizon = 8192.0f;
+  P.adv_per_token = 0;
+  DevBuf<float> dnw(nw), dod(od), dadv(adv), dmet(UNIRL_M_COUNT), dmet2(UNIRL_M_COUNT), dgrad(n_seq * L);
+  DevBuf<int64_t> dlen(len);
+  expect_status("unirl_ratio_loss_fwd", unirl_ratio_loss_fwd(dnw.p, dod.p, dadv.p, dlen.p, nullptr, n_seq, L, n_seq * L,
+                                                             &P, nullptr, dmet.p, ws, ws_bytes, st));
+  const float loss_scale = 0.5f;
+  expect_status("unirl_ratio_loss_fwd_bwd",
+                unirl_ratio_loss_fwd_bwd(dnw.p, dod.p, dadv.p, dlen.p, nullptr, n_seq, L, n_seq * L, &P, loss_scale, -1,
+                                         dgrad.p, dmet2.p, ws, ws_bytes, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto met = dmet.host(), met2 = dmet2.host(), grad = dgrad.host();
+  const double lo = (double)(float)(1.0 - eps_lo), hi = (double)(float)(1.0 + eps_hi);
+  double N = 0.0, loss = 0.0, rsum = 0.0, kl = 0.0, clip = 0.0;
+  std::vector<double> gref(n_seq * L, 0.0);
+  for (int64_t r = 0; r < n_seq; ++r) N += (double)len[r];
+  for (int64_t r = 0; r < n_seq; ++r) {
+    for (int64_t j = 0; j < len[r]; ++j) {
+      const int64_t i = r * L + j;
+      const double ld = (double)(nw[i] - od[i]), ratio = std::exp(ld), A = (double)adv[r];
+      const double u = -A * ratio, c = -A * std::fmin(std::fmax(ratio, lo), hi);
+      loss += std::fmax(u, c);
+      rsum += ratio;
+      kl += 0.5 * ld * ld;
+      clip += (ratio - 1.0 > eps_hi || 1.0 - ratio > eps_lo) ? 1.0 : 0.0;
+      const bool inside = ratio >= lo && ratio <= hi;
+      gref[i] = (u >= c ? u : (inside ? c : 0.0)) * (double)loss_scale / N;  // ties do not occur on these inputs
+    }
+  }
+  expect_close("grpo loss", met[UNIRL_M_LOSS], loss / N, 2e-5, 1e-6);
+  expect_close("grpo ratio_mean", met[UNIRL_M_RATIO_MEAN], rsum / N, 1e-5, 0);
+  expect_close("grpo approx_kl", met[UNIRL_M_APPROX_KL], kl / N, 2e-5, 1e-9);
+  expect_close("grpo clip_fraction", met[UNIRL_M_CLIP_FRACTION], clip / N, 0, 1.5 / N);
+  expect_close("grpo token count", met[UNIRL_M_NUM_TOKENS], N, 0, 0);
+  for (int k = 0; k < UNIRL_M_COUNT; ++k)
+    if (k <= UNIRL_M_NUM_TOKENS) expect_close("one-pass metrics equal the forward's", met2[k], met[k], 1e-6, 1e-9);
+  for (int64_t i = 0; i < n_seq * L; ++i) expect_close("grpo grad_new", grad[i], gref[i], 3e-5, 1e-9);
+  std::printf("grpo clipped-ratio loss: checked metrics and %lld gradients\n", (long long)(n_seq * L));
+}
+
+// RolloutTrack.compute_advantages (unirl/types/rollout_resp.py:314-333): (r - mean_g) / sqrt(var_pop_g + eps).
+void check_advantages(hipStream_t st) {
+  const int64_t G = 6, b = 5;
+  Rng rng(15);
+  std::vector<float> r(G * b);
+  for (auto& v : r) v = rng.uniform() < 0.5 ? 0.0f : 1.0f;
+  for (int64_t j = 0; j < b; ++j) r[2 * b + j] = 1.0f;  // an all-equal group: exactly 0
+  DevBuf<float> dr(r), dout(G * b);
+  expect_status("unirl_group_advantages", unirl_group_advantages(dr.p, G, b, 1, 1e-8f, 0, 0, dout.p, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto out = dout.host();
+  for (int64_t g = 0; g < G; ++g) {
+    double m = 0.0, var = 0.0;
+    for (int64_t j = 0; j < b; ++j) m += (double)r[g * b + j];
+    m /= (double)b;
+    for (int64_t j = 0; j < b; ++j) var += ((double)r[g * b + j] - m) * ((double)r[g * b + j] - m);
+    var /= (double)b;
+    for (int64_t j = 0; j < b; ++j)
+      expect_close("group advantage", out[g * b + j], ((double)r[g * b + j] - m) / std::sqrt(var + 1e-8), 2e-5, 1e-6);
+  }
+  std::printf("group advantages: checked %lld rewards\n", (long long)(G * b));
+}
+
+}  // namespace
+
+int main() {
+  int n_dev = 0;
+  if (hipGetDeviceCount(&n_dev) != hipSuccess || n_dev < 1) {
+    std::printf("no HIP device\n");
+    return 3;
+  }
+  HIP_OK(hipSetDevice(0));
+  if (unirl_abi_version() != UNIRL_ABI_VERSION) {
+    std::printf("library ABI %d, header ABI %d\n", unirl_abi_version(), UNIRL_ABI_VERSION);
+    return 4;
+  }
+  hipStream_t st;
+  HIP_OK(hipStreamCreate(&st));
+  const size_t ws_bytes = unirl_workspace_bytes();
+  void* ws = nullptr;
+  HIP_OK(hipMalloc(&ws, ws_bytes));
+  check_token_logp(st);
+  check_sde_step(st, ws, ws_bytes);
+  check_kl(st, ws, ws_bytes);
+  check_grpo(st, ws, ws_bytes);
+  check_advantages(st);
+  HIP_OK(hipStreamSynchronize(st));
+  HIP_OK(hipFree(ws));
+  HIP_OK(hipStreamDestroy(st));
+  std::printf(g_failures ? "FAILED: %d checks\n" : "all checks passed\n", g_failures);
+  return g_failures ? 1 : 0;
+}
