@@ -37,7 +37,7 @@ extern "C" {
 
 /* 2: typed gradient outputs in unirl_sde_step_logp_bwd; unirl_ratio_loss_fwd_bwd and
  * unirl_flowdppo_step added. */
-#define UNIRL_ABI_VERSION 2
+#define UNIRL_ABI_VERSION 3
 
 enum unirl_dtype { UNIRL_F32 = 0, UNIRL_BF16 = 1, UNIRL_F16 = 2 };
 
@@ -184,6 +184,34 @@ int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* const* v_ste
                            float sigma_max_val, int kind, int64_t B, int64_t D, float* x_out,
                            float* traj_out, float* logp_out, int logp_sum, void* workspace,
                            size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * One step of the deterministic DPM-Solver-2 sampler: DPM2Strategy.step ->
+ * _dpm_step (unirl/sde/kernels.py:360-471).  No log-prob (the reference
+ * returns None for it).  The caller keeps the solver's state -- the previous
+ * step's x0 prediction -- and derives the step's scalar coefficients from the
+ * sigma schedule the way the reference does (0-dim tensor arithmetic, float64
+ * for the two DPM updates), rounded to f32:
+ *   x0   = sample - sigma * model_output                      (:366-367)
+ *   DDIM   (first / last step)  eps = (sample - one_minus_s*x0) / s;
+ *                               prev = one_minus_t*x0 + sqrt_t2*eps   (:449-453)
+ *   FIRST  (first order)        prev = c1*sample - c2*x0               (:391)
+ *   SECOND (multistep)          D1 = inv_r0*(x0 - x0_prev);
+ *                               prev = c1*sample - c2*x0 - half_c2*D1  (:416-425)
+ * model_output / sample [n] in their dtypes (upcast in registers, as
+ * StepStrategy.denoise's .float()); x0_prev f32 [n], SECOND only; x0_out and
+ * prev_out f32 [n].  x0_out must not alias x0_prev.
+ * ---------------------------------------------------------------------- */
+enum unirl_dpm2_branch { UNIRL_DPM2_DDIM = 0, UNIRL_DPM2_FIRST = 1, UNIRL_DPM2_SECOND = 2 };
+struct unirl_dpm2_coeffs {
+  float sigma;                                 /* sigmas[step] */
+  float one_minus_s, s, one_minus_t, sqrt_t2;  /* DDIM */
+  float c1, c2;                                /* sigma_t/sigma_s, alpha_t*(exp(-h)-1) */
+  float half_c2, inv_r0;                       /* SECOND */
+};
+int unirl_dpm2_step(const void* model_output, int dtype_v, const void* sample, int dtype_x,
+                    const float* x0_prev, int branch, const struct unirl_dpm2_coeffs* coeffs /* host */,
+                    int64_t n, float* x0_out, float* prev_out, void* stream);
 
 /* ------------------------------------------------------------------------
  * Gaussian KL between transition means, reduced per (sample, step), and the

@@ -37,7 +37,7 @@ def test_version_status_strings_and_workspace(built_lib):
     from unirl_amd import _native as N
 
     L = N.lib()
-    assert L.unirl_abi_version() == N.ABI_VERSION == 2
+    assert L.unirl_abi_version() == N.ABI_VERSION == 3
     assert f"#define UNIRL_ABI_VERSION {N.ABI_VERSION}" in (ROOT / "include" / "unirl_hip.h").read_text()
     assert L.unirl_workspace_bytes() >= 64 * 1024
     assert L.unirl_status_string(0) == b"ok"
@@ -154,6 +154,10 @@ def test_strategy_surface():
         obj.init_schedule(torch.ones(3))
     with pytest.raises(TypeError):
         sde.FlowSDEStrategy(None)  # config is keyword-only
+    ode = sde.DPM2Strategy(config=None)
+    assert ode.canonical_name == "dpm2" and isinstance(ode, sde.StepStrategy) and not isinstance(ode, sde.SDEStrategy)
+    ode.init_schedule(torch.linspace(1, 0, 5))
+    ode.reset()
 
 
 def test_clip_schedule():
@@ -273,3 +277,43 @@ def test_header_is_plain_c_and_a_c_program_links(built_lib, tmp_path):
     subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", f"-I{HEADER.parent}", str(src),
                     f"-L{lib_dir}", "-lunirl_hip", f"-Wl,-rpath,{lib_dir}", "-o", str(exe)], check=True)
     assert subprocess.run([str(exe)]).returncode == 0
+
+
+def test_dpm2_coefficients_reproduce_the_oracle_on_the_host():
+    """Branch selection and scalar coefficients of the DPM-Solver-2 step are host logic: evaluated
+    with the kernel's fp32 operation order in torch on the CPU, they reproduce the oracle's
+    trajectory bit for bit, for an fp32 and a float64 schedule and for a solver restarted mid-way."""
+    from oracle import dpm2 as odpm
+    from unirl_amd import _native as N
+    from unirl_amd.sde.kernels import dpm2_coefficients
+
+    def emulate(branch, c, v, x, m1):
+        x0 = x - c.sigma * v
+        if branch == N.DPM2_DDIM:
+            eps = (x - c.one_minus_s * x0) / c.s
+            return x0, c.one_minus_t * x0 + c.sqrt_t2 * eps
+        if branch == N.DPM2_FIRST:
+            return x0, c.c1 * x - c.c2 * x0
+        d1 = c.inv_r0 * (x0 - m1)
+        return x0, (c.c1 * x - c.c2 * x0) - c.half_c2 * d1
+
+    g = torch.Generator().manual_seed(8)
+    for sig, start in ((osch.sigma_schedule(12, 3.0), 0), (osch.sigma_schedule(9, 1.0).double(), 0),
+                       (osch.sigma_schedule(12, 3.0), 4)):
+        solver = odpm.Dpm2Solver(sig)
+        x = torch.randn(3, 50, generator=g)
+        warm, m1, seen = 0, None, []
+        for i in range(start, sig.numel() - 1):
+            v = torch.randn(3, 50, generator=g)
+            want = solver.step(v, x, i)
+            branch, c = dpm2_coefficients(sig, i, warm)
+            seen.append(branch)
+            m1, got = emulate(branch, c, v, x, m1)
+            assert torch.equal(got, want), (i, branch)
+            warm = min(2, warm + 1)
+            x = want
+        n = sig.numel() - 1 - start
+        first = N.DPM2_DDIM if start == 0 else N.DPM2_FIRST
+        assert seen == [first] + [N.DPM2_SECOND] * (n - 2) + [N.DPM2_DDIM]
+    with pytest.raises(IndexError):
+        dpm2_coefficients(osch.sigma_schedule(4, 3.0), 4, 0)

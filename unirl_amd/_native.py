@@ -91,8 +91,19 @@ class SdeStepDesc(Structure):
     ]
 
 
+# enum unirl_dpm2_branch
+DPM2_DDIM, DPM2_FIRST, DPM2_SECOND = 0, 1, 2
+
+
+class Dpm2Coeffs(Structure):
+    """struct unirl_dpm2_coeffs."""
+
+    _fields_ = [(name, c_float) for name in
+                ("sigma", "one_minus_s", "s", "one_minus_t", "sqrt_t2", "c1", "c2", "half_c2", "inv_r0")]
+
+
 # UNIRL_ABI_VERSION of include/unirl_hip.h that the signatures below describe
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _SIGNATURES = {
     "unirl_abi_version": (c_int, []),
@@ -118,6 +129,10 @@ _SIGNATURES = {
         [c_void_p, c_int, POINTER(c_void_p), c_int, POINTER(c_void_p), c_void_p, POINTER(c_double), c_int,
          c_void_p, c_float, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t,
          c_void_p],
+    ),
+    "unirl_dpm2_step": (
+        c_int,
+        [c_void_p, c_int, c_void_p, c_int, c_void_p, c_int, POINTER(Dpm2Coeffs), c_int64, c_void_p, c_void_p, c_void_p],
     ),
     "unirl_gaussian_kl_mask": (
         c_int,

@@ -385,6 +385,47 @@ def sde_rollout_logp(
     return x_out, logp, traj
 
 
+def dpm2_step(
+    model_output: torch.Tensor,
+    sample: torch.Tensor,
+    x0_prev: Optional[torch.Tensor],
+    branch: int,
+    coeffs: "N.Dpm2Coeffs",
+    x0_out: Optional[torch.Tensor] = None,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """One DPM-Solver-2 update: ``(x0 prediction, prev_sample)``, both fp32 in ``sample``'s shape.
+
+    ``x0_prev`` is the previous step's prediction (second-order branch only); ``x0_out`` may name
+    a reusable fp32 buffer for the new one (not ``x0_prev``)."""
+    N.require_device(sample, "sample")
+    if model_output.shape != sample.shape:
+        raise ValueError(f"model_output {tuple(model_output.shape)} != sample {tuple(sample.shape)}")
+    device = sample.device
+    v = model_output.detach().to(device).contiguous()
+    x = sample.detach().contiguous()
+    if v.dtype not in N._DTYPE_CODE:
+        v = v.float()
+    if x.dtype not in N._DTYPE_CODE:
+        x = x.float()
+    m1 = None
+    if branch == N.DPM2_SECOND:
+        if x0_prev is None or x0_prev.shape != sample.shape:
+            raise ValueError("the second-order update needs the previous x0 prediction in the sample's shape")
+        m1 = x0_prev.detach().to(device=device, dtype=torch.float32).contiguous()
+    if x0_out is None or x0_out.shape != sample.shape or x0_out.dtype != torch.float32 or not x0_out.is_contiguous():
+        x0_out = torch.empty(sample.shape, dtype=torch.float32, device=device)
+    if m1 is not None and x0_out.data_ptr() == m1.data_ptr():
+        raise ValueError("x0_out must not alias x0_prev")
+    prev = torch.empty(sample.shape, dtype=torch.float32, device=device)
+    with N.on_device(device):
+        rc = N.lib().unirl_dpm2_step(
+            N.ptr(v), N.dtype_code(v.dtype), N.ptr(x), N.dtype_code(x.dtype), N.ptr(m1), int(branch),
+            ctypes.byref(coeffs), x.numel(), N.ptr(x0_out), N.ptr(prev), N.current_stream(device),
+        )
+    N.check(rc, "unirl_dpm2_step")
+    return x0_out, prev
+
+
 def gaussian_kl_mask(
     p: torch.Tensor,
     q: torch.Tensor,

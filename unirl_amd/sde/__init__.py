@@ -4,6 +4,7 @@ from .kernels import (
     STRATEGIES,
     CPSSDEStrategy,
     DanceSDEStrategy,
+    DPM2Strategy,
     FlowSDEStrategy,
     SDEStrategy,
     StepStrategy,
@@ -15,6 +16,7 @@ from .runtime import calculate_dynamic_mu, get_sigma_schedule
 
 __all__ = [
     "CPSSDEStrategy",
+    "DPM2Strategy",
     "DanceSDEStrategy",
     "FlowSDEStrategy",
     "SDEStrategy",

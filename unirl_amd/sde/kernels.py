@@ -14,8 +14,10 @@ ops and a reduction per call, ``denoise`` here is one kernel launch
 Additions over the reference signature (keyword-only, optional): ``noise`` lets
 the caller supply the sampling noise instead of drawing it inside the step.
 
-The DPM2 ODE solver of the reference (eval-only, no log-prob) is not part of
-this package.
+``DPM2Strategy`` (:474-516, the deterministic second-order sampler: no log-prob,
+``prev_sample_mean`` and ``std_var`` are ``None``) runs its element-wise update as
+one kernel per step (``unirl_dpm2_step``) with the scalar coefficients derived on
+the host from the schedule.
 """
 
 from __future__ import annotations
@@ -24,8 +26,10 @@ import math
 from abc import ABC, abstractmethod
 from typing import Any, ClassVar, Optional, Tuple, Union
 
+import numpy as np
 import torch
 
+from .. import _native as N
 from .. import ops
 
 SigmaMax = Union[float, torch.Tensor]
@@ -324,6 +328,114 @@ class CPSSDEStrategy(SDEStrategy):
 STRATEGIES = {cls.canonical_name: cls for cls in (FlowSDEStrategy, DanceSDEStrategy, CPSSDEStrategy)}
 
 
+def _half_log_snr(sigma: torch.Tensor) -> torch.Tensor:
+    return torch.log(1 - sigma) - torch.log(sigma)
+
+
+def _f32(t: torch.Tensor) -> float:
+    """A 0-dim tensor rounded to fp32: the value torch multiplies an fp32 tensor by."""
+    return float(t.to(torch.float32))
+
+
+def dpm2_coefficients(sigmas: torch.Tensor, step_index: int, warm: int) -> Tuple[int, "N.Dpm2Coeffs"]:
+    """Branch and scalar coefficients of one DPM-Solver-2 step (``_dpm_step``,
+    ``unirl/sde/kernels.py:428-471``) from a host copy of the schedule: the DDIM update on the
+    first and the last step (scalars in the schedule's dtype), else the first-order update until
+    one step has been taken and the multistep second-order update afterwards (scalars in
+    float64, :377-425).  ``warm`` counts the steps taken since the last reset."""
+    n_steps = int(sigmas.shape[0]) - 1
+    i = int(step_index)
+    if not 0 <= i < n_steps:
+        raise IndexError(f"step_index {i} outside the schedule's {n_steps} steps")
+    c = N.Dpm2Coeffs()
+    c.sigma = _f32(sigmas[i])
+    last = i == n_steps - 1
+    if (warm < 1 or last) and (i == 0 or last):
+        t, s = sigmas[i + 1], sigmas[i]
+        c.one_minus_s, c.s, c.one_minus_t = _f32(1 - s), _f32(s), _f32(1 - t)
+        # sqrt(t**2) in the schedule's dtype; numpy's root is correctly rounded on every host
+        c.sqrt_t2 = float(np.float32(np.sqrt((t**2).numpy())))
+        return N.DPM2_DDIM, c
+    sig = sigmas.to(torch.float64)
+    s_t, s_0 = sig[i + 1], sig[i]
+    lam_t, lam_0 = _half_log_snr(s_t), _half_log_snr(s_0)
+    h = lam_t - lam_0
+    growth = (1 - s_t) * (torch.exp(-h) - 1.0)
+    c.c1, c.c2 = _f32(s_t / s_0), _f32(growth)
+    if warm < 1 or last:
+        return N.DPM2_FIRST, c
+    r0 = (lam_0 - _half_log_snr(sig[i - 1])) / h
+    c.inv_r0, c.half_c2 = _f32(1.0 / r0), _f32(0.5 * growth)
+    return N.DPM2_SECOND, c
+
+
+class DPM2Strategy(StepStrategy):
+    """DPM-Solver-2 multistep ODE sampler (deterministic, stateful): ``init_schedule`` before the
+    first step, consecutive ``step_index`` values afterwards.  No log-prob, so it cannot train."""
+
+    canonical_name: ClassVar[str] = "dpm2"
+
+    def __init__(self, *, config: Optional[Any] = None) -> None:
+        del config
+        self.reset()
+
+    def reset(self) -> None:
+        self._sigmas: Optional[torch.Tensor] = None  # host copy of the schedule
+        self._x0: list = [None, None]  # x0 predictions, oldest first; the buffers alternate
+        self._warm = 0
+
+    def init_schedule(self, sigmas: torch.Tensor) -> None:
+        self.reset()
+        self._sigmas = sigmas.detach().cpu()
+
+    def _advance(self, noise_pred: torch.Tensor, sample: torch.Tensor, step_index: int) -> torch.Tensor:
+        if self._sigmas is None:
+            raise RuntimeError("DPM2Strategy requires init_schedule() before stepping.")
+        if not sample.is_cuda:
+            raise RuntimeError(
+                f"DPM2Strategy: sample lives on {sample.device}; the fused kernel runs on a HIP device only "
+                "and there is no CPU fallback"
+            )
+        branch, coeffs = dpm2_coefficients(self._sigmas, step_index, self._warm)
+        older, newer = self._x0
+        x0, prev = ops.dpm2_step(noise_pred, sample, newer, branch, coeffs, x0_out=older)
+        self._x0 = [newer, x0]
+        self._warm = min(2, self._warm + 1)
+        return prev
+
+    def step(
+        self,
+        noise_pred: torch.Tensor,
+        sample: torch.Tensor,
+        sigma: torch.Tensor,
+        sigma_next: torch.Tensor,
+        eta: float = 1.0,
+        prev_sample: Optional[torch.Tensor] = None,
+        generator: Optional[torch.Generator] = None,
+        sigma_max: SigmaMax = 0.99,
+        step_index: int = 0,
+    ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+        del sigma, sigma_next, eta, prev_sample, generator, sigma_max  # the schedule and the index say it all
+        return self._advance(noise_pred, sample, step_index), None, None
+
+    def denoise(
+        self,
+        noise_pred: torch.Tensor,
+        sample: torch.Tensor,
+        sigma: torch.Tensor,
+        sigma_next: torch.Tensor,
+        *,
+        eta: float = 1.0,
+        prev_sample: Optional[torch.Tensor] = None,
+        sigma_max: SigmaMax = 0.99,
+        step_index: int = 0,
+        noise: Optional[torch.Tensor] = None,
+    ) -> Tuple[torch.Tensor, Optional[torch.Tensor], Optional[torch.Tensor]]:
+        """``(prev_sample fp32, None, None)``: an ODE step has no log-prob and no transition mean."""
+        del sigma, sigma_next, eta, prev_sample, sigma_max, noise
+        return self._advance(noise_pred, sample, step_index), None, None
+
+
 def sde_rollout(
     strategy: SDEStrategy,
     latents: torch.Tensor,
@@ -353,6 +465,7 @@ def sde_rollout(
 
 __all__ = [
     "CPSSDEStrategy",
+    "DPM2Strategy",
     "DanceSDEStrategy",
     "FlowSDEStrategy",
     "SDEStrategy",
