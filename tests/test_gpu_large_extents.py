@@ -102,3 +102,58 @@ def test_sde_step_and_kl_rows_past_2g(dev):
     kl2, _ = ops.gaussian_kl_mask(mean.view(2, h), prev.view(2, h), torch.tensor([0.5], device=dev), 0.01,
                                   reduce_from_dim=1)
     assert abs(float(kl[0]) - float(kl2.double().mean())) <= 1e-5 * abs(float(kl[0]))
+
+
+def test_more_rows_than_one_launch_can_index(dev):
+    """70 001 samples / rows of a few elements each: the second grid dimension holds at most 65 535
+    workgroups, so every per-row entry point walks the rows in several launches.  Against the oracle."""
+    from oracle import flowdppo as ofd
+    from oracle import schedule as osch
+    from oracle import sde as osde
+    from oracle import token_logp as otok
+    from tests._util import assert_close
+    from unirl_amd import ops, sde
+
+    R = 70001
+    g = torch.Generator().manual_seed(12)
+    sig = osch.sigma_schedule(28, 3.0)
+    # SDE step, sampling and replay, and its backward
+    x, v, n = (torch.randn(R, 8, generator=g) for _ in range(3))
+    ref_prev, ref_lp, ref_mean = osde.sde_denoise("flow", v, x, sig[10], sig[11], eta=0.7, noise=n, sigma_max=sig[1],
+                                                  ieee_sqrt=True)
+    st = sde.FlowSDEStrategy()
+    vd = v.to(dev).requires_grad_(True)
+    prev, lp, mean = st.denoise(vd, x.to(dev), sig[10].to(dev), sig[11].to(dev), eta=0.7, sigma_max=sig[1].to(dev),
+                                noise=n.to(dev))
+    assert torch.equal(prev.cpu(), ref_prev) and torch.equal(mean.cpu(), ref_mean)
+    assert_close(lp, ref_lp, 1e-5, 2e-6, "log-prob of 70 001 samples")
+    gl = torch.randn(R, generator=g)
+    vr = v.clone().requires_grad_(True)
+    _, rl, _ = osde.sde_denoise("flow", vr, x, sig[10], sig[11], eta=0.7, prev_sample=ref_prev, sigma_max=sig[1])
+    (rl * gl).sum().backward()
+    _, lp2, _ = st.denoise(vd, x.to(dev), sig[10].to(dev), sig[11].to(dev), eta=0.7, sigma_max=sig[1].to(dev),
+                           prev_sample=ref_prev.to(dev))
+    (lp2 * gl.to(dev)).sum().backward()
+    assert_close(vd.grad, vr.grad, 5e-5, 1e-7, "gradient over 70 001 samples")
+    # Gaussian KL and mask, one sigma per row modulo 3
+    base = torch.randn(23334, 3, 8, generator=g)  # 70 002 rows
+    p = (base + 0.02 * torch.randn(base.shape, generator=g)).bfloat16()
+    q = (base + 0.02 * torch.randn(base.shape, generator=g)).bfloat16()
+    sg = torch.tensor([0.3, 0.2, 0.1]).view(1, 3, 1)
+    ref = ofd.kl_per_sample(p, q, sg)
+    kl, _ = ops.gaussian_kl_mask(p.to(dev), q.to(dev), sg.to(dev), 0.01)
+    assert kl.shape == ref.shape and kl.numel() > 65535
+    assert_close(kl, ref, 2e-3, 1e-9, "kl of 70 002 rows")
+    # token log-prob, entropy and backward on 70 001 short rows
+    logits = (2 * torch.randn(R, 24, generator=g)).bfloat16()
+    ids = torch.randint(0, 24, (R,), generator=g)
+    tlp, ent, lse = ops.token_logp_entropy(logits.to(dev), ids.to(dev), 0.7, want_lse=True)
+    assert_close(tlp, otok.token_logp(logits, ids, 0.7), 2e-5, 2e-6, "token log-prob of 70 001 rows")
+    assert_close(ent, otok.token_entropy(logits, 0.7), 2e-5, 2e-6, "entropy of 70 001 rows")
+    lf = logits.float().requires_grad_(True)
+    torch.log_softmax(lf / 0.7, -1).gather(-1, ids[:, None])[:, 0].backward(gl)
+    grad = ops.token_logp_bwd(logits.to(dev), ids.to(dev), 0.7, lse, gl.to(dev))
+    assert_close(grad.float(), lf.grad, 1e-2, 1e-3, "token gradient of 70 001 rows")
+    # gather of 70 001 samples
+    t = torch.randn(R, 3, 4, generator=g)
+    assert torch.equal(ops.gather_steps(t.to(dev), [2, 0]).cpu(), t[:, [2, 0]])
