@@ -317,3 +317,21 @@ def test_dpm2_coefficients_reproduce_the_oracle_on_the_host():
         assert seen == [first] + [N.DPM2_SECOND] * (n - 2) + [N.DPM2_DDIM]
     with pytest.raises(IndexError):
         dpm2_coefficients(osch.sigma_schedule(4, 3.0), 4, 0)
+
+
+def test_metric_names_are_the_references():
+    """Metric keys become W&B series, so they are part of the contract: the names below are the
+    reference's (unirl/algorithms/base.py:98-103, :147-156; drpo.py:151-158; flowdppo.py:124-137)."""
+    from unirl_amd import ops
+    from unirl_amd.algorithms._fused import ABSDIFF_METRICS, DRPO_METRICS, GRPO_METRICS
+
+    assert set(GRPO_METRICS) == {"ratio_mean", "ratio_std", "ratio_min", "ratio_max", "clip_fraction",
+                                 "clipfrac_gt_one", "clipfrac_lt_one", "approx_kl"}
+    assert set(DRPO_METRICS) == {"ratio_mean", "ratio_max", "approx_kl", "drpo_penalty_mean", "clipfrac_upper",
+                                 "clipfrac_lower"}
+    assert set(ABSDIFF_METRICS) == {"rollout_replay_logp_absdiff_mean", "rollout_replay_logp_absdiff_max"}
+    assert set(ops.FLOWDPPO_METRIC_SLOTS) - {"loss_mean"} == {
+        "ratio_mean", "ratio_std", "ratio_min", "ratio_max", "approx_kl", "kl_new_old_mean", "kl_new_old_max",
+        "kl_mask_fraction", "pos_rm_fraction", "neg_rm_fraction", "masked_fraction", "unmasked_fraction"}
+    for table in (GRPO_METRICS, DRPO_METRICS, ABSDIFF_METRICS, ops.FLOWDPPO_METRIC_SLOTS):
+        assert len(set(table.values())) == len(table)  # one slot of the metrics vector each
