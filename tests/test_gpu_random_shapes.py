@@ -148,3 +148,95 @@ def test_kl_mask_random(dev, seed):
         assert_close(kl, ref, rtol, 1e-9, f"kl {tuple(base.shape)} {dtype}")
         near = (ref - thr).abs() <= 4 * torch.finfo(torch.float32).eps * abs(thr) + rtol * abs(thr) * (dtype != torch.float32)
         assert torch.equal(mask.cpu()[~near], (ref < thr)[~near])
+
+
+def _offset(t, k, dev):
+    """The same values in a device tensor whose storage starts ``k`` elements into a buffer."""
+    buf = torch.empty(t.numel() + k, dtype=t.dtype, device=dev)
+    view = buf[k:].view(t.shape)
+    view.copy_(t)
+    return view
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_misaligned_base_pointers(dev, seed):
+    """Every operand starts a few elements into its buffer (4- or 2-byte aligned only), each by its
+    own amount, so the kernels cannot take their 16-byte paths on all of them."""
+    from oracle import dpm2 as odpm
+    from unirl_amd import ops, sde
+    from unirl_amd.algorithms import fused_token_loss_backward
+
+    rng = random.Random(9000 + seed)
+    for _ in range(4):
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        k = [rng.randint(0, 7) for _ in range(4)]
+        # SDE step, sampling and replay
+        B, D, kind = rng.randint(1, 4), rng.choice((5, 64, 1000, 4099)), rng.choice(("flow", "dance", "cps"))
+        dtype, vdtype, i = rng.choice(DTYPES), rng.choice(DTYPES), rng.randint(0, 27)
+        x, v, n = torch.randn(B, D, generator=g).to(dtype), torch.randn(B, D, generator=g).to(vdtype), torch.randn(B, D, generator=g)
+        ref_prev, ref_lp, ref_mean = osde.sde_denoise(kind, v, x, SIG[i], SIG[i + 1], eta=0.7, noise=n, sigma_max=SIG[1],
+                                                      ieee_sqrt=True)
+        st = sde.STRATEGIES[kind]()
+        prev, lp, mean = st.denoise(_offset(v, k[0], dev), _offset(x, k[1], dev), SIG[i].to(dev), SIG[i + 1].to(dev),
+                                    eta=0.7, sigma_max=SIG[1].to(dev), noise=_offset(n, k[2], dev))
+        what = f"{kind} [{B},{D}] {dtype}/{vdtype} offsets {k}"
+        rtol = FP32_RTOL if dtype == vdtype == torch.float32 else BF16_RTOL
+        assert torch.equal(mean.cpu(), ref_mean) and torch.equal(prev.cpu(), ref_prev), what
+        assert_close(lp, ref_lp, rtol, 2e-6, what)
+        _, r_lp, r_mean = osde.sde_denoise(kind, v, x, SIG[i], SIG[i + 1], eta=0.7, prev_sample=ref_prev.to(dtype),
+                                           sigma_max=SIG[1], ieee_sqrt=True)
+        _, lp2, mean2 = st.denoise(_offset(v, k[0], dev), _offset(x, k[1], dev), SIG[i].to(dev), SIG[i + 1].to(dev), eta=0.7,
+                                   sigma_max=SIG[1].to(dev), prev_sample=_offset(ref_prev.to(dtype), k[3], dev))
+        assert torch.equal(mean2.cpu(), r_mean), what + " replay"
+        assert_close(lp2, r_lp, rtol, 2e-6, what + " replay")
+        # Gaussian KL
+        p = (x.float() + 0.02 * torch.randn(B, D, generator=g)).to(dtype)
+        ref = ofd.kl_per_sample(p.view(B, 1, D), x.view(B, 1, D), torch.tensor([0.3]).view(1, 1, 1))
+        kl, _ = ops.gaussian_kl_mask(_offset(p.view(B, 1, D), k[0], dev), _offset(x.view(B, 1, D), k[3], dev),
+                                     torch.tensor([0.3], device=dev), 0.01)
+        assert_close(kl, ref, FP32_RTOL if dtype == torch.float32 else BF16_RTOL, 1e-9, what + " kl")
+        # one-pass ratio loss, packed
+        n_seq, max_len, lk = rng.randint(1, 20), rng.choice((3, 4, 31, 257, 1024)), rng.choice(("grpo", "drpo"))
+        old = -8 * torch.rand(n_seq, max_len, generator=g)
+        new = old + 0.05 * torch.randn(n_seq, max_len, generator=g)
+        lengths = torch.randint(1, max_len + 1, (n_seq,), generator=g)
+        adv = torch.randn(n_seq, generator=g)
+        newp, oldp = olos.pack_padded(new, lengths), olos.pack_padded(old, lengths)
+        npk = newp.clone().requires_grad_(True)
+        ref_loss, _ = olos.token_loss(lk, npk, oldp, adv, lengths, mode="token-mean", clip_range=0.2, clip_range_high=0.28,
+                                      epsilon=5.0)
+        ref_loss.backward()
+        cu = torch.cat([torch.zeros(1, dtype=torch.int64), lengths.cumsum(0)])
+        nd = _offset(newp, k[0], dev).requires_grad_(True)
+        mvec = fused_token_loss_backward(lk, nd * 1.0, _offset(oldp, k[1], dev), _offset(adv, k[2], dev), cu_seqlens=cu.to(dev),
+                                         loss_scale=1.0, clip_range=0.2, clip_range_high=0.28, drpo_epsilon=5.0,
+                                         adv_per_token=False)
+        scale = float(ref_loss.detach().abs()) + float(adv.abs().mean())
+        assert_close(mvec[0], ref_loss.detach(), 2e-5, 4e-6 * scale, f"{lk} [{n_seq},{max_len}] offsets {k}")
+        assert_close(nd.grad, npk.grad, 2e-5, 2e-6 * float(npk.grad.abs().max()), f"{lk} gradient, offsets {k}")
+        # token log-prob and backward
+        rows, V, T = rng.randint(1, 6), rng.choice((7, 64, 1000, 4099)), rng.choice((1.0, 0.7))
+        logits = (2 * torch.randn(rows, V, generator=g)).to(dtype)
+        ids = torch.randint(0, V, (rows,), generator=g)
+        ld = _offset(logits, k[3], dev)
+        tlp, ent, lse = ops.token_logp_entropy(ld, ids.to(dev), T, want_lse=True)
+        assert_close(tlp, otok.token_logp(logits, ids, T), 2e-5, 2e-6, f"token [{rows},{V}] {dtype} offset {k[3]}")
+        assert_close(ent, otok.token_entropy(logits, T), 2e-5, 2e-6, f"entropy [{rows},{V}] {dtype} offset {k[3]}")
+        gl = torch.randn(rows, generator=g)
+        lf = logits.float().requires_grad_(True)
+        torch.log_softmax(lf / T, -1).gather(-1, ids[:, None])[:, 0].backward(gl)
+        tol = 2e-5 if dtype == torch.float32 else (1e-2 if dtype == torch.bfloat16 else 2e-3)
+        grad = ops.token_logp_bwd(ld, ids.to(dev), T, lse, gl.to(dev))
+        assert_close(grad.float(), lf.grad, tol, tol * float(gl.abs().max()) * 0.1 + 1e-7, f"token gradient offset {k[3]}")
+        # DPM-Solver-2 step (second order needs two steps of history)
+        sig = osch.sigma_schedule(6, 3.0)
+        strategy, solver = sde.DPM2Strategy(), odpm.Dpm2Solver(sig)
+        strategy.init_schedule(sig)
+        xs = x
+        for step in range(3):
+            vs = torch.randn(B, D, generator=g).to(vdtype)
+            want = solver.step(vs, xs, step)
+            got, _, _ = strategy.denoise(_offset(vs, k[step], dev), _offset(xs, k[3 - step], dev), sig[step], sig[step + 1],
+                                         step_index=step)
+            assert torch.equal(got.cpu(), want), f"dpm2 step {step}, offsets {k}"
+            xs = want.to(dtype)
