@@ -324,6 +324,65 @@ def make_headline(torch, dev, rows: int, vocab: int):
     return x, ids, spiked
 
 
+def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
+    """The caller of the headline kernel in training: `lm_head` on a chunk of response tokens, their
+    log-probs, and the backward with the chunk's logits rebuilt (unirl/models/qwen3/ar.py:82-99).
+    One sequence of `rows` tokens, a bf16 head of Qwen3-4B's size; the fused path against the
+    reference's own ops (`.float() / T`, gather, logsumexp under torch's checkpoint)."""
+    from torch.utils.checkpoint import checkpoint
+
+    from unirl_amd import models
+
+    torch.manual_seed(0)
+    head = torch.nn.Linear(hidden, vocab, bias=False).to(dev).to(torch.bfloat16)
+    hidden_states = torch.randn(1, rows, hidden, device=dev, dtype=torch.bfloat16)
+    tokens = torch.randint(0, vocab, (1, rows), device=dev)
+    upstream = torch.randn(1, rows, device=dev)
+
+    def reference(h_all):
+        def logp_chunk(h, tok):
+            lf = head(h).float() / 1.0
+            return lf.gather(-1, tok.unsqueeze(-1)).squeeze(-1) - torch.logsumexp(lf, dim=-1)
+
+        chunk = max(64, 2048 // int(h_all.shape[0]))
+        parts = [checkpoint(logp_chunk, h_all[:, s : s + chunk], tokens[:, s : s + chunk], use_reentrant=False)
+                 for s in range(0, rows, chunk)]
+        return torch.cat(parts, dim=1)
+
+    def timed(fn):
+        for _ in range(3):  # the last of three passes is reported
+            head.zero_grad(set_to_none=True)
+            h = hidden_states.clone().requires_grad_(True)
+            torch.cuda.synchronize()
+            torch.cuda.reset_peak_memory_stats()
+            base = torch.cuda.memory_allocated()
+            a, b, c = (torch.cuda.Event(enable_timing=True) for _ in range(3))
+            a.record()
+            out = fn(h)
+            b.record()
+            (out * upstream).sum().backward()
+            c.record()
+            torch.cuda.synchronize()
+        stats = {"forward_ms": round(a.elapsed_time(b), 2), "backward_ms": round(b.elapsed_time(c), 2),
+                 "total_ms": round(a.elapsed_time(c), 2),
+                 "peak_transient_gib": round((torch.cuda.max_memory_allocated() - base) / 2**30, 2)}
+        return stats, out.detach(), h.grad.detach().float(), head.weight.grad.detach().float()
+
+    out = {"rows": rows, "vocab": vocab, "hidden": hidden}
+    ref = timed(reference)
+    out["reference_torch_checkpoint_chunk2048"] = ref[0]
+    for name, kw in (("fused_chunk2048", dict(chunk=2048)), ("fused_default_chunk4096", dict()),
+                     ("fused_keep_logits_chunk8192", dict(chunk=8192, keep_logits=True))):
+        got = timed(lambda h: models.chunked_replay_logp(head, h, tokens, 1.0, **kw))
+        got[0]["max_abs_logp_diff"] = float((got[1] - ref[1]).abs().max())
+        got[0]["grad_hidden_rel"] = float((got[2] - ref[2]).norm() / ref[2].norm())
+        got[0]["grad_weight_rel"] = float((got[3] - ref[3]).norm() / ref[3].norm())
+        out[name] = got[0]
+        log(f"replay {name}: {got[0]}")
+    log(f"replay reference: {ref[0]}")
+    return out
+
+
 # ----------------------------------------------------------------------------------------------
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
@@ -338,6 +397,11 @@ def main() -> int:
                     help="run 3 calibration copies of 1 GiB, 3 headline launches and 3 launches of every "
                          "other shape, then exit "
                          "(the command `rocprofv3 --pmc FETCH_SIZE|WRITE_SIZE` is pointed at)")
+    ap.add_argument("--replay-probe", action="store_true",
+                    help="forward + backward of the chunked lm_head + log-prob replay (bf16 Linear(2560, vocab), "
+                         "--rows response tokens) through the fused kernels and through the reference's torch ops "
+                         "under checkpoint, then exit (time, peak transient memory; a kernel trace of this command "
+                         "shows the split between the head's GEMMs and the log-prob kernels)")
     ap.add_argument("--skip-shapes", action="store_true", help="headline only")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
     args = ap.parse_args()
@@ -366,6 +430,10 @@ def main() -> int:
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     log(f"device {torch.cuda.get_device_name(0)}, torch {torch.__version__}, host threads {torch.get_num_threads()}")
+
+    if args.replay_probe:
+        print(json.dumps({"replay_probe": replay_probe(torch, dev, args.rows, args.vocab)}), flush=True)
+        return 0
 
     # ---------------- headline: token log-prob + entropy ----------------
     x, ids, spiked = make_headline(torch, dev, args.rows, args.vocab)
