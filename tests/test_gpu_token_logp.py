@@ -274,6 +274,31 @@ def test_chunked_replay_recomputes_logits_in_backward(dev, dtype):
     with torch.no_grad():
         hd.weight.copy_(head.weight)
         hd.bias.copy_(head.bias)
-    out = models.chunked_replay_logp(hd, hidden.to(dev), toks.to(dev), temperature=T, chunk=64)
+    out = models.chunked_replay_logp(hd, hidden.to(dev), toks.to(dev), temperature=T, chunk=64, keep_logits=False)
+    assert "RecomputedChunk" in type(out.grad_fn.next_functions[0][0]).__name__
     (out * upstream.to(dev)).sum().backward()
     assert_close(hd.weight.grad.cpu(), ref_grads[1], 1e-4, 1e-5 * float(ref_grads[1].abs().max()), "weight grad only")
+
+
+def test_chunked_replay_keeps_logits_only_within_its_budget(dev, monkeypatch):
+    """Left to itself the replay keeps an ``nn.Linear`` head's logits for the backward while all of them
+    fit the byte budget and recomputes them beyond it; a bare callable's logits are never kept by default
+    when the hidden states need a gradient."""
+    from unirl_amd import models
+    from unirl_amd.models import ar_logp
+
+    B, T_max, H, V = 2, 40, 16, 300
+    g = torch.Generator().manual_seed(12)
+    head = torch.nn.Linear(H, V).to(dev)
+    toks = torch.randint(0, V, (B, T_max), generator=g).to(dev)
+
+    def path(lm_head):
+        h = torch.randn(B, T_max, H, generator=g).to(dev).requires_grad_(True)
+        out = models.chunked_replay_logp(lm_head, h, toks, chunk=16)
+        return {type(fn).__name__ for fn, _ in out.grad_fn.next_functions}  # out = cat(per-chunk parts)
+
+    assert B * T_max * V * 4 < ar_logp.KEEP_LOGITS_BYTES
+    assert not any("RecomputedChunk" in n for n in path(head))
+    monkeypatch.setattr(ar_logp, "KEEP_LOGITS_BYTES", B * T_max * V * 4 - 1)
+    assert all("RecomputedChunk" in n for n in path(head))
+    assert all("RecomputedChunk" in n for n in path(lambda h: h @ head.weight.t()))

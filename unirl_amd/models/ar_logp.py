@@ -124,13 +124,17 @@ def token_entropy(logits: torch.Tensor, temperature: float = 1.0) -> torch.Tenso
     return ent
 
 
+#: all of a replay's logits are kept for the backward (no second ``lm_head`` pass) up to this size
+KEEP_LOGITS_BYTES = 4 << 30
+
+
 def chunked_replay_logp(
     lm_head: Callable[[torch.Tensor], torch.Tensor],
     resp_hidden: torch.Tensor,
     response_tokens: torch.Tensor,
     temperature: float = 1.0,
     chunk: Optional[int] = None,
-    keep_logits: bool = False,
+    keep_logits: Optional[bool] = None,
 ) -> torch.Tensor:
     """Padded ``[B, T_max]`` fp32 log-probs of ``response_tokens`` under ``lm_head(resp_hidden)``.
 
@@ -142,14 +146,24 @@ def chunked_replay_logp(
     faster on the larger block.  Under autograd
     the logits of a chunk are dropped and recomputed in the backward, like the reference's
     per-chunk checkpoint (``keep_logits=True`` keeps them instead: no second ``lm_head``
-    pass, ``B * T_max * V`` elements of memory).  The recomputing path is taken when
-    ``resp_hidden`` or a parameter of an ``nn.Module`` head requires grad; a bare callable whose
-    captured weights alone require grad keeps its logits.
+    pass, ``B * T_max * V`` elements of memory).  Left at ``None``, the logits of an
+    ``nn.Linear`` head are kept when all of them together take at most ``KEEP_LOGITS_BYTES``
+    (4 GiB: with the gradient block of one chunk that is what the reference's checkpointed
+    chunks hold in fp32 transients anyway) and recomputed otherwise; kept logits allow chunks
+    of ``8192 // B`` rows.  The recomputing path is taken when ``resp_hidden`` or a parameter of
+    an ``nn.Module`` head requires grad; a bare callable whose captured weights alone require
+    grad keeps its logits.
     """
     bsz, t_max = int(resp_hidden.size(0)), int(response_tokens.size(1))
     if t_max == 0:
         return resp_hidden.new_zeros((bsz, 0), dtype=torch.float32)
-    step = int(chunk) if chunk is not None else max(64, 4096 // max(1, bsz))
+    if keep_logits is None:
+        keep_logits = (
+            isinstance(lm_head, torch.nn.Linear)
+            and bsz * t_max * lm_head.out_features * lm_head.weight.element_size() <= KEEP_LOGITS_BYTES
+        )
+    rows_per_chunk = 8192 if keep_logits else 4096
+    step = int(chunk) if chunk is not None else max(64, rows_per_chunk // max(1, bsz))
     T = float(temperature) if float(temperature) > 0.0 else 1.0
     params = tuple(lm_head.parameters()) if isinstance(lm_head, torch.nn.Module) else ()
     recompute = (
