@@ -12,6 +12,11 @@ figures for all five synthetic shapes (small ones timed as back-to-back launches
 a HIP graph over rotating buffer sets, so neither the launch path nor the 256 MB
 last-level cache hides the kernel time); `cpu_baseline` is the eager-torch CPU oracle of
 the headline path on a bounded row sample, timed on this host's cores.
+
+Two probe modes print their own JSON line and exit: `--traffic-probe` (three launches of every
+kernel after three calibration copies, the command the hardware byte counters are collected on)
+and `--replay-probe` (the kernel's caller in training, the chunked lm_head + log-prob replay,
+forward + backward, against the reference's torch ops under checkpoint).
 """
 
 from __future__ import annotations
