@@ -297,6 +297,14 @@ def test_chunked_replay_keeps_logits_only_within_its_budget(dev, monkeypatch):
         out = models.chunked_replay_logp(lm_head, h, toks, chunk=16)
         return {type(fn).__name__ for fn, _ in out.grad_fn.next_functions}  # out = cat(per-chunk parts)
 
+    # kept logits of a Linear head are overwritten by their gradient: a second backward says so
+    h = torch.randn(B, T_max, H, generator=g).to(dev).requires_grad_(True)
+    out = models.chunked_replay_logp(head, h, toks, chunk=16)
+    out.sum().backward(retain_graph=True)
+    with pytest.raises(RuntimeError, match="overwritten by their gradient"):
+        out.sum().backward()
+    head.zero_grad()
+
     assert B * T_max * V * 4 < ar_logp.KEEP_LOGITS_BYTES
     assert not any("RecomputedChunk" in n for n in path(head))
     monkeypatch.setattr(ar_logp, "KEEP_LOGITS_BYTES", B * T_max * V * 4 - 1)

@@ -29,12 +29,17 @@ class _TokenLogpFn(torch.autograd.Function):
     """Log-prob (differentiable) and, on request, entropy (detached) from one pass over the logits."""
 
     @staticmethod
-    def forward(ctx, logits: torch.Tensor, tokens: torch.Tensor, temperature: float, want_entropy: bool):
+    def forward(ctx, logits: torch.Tensor, tokens: torch.Tensor, temperature: float, want_entropy: bool,
+                consume: bool = False):
         logp, ent, lse = ops.token_logp_entropy(
             logits, tokens, temperature, want_logp=True, want_entropy=want_entropy, want_lse=True
         )
         ctx.save_for_backward(logits, tokens, lse)
         ctx.temperature = temperature
+        # `consume`: the caller owns the logits and nobody reads them after this node's backward, so
+        # the gradient may overwrite them (no second [rows, V] buffer)
+        ctx.consume = bool(consume) and logits.is_contiguous() and logits.dtype in _KERNEL_DTYPES
+        ctx.consumed = False
         if not want_entropy:
             return logp
         ctx.mark_non_differentiable(ent)
@@ -43,7 +48,14 @@ class _TokenLogpFn(torch.autograd.Function):
     @staticmethod
     def backward(ctx, g_logp, *_g_entropy):
         logits, tokens, lse = ctx.saved_tensors
-        return ops.token_logp_bwd(logits, tokens, ctx.temperature, lse, g_logp), None, None, None
+        if ctx.consumed:
+            raise RuntimeError(
+                "the logits of this replay were overwritten by their gradient in the first backward; "
+                "a second backward through the same graph needs chunked_replay_logp(..., keep_logits=False)"
+            )
+        ctx.consumed = ctx.consume
+        grad = ops.token_logp_bwd(logits, tokens, ctx.temperature, lse, g_logp, in_place=ctx.consume)
+        return grad, None, None, None, None
 
 
 class _RecomputedChunkFn(torch.autograd.Function):
@@ -146,10 +158,12 @@ def chunked_replay_logp(
     faster on the larger block.  Under autograd
     the logits of a chunk are dropped and recomputed in the backward, like the reference's
     per-chunk checkpoint (``keep_logits=True`` keeps them instead: no second ``lm_head``
-    pass, ``B * T_max * V`` elements of memory).  Left at ``None``, the logits of an
+    pass, ``B * T_max * V`` elements of memory; an ``nn.Linear`` head's kept logits are overwritten
+    by their gradient in the backward, so a second backward through the same graph raises).
+    Left at ``None``, the logits of an
     ``nn.Linear`` head are kept when all of them together take at most ``KEEP_LOGITS_BYTES``
-    (4 GiB: with the gradient block of one chunk that is what the reference's checkpointed
-    chunks hold in fp32 transients anyway) and recomputed otherwise; kept logits allow chunks
+    (4 GiB, below what the reference's checkpointed chunks hold in fp32 transients) and
+    recomputed otherwise; kept logits allow chunks
     of ``8192 // B`` rows.  The recomputing path is taken when ``resp_hidden`` or a parameter of
     an ``nn.Module`` head requires grad; a bare callable whose captured weights alone require
     grad keeps its logits.
@@ -176,7 +190,12 @@ def chunked_replay_logp(
         if recompute:
             parts.append(_RecomputedChunkFn.apply(h, tok, lm_head, T, *params))
         else:
-            parts.append(token_logp(lm_head(h), tok, temperature))
+            logits = lm_head(h)
+            if isinstance(lm_head, torch.nn.Linear) and torch.is_grad_enabled() and logits.requires_grad:
+                # a Linear's output is saved by nothing but this node: its gradient may take its place
+                parts.append(_TokenLogpFn.apply(logits, tok, T, False, True))
+            else:
+                parts.append(token_logp(logits, tok, temperature))
     return torch.cat(parts, dim=1)
 
 
