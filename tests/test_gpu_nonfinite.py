@@ -130,6 +130,20 @@ def test_token_rows_where_a_nan_precedes_every_finite_logit(dev):
         lp, ent = models.token_logp_entropy(xd.to(dev), ids.to(dev), 0.7)
         same(lp, otok.token_logp(xd, ids, 0.7), f"log-prob {dtype}", 2e-5, 2e-6)
         same(ent, otok.token_entropy(xd, 0.7), f"entropy {dtype}", 2e-5, 2e-6)
+    # several +inf logits in one row: the log-sum-exp is +inf, so a finite or masked target has
+    # log-prob -inf (not NaN), the +inf tokens themselves inf - inf = NaN
+    many = torch.randn(4, 6000)
+    many[0, [5, 4000]] = INF
+    many[1, [7, 2500, 5999]] = INF
+    many[1, 9] = -INF
+    many[2, [1, 3000]] = INF
+    many[3, [10, 5000]] = INF
+    many[3, 77] = NAN
+    ids = torch.tensor([100, 9, 3000, 100])
+    lp, ent = models.token_logp_entropy(many.to(dev), ids.to(dev), 1.0)
+    same(lp, otok.token_logp(many, ids), "log-prob, several +inf", 2e-5, 2e-6)
+    assert lp.cpu().tolist()[:2] == [-INF, -INF] and math.isnan(float(lp[2])) and math.isnan(float(lp[3]))
+    same(ent, otok.token_entropy(many), "entropy, several +inf", 2e-5, 2e-6)
     big = torch.randn(3, 5000)
     big[1, :700] = NAN          # the first chunks of several wavefronts hold nothing but NaN
     big[2, :300] = -INF

@@ -110,7 +110,17 @@ __device__ __forceinline__ void tok_update(TokRef& ref, TokAcc& acc, const float
       }
     }
   } else if (ref.m != -INFINITY) {
-    if (active) {
+    if (SAFE && ref.m == INFINITY) {
+      // a +inf logit has been met: every other term is 0 against it, a further +inf is one more
+      // maximum (inf - inf above would make it a NaN), and only a NaN still matters
+      if (active) {
+#pragma unroll
+        for (int k = 0; k < N; ++k) {
+          if (x[k] == INFINITY) acc.cnt += 1.0f;
+          else if (x[k] != x[k]) acc.s = x[k];
+        }
+      }
+    } else if (active) {
 #pragma unroll
       for (int k = 0; k < N; ++k) {
         float a = fmaf(x[k], c, -ref.r);
