@@ -335,3 +335,28 @@ def test_metric_names_are_the_references():
         "kl_mask_fraction", "pos_rm_fraction", "neg_rm_fraction", "masked_fraction", "unmasked_fraction"}
     for table in (GRPO_METRICS, DRPO_METRICS, ABSDIFF_METRICS, ops.FLOWDPPO_METRIC_SLOTS):
         assert len(set(table.values())) == len(table)  # one slot of the metrics vector each
+
+
+def test_per_sample_view_never_hands_stride_zero_for_several_samples(monkeypatch):
+    """A sample stride of 0 means "densely packed" in the C ABI: a tensor broadcast over the
+    samples must be copied, not passed with its stride of 0 (the kernel would then read B blocks
+    from a buffer that holds one)."""
+    from unirl_amd import _native as N
+    from unirl_amd import ops
+
+    monkeypatch.setattr(N, "require_device", lambda t, name: None)
+    one = torch.arange(12.0).reshape(1, 3, 4)
+    for B in (2, 7):
+        t, stride = ops._per_sample_view(one.expand(B, 3, 4), "noise")
+        assert stride == 12 and t.is_contiguous() and t.shape == (B, 3, 4)
+        assert torch.equal(t[B - 1], one[0])
+    # one sample: any stride is harmless and reported as D
+    t, stride = ops._per_sample_view(one.expand(1, 3, 4), "noise")
+    assert stride == 12
+    # slices of a stack keep their stride and are not copied
+    stack = torch.zeros(4, 5, 3, 4)
+    t, stride = ops._per_sample_view(stack[:, 2], "sample")
+    assert stride == 60 and t.data_ptr() == stack[:, 2].data_ptr()
+    # outputs may not overlap across samples
+    with pytest.raises(ValueError):
+        ops._per_sample_view(one.expand(3, 3, 4), "prev_out", writable=True)

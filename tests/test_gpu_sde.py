@@ -433,3 +433,35 @@ def test_stage_loops_on_stacks_match_oracle(dev, kind, traj_dtype, shape):
     with pytest.raises(ValueError):
         st.denoise_into(v2[0].to(dev), stack[:, 0], SIG[0].to(dev), SIG[1].to(dev), eta=0.7,
                         mean_out=means[:, 0].transpose(-1, -2), logp_out=rlp[:, 0])
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_inputs_broadcast_over_the_samples(dev, kind):
+    """noise / noise_pred / sample given as expand(B, ...) views (sample stride 0): every sample
+    must see the one block, and nothing past it is read."""
+    st = strategy(kind)
+    B, shape = 5, (1, 4, 24, 24)
+    g = torch.Generator().manual_seed(77)
+    x1, v, n1 = (torch.randn(shape, generator=g) for _ in range(3))
+    v = torch.randn((B,) + shape[1:], generator=g)
+    xe, ne = x1.expand(B, *shape[1:]), n1.expand(B, *shape[1:])
+    ref_prev, ref_lp, ref_mean = osde.sde_denoise(kind, v, xe, SIG[3], SIG[4], eta=0.7, noise=ne, sigma_max=SIG[1],
+                                                  ieee_sqrt=True)
+    prev = torch.empty((B,) + shape[1:], device=dev)
+    mean = torch.empty_like(prev)
+    lp = torch.empty(B, device=dev)
+    # the expanded operands sit at the very end of their allocations
+    xd, nd = x1.to(dev).expand(B, *shape[1:]), n1.to(dev).expand(B, *shape[1:])
+    assert xd.stride(0) == 0 and nd.stride(0) == 0
+    assert st.denoise_into(v.to(dev), xd, SIG[3].to(dev), SIG[4].to(dev), eta=0.7, sigma_max=SIG[1].to(dev),
+                           noise=nd, prev_out=prev, mean_out=mean, logp_out=lp)
+    assert torch.equal(prev.cpu(), ref_prev) and torch.equal(mean.cpu(), ref_mean)
+    assert_close(lp, ref_lp, FP32_RTOL, 2e-6, "log-prob with broadcast inputs")
+    # replay with a broadcast velocity
+    ve = v[:1].expand(B, *shape[1:])
+    _, ref_lp2, ref_mean2 = osde.sde_denoise(kind, ve, xe, SIG[3], SIG[4], eta=0.7, prev_sample=ref_prev,
+                                             sigma_max=SIG[1], ieee_sqrt=True)
+    st.denoise_into(v[:1].to(dev).expand(B, *shape[1:]), xd, SIG[3].to(dev), SIG[4].to(dev), eta=0.7,
+                    sigma_max=SIG[1].to(dev), prev_sample=ref_prev.to(dev), mean_out=mean, logp_out=lp)
+    assert torch.equal(mean.cpu(), ref_mean2)
+    assert_close(lp, ref_lp2, FP32_RTOL, 2e-6, "replay log-prob with broadcast inputs")

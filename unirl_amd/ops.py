@@ -133,7 +133,9 @@ def _per_sample_view(t: torch.Tensor, name: str, *, writable: bool = False) -> T
     B = t.shape[0]
     D = t.numel() // B if B else 0
     inner_ok = B == 0 or t[0].is_contiguous()
-    if inner_ok and (B <= 1 or t.stride(0) >= (D if writable else 0)):
+    # A sample stride of 0 means "densely packed" in the C ABI, so a tensor broadcast over the
+    # samples (expand(B, ...), stride 0) cannot be handed over as it is: it is copied.
+    if inner_ok and (B <= 1 or t.stride(0) >= (D if writable else 1)):
         return t, (t.stride(0) if B > 1 else D)
     if writable:
         raise ValueError(f"{name}: each sample must be one contiguous, non-overlapping block; got strides {t.stride()}")
