@@ -36,8 +36,9 @@ extern "C" {
 #endif
 
 /* 2: typed gradient outputs in unirl_sde_step_logp_bwd; unirl_ratio_loss_fwd_bwd and
- * unirl_flowdppo_step added. */
-#define UNIRL_ABI_VERSION 3
+ * unirl_flowdppo_step added.  3: unirl_dpm2_step added.  4: unirl_gaussian_kl_mask_static
+ * added. */
+#define UNIRL_ABI_VERSION 4
 
 enum unirl_dtype { UNIRL_F32 = 0, UNIRL_BF16 = 1, UNIRL_F16 = 2 };
 
@@ -231,6 +232,21 @@ int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, const float*
                            int64_t n_sigma, int64_t R, int64_t D, float threshold, float* kl_out,
                            uint8_t* mask_out, void* workspace, size_t workspace_bytes,
                            void* stream);
+
+/* unirl_gaussian_kl_mask without a workspace and without any allocation.  It has no
+ * counterpart in the reference; it exists for callers that cannot allocate device memory: code
+ * under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  The
+ * per-workgroup partials go to a static device array inside the library (256 KiB, held by every
+ * GPU the library runs on until the process ends) instead of a caller-owned workspace; its
+ * address is looked up once per device, on the first call made with that device current, which
+ * is best made outside a graph capture.  Same kernels, same launch shape and bit-identical
+ * results as unirl_gaussian_kl_mask.  Limit: R <= UNIRL_KL_STATIC_MAX_ROWS (UNIRL_E_LIMIT
+ * beyond).  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU
+ * (different streams or threads) race; calls ordered on one stream do not. */
+#define UNIRL_KL_STATIC_MAX_ROWS 32768
+int unirl_gaussian_kl_mask_static(const void* p, const void* q, int dtype, const float* sigma,
+                                  int64_t n_sigma, int64_t R, int64_t D, float threshold,
+                                  float* kl_out, uint8_t* mask_out, void* stream);
 
 /* The [B,S'] part of _flowdppo_kl_adv_loss (flowdppo.py:86-137) given the row
  * KLs from unirl_gaussian_kl_mask: ratio, the KL / advantage-sign masks,

@@ -210,6 +210,22 @@ void check_kl(hipStream_t st, void* ws, size_t ws_bytes) {
       ++g_failures;
     }
   }
+  // the allocation-free entry (static scratch inside the library) gives the same bits, twice
+  for (int call = 0; call < 2; ++call) {
+    DevBuf<float> dkl2(R);
+    DevBuf<uint8_t> dmask2(R);
+    expect_status("unirl_gaussian_kl_mask_static", unirl_gaussian_kl_mask_static(dp.p, dq.p, UNIRL_BF16, dsig.p, 2, R, D,
+                                                                                 thr, dkl2.p, dmask2.p, st));
+    HIP_OK(hipStreamSynchronize(st));
+    const auto kl2 = dkl2.host();
+    const auto mask2 = dmask2.host();
+    for (int64_t r = 0; r < R; ++r) {
+      if (std::memcmp(&kl2[r], &kl[r], sizeof(float)) != 0 || mask2[r] != mask[r]) {
+        std::printf("FAIL static-scratch kl row %lld call %d\n", (long long)r, call);
+        ++g_failures;
+      }
+    }
+  }
   std::printf("gaussian kl + mask: checked %lld rows\n", (long long)R);
 }
 

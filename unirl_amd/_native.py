@@ -103,7 +103,7 @@ class Dpm2Coeffs(Structure):
 
 
 # UNIRL_ABI_VERSION of include/unirl_hip.h that the signatures below describe
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _SIGNATURES = {
     "unirl_abi_version": (c_int, []),
@@ -138,6 +138,10 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p,
          c_size_t, c_void_p],
+    ),
+    "unirl_gaussian_kl_mask_static": (
+        c_int,
+        [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_float, c_void_p, c_void_p, c_void_p],
     ),
     "unirl_flowdppo_loss": (
         c_int,

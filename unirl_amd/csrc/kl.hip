@@ -11,12 +11,16 @@
 //
 // HBM traffic: 2 * D * sizeof(T) bytes read per row, 5 bytes written per row.
 
+#include <mutex>
+
 #include "common.cuh"
 #include "unirl_internal.h"
 
 namespace unirl {
 
 constexpr int kKlThreads = 256;
+// Rows (and partial slots) the allocation-free entry point accepts: 32768 doubles = 256 KiB per GPU.
+constexpr int64_t kKlStaticRows = UNIRL_KL_STATIC_MAX_ROWS;
 
 struct KlArgs {
   const void* p;
@@ -383,14 +387,10 @@ extern "C" int unirl_flowdppo_loss(const float* new_logp, const float* old_logp,
   return (int)hipGetLastError();
 }
 
-extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, const float* sigma, int64_t n_sigma,
-                                      int64_t R, int64_t D, float threshold, float* kl_out, uint8_t* mask_out,
-                                      void* workspace, size_t workspace_bytes, void* stream) {
-  if (!dtype_ok(dtype)) return UNIRL_E_DTYPE;
-  if (R < 0 || D <= 0 || n_sigma <= 0) return UNIRL_E_SHAPE;
-  if (R == 0) return UNIRL_OK;
-  if (!p || !q || !sigma || !kl_out) return UNIRL_E_NULL;
-  if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
+// Shared body of the two row-KL entry points; `partials` holds `capacity` doubles.
+static int kl_mask_run(const void* p, const void* q, int dtype, const float* sigma, int64_t n_sigma, int64_t R,
+                       int64_t D, float threshold, float* kl_out, uint8_t* mask_out, double* partials,
+                       int64_t capacity, hipStream_t st) {
   const size_t sz = dtype_size(dtype);
   if (!aligned_to(p, sz) || !aligned_to(q, sz)) return UNIRL_E_ALIGN;
   int vec = 4;
@@ -398,9 +398,9 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
   if (sz == 2 && D % 8 == 0 && aligned_to(p, 16) && aligned_to(q, 16)) vec = 8;
   const int items = (vec >= 4) ? (int)tune_int("UNIRL_KL_ITEMS", 2) : 2;
   const unsigned int nblk = kl_blocks_per_row(D / vec, items, R);
-  int64_t per_launch = kPartialCapacity / nblk;
+  int64_t per_launch = capacity / nblk;
   if (per_launch > 32768) per_launch = 32768;
-  hipStream_t st = (hipStream_t)stream;
+  if (per_launch < 1) return UNIRL_E_LIMIT;
   for (int64_t r0 = 0; r0 < R; r0 += per_launch) {
     const int64_t nr = (R - r0 < per_launch) ? (R - r0) : per_launch;
     KlArgs A = {};
@@ -414,7 +414,7 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
     A.kl = kl_out + r0;
     A.mask = mask_out ? mask_out + r0 : nullptr;
     A.elem_out = nullptr;
-    A.partials = ws_partials(workspace);
+    A.partials = partials;
     int rc = UNIRL_E_DTYPE;
     switch (dtype) {
       case UNIRL_F32: rc = launch_kl<float>(A, nr, vec, nblk, items, st); break;
@@ -431,6 +431,66 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
     }
   }
   return UNIRL_OK;
+}
+
+extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, const float* sigma, int64_t n_sigma,
+                                      int64_t R, int64_t D, float threshold, float* kl_out, uint8_t* mask_out,
+                                      void* workspace, size_t workspace_bytes, void* stream) {
+  if (!dtype_ok(dtype)) return UNIRL_E_DTYPE;
+  if (R < 0 || D <= 0 || n_sigma <= 0) return UNIRL_E_SHAPE;
+  if (R == 0) return UNIRL_OK;
+  if (!p || !q || !sigma || !kl_out) return UNIRL_E_NULL;
+  if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
+  return kl_mask_run(p, q, dtype, sigma, n_sigma, R, D, threshold, kl_out, mask_out, ws_partials(workspace),
+                     kPartialCapacity, (hipStream_t)stream);
+}
+
+// ---------------------------------------------------------------------------
+// The same call for callers that cannot allocate (a HIP graph under capture, a serving loop, a
+// harness that forbids hipMalloc): the per-workgroup partials live in a static device array of
+// this library instead of a caller-owned workspace.  Every GPU holds its own copy of the array
+// at its own address, looked up once per device; host code only ever uses that address, never
+// the array's name.  The kernels overwrite every partial they read back, so nothing needs
+// clearing between calls; calls that overlap on one GPU share the array and race.
+// ---------------------------------------------------------------------------
+static __device__ __align__(256) double scratch[kKlStaticRows];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+double* g_scratch_ptr[kMaxDevices];  // device address of `scratch` on each GPU, null until looked up
+
+int kl_static_scratch(double** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= kMaxDevices) return UNIRL_E_LIMIT;
+  std::lock_guard<std::mutex> hold(g_scratch_mutex);
+  if (!g_scratch_ptr[dev]) {
+    void* addr = nullptr;
+    e = hipGetSymbolAddress(&addr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return (int)e;
+    if (!addr) return UNIRL_E_NULL;
+    g_scratch_ptr[dev] = reinterpret_cast<double*>(addr);
+  }
+  *out = g_scratch_ptr[dev];
+  return UNIRL_OK;
+}
+}  // namespace
+
+extern "C" int unirl_gaussian_kl_mask_static(const void* p, const void* q, int dtype, const float* sigma,
+                                             int64_t n_sigma, int64_t R, int64_t D, float threshold, float* kl_out,
+                                             uint8_t* mask_out, void* stream) {
+  if (!dtype_ok(dtype)) return UNIRL_E_DTYPE;
+  if (R < 0 || D <= 0 || n_sigma <= 0) return UNIRL_E_SHAPE;
+  if (R > kKlStaticRows) return UNIRL_E_LIMIT;  // one launch pair, partials within the static array
+  if (R == 0) return UNIRL_OK;
+  if (!p || !q || !sigma || !kl_out) return UNIRL_E_NULL;
+  double* partials = nullptr;
+  const int rc = kl_static_scratch(&partials);
+  if (rc != 0) return rc;
+  return kl_mask_run(p, q, dtype, sigma, n_sigma, R, D, threshold, kl_out, mask_out, partials, kKlStaticRows,
+                     (hipStream_t)stream);
 }
 
 extern "C" int unirl_flowdppo_step(const void* p, const void* q, int dtype, const float* sigma, int64_t n_sigma,
