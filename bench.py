@@ -13,10 +13,13 @@ a HIP graph over rotating buffer sets, so neither the launch path nor the 256 MB
 last-level cache hides the kernel time); `cpu_baseline` is the eager-torch CPU oracle of
 the headline path on a bounded row sample, timed on this host's cores.
 
-Two probe modes print their own JSON line and exit: `--traffic-probe` (three launches of every
-kernel after three calibration copies, the command the hardware byte counters are collected on)
-and `--replay-probe` (the kernel's caller in training, the chunked lm_head + log-prob replay,
-forward + backward, against the reference's torch ops under checkpoint).
+Three probe modes print their own JSON line and exit: `--traffic-probe` (three launches of every
+kernel after three calibration copies, the command the hardware byte counters are collected on),
+`--replay-probe` (the kernel's caller in training, the chunked lm_head + log-prob replay,
+forward + backward, against the reference's torch ops under checkpoint) and `--timeline` (where
+the time of a small shape goes inside the 64-launch graph: launch gaps and kernel bodies from
+clock readings the kernels of the measurement build take themselves; needs
+`python -m unirl_amd.build --tune`).
 """
 
 from __future__ import annotations
@@ -120,15 +123,22 @@ def n_sets_for(bytes_per_set: int) -> int:
 
 
 def make_shapes(torch, dev):
-    from oracle import advantages as oadv
-    from oracle import flowdppo as ofd
-    from oracle import losses as olos
-    from oracle import schedule as osch
-    from oracle import sde as osde
+    """The synthetic shapes.  Every input the GPU sees comes from the package's own functions; the
+    oracle is imported only inside the `cpu` callables (the CPU baseline of each shape)."""
     from unirl_amd import _native as N
     from unirl_amd import ops
+    from unirl_amd.sde.runtime import get_sigma_schedule
+    from unirl_amd.types import compute_advantages
 
-    sig = osch.sigma_schedule(28, 3.0)
+    def oracle(name):
+        import importlib
+
+        return importlib.import_module(f"oracle.{name}")
+
+    def pack_padded(x, lengths):
+        return torch.cat([x[r, : int(lengths[r])] for r in range(x.shape[0])], dim=0)
+
+    sig = get_sigma_schedule(28, 3.0)
     sig_d = sig.to(dev)
     shapes = []
 
@@ -149,15 +159,15 @@ def make_shapes(torch, dev):
     shapes.append(dict(
         name="sde_step_logp", config=1, shape="fp32 [8,16,128,128], step 10/28, shift 3, eta 0.7, sampling",
         bytes=bytes1, read_bytes=3 * numel * 4, write_bytes=2 * numel * 4, elements=numel, run=run1, sets=ns,
-        cpu=lambda: osde.sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7, noise=host1[2],
-                                     sigma_max=sig[1]),
+        cpu=lambda: oracle("sde").sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7, noise=host1[2],
+                                              sigma_max=sig[1]),
         cpu_bytes=bytes1,
     ))
 
     # the same step in replay mode: the stored next latent is given, mean and log-prob come back
-    prev_host = osde.sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7, noise=host1[2],
-                                 sigma_max=sig[1])[0]
-    prev1 = [prev_host.to(dev) + 0.0 * k for k in range(ns)]
+    prev_dev = run1(0)[0]
+    prev_host = prev_dev.cpu()
+    prev1 = [prev_dev + 0.0 * k for k in range(ns)]
     bytes1r = 4 * numel * 4  # reads noise_pred, sample, prev_sample; writes the mean
 
     def run1r(i):
@@ -169,8 +179,8 @@ def make_shapes(torch, dev):
         name="sde_step_logp_replay", config=1,
         shape="fp32 [8,16,128,128], step 10/28, replay of a stored transition (3 reads, 1 write)",
         bytes=bytes1r, read_bytes=3 * numel * 4, write_bytes=numel * 4, elements=numel, run=run1r, sets=ns,
-        cpu=lambda: osde.sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7,
-                                     prev_sample=prev_host, sigma_max=sig[1]),
+        cpu=lambda: oracle("sde").sde_denoise("flow", host1[1], host1[0], sig[10], sig[11], eta=0.7,
+                                              prev_sample=prev_host, sigma_max=sig[1]),
         cpu_bytes=bytes1r,
     ))
 
@@ -180,7 +190,7 @@ def make_shapes(torch, dev):
     new = old + 0.05 * torch.randn(256, 8192, generator=g)
     lengths = torch.randint(512, 8193, (256,), generator=g)
     rewards = (torch.rand(256, generator=g) < 0.5).float()
-    adv = oadv.compute_advantages(rewards, [i // 16 for i in range(256)])
+    adv = compute_advantages(rewards.to(dev), [i // 16 for i in range(256)]).cpu()
     n_valid = int(lengths.sum())
     bytes3_padded = 2 * new.numel() * 4
     bytes3_valid = 2 * n_valid * 4
@@ -191,7 +201,7 @@ def make_shapes(torch, dev):
     for kind, code, kw in (("grpo", N.LOSS_GRPO, dict(clip_low=0.2, clip_high=0.28)),
                            ("drpo", N.LOSS_DRPO, dict(drpo_epsilon=5.0))):
         plans[kind] = [ops.RatioLossPlan(a, b, adv_d, kind=code, lengths=len_d, **kw) for a, b in sets3]
-    newp, oldp = olos.pack_padded(new, lengths), olos.pack_padded(old, lengths)
+    newp, oldp = pack_padded(new, lengths), pack_padded(old, lengths)
     for kind, okw in (("grpo", dict(clip_range=0.2, clip_range_high=0.28)), ("drpo", dict(epsilon=5.0))):
         shapes.append(dict(
             name=f"ratio_loss_{kind}", config=3,
@@ -199,7 +209,8 @@ def make_shapes(torch, dev):
             bytes=bytes3_valid, bytes_padded=bytes3_padded, read_bytes=bytes3_valid, write_bytes=0,
             elements=n_valid,
             run=(lambda i, k=kind: plans[k][i % ns3].forward(False)), sets=ns3,
-            cpu=(lambda k=kind, o=okw: olos.token_loss(k, newp, oldp, adv, lengths, **o)), cpu_bytes=bytes3_valid,
+            cpu=(lambda k=kind, o=okw: oracle("losses").token_loss(k, newp, oldp, adv, lengths, **o)),
+            cpu_bytes=bytes3_valid,
         ))
     # the whole training micro-step: loss, metrics and the gradient w.r.t. new_logp in one pass
     # (the gradient tensor has the padded shape; the padding is written as zeros)
@@ -207,7 +218,7 @@ def make_shapes(torch, dev):
 
     def cpu_step(k, o):
         leaf = newp.clone().requires_grad_(True)
-        olos.token_loss(k, leaf, oldp, adv, lengths, **o)[0].backward()
+        oracle("losses").token_loss(k, leaf, oldp, adv, lengths, **o)[0].backward()
 
     for kind, okw in (("grpo", dict(clip_range=0.2, clip_range_high=0.28)), ("drpo", dict(epsilon=5.0))):
         shapes.append(dict(
@@ -254,7 +265,8 @@ def make_shapes(torch, dev):
     shapes.append(dict(
         name="gaussian_kl_mask", config=4, shape="bf16 [2,16,21,60,104] old/new means, threshold 0.01",
         bytes=bytes4, read_bytes=bytes4, write_bytes=0, elements=old_m.numel(), run=run4, sets=ns4,
-        cpu=lambda: ofd.kl_per_sample(new_m, old_m, sig_t.reshape(1, 1, 1, 1, 1, 1)) < 0.01, cpu_bytes=bytes4,
+        cpu=lambda: oracle("flowdppo").kl_per_sample(new_m, old_m, sig_t.reshape(1, 1, 1, 1, 1, 1)) < 0.01,
+        cpu_bytes=bytes4,
     ))
 
     # the loss step of Flow-DPPO around that kernel: KL, masks, loss, metrics and the gradient
@@ -269,7 +281,8 @@ def make_shapes(torch, dev):
 
     def cpu4s():
         leaf = new_lp.clone().requires_grad_(True)
-        ofd.flowdppo_loss(leaf, old_lp, new_m, old_m, adv4, sig_t.reshape(1, 1, 1, 1, 1, 1), 0.01)[0].mean().backward()
+        oracle("flowdppo").flowdppo_loss(leaf, old_lp, new_m, old_m, adv4, sig_t.reshape(1, 1, 1, 1, 1, 1),
+                                         0.01)[0].mean().backward()
 
     shapes.append(dict(
         name="flowdppo_step", config=4,
@@ -294,7 +307,7 @@ def make_shapes(torch, dev):
         name="sde_rollout_logp", config=5, shape="fp32 [16,4096,64], 10 steps from step 0, eta 0.7",
         bytes=bytes5, read_bytes=21 * x0.numel() * 4, write_bytes=x0.numel() * 4, elements=10 * x0.numel(),
         run=run5, sets=1,
-        cpu=lambda: osde.sde_rollout("flow", x0, vs, nz, sig, 0.7), cpu_bytes=bytes5, cpu_reps=3,
+        cpu=lambda: oracle("sde").sde_rollout("flow", x0, vs, nz, sig, 0.7), cpu_bytes=bytes5, cpu_reps=3,
     ))
     return shapes
 
@@ -313,6 +326,16 @@ def make_floor(torch, dev, read_bytes: int, write_bytes: int, n_sets: int, tail_
         ops.calib_stream(srcs[i % n_sets], rb, dsts[i % n_sets], wb, sink, tail_launch=tail_launch)
 
     return run
+
+
+def kernel_source_sha256() -> str:
+    """Hash of the token kernel's source text (the kernel file and the helpers it includes)."""
+    import hashlib
+
+    h = hashlib.sha256()
+    for name in ("token_logp.hip", "common.cuh"):
+        h.update((ROOT / "unirl_amd" / "csrc" / name).read_bytes())
+    return h.hexdigest()
 
 
 def make_headline(torch, dev, rows: int, vocab: int):
@@ -388,6 +411,137 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
     return out
 
 
+def tail_probe(torch, dev):
+    """What finishing a grid-wide reduction costs after its streaming part, at the byte counts of the
+    three small reducing shapes: the streaming kernel alone, plus a dependent second launch (the
+    library's scheme), and finished inside the one launch by a polling workgroup
+    (`unirl_calib_reduce` modes 0 / 1 / 2), each as 64 back-to-back calls in a HIP graph over
+    rotating inputs."""
+    from unirl_amd import ops
+
+    pool = torch.ones(160 * 2**20, dtype=torch.float32, device=dev)  # 640 MiB: beyond L2 + last-level cache
+    out = torch.zeros(1, dtype=torch.float64, device=dev)
+    rows = []
+    for label, nbytes in (("ratio loss, config 3 (valid tokens)", 8915200), ("gaussian KL, config 4", 16773120),
+                          ("SDE step replay reads, config 1", 25165824)):
+        n_sets = pool.numel() * 4 // nbytes
+        views = [pool.view(torch.uint8)[k * nbytes : (k + 1) * nbytes] for k in range(n_sets)]
+        for nwg in (256, 512):
+            scratch = torch.zeros(16 + 16 * nwg, dtype=torch.uint8, device=dev)
+            got = {}
+            for mode in (1, 2):  # same sum both ways, also on a second call that meets the first one's tags
+                for _ in range(2):
+                    ops.calib_reduce(views[0], nbytes, mode, nwg, scratch, out)
+                torch.cuda.synchronize()
+                got[mode] = float(out.item())
+            row = {"shape": label, "bytes": nbytes, "workgroups": nwg, "results_agree": got[1] == got[2]}
+            for mode, key in ((0, "stream_only_us"), (1, "two_launches_us"), (2, "one_launch_polled_us")):
+                row[key] = round(time_in_graph(torch, lambda i, m=mode: ops.calib_reduce(views[i % n_sets], nbytes, m, nwg,
+                                                                                         scratch, out), n_sets), 2)
+            log(f"tail probe: {row}")
+            rows.append(row)
+    empty = torch.zeros(4, dtype=torch.int32, device=dev)
+    rows.append({"shape": "one-wavefront kernel with one store, alone",
+                 "us": round(time_in_graph(torch, lambda i: ops.calib_stream(None, 0, None, 0, empty, tail_launch=True), 2), 2)})
+    return rows
+
+
+def timeline_probe(torch, dev, names):
+    """Device-side timeline of the small shapes inside the 64-launch graph the bench times them in.
+
+    A kernel-trace profiler serialises the dispatches of a graph and so cannot show the gaps
+    between them; here the kernels of the measurement build (`python -m unirl_amd.build --tune`)
+    read the 100 MHz device clock at entry, after their streaming loop and at exit, every
+    workgroup for itself, into a buffer.  Per launch: gap = first workgroup's start minus the
+    previous launch's last end; body = last end minus first start.  The marks cost about 0.5 us
+    per call, so the sum sits that much above the release library's time."""
+    import ctypes
+
+    from unirl_amd import _native as N
+    from unirl_amd.build import TUNE_LIB_PATH
+
+    if not TUNE_LIB_PATH.exists():
+        raise SystemExit(f"bench.py --timeline needs {TUNE_LIB_PATH}: build it with `python -m unirl_amd.build --tune`")
+    N.LIB_PATH = TUNE_LIB_PATH  # before the first call binds the library
+    lib = N.lib()
+    lib.unirl_trace_begin.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
+    lib.unirl_trace_entry.restype = ctypes.c_char_p
+    lib.unirl_trace_entry.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_size_t)]
+    tick_ns = 10.0
+    buf = torch.zeros(8 * 2**20, dtype=torch.int64, device=dev)
+    spin = torch.randn(64 * 2**20, device=dev)
+    for _ in range(300):  # bring the clocks up
+        spin.mul_(1.0001)
+    torch.cuda.synchronize()
+    out = {}
+    med = lambda v: round(statistics.median(v) / 1e3, 2) if v else None
+    for sh in make_shapes(torch, dev):
+        if names and sh["name"] not in names:
+            continue
+        fn, n_sets = sh["run"], sh["sets"]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for i in range(n_sets):
+                fn(i)
+        torch.cuda.synchronize()
+        lib.unirl_trace_begin(buf.data_ptr(), buf.numel() * 8)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for i in range(64):
+                fn(i % n_sets)
+        torch.cuda.synchronize()
+        entries = []
+        for i in range(lib.unirl_trace_count()):
+            nb, off = ctypes.c_uint(), ctypes.c_size_t()
+            name = lib.unirl_trace_entry(i, ctypes.byref(nb), ctypes.byref(off)).decode()
+            entries.append((name, nb.value, off.value))
+        lib.unirl_trace_begin(None, 0)
+        per, events = {}, []
+        for rep in range(6):
+            buf.zero_()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            if rep == 0:
+                continue
+            events.append(e0.elapsed_time(e1) * 1e3 / 64)
+            host = buf.cpu()
+            prev_end = None
+            for name, nb, off in entries:
+                t = host[off : off + nb * 4].view(nb, 4)
+                t = t[t[:, 3] > 0]
+                if t.numel() == 0:
+                    continue
+                start, end = int(t[:, 0].min()), int(t[:, 3].max())
+                d = per.setdefault(name, dict(gap=[], body=[], first_wg_done=[], stream_done=[]))
+                d["body"].append((end - start) * tick_ns)
+                d["first_wg_done"].append((int(t[:, 3].min()) - start) * tick_ns)
+                marks = t[:, 1][t[:, 1] > 0]
+                if marks.numel():
+                    d["stream_done"].append((int(marks.max()) - start) * tick_ns)
+                if prev_end is not None:
+                    d["gap"].append((start - prev_end) * tick_ns)
+                prev_end = end
+        del graph
+        row = {"us_per_call_hip_events": round(statistics.median(events), 2), "launches": {}}
+        total = 0.0
+        for name, d in per.items():
+            row["launches"][name] = {
+                "gap_before_us": med(d["gap"]), "body_us": med(d["body"]),
+                "first_workgroup_done_at_us": med(d["first_wg_done"]),
+                "last_workgroup_past_its_loop_at_us": med(d["stream_done"]),
+            }
+            total += (med(d["gap"]) or 0.0) + (med(d["body"]) or 0.0)
+        row["sum_of_gaps_and_bodies_us"] = round(total, 2)
+        log(f"timeline {sh['name']}: {row}")
+        out[sh["name"]] = row
+    return out
+
+
 # ----------------------------------------------------------------------------------------------
 def main() -> int:
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
@@ -407,6 +561,13 @@ def main() -> int:
                          "--rows response tokens) through the fused kernels and through the reference's torch ops "
                          "under checkpoint, then exit (time, peak transient memory; a kernel trace of this command "
                          "shows the split between the head's GEMMs and the log-prob kernels)")
+    ap.add_argument("--timeline", nargs="?", const="", default=None, metavar="SHAPES",
+                    help="device-side timeline (launch gaps, kernel bodies) of the small shapes inside the 64-launch "
+                         "graph, from the measurement build's own clock readings; optional comma-separated shape "
+                         "names; needs `python -m unirl_amd.build --tune`")
+    ap.add_argument("--tail-probe", action="store_true",
+                    help="cost of finishing a grid-wide reduction after its streaming part: nothing, a second "
+                         "launch, or polled inside the one launch (unirl_calib_reduce), then exit")
     ap.add_argument("--skip-shapes", action="store_true", help="headline only")
     ap.add_argument("--skip-cpu", action="store_true", help="no CPU baselines")
     args = ap.parse_args()
@@ -435,6 +596,15 @@ def main() -> int:
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     log(f"device {torch.cuda.get_device_name(0)}, torch {torch.__version__}, host threads {torch.get_num_threads()}")
+
+    if args.timeline is not None:
+        names = [n for n in args.timeline.split(",") if n]
+        print(json.dumps({"timeline": timeline_probe(torch, dev, names)}), flush=True)
+        return 0
+
+    if args.tail_probe:
+        print(json.dumps({"tail_probe": tail_probe(torch, dev)}), flush=True)
+        return 0
 
     if args.replay_probe:
         print(json.dumps({"replay_probe": replay_probe(torch, dev, args.rows, args.vocab)}), flush=True)
@@ -569,15 +739,22 @@ def main() -> int:
                 f"floor {row.get('floor_us', float('nan')):.2f} us, wrapper {lat:.0f} us")
             shapes_out.append(row)
 
-    # HBM bytes per launch from hardware counters, when a committed counter summary covers this workload
-    traffic = None
+    # HBM bytes per launch from hardware counters.  Counter runs cannot be made from inside the bench,
+    # so the figure comes from the committed counter summary -- and only while that summary still
+    # describes this kernel: same workload, and the same text of the kernel's two source files.
+    traffic, traffic_source = None, None
     traffic_file = ROOT / "profiles" / "token_logp_entropy_traffic.json"
     if traffic_file.exists():
         try:
             rec = json.loads(traffic_file.read_text())
-            if rec.get("rows") == args.rows and rec.get("vocab") == args.vocab:
+            same_kernel = rec.get("kernel_source_sha256") == kernel_source_sha256()
+            if rec.get("rows") == args.rows and rec.get("vocab") == args.vocab and same_kernel:
                 traffic = rec.get("hbm_bytes_per_launch")
-        except (ValueError, OSError):
+                traffic_source = (f"committed counter summary profiles/{traffic_file.name} "
+                                  f"(kernel sources sha256 {rec['kernel_source_sha256'][:12]}), not measured in this run")
+            elif not same_kernel:
+                traffic_source = "none: the kernel's sources changed since the committed counter summary was taken"
+        except (ValueError, OSError, KeyError):
             traffic = None
 
     result = {
@@ -592,6 +769,7 @@ def main() -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
+        "storage_dtype": "bf16",
         "data": "synthetic",
         "config": {
             "workload": f"token log-prob + entropy, logits bf16 [{args.rows},{args.vocab}] ~N(0,2) with 1% spiked "
@@ -600,7 +778,7 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
+            "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
             "kernel": "token_logp_entropy_kernel<bf16>", "algorithmic_bytes_per_launch": alg_bytes,
             "launch_ms": round(event_ms, 4),
         },

@@ -80,6 +80,21 @@ int unirl_calib_copy(const void* src, void* dst, size_t bytes, void* stream);
 int unirl_calib_stream(const void* src, size_t read_bytes, void* dst, size_t write_bytes,
                        int tail_launch, void* sink, void* stream);
 
+/* Measurement aid, no counterpart in the reference: what finishing a grid-wide reduction costs.
+ * Sums the `read_bytes / 4` floats at src (a multiple of 16 bytes, 16-byte aligned) over
+ * n_workgroups workgroups of 256 threads and finishes in one of three ways:
+ *   mode 0  the streaming kernel only (per-workgroup partials stored, *out untouched);
+ *   mode 1  plus a dependent second launch that adds the partials -- the scheme of every
+ *           reducing entry point of this library;
+ *   mode 2  a single launch: the partials are published as self-validating tagged 8-byte units
+ *           (relaxed device-scope atomics) and polled by the last workgroup, bounded by a
+ *           one-second clock budget (*out is NaN if it ever runs out).
+ * scratch: at least 16 + 16 * n_workgroups bytes, zero-filled ONCE before its first use with
+ * mode 2 (its first word carries the call tag from call to call) and used by one call at a
+ * time.  Modes 1 and 2 return the same bits in *out. */
+int unirl_calib_reduce(const void* src, size_t read_bytes, int mode, unsigned int n_workgroups,
+                       void* scratch, size_t scratch_bytes, double* out, void* stream);
+
 /* ------------------------------------------------------------------------
  * One SDE transition + per-sample Gaussian log-prob.
  * Replaces StepStrategy.denoise -> SDEStrategy.step -> _finalize_logp

@@ -360,3 +360,12 @@ def test_per_sample_view_never_hands_stride_zero_for_several_samples(monkeypatch
     # outputs may not overlap across samples
     with pytest.raises(ValueError):
         ops._per_sample_view(one.expand(3, 3, 4), "prev_out", writable=True)
+
+
+def test_release_library_reads_no_environment_knobs(built_lib):
+    """The launch-shape knobs of the measurement build (UNIRL_* environment variables) must not
+    exist in the shipped library: an exported variable must never change a production launch."""
+    blob = built_lib.read_bytes()
+    names = set(re.findall(rb"UNIRL_[A-Z0-9_]{3,}", blob))
+    assert not names, f"environment knob names in the release library: {sorted(names)}"
+    assert b"getenv" not in blob or b"UNIRL_" not in blob

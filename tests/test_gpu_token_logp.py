@@ -120,6 +120,43 @@ def test_out_of_range_id_gives_nan_not_a_fault(dev):
     assert torch.isnan(lp[1]) and torch.isnan(lp[2]) and torch.isfinite(lp[0]) and torch.isfinite(lp[3])
 
 
+def test_out_of_range_id_gets_a_zero_gradient_row(dev):
+    """A padding id (e.g. -100) has no log-prob; its row of the gradient is zero, whatever the
+    upstream gradient holds (NaN included), and the other rows are untouched by it."""
+    from unirl_amd import ops
+
+    V = 1000
+    x, ids = logits(6, V, 9, torch.bfloat16)
+    bad = ids.clone()
+    bad[1], bad[4] = -100, V
+    xd = x.to(dev)
+    _, _, lse = ops.token_logp_entropy(xd, bad.to(dev), 1.0, want_logp=False, want_entropy=False, want_lse=True)
+    g = torch.randn(6)
+    g[4] = float("nan")
+    grad = ops.token_logp_bwd(xd, bad.to(dev), 1.0, lse, g.to(dev)).float().cpu()
+    assert torch.count_nonzero(grad[1]) == 0 and torch.count_nonzero(grad[4]) == 0
+    good = ops.token_logp_bwd(xd, ids.to(dev), 1.0, lse, torch.nan_to_num(g).to(dev)).float().cpu()
+    keep = [0, 2, 3, 5]
+    assert torch.equal(grad[keep], good[keep])
+    # in place on the same buffer gives the same bits
+    buf = xd.clone()
+    ops.token_logp_bwd(buf, bad.to(dev), 1.0, lse, g.to(dev), in_place=True)
+    assert torch.equal(buf.float().cpu(), grad)
+
+
+def test_all_minus_inf_row_has_lse_minus_inf(dev):
+    """torch.logsumexp of a row of -inf is -inf (and the log-prob -inf - (-inf) = NaN)."""
+    from unirl_amd import ops
+
+    x = torch.randn(3, 500)
+    x[1] = float("-inf")
+    ids = torch.tensor([3, 4, 5])
+    lp, ent, lse = ops.token_logp_entropy(x.to(dev), ids.to(dev), 1.0, want_lse=True)
+    ref = torch.logsumexp(x, dim=-1)
+    assert float(lse[1]) == float("-inf") and torch.isnan(lp[1]) and torch.isnan(ent[1])
+    assert torch.allclose(lse.cpu()[[0, 2]], ref[[0, 2]], rtol=1e-6)
+
+
 def test_shape_errors(dev):
     from unirl_amd import models
 
@@ -304,6 +341,31 @@ def test_chunked_replay_keeps_logits_only_within_its_budget(dev, monkeypatch):
     with pytest.raises(RuntimeError, match="overwritten by their gradient"):
         out.sum().backward()
     head.zero_grad()
+
+    # a Linear subclass, or a Linear with a forward hook, may hold its output elsewhere: its logits are
+    # never overwritten, so the captured output still holds logits after the backward and a second
+    # backward through the same graph works
+    class MyLinear(torch.nn.Linear):
+        pass
+
+    sub = MyLinear(H, V).to(dev)
+    hooked = torch.nn.Linear(H, V).to(dev)
+    seen = []
+    hooked.register_forward_hook(lambda mod, args, out: seen.append(out))
+    for lm_head in (sub, hooked):
+        assert not ar_logp._is_plain_linear(lm_head)
+        h = torch.randn(B, T_max, H, generator=g).to(dev).requires_grad_(True)
+        out = models.chunked_replay_logp(lm_head, h, toks, chunk=16, keep_logits=True)
+        out.sum().backward(retain_graph=True)
+        first = h.grad.clone()
+        h.grad = None
+        out.sum().backward()
+        assert torch.equal(h.grad, first)
+    assert ar_logp._is_plain_linear(head)
+    captured = seen[0].detach()
+    with torch.no_grad():
+        again = torch.nn.functional.linear(h[:, :16].detach(), hooked.weight, hooked.bias)
+    assert torch.allclose(captured, again), "a hooked head's captured logits were overwritten"
 
     assert B * T_max * V * 4 < ar_logp.KEEP_LOGITS_BYTES
     assert not any("RecomputedChunk" in n for n in path(head))

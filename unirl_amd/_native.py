@@ -112,6 +112,7 @@ _SIGNATURES = {
     "unirl_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
     "unirl_calib_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "unirl_calib_stream": (c_int, [c_void_p, c_size_t, c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
+    "unirl_calib_reduce": (c_int, [c_void_p, c_size_t, c_int, ctypes.c_uint, c_void_p, c_size_t, c_void_p, c_void_p]),
     "unirl_sde_step_logp": (
         c_int,
         [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,

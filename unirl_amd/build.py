@@ -1,6 +1,7 @@
 """Build libunirl_hip.so for gfx950 with hipcc, in-tree.
 
     python -m unirl_amd.build            # compile every csrc/*.hip and link
+    python -m unirl_amd.build --tune     # measurement build beside it (libunirl_hip_tune.so)
 
 hipcc cross-compiles without a GPU.  Objects go to ``unirl_amd/lib/obj`` and the
 shared library to ``unirl_amd/lib/libunirl_hip.so``; both are git-ignored build
@@ -65,32 +66,50 @@ def sources() -> List[Path]:
     return sorted(CSRC_DIR.glob("*.hip"))
 
 
-def build(verbose: bool = True, jobs: int | None = None) -> Path:
-    """Compile every kernel source and link the shared library. Always recompiles."""
+def build(verbose: bool = True, jobs: int | None = None, *, tune: bool = False, out: Path | None = None,
+          extra_flags: List[str] | None = None) -> Path:
+    """Compile every kernel source and link the shared library. Always recompiles.
+
+    ``tune=True`` makes a measurement build (``-DUNIRL_TUNE -DUNIRL_TRACE``: launch-shape knobs read
+    from the environment, device-side timeline marks); it must be given its own ``out`` path and is
+    never the library the package loads.
+    """
     hipcc = _hipcc()
-    OBJ_DIR.mkdir(parents=True, exist_ok=True)
+    if tune and out is None:
+        raise ValueError("a tune build needs its own output path (out=...)")
+    lib_path = Path(out) if out is not None else LIB_PATH
+    obj_dir = OBJ_DIR if out is None else lib_path.parent / (lib_path.stem + "_obj")
+    obj_dir.mkdir(parents=True, exist_ok=True)
     srcs = sources()
     if not srcs:
         raise RuntimeError(f"no .hip sources under {CSRC_DIR}")
-    objs = [OBJ_DIR / (s.stem + ".o") for s in srcs]
+    objs = [obj_dir / (s.stem + ".o") for s in srcs]
     jobs = jobs or min(len(srcs), max(1, (os.cpu_count() or 2) // 2))
+    flags = list(HIPCC_FLAGS) + (["-DUNIRL_TUNE", "-DUNIRL_TRACE"] if tune else []) + list(extra_flags or [])
 
     def compile_one(pair):
         src, obj = pair
         if verbose:
             print(f"[unirl_amd.build] hipcc {src.name}", flush=True)
-        _run([hipcc, *HIPCC_FLAGS, "-c", str(src), "-o", str(obj)])
+        _run([hipcc, *flags, "-c", str(src), "-o", str(obj)])
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         list(pool.map(compile_one, zip(srcs, objs)))
 
-    tmp = LIB_PATH.with_suffix(".so.tmp")
+    tmp = lib_path.with_suffix(".so.tmp")
     _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(tmp), *map(str, objs)])
-    os.replace(tmp, LIB_PATH)
+    os.replace(tmp, lib_path)
     if verbose:
-        print(f"[unirl_amd.build] linked {LIB_PATH}", flush=True)
-    return LIB_PATH
+        print(f"[unirl_amd.build] linked {lib_path}", flush=True)
+    return lib_path
+
+
+TUNE_LIB_PATH = LIB_DIR / "libunirl_hip_tune.so"
 
 
 if __name__ == "__main__":
-    build()
+    if "--tune" in sys.argv[1:]:
+        # the measurement build `bench.py --timeline` and the launch-shape sweeps load
+        build(tune=True, out=TUNE_LIB_PATH)
+    else:
+        build()

@@ -413,6 +413,29 @@ __device__ __forceinline__ float block_min(float v, float* lds) {
 }
 
 // ---------------------------------------------------------------------------
+// Timeline marks of measurement builds (-DUNIRL_TRACE); nothing otherwise.  T0 reads the clock
+// at kernel entry, MARK reads it again, END has thread 0 of the workgroup store
+// {start, mark1, mark2, end} at slot (workgroup index) of the launch's trace slice.
+// ---------------------------------------------------------------------------
+#ifdef UNIRL_TRACE
+#define UNIRL_TRACE_T0() const unsigned long long trace_t0_ = wall_clock64(); unsigned long long trace_m1_ = 0, trace_m2_ = 0
+#define UNIRL_TRACE_MARK1() trace_m1_ = wall_clock64()
+#define UNIRL_TRACE_MARK2() trace_m2_ = wall_clock64()
+#define UNIRL_TRACE_END(tr)                                                                      \
+  do {                                                                                           \
+    if ((tr) && threadIdx.x == 0) {                                                              \
+      unsigned long long* q_ = (tr) + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 4;         \
+      q_[0] = trace_t0_; q_[1] = trace_m1_; q_[2] = trace_m2_; q_[3] = wall_clock64();           \
+    }                                                                                            \
+  } while (0)
+#else
+#define UNIRL_TRACE_T0() ((void)0)
+#define UNIRL_TRACE_MARK1() ((void)0)
+#define UNIRL_TRACE_MARK2() ((void)0)
+#define UNIRL_TRACE_END(tr) ((void)0)
+#endif
+
+// ---------------------------------------------------------------------------
 // Grid-wide sums are two launches: the streaming kernel stores one partial per
 // workgroup (plain stores), and a finalize kernel of a few wavefronts -- ordered
 // after it on the stream -- adds them in index order.  In-kernel alternatives

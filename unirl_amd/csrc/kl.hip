@@ -35,6 +35,7 @@ struct KlArgs {
   float* elem_out;
   double* partials;
   int always_partials;  // store workgroup partials even when one workgroup covers a row
+  UNIRL_TRACE_FIELD
 };
 
 template <typename T>
@@ -57,6 +58,7 @@ __device__ __forceinline__ void kl_finish(const KlArgs& A, int64_t row, double q
 template <typename T, int VEC, int ITEMS>
 __global__ __launch_bounds__(kKlThreads) void gaussian_kl_kernel(KlArgs A) {
   __shared__ double lds[kKlThreads / kWave];
+  UNIRL_TRACE_T0();
   const int64_t row = blockIdx.y;
   const int64_t D = A.D;
   const T* __restrict__ pp = reinterpret_cast<const T*>(A.p) + row * D;
@@ -83,6 +85,7 @@ __global__ __launch_bounds__(kKlThreads) void gaussian_kl_kernel(KlArgs A) {
       }
     }
   }
+  UNIRL_TRACE_MARK1();
   const double part = block_sum<double>((double)acc, lds);
   if (threadIdx.x != 0) return;
   if (gridDim.x == 1 && !A.always_partials) {
@@ -90,15 +93,19 @@ __global__ __launch_bounds__(kKlThreads) void gaussian_kl_kernel(KlArgs A) {
   } else {
     A.partials[row * gridDim.x + blockIdx.x] = part;  // summed by gaussian_kl_finalize_kernel
   }
+  UNIRL_TRACE_END(A.trace);
 }
 
 // One wavefront per row: adds the workgroup partials in index order, divides, thresholds.
 __global__ __launch_bounds__(kKlThreads) void gaussian_kl_finalize_kernel(KlArgs A, int64_t R, unsigned int nblk) {
+  UNIRL_TRACE_T0();
   const int64_t row = (int64_t)blockIdx.x * (kKlThreads / kWave) + threadIdx.x / kWave;
   if (row >= R) return;
   const float den = kl_den(A, row);  // issued with the partial loads, not after them
   const double q = wave_ordered_sum(A.partials + row * nblk, nblk);
+  UNIRL_TRACE_MARK1();
   if ((threadIdx.x & (kWave - 1)) == 0) kl_finish(A, row, q, den);
+  UNIRL_TRACE_END(A.trace);
 }
 
 template <typename T, int VEC>
@@ -342,6 +349,7 @@ __global__ __launch_bounds__(kKlThreads) void flowdppo_loss_kernel(DppoArgs A) {
 // first wavefront runs the [B,S'] problem on it.  R <= kDppoWaveMax.
 __global__ __launch_bounds__(kKlThreads) void flowdppo_finish_kernel(KlArgs K, DppoArgs A, unsigned int nblk) {
   __shared__ float lds_kl[kDppoWaveMax];
+  UNIRL_TRACE_T0();
   const int wave = threadIdx.x / kWave;
   const int64_t R = A.n;
   for (int64_t row = wave; row < R; row += kKlThreads / kWave) {
@@ -354,8 +362,10 @@ __global__ __launch_bounds__(kKlThreads) void flowdppo_finish_kernel(KlArgs K, D
       lds_kl[row] = kl;
     }
   }
+  UNIRL_TRACE_MARK1();
   __syncthreads();
   if (wave == 0) dppo_on_one_wave(A, lds_kl);
+  UNIRL_TRACE_END(K.trace);
 }
 
 }  // namespace unirl
@@ -415,6 +425,7 @@ static int kl_mask_run(const void* p, const void* q, int dtype, const float* sig
     A.mask = mask_out ? mask_out + r0 : nullptr;
     A.elem_out = nullptr;
     A.partials = partials;
+    UNIRL_TRACE_SET(A, "kl", nblk * (unsigned int)nr);
     int rc = UNIRL_E_DTYPE;
     switch (dtype) {
       case UNIRL_F32: rc = launch_kl<float>(A, nr, vec, nblk, items, st); break;
@@ -424,6 +435,7 @@ static int kl_mask_run(const void* p, const void* q, int dtype, const float* sig
     if (rc != 0) return rc;
     if (nblk > 1) {
       const int per_block = kKlThreads / kWave;
+      UNIRL_TRACE_SET(A, "kl_finalize", (unsigned int)((nr + per_block - 1) / per_block));
       hipLaunchKernelGGL(gaussian_kl_finalize_kernel, dim3((unsigned int)((nr + per_block - 1) / per_block)),
                          dim3(kKlThreads), 0, st, A, nr, nblk);
       rc = (int)hipGetLastError();
@@ -526,6 +538,7 @@ extern "C" int unirl_flowdppo_step(const void* p, const void* q, int dtype, cons
   K.kl = kl_out;
   K.partials = ws_partials(workspace);
   K.always_partials = 1;
+  UNIRL_TRACE_SET(K, "kl", nblk * (unsigned int)R);
   int rc = UNIRL_E_DTYPE;
   switch (dtype) {
     case UNIRL_F32: rc = launch_kl<float>(K, R, vec, nblk, items, st); break;
@@ -544,6 +557,7 @@ extern "C" int unirl_flowdppo_step(const void* p, const void* q, int dtype, cons
   A.metrics = metrics;
   A.grad_new = grad_new;
   A.grad_scale = loss_scale / (float)R;  // d(loss_scale * mean(elem)) / d elem
+  UNIRL_TRACE_SET(K, "dppo_finish", 1);
   hipLaunchKernelGGL(flowdppo_finish_kernel, dim3(1), dim3(kKlThreads), 0, st, K, A, nblk);
   return (int)hipGetLastError();
 }

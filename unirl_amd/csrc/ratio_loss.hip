@@ -79,6 +79,7 @@ struct RatioArgs {
   float loss_scale;      // gradient arriving at the aggregated loss
   int64_t n_valid_host;  // token-mean denominator when the host knows it, else < 0
   int64_t per_wave;      // packed kernel: vectors in a wavefront's run (a multiple of 64)
+  UNIRL_TRACE_FIELD
 };
 
 // exp(x) for fp32 within ~1.5 ulp: 2^(x*log2(e)) on the hardware exp2, with the rounding error
@@ -420,19 +421,19 @@ __device__ __forceinline__ void fill_ones(float (&m)[VEC]) {
   for (int k = 0; k < VEC; ++k) m[k] = 1.0f;
 }
 
-#ifndef UNIRL_RATIO_ITEMS
-#define UNIRL_RATIO_ITEMS 2  // 4 measured slower on large inputs (registers), equal on small ones
-#endif
-
 // FLAGS >= 0 fixes at compile time whether a loss mask (bit 0) and per-token advantages (bit 1)
 // are read, which keeps the loads of a pass straight-line code (all of them in flight before the
 // first use); FLAGS < 0 reads both switches at run time.
 // With GRAD the kernel also writes grad_new = loss_scale * w_tok * dloss/dnew (the aggregation
 // weights of ratio_loss_bwd_kernel with aggregate set), so a training step reads new / old once.
-template <int KIND, int VEC, bool PACKED, int FLAGS, bool GRAD>
+// ITEMS: vectors in flight per lane and pass.  Two on large inputs (four cost registers: 10 %
+// slower for DRPO on 8 M tokens); four when that covers every row in a single pass, because a
+// second pass cannot start before the first has come back and at a few MB a trip to memory is
+// most of the kernel (9.2 -> 8.7 us on 1.1 M tokens in 256 ragged rows).
+template <int KIND, int VEC, bool PACKED, int FLAGS, bool GRAD, int ITEMS = 2>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A) {
-  constexpr int ITEMS = UNIRL_RATIO_ITEMS;  // vectors in flight per lane
   __shared__ double lds_v[kRlVals][kRlThreads];
+  UNIRL_TRACE_T0();
   const RatioConsts C = A.C;
   const bool has_mask = (FLAGS < 0) ? (A.mask != nullptr) : ((FLAGS & 1) != 0);
   const bool adv_tok = (FLAGS < 0) ? (C.adv_per_token != 0) : ((FLAGS & 2) != 0);
@@ -564,7 +565,9 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
       }
     }
   }
+  UNIRL_TRACE_MARK1();
   store_block_partials(A, acc, wc, lds_v);
+  UNIRL_TRACE_END(A.trace);
 }
 
 // Largest s in [lo, n_seq) with cu(s) <= tok, found by the whole wavefront: every round 64 lanes
@@ -603,6 +606,7 @@ template <int KIND, int FLAGS, bool GRAD, int ITEMS>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs A) {
   constexpr int VEC = 4;
   __shared__ double lds_v[kRlVals][kRlThreads];
+  UNIRL_TRACE_T0();
   const RatioConsts C = A.C;
   const bool has_mask = (FLAGS & 1) != 0;
   const bool adv_tok = (FLAGS & 2) != 0;
@@ -722,10 +726,10 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs
             const int64_t t = i * VEC + k;
             while (t >= lend && ls + 1 < n_seq) {
               ++ls;
-              const int64_t e = A.seq[ls + 1];
+              const int64_t e = cu(ls + 1);
               lw = seq_weight(C, e - lend);
               lend = e;
-              if (!adv_tok) ladv = A.adv[ls];
+              if (!adv_tok) ladv = seq_adv(ls);
             }
             bool hi, lo;
             float dl;
@@ -767,7 +771,9 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs
     }
     acc.flush(1.0);
   }
+  UNIRL_TRACE_MARK1();
   if (A.partials) store_block_partials(A, acc, wc, lds_v);  // absent when only the gradient is wanted
+  UNIRL_TRACE_END(A.trace);
 }
 
 // One workgroup of T threads (256, or 1024 when there are more than 512 partial vectors, so that
@@ -779,6 +785,7 @@ __global__ __launch_bounds__(T) void ratio_loss_finalize_kernel(RatioArgs A, uns
   static_assert(kSlices == kRlParts || kSlices == kWave, "a slot's slices fill a 16-lane row or a wavefront");
   __shared__ double lds_t[T];
   __shared__ double lds_tot[kRlVals];
+  UNIRL_TRACE_T0();
   const RatioConsts C = A.C;
   const int t = threadIdx.x;
   {
@@ -807,6 +814,7 @@ __global__ __launch_bounds__(T) void ratio_loss_finalize_kernel(RatioArgs A, uns
     }
     lds_t[v * kSlices + j0] = x;  // transposed: the slices of a slot side by side
   }
+  UNIRL_TRACE_MARK1();
   __syncthreads();
   {
     // thread = (slot, slice) again, now with a slot's slices in one 16-lane row / one wavefront
@@ -866,6 +874,7 @@ __global__ __launch_bounds__(T) void ratio_loss_finalize_kernel(RatioArgs A, uns
       ((unsigned long long)UNIRL_M_RATIO_MIN << (4 * P_NRMIN)) | ((unsigned long long)UNIRL_M_RATIO_MAX << (4 * P_RMAX)) |
       ((unsigned long long)UNIRL_M_ABSDIFF_MAX << (4 * P_AMAX)) | (15ull << (4 * 15));
   A.metrics[(kMetricOf >> (4 * v)) & 15u] = (float)y;
+  UNIRL_TRACE_END(A.trace);
 }
 
 template <int KIND, int VEC>
@@ -1057,6 +1066,10 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
   // to whole spans of 64; only the workgroups whose wavefronts have a run are launched, and a run
   // of up to four spans goes out as a single pass of loads
   bool one_pass = false;
+  // padded / flat layout: four vectors per lane when one pass of four then covers a whole row
+  const int64_t row_vec = ((A.layout == LAYOUT_PADDED ? A.seq_stride : A.n_tok) + 3) / 4;
+  const bool four_items = !packed && S.vec == 4 && row_vec > (int64_t)S.grid.x * kRlThreads * 2 &&
+                          row_vec <= (int64_t)S.grid.x * kRlThreads * 4 && tune_int("UNIRL_RATIO_ITEMS4", 1) == 1;
   if (packed && S.vec == 4) {
     const int64_t waves_per_wg = kRlThreads / kWave;
     const int64_t n_waves = (int64_t)S.grid.x * waves_per_wg;
@@ -1069,12 +1082,17 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
     S.grid.x = (unsigned int)nwg;
     one_pass = A.per_wave / kWave <= 4;
   }
-#define UNIRL_LAUNCH_FWD4(KIND, VEC, PACKED, FLAGS)                                                            \
+#define UNIRL_LAUNCH_FWD5(KIND, VEC, PACKED, FLAGS, ITEMS)                                                     \
   do {                                                                                                         \
     if (grad)                                                                                                  \
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, PACKED, FLAGS, true>), S.grid, block, 0, st, A);    \
+      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, PACKED, FLAGS, true, ITEMS>), S.grid, block, 0, st, A);  \
     else                                                                                                       \
-      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, PACKED, FLAGS, false>), S.grid, block, 0, st, A);   \
+      hipLaunchKernelGGL((ratio_loss_fwd_kernel<KIND, VEC, PACKED, FLAGS, false, ITEMS>), S.grid, block, 0, st, A); \
+  } while (0)
+#define UNIRL_LAUNCH_FWD4(KIND, VEC, PACKED, FLAGS)                                                            \
+  do {                                                                                                         \
+    if (VEC == 4 && !PACKED && four_items) UNIRL_LAUNCH_FWD5(KIND, VEC, PACKED, FLAGS, 4);                     \
+    else UNIRL_LAUNCH_FWD5(KIND, VEC, PACKED, FLAGS, 2);                                                       \
   } while (0)
 #define UNIRL_LAUNCH_PACKED2(KIND, FLAGS, ITEMS)                                                               \
   do {                                                                                                         \
@@ -1103,7 +1121,9 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
     else if (flags == 2) UNIRL_LAUNCH_FWD4(KIND, 4, false, 2);                                                 \
     else UNIRL_LAUNCH_FWD4(KIND, 4, false, 3);                                                                 \
   } while (0)
+  UNIRL_TRACE_SET(A, packed ? "ratio_packed" : "ratio_fwd", S.grid.x * S.grid.y);
   if (A.C.kind == UNIRL_LOSS_GRPO) UNIRL_LAUNCH_FWD(UNIRL_LOSS_GRPO); else UNIRL_LAUNCH_FWD(UNIRL_LOSS_DRPO);
+#undef UNIRL_LAUNCH_FWD5
 #undef UNIRL_LAUNCH_FWD4
 #undef UNIRL_LAUNCH_PACKED
 #undef UNIRL_LAUNCH_PACKED2
@@ -1112,6 +1132,7 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
   const int launch_rc = (int)hipGetLastError();
   if (launch_rc != 0 || !A.metrics) return launch_rc;
   const unsigned int nblk = S.grid.x * S.grid.y;
+  UNIRL_TRACE_SET(A, "ratio_finalize", 1);
   if (nblk <= 512)
     hipLaunchKernelGGL(ratio_loss_finalize_kernel<256>, dim3(1), dim3(256), 0, st, A, nblk);
   else

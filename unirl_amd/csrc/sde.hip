@@ -133,6 +133,7 @@ struct SdeStepArgs {
   double* partials;        // [B][gridDim.x]
   unsigned int nblk;       // host only: grid.x
   int items;               // host only: vectors in flight per lane
+  UNIRL_TRACE_FIELD
 };
 
 // Store VEC floats as `dtype` (wave-uniform switch) at element index `idx` of `base`.
@@ -150,6 +151,7 @@ template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING>
 __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
   __shared__ double lds[kSdeThreads / kWave];
   using T3 = typename std::conditional<SAMPLING, float, TX>::type;
+  UNIRL_TRACE_T0();
 
   const int64_t b = blockIdx.y;
   const int64_t D = A.D;
@@ -214,7 +216,11 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
     if (i0 < nvec) load_pass(i0);
   }
 
-  if (!A.want_logp) return;  // uniform across the grid
+  UNIRL_TRACE_MARK1();
+  if (!A.want_logp) {  // uniform across the grid
+    UNIRL_TRACE_END(A.trace);
+    return;
+  }
 
   const double part = block_sum<double>((double)acc, lds);
   if (threadIdx.x != 0) return;
@@ -223,10 +229,12 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
   } else {
     A.partials[b * gridDim.x + blockIdx.x] = part;  // summed by sde_step_finalize_kernel
   }
+  UNIRL_TRACE_END(A.trace);
 }
 
 // One wavefront per sample: adds the workgroup partials in index order and finishes the log-prob.
 __global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepArgs A, int64_t B, unsigned int nblk) {
+  UNIRL_TRACE_T0();
   const int64_t b = (int64_t)blockIdx.x * (kSdeThreads / kWave) + threadIdx.x / kWave;
   if (b >= B) return;
   // the partial loads are issued first; the coefficients are worked out while they are in flight
@@ -239,8 +247,10 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepA
   const SdeCoef c = sde_coef(A.kind, s, sn, smax, A.sc);
   for (int64_t j = lane + kWave; j < nblk; j += kWave) q += pp[j];
   q = wave_sum(q);
+  UNIRL_TRACE_MARK1();
   if (lane != 0) return;
   A.logp_out[b * A.stride_logp] = sde_finish_logp(A.kind, c, q, (double)A.D, A.logp_sum);
+  UNIRL_TRACE_END(A.trace);
 }
 
 // ---------------------------------------------------------------------------
@@ -714,6 +724,7 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
     A.partials = ws_partials(workspace);
     A.nblk = nblk;
     A.items = items;
+    UNIRL_TRACE_SET(A, "sde_step", nblk * (unsigned int)nb);
     int rc = UNIRL_E_DTYPE;
     switch (dtype_v) {
       case UNIRL_F32: rc = launch_step_x<float>(A, dtype_x, nb, vec, sampling, st); break;
@@ -723,6 +734,7 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
     if (rc != 0) return rc;
     if (want_logp && nblk > 1) {
       const int per_block = kSdeThreads / kWave;
+      UNIRL_TRACE_SET(A, "sde_finalize", (unsigned int)((nb + per_block - 1) / per_block));
       hipLaunchKernelGGL(sde_step_finalize_kernel, dim3((unsigned int)((nb + per_block - 1) / per_block)),
                          dim3(kSdeThreads), 0, st, A, nb, nblk);
       rc = (int)hipGetLastError();

@@ -365,6 +365,14 @@ __global__ __launch_bounds__(TPB) void token_logp_entropy_kernel(TokArgs A) {
     }
     return;
   }
+  if (st.m == -INFINITY) {
+    // every logit is -inf: logsumexp is -inf (torch.logsumexp), the log-prob -inf - (-inf) = NaN
+    // and the softmax 0/0, so the entropy is NaN too
+    if (A.lse) A.lse[row] = -INFINITY;
+    if (A.ent) A.ent[row] = quiet_nan();
+    if (A.logp) A.logp[row] = quiet_nan();
+    return;
+  }
   // sum = cnt*2^r0 + s relative to the reference r;  ln sum = r0 ln2 + ln cnt + log1p(s 2^-r0 / cnt)
   const double r0 = (double)fmaf(st.m, c, -st.r);
   const double cnt = (double)st.cnt;
@@ -410,14 +418,19 @@ template <typename T, int UNROLL>
 __global__ __launch_bounds__(kTokThreads) void token_logp_bwd_kernel(TokBwdArgs A) {
   constexpr int VEC = Stream16<T>::N;
   const int64_t row = blockIdx.x;
-  const T* __restrict__ p = reinterpret_cast<const T*>(A.logits) + row * A.row_stride;
-  T* __restrict__ gp = reinterpret_cast<T*>(A.grad) + row * A.grad_row_stride;
-  const float lse2 = A.lse[row] * kLog2e;
-  const float gs = A.g[row] * A.inv_t;
+  // No __restrict__ on the logits and the gradient: the caller may pass one buffer for both (the
+  // gradient then overwrites the logits it was computed from, element for element).
+  const T* p = reinterpret_cast<const T*>(A.logits) + row * A.row_stride;
+  T* gp = reinterpret_cast<T*>(A.grad) + row * A.grad_row_stride;
   const float c = A.c;
   const int64_t id = A.ids[row];
   const int64_t V = A.V;
   const int tid = threadIdx.x;
+  // A target outside [0, V) has no log-prob (the forward returns NaN for it): its row gets a zero
+  // gradient rather than -g*softmax.  lse = +inf makes every softmax term exactly 0.
+  const bool id_ok = id >= 0 && id < V;
+  const float lse2 = id_ok ? A.lse[row] * kLog2e : INFINITY;
+  const float gs = id_ok ? A.g[row] * A.inv_t : 0.0f;
 
   const unsigned mis_p = (unsigned)(reinterpret_cast<uintptr_t>(p) & 15u);
   const unsigned mis_g = (unsigned)(reinterpret_cast<uintptr_t>(gp) & 15u);
@@ -436,8 +449,8 @@ __global__ __launch_bounds__(kTokThreads) void token_logp_bwd_kernel(TokBwdArgs 
     Elem<T>::store(gp + j, tok_bwd_elem(Elem<T>::load(p + j), c, lse2, gs, (j == id) ? 1.0f : 0.0f));
   }
 
-  const T* __restrict__ pv = p + head;
-  T* __restrict__ gv = gp + head;
+  const T* pv = p + head;
+  T* gv = gp + head;
   const int64_t idv = id - head;  // position of the gathered column in the vector region
   const int64_t per_iter = (int64_t)kTokThreads * UNROLL;
   const int64_t n_full = nvec / per_iter;

@@ -25,6 +25,20 @@ import torch
 from .. import ops
 
 
+def _is_plain_linear(lm_head) -> bool:
+    """True for an ``nn.Linear`` proper whose output nobody else can be holding: not a subclass
+    (a quantised or custom Linear's autograd may save its output) and no forward hook (a hook
+    sees, and may keep, the output).  Only then may a gradient be written over the logits."""
+    from torch.nn.modules import module as _m
+
+    return (
+        type(lm_head) is torch.nn.Linear
+        and not lm_head._forward_hooks
+        and not lm_head._forward_hooks_with_kwargs
+        and not _m._global_forward_hooks
+    )
+
+
 class _TokenLogpFn(torch.autograd.Function):
     """Log-prob (differentiable) and, on request, entropy (detached) from one pass over the logits."""
 
@@ -47,14 +61,18 @@ class _TokenLogpFn(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_logp, *_g_entropy):
-        logits, tokens, lse = ctx.saved_tensors
         if ctx.consumed:
             raise RuntimeError(
                 "the logits of this replay were overwritten by their gradient in the first backward; "
                 "a second backward through the same graph needs chunked_replay_logp(..., keep_logits=False)"
             )
+        logits, tokens, lse = ctx.saved_tensors
         ctx.consumed = ctx.consume
         grad = ops.token_logp_bwd(logits, tokens, ctx.temperature, lse, g_logp, in_place=ctx.consume)
+        if ctx.consume:
+            # the kernel wrote through a raw pointer: tell autograd, so that anything else that saved
+            # these logits fails loudly instead of reading their gradient
+            torch.autograd.graph.increment_version(logits)
         return grad, None, None, None, None
 
 
@@ -89,7 +107,7 @@ class _RecomputedChunkFn(torch.autograd.Function):
         h = hidden.detach().requires_grad_(hidden.requires_grad)
         with torch.enable_grad(), torch.autocast("cuda", dtype=dtype, enabled=enabled):
             logits = ctx.lm_head(h)
-        plain = isinstance(ctx.lm_head, torch.nn.Linear) and logits.is_contiguous()
+        plain = _is_plain_linear(ctx.lm_head) and logits.is_contiguous()
         d_logits = ops.token_logp_bwd(
             logits.detach(), tokens, ctx.temperature, lse, g_logp, in_place=plain and logits.dtype in _KERNEL_DTYPES
         )
@@ -173,7 +191,7 @@ def chunked_replay_logp(
         return resp_hidden.new_zeros((bsz, 0), dtype=torch.float32)
     if keep_logits is None:
         keep_logits = (
-            isinstance(lm_head, torch.nn.Linear)
+            _is_plain_linear(lm_head)
             and bsz * t_max * lm_head.out_features * lm_head.weight.element_size() <= KEEP_LOGITS_BYTES
         )
     rows_per_chunk = 8192 if keep_logits else 4096
@@ -191,8 +209,8 @@ def chunked_replay_logp(
             parts.append(_RecomputedChunkFn.apply(h, tok, lm_head, T, *params))
         else:
             logits = lm_head(h)
-            if isinstance(lm_head, torch.nn.Linear) and torch.is_grad_enabled() and logits.requires_grad:
-                # a Linear's output is saved by nothing but this node: its gradient may take its place
+            if _is_plain_linear(lm_head) and torch.is_grad_enabled() and logits.requires_grad:
+                # a plain Linear's output is saved by nothing but this node: its gradient may take its place
                 parts.append(_TokenLogpFn.apply(logits, tok, T, False, True))
             else:
                 parts.append(token_logp(logits, tok, temperature))

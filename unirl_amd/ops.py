@@ -1045,6 +1045,24 @@ def calib_stream(src: Optional[torch.Tensor], read_bytes: int, dst: Optional[tor
     N.check(rc, "unirl_calib_stream")
 
 
+def calib_reduce(src: torch.Tensor, read_bytes: int, mode: int, n_workgroups: int, scratch: torch.Tensor,
+                 out: torch.Tensor) -> None:
+    """Measurement aid: the sum of ``read_bytes // 4`` floats of ``src``, finished by nothing (mode 0),
+    a second launch (mode 1) or inside the one kernel by polling tagged partials (mode 2).
+    ``scratch``: zero-filled once, at least ``16 + 16 * n_workgroups`` bytes; ``out``: float64 [1]."""
+    for t, name in ((src, "src"), (scratch, "scratch"), (out, "out")):
+        N.require_device(t, name)
+    if not src.is_contiguous() or src.numel() * src.element_size() < read_bytes:
+        raise ValueError(f"src must be contiguous and hold at least {read_bytes} bytes")
+    if out.dtype != torch.float64 or out.numel() < 1:
+        raise ValueError("out must be a float64 tensor")
+    with N.on_device(src.device):
+        rc = N.lib().unirl_calib_reduce(N.ptr(src), int(read_bytes), int(mode), int(n_workgroups), N.ptr(scratch),
+                                        scratch.numel() * scratch.element_size(), N.ptr(out),
+                                        N.current_stream(src.device))
+    N.check(rc, "unirl_calib_reduce")
+
+
 def gather_steps(tensor: torch.Tensor, positions: Sequence[int]) -> torch.Tensor:
     """``tensor[:, positions]`` for a ``[B, S, ...]`` tensor, as one gather kernel."""
     N.require_device(tensor, "tensor")
