@@ -184,6 +184,57 @@ def make_shapes(torch, dev):
         cpu_bytes=bytes1r,
     ))
 
+    # the replay of S' recorded steps of a whole micro-batch as one launch (what the [B,S'] losses
+    # consume), against the same work as one call per step: SD3 recipe (bf16 trajectory of 10 steps,
+    # 3 trained steps, micro-batch 8) and WAN recipe (fp16 trajectory of 14 steps, 7 trained, batch 2)
+    from unirl_amd import sde as psde
+
+    strat = psde.FlowSDEStrategy()
+    for tag, B, tail, n_steps, shift, steps, tdt in (
+            ("sd3", 8, (16, 128, 128), 10, 3.0, [0, 2, 4], torch.bfloat16),
+            ("wan", 2, (16, 21, 60, 104), 14, 5.0, list(range(7)), torch.float16)):
+        g = torch.Generator().manual_seed(1011)
+        sg = get_sigma_schedule(n_steps, shift)
+        K, S = n_steps + 1, len(steps)
+        D = math.prod(tail)
+        bytes_r = B * S * D * 2 * 4  # velocity, start latent, stored next latent read; mean written (16-bit each)
+        nsr = n_sets_for(bytes_r)
+        stacks = [torch.randn((B, K) + tail, generator=g).to(tdt).to(dev) for _ in range(min(nsr, 4))]
+        vels = [torch.randn((B, S) + tail, generator=g).bfloat16().to(dev) for _ in range(min(nsr, 4))]
+        nsr = len(stacks)
+        slot_x, slot_p = psde.replay_slots(list(range(K)), steps)
+        sg_a = torch.stack([sg[i] for i in steps]).to(dev)
+        sg_b = torch.stack([sg[i + 1] for i in steps]).to(dev)
+        smax_r = sg[1].to(dev)
+        sg_d = sg.to(dev)
+
+        def run_replay(i, stacks=stacks, vels=vels, nsr=nsr, slot_x=slot_x, slot_p=slot_p, sg_a=sg_a, sg_b=sg_b,
+                       smax_r=smax_r):
+            return strat.replay_steps(vels[i % nsr], stacks[i % nsr], slot_x, slot_p, sg_a, sg_b, eta=0.7,
+                                      sigma_max=smax_r)
+
+        out_lp = torch.empty(B, S, device=dev)
+        out_mean = torch.empty((B, S) + tail, dtype=tdt, device=dev)
+
+        def run_loop(i, stacks=stacks, vels=vels, nsr=nsr, steps=steps, slot_x=slot_x, slot_p=slot_p, sg_d=sg_d,
+                     smax_r=smax_r, out_lp=out_lp, out_mean=out_mean):
+            st_, v_ = stacks[i % nsr], vels[i % nsr]
+            for j, k in enumerate(steps):
+                strat.denoise_into(v_[:, j], st_[:, slot_x[j]], sg_d[k], sg_d[k + 1], eta=0.7, prev_sample=st_[:, slot_p[j]],
+                                   sigma_max=smax_r, mean_out=out_mean[:, j], logp_out=out_lp[:, j])
+
+        shape_txt = f"{str(tdt).split('.')[-1]} stack [{B},{K},{','.join(map(str, tail))}], bf16 velocities, S'={S} steps"
+        shapes.append(dict(
+            name=f"sde_replay_BxS_{tag}", config=1, shape=shape_txt + ": one launch over the B*S' transitions",
+            bytes=bytes_r, read_bytes=bytes_r * 3 // 4, write_bytes=bytes_r // 4, elements=B * S * D, run=run_replay,
+            sets=nsr,
+        ))
+        shapes.append(dict(
+            name=f"sde_replay_per_step_{tag}", config=1, shape=shape_txt + ": one call per step (S' launch pairs)",
+            bytes=bytes_r, read_bytes=bytes_r * 3 // 4, write_bytes=bytes_r // 4, elements=B * S * D, run=run_loop,
+            sets=nsr,
+        ))
+
     # -- config 3: GRPO / DRPO token loss, fp32 [256, 8192], lengths U[512, 8192] -----------------
     g = torch.Generator().manual_seed(1003)
     old = -8 * torch.rand(256, 8192, generator=g)

@@ -37,8 +37,8 @@ extern "C" {
 
 /* 2: typed gradient outputs in unirl_sde_step_logp_bwd; unirl_ratio_loss_fwd_bwd and
  * unirl_flowdppo_step added.  3: unirl_dpm2_step added.  4: unirl_gaussian_kl_mask_static
- * added. */
-#define UNIRL_ABI_VERSION 4
+ * added.  5: unirl_sde_replay_logp, unirl_sde_replay_logp_bwd, unirl_calib_reduce added. */
+#define UNIRL_ABI_VERSION 5
 
 enum unirl_dtype { UNIRL_F32 = 0, UNIRL_BF16 = 1, UNIRL_F16 = 2 };
 
@@ -162,6 +162,61 @@ struct unirl_sde_step_desc {
 };
 int unirl_sde_step_logp_ex(const struct unirl_sde_step_desc* desc /* host */, void* workspace,
                            size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * The replay of S recorded steps of every sample as ONE launch (+ its finalize)
+ * over the B*S (sample, step) rows, instead of one call per step: the loop of
+ * DiffusionStage.replay (unirl/models/sd3/diffusion.py:467-497, which ends in
+ * stack(log_probs, dim=1) and stack(means, dim=1).to(trajectory_dtype)) for
+ * velocities that are all known, e.g. from one model pass over the steps
+ * stacked into the batch.  The consumer is the [B,S'] loss of
+ * unirl/algorithms/flowdppo.py:286-320 / flowgrpo.py:160-193.
+ *
+ *   noise_pred  velocities; step j of sample b at
+ *               ptr + b*sample_stride + j*noise_pred_step_stride elements
+ *               (0 = dense [B,S,D]: S*D and D; [S,B,D] is sample_stride = D,
+ *               step stride = B*D)
+ *   latents     the trajectory stack [B,K,D] (segment.latents): slot k of
+ *               sample b at ptr + b*sample_stride + k*latents_slot_stride
+ *               (0 = K*slot stride and D).  Read in place, twice per row.
+ *   slot_sample host int64 [S]: slot of the latent step j starts from
+ *               (LatentSegment.latents_at(step), unirl/types/segments/latent.py:82-97)
+ *   slot_prev   host int64 [S]: slot of the stored next latent (prev_sample)
+ *   sigma, sigma_next  device f32 [S]: the step's sigma pair
+ *   mean_out    [B,S,D] dense in mean_dtype, or NULL
+ *   logp_out    [B,S] dense f32, or NULL (left untouched when eta < 1e-7)
+ * Per row the arithmetic is unirl_sde_step_logp_ex's in replay mode, bit for
+ * bit.  Limits: S <= UNIRL_MAX_ROLLOUT_STEPS, B*S <= 32768 (UNIRL_E_LIMIT).
+ * ---------------------------------------------------------------------- */
+struct unirl_sde_replay_desc {
+  struct unirl_sde_tensor noise_pred;
+  int64_t noise_pred_step_stride;
+  struct unirl_sde_tensor latents;
+  int64_t latents_slot_stride;
+  int64_t K;
+  const int64_t* slot_sample; /* host */
+  const int64_t* slot_prev;   /* host */
+  const float* sigma;
+  const float* sigma_next;
+  const float* sigma_max_ptr;
+  float sigma_max_val;
+  double eta;
+  int kind;
+  int64_t B, S, D;
+  void* mean_out;
+  int mean_dtype;
+  float* logp_out;
+  int logp_sum;
+};
+int unirl_sde_replay_logp(const struct unirl_sde_replay_desc* desc /* host */, void* workspace,
+                          size_t workspace_bytes, void* stream);
+
+/* Its backward with respect to the velocities (the latents are stored data): g_logp f32 [B,S]
+ * (NULL = 0), g_mean f32 [B,S,D] dense (NULL = 0; the Flow-DPPO loss sends none, its KL mask is
+ * detached); grad_v in dtype_gv, laid out like noise_pred (same strides).  mean_out / logp_out
+ * of the descriptor are ignored. */
+int unirl_sde_replay_logp_bwd(const struct unirl_sde_replay_desc* desc /* host */, const float* g_logp,
+                              const float* g_mean, void* grad_v, int dtype_gv, void* stream);
 
 /* Backward of unirl_sde_step_logp with respect to noise_pred and sample, for
  * the autograd graph the reference builds through kernels.py:225-228 and

@@ -37,7 +37,7 @@ def test_version_status_strings_and_workspace(built_lib):
     from unirl_amd import _native as N
 
     L = N.lib()
-    assert L.unirl_abi_version() == N.ABI_VERSION == 4
+    assert L.unirl_abi_version() == N.ABI_VERSION == 5
     assert f"#define UNIRL_ABI_VERSION {N.ABI_VERSION}" in (ROOT / "include" / "unirl_hip.h").read_text()
     assert L.unirl_workspace_bytes() >= 64 * 1024
     assert L.unirl_status_string(0) == b"ok"

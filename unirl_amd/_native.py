@@ -91,6 +91,33 @@ class SdeStepDesc(Structure):
     ]
 
 
+class SdeReplayDesc(Structure):
+    """struct unirl_sde_replay_desc."""
+
+    _fields_ = [
+        ("noise_pred", SdeTensor),
+        ("noise_pred_step_stride", c_int64),
+        ("latents", SdeTensor),
+        ("latents_slot_stride", c_int64),
+        ("K", c_int64),
+        ("slot_sample", POINTER(c_int64)),
+        ("slot_prev", POINTER(c_int64)),
+        ("sigma", c_void_p),
+        ("sigma_next", c_void_p),
+        ("sigma_max_ptr", c_void_p),
+        ("sigma_max_val", c_float),
+        ("eta", c_double),
+        ("kind", c_int),
+        ("B", c_int64),
+        ("S", c_int64),
+        ("D", c_int64),
+        ("mean_out", c_void_p),
+        ("mean_dtype", c_int),
+        ("logp_out", c_void_p),
+        ("logp_sum", c_int),
+    ]
+
+
 # enum unirl_dpm2_branch
 DPM2_DDIM, DPM2_FIRST, DPM2_SECOND = 0, 1, 2
 
@@ -103,7 +130,7 @@ class Dpm2Coeffs(Structure):
 
 
 # UNIRL_ABI_VERSION of include/unirl_hip.h that the signatures below describe
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _SIGNATURES = {
     "unirl_abi_version": (c_int, []),
@@ -119,6 +146,8 @@ _SIGNATURES = {
          c_double, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "unirl_sde_step_logp_ex": (c_int, [POINTER(SdeStepDesc), c_void_p, c_size_t, c_void_p]),
+    "unirl_sde_replay_logp": (c_int, [POINTER(SdeReplayDesc), c_void_p, c_size_t, c_void_p]),
+    "unirl_sde_replay_logp_bwd": (c_int, [POINTER(SdeReplayDesc), c_void_p, c_void_p, c_void_p, c_int, c_void_p]),
     "unirl_sde_step_logp_bwd": (
         c_int,
         [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,

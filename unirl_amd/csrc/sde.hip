@@ -136,6 +136,19 @@ struct SdeStepArgs {
   UNIRL_TRACE_FIELD
 };
 
+// Rows of a batched replay.  A launch of the step kernels covers `rows` independent transitions
+// (grid.y); in the plain step a row is a sample.  In a replay of S recorded steps per sample, row
+// = b * S + j is step j of sample b: the velocity sits at v + b*stride_v + j*v_step, the latent
+// the step starts from and the stored next latent at their slots of the sample's trajectory
+// stack (element offsets off_x[j], off_t[j] from the sample's base), sigma at index j, and the
+// outputs are dense in the row index.
+struct SdeRowMap {
+  int S;
+  int64_t v_step;
+  int64_t off_x[UNIRL_MAX_ROLLOUT_STEPS];
+  int64_t off_t[UNIRL_MAX_ROLLOUT_STEPS];
+};
+
 // Store VEC floats as `dtype` (wave-uniform switch) at element index `idx` of `base`.
 template <int VEC>
 __device__ __forceinline__ void sde_store_as(void* base, int dtype, int64_t idx, const float (&o)[VEC]) {
@@ -147,22 +160,32 @@ __device__ __forceinline__ void sde_store_as(void* base, int dtype, int64_t idx,
     Vec<f16_t, VEC>::store(reinterpret_cast<f16_t*>(base) + idx, o);
 }
 
-template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING>
-__global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
+template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING, bool ROWS>
+__device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRowMap* M) {
   __shared__ double lds[kSdeThreads / kWave];
   using T3 = typename std::conditional<SAMPLING, float, TX>::type;
   UNIRL_TRACE_T0();
 
-  const int64_t b = blockIdx.y;
+  const int64_t row = blockIdx.y;
   const int64_t D = A.D;
   const int kind = A.kind;
 
-  const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + b * A.stride_v;
-  const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + b * A.stride_x;
-  const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + b * A.stride_third : nullptr;
+  // plain step: the row is the sample; replay rows: (sample, step)
+  int64_t b = row, off_v = 0, off_x = 0, off_t = 0, sig_idx = row * A.sigma_stride;
+  if (ROWS) {
+    b = row / M->S;
+    const int j = (int)(row - b * M->S);
+    off_v = j * M->v_step;
+    off_x = M->off_x[j];
+    off_t = M->off_t[j];
+    sig_idx = j;
+  }
+  const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + b * A.stride_v + off_v;
+  const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + b * A.stride_x + off_x;
+  const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + b * A.stride_third + off_t : nullptr;
   void* const po = A.prev_out;
   void* const mo = A.mean_out;
-  const int64_t po0 = b * A.stride_prev, mo0 = b * A.stride_mean;
+  const int64_t po0 = row * A.stride_prev, mo0 = row * A.stride_mean;
   const int pdt = A.prev_dtype, mdt = A.mean_dtype;
 
   const int64_t nvec = D / VEC;  // VEC == 1 or D % VEC == 0 (checked on the host)
@@ -192,8 +215,8 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
   // and at small sizes (one pass per lane) the two would otherwise run back to back.
   int64_t i0 = (int64_t)blockIdx.x * kSdeThreads + threadIdx.x;
   load_pass(i0);
-  const float s = A.sigma[b * A.sigma_stride];
-  const float sn = A.sigma_next[b * A.sigma_stride];
+  const float s = A.sigma[sig_idx];
+  const float sn = A.sigma_next[sig_idx];
   const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
   const SdeCoef c = sde_coef(kind, s, sn, smax, A.sc);
 
@@ -225,15 +248,29 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
   const double part = block_sum<double>((double)acc, lds);
   if (threadIdx.x != 0) return;
   if (gridDim.x == 1) {
-    A.logp_out[b * A.stride_logp] = sde_finish_logp(kind, c, part, (double)D, A.logp_sum);
+    A.logp_out[row * A.stride_logp] = sde_finish_logp(kind, c, part, (double)D, A.logp_sum);
   } else {
-    A.partials[b * gridDim.x + blockIdx.x] = part;  // summed by sde_step_finalize_kernel
+    A.partials[row * gridDim.x + blockIdx.x] = part;  // summed by sde_step_finalize_kernel
   }
   UNIRL_TRACE_END(A.trace);
 }
 
-// One wavefront per sample: adds the workgroup partials in index order and finishes the log-prob.
-__global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepArgs A, int64_t B, unsigned int nblk) {
+template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING>
+__global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
+  sde_step_body<TV, TX, VEC, ITEMS, SAMPLING, false>(A, nullptr);
+}
+
+// The replay of S recorded steps per sample as one launch over the (sample, step) rows.
+template <typename TV, typename TX, int VEC, int ITEMS>
+__global__ __launch_bounds__(kSdeThreads) void sde_replay_kernel(SdeStepArgs A, SdeRowMap M) {
+  sde_step_body<TV, TX, VEC, ITEMS, false, true>(A, &M);
+}
+
+// One wavefront per row: adds the workgroup partials in index order and finishes the log-prob.
+// sigma_mod: rows per sample of a batched replay (sigma is then indexed by the step, row modulo
+// sigma_mod), 0 for the plain step (sigma indexed by the sample through sigma_stride).
+__global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepArgs A, int64_t B, unsigned int nblk,
+                                                                       int sigma_mod) {
   UNIRL_TRACE_T0();
   const int64_t b = (int64_t)blockIdx.x * (kSdeThreads / kWave) + threadIdx.x / kWave;
   if (b >= B) return;
@@ -241,8 +278,9 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepA
   const int lane = threadIdx.x & (kWave - 1);
   const double* __restrict__ pp = A.partials + b * nblk;
   double q = (lane < (int)nblk) ? pp[lane] : 0.0;
-  const float s = A.sigma[b * A.sigma_stride];
-  const float sn = A.sigma_next[b * A.sigma_stride];
+  const int64_t sig_idx = sigma_mod ? b % sigma_mod : b * A.sigma_stride;
+  const float s = A.sigma[sig_idx];
+  const float sn = A.sigma_next[sig_idx];
   const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
   const SdeCoef c = sde_coef(A.kind, s, sn, smax, A.sc);
   for (int64_t j = lane + kWave; j < nblk; j += kWave) q += pp[j];
@@ -280,22 +318,35 @@ struct SdeBwdArgs {
   void* grad_v;
   void* grad_x;
   int dtype_gv, dtype_gx;  // unirl_dtype of the two outputs
+  int64_t stride_v, stride_x;  // replay rows only: elements between consecutive samples
 };
 
-template <typename TV, typename TX, int VEC, bool SAMPLING>
-__global__ __launch_bounds__(kSdeThreads) void sde_step_bwd_kernel(SdeBwdArgs A) {
+template <typename TV, typename TX, int VEC, bool SAMPLING, bool ROWS>
+__device__ __forceinline__ void sde_step_bwd_body(const SdeBwdArgs& A, const SdeRowMap* M) {
   using T3 = typename std::conditional<SAMPLING, float, TX>::type;
-  const int64_t b = blockIdx.y;
+  const int64_t b = blockIdx.y;  // the row: a sample, or (sample, step) of a batched replay
   const int64_t D = A.D;
-  const float s = A.sigma[b * A.sigma_stride];
-  const float sn = A.sigma_next[b * A.sigma_stride];
+  // plain: dense [B, D] operands; replay rows: velocity / latents addressed through the row map
+  // (the velocity's gradient takes the velocity's layout), the incoming mean gradient dense in
+  // the row index
+  int64_t base_v = b * D, base_x = b * D, base_t = b * D, sig_idx = b * A.sigma_stride;
+  if (ROWS) {
+    const int64_t smp = b / M->S;
+    const int j = (int)(b - smp * M->S);
+    base_v = smp * A.stride_v + j * M->v_step;
+    base_x = smp * A.stride_x + M->off_x[j];
+    base_t = smp * A.stride_x + M->off_t[j];
+    sig_idx = j;
+  }
+  const float s = A.sigma[sig_idx];
+  const float sn = A.sigma_next[sig_idx];
   const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
   const int kind = A.kind;
   const SdeCoef c = sde_coef(kind, s, sn, smax, A.sc);
 
-  const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + b * D;
-  const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + b * D;
-  const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + b * D : nullptr;
+  const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + base_v;
+  const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + base_x;
+  const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + base_t : nullptr;
   const float* __restrict__ gm = A.g_mean ? A.g_mean + b * D : nullptr;
   const float* __restrict__ gp = A.g_prev ? A.g_prev + b * D : nullptr;
   void* const gv = A.grad_v;
@@ -340,9 +391,20 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_bwd_kernel(SdeBwdArgs A)
       ov[k] = g * dmean_dv;
       ox[k] = g * dmean_dx;
     }
-    if (gv) sde_store_as<VEC>(gv, dgv, b * D + i * VEC, ov);
+    if (gv) sde_store_as<VEC>(gv, dgv, (ROWS ? base_v : b * D) + i * VEC, ov);
     if (gx) sde_store_as<VEC>(gx, dgx, b * D + i * VEC, ox);
   }
+}
+
+template <typename TV, typename TX, int VEC, bool SAMPLING>
+__global__ __launch_bounds__(kSdeThreads) void sde_step_bwd_kernel(SdeBwdArgs A) {
+  sde_step_bwd_body<TV, TX, VEC, SAMPLING, false>(A, nullptr);
+}
+
+// Backward of the batched replay with respect to the velocities (the latents are stored data).
+template <typename TV, typename TX, int VEC>
+__global__ __launch_bounds__(kSdeThreads) void sde_replay_bwd_kernel(SdeBwdArgs A, SdeRowMap M) {
+  sde_step_bwd_body<TV, TX, VEC, false, true>(A, &M);
 }
 
 // ---------------------------------------------------------------------------
@@ -589,6 +651,124 @@ static int launch_bwd_x(const SdeBwdArgs& A, int dtype_x, int64_t B, int vec, bo
 }
 
 template <typename TV, typename TX>
+static int launch_replay(const SdeStepArgs& A, const SdeRowMap& M, int64_t rows, int vec, hipStream_t st) {
+  dim3 grid(A.nblk, (unsigned int)rows), block(kSdeThreads);
+  if (vec == 8) {
+    if constexpr (sizeof(TV) == 2 || sizeof(TX) == 2)
+      hipLaunchKernelGGL((sde_replay_kernel<TV, TX, 8, 2>), grid, block, 0, st, A, M);
+    else
+      return UNIRL_E_DTYPE;
+  } else if (vec == 4) {
+    hipLaunchKernelGGL((sde_replay_kernel<TV, TX, 4, 4>), grid, block, 0, st, A, M);
+  } else {
+    hipLaunchKernelGGL((sde_replay_kernel<TV, TX, 1, 2>), grid, block, 0, st, A, M);
+  }
+  return (int)hipGetLastError();
+}
+
+template <typename TV>
+static int launch_replay_x(const SdeStepArgs& A, const SdeRowMap& M, int dtype_x, int64_t rows, int vec, hipStream_t st) {
+  switch (dtype_x) {
+    case UNIRL_F32: return launch_replay<TV, float>(A, M, rows, vec, st);
+    case UNIRL_BF16: return launch_replay<TV, bf16_t>(A, M, rows, vec, st);
+    case UNIRL_F16: return launch_replay<TV, f16_t>(A, M, rows, vec, st);
+  }
+  return UNIRL_E_DTYPE;
+}
+
+template <typename TV, typename TX>
+static int launch_replay_bwd(const SdeBwdArgs& A, const SdeRowMap& M, int64_t rows, int vec, hipStream_t st) {
+  const unsigned int nblk = sde_blocks_per_sample(A.D / vec, 1, rows);
+  dim3 grid(nblk, (unsigned int)rows), block(kSdeThreads);
+  if (vec == 8) {
+    if constexpr (sizeof(TV) == 2 || sizeof(TX) == 2)
+      hipLaunchKernelGGL((sde_replay_bwd_kernel<TV, TX, 8>), grid, block, 0, st, A, M);
+    else
+      return UNIRL_E_DTYPE;
+  } else if (vec == 4) {
+    hipLaunchKernelGGL((sde_replay_bwd_kernel<TV, TX, 4>), grid, block, 0, st, A, M);
+  } else {
+    hipLaunchKernelGGL((sde_replay_bwd_kernel<TV, TX, 1>), grid, block, 0, st, A, M);
+  }
+  return (int)hipGetLastError();
+}
+
+template <typename TV>
+static int launch_replay_bwd_x(const SdeBwdArgs& A, const SdeRowMap& M, int dtype_x, int64_t rows, int vec,
+                               hipStream_t st) {
+  switch (dtype_x) {
+    case UNIRL_F32: return launch_replay_bwd<TV, float>(A, M, rows, vec, st);
+    case UNIRL_BF16: return launch_replay_bwd<TV, bf16_t>(A, M, rows, vec, st);
+    case UNIRL_F16: return launch_replay_bwd<TV, f16_t>(A, M, rows, vec, st);
+  }
+  return UNIRL_E_DTYPE;
+}
+
+// Argument checks and the row map shared by the replay's forward and backward entry points.
+struct ReplayPlan {
+  int64_t stride_v, v_step, stride_x, slot_stride;
+  int vec;
+  SdeRowMap M;
+};
+
+static int plan_replay(const unirl_sde_replay_desc* d, const void* extra_f32_a, const void* extra_b, size_t extra_b_size,
+                       ReplayPlan& P) {
+  if (!d) return UNIRL_E_NULL;
+  const int dtype_v = d->noise_pred.dtype, dtype_x = d->latents.dtype;
+  const int64_t B = d->B, S = d->S, D = d->D, K = d->K;
+  if (!dtype_ok(dtype_v) || !dtype_ok(dtype_x)) return UNIRL_E_DTYPE;
+  if (d->kind < UNIRL_SDE_FLOW || d->kind > UNIRL_SDE_CPS) return UNIRL_E_DTYPE;
+  if (d->mean_out && !dtype_ok(d->mean_dtype)) return UNIRL_E_DTYPE;
+  if (B < 0 || S < 1 || D <= 0 || K < 1) return UNIRL_E_SHAPE;
+  if (S > UNIRL_MAX_ROLLOUT_STEPS) return UNIRL_E_LIMIT;
+  if (B * S > 32768) return UNIRL_E_LIMIT;  // one row per grid.y index
+  if (!d->slot_sample || !d->slot_prev) return UNIRL_E_NULL;
+  P.v_step = d->noise_pred_step_stride ? d->noise_pred_step_stride : D;
+  P.stride_v = d->noise_pred.sample_stride ? d->noise_pred.sample_stride : S * D;
+  P.slot_stride = d->latents_slot_stride ? d->latents_slot_stride : D;
+  P.stride_x = d->latents.sample_stride ? d->latents.sample_stride : K * P.slot_stride;
+  if (P.v_step < D || P.stride_v < 0 || P.slot_stride < D || P.stride_x < 0) return UNIRL_E_SHAPE;
+  const size_t sv = dtype_size(dtype_v), sx = dtype_size(dtype_x);
+  const size_t smo = d->mean_out ? dtype_size(d->mean_dtype) : 4;
+  if (!aligned_to(d->noise_pred.ptr, sv) || !aligned_to(d->latents.ptr, sx) || !aligned_to(d->mean_out, smo) ||
+      !aligned_to(d->logp_out, 4) || !aligned_to(extra_f32_a, 4) || !aligned_to(extra_b, extra_b_size))
+    return UNIRL_E_ALIGN;
+  P.M.S = (int)S;
+  P.M.v_step = P.v_step;
+  for (int64_t j = 0; j < S; ++j) {
+    const int64_t a = d->slot_sample[j], b = d->slot_prev[j];
+    if (a < 0 || a >= K || b < 0 || b >= K) return UNIRL_E_SHAPE;
+    P.M.off_x[j] = a * P.slot_stride;
+    P.M.off_t[j] = b * P.slot_stride;
+  }
+  // vectors of four (or eight, when the 16-bit tensors carry at least as many bytes as the fp32
+  // ones: same rule as the single step) need every row base on the vector's boundary
+  int vec = 4;
+  if (D % 4 != 0 || P.v_step % 4 || P.stride_v % 4 || P.slot_stride % 4 || P.stride_x % 4 ||
+      !aligned_to(d->noise_pred.ptr, 4 * sv) || !aligned_to(d->latents.ptr, 4 * sx) ||
+      !aligned_to(d->mean_out, 4 * smo) || !aligned_to(extra_f32_a, 16) || !aligned_to(extra_b, 4 * extra_b_size))
+    vec = 1;
+  if (vec == 4 && (sv == 2 || sx == 2) && D % 8 == 0) {
+    size_t narrow = 0, wide = 0;
+    bool ok = true;
+    auto visit = [&](const void* p, size_t es, bool strides_ok) {
+      if (!p) return;
+      (es == 2 ? narrow : wide) += es;
+      ok = ok && aligned_to(p, 16) && (es == 4 || strides_ok);
+    };
+    visit(d->noise_pred.ptr, sv, P.v_step % 8 == 0 && P.stride_v % 8 == 0);
+    visit(d->latents.ptr, sx, P.slot_stride % 8 == 0 && P.stride_x % 8 == 0);
+    visit(d->latents.ptr, sx, true);  // read twice: the step's input and the stored next latent
+    visit(d->mean_out, smo, true);
+    visit(extra_f32_a, 4, true);
+    visit(extra_b, extra_b_size, P.v_step % 8 == 0 && P.stride_v % 8 == 0);
+    if (ok && narrow >= wide) vec = 8;
+  }
+  P.vec = vec;
+  return UNIRL_OK;
+}
+
+template <typename TV, typename TX>
 static int launch_rollout(const SdeRolloutArgs& A, int64_t B, int vec, hipStream_t st) {
   dim3 grid(A.nblk, (unsigned int)B), block(kSdeThreads);
   const int items = A.items;
@@ -736,12 +916,122 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
       const int per_block = kSdeThreads / kWave;
       UNIRL_TRACE_SET(A, "sde_finalize", (unsigned int)((nb + per_block - 1) / per_block));
       hipLaunchKernelGGL(sde_step_finalize_kernel, dim3((unsigned int)((nb + per_block - 1) / per_block)),
-                         dim3(kSdeThreads), 0, st, A, nb, nblk);
+                         dim3(kSdeThreads), 0, st, A, nb, nblk, 0);
       rc = (int)hipGetLastError();
       if (rc != 0) return rc;
     }
   }
   return UNIRL_OK;
+}
+
+extern "C" int unirl_sde_replay_logp(const unirl_sde_replay_desc* d, void* workspace, size_t workspace_bytes,
+                                     void* stream) {
+  ReplayPlan P;
+  int rc = plan_replay(d, nullptr, nullptr, 4, P);
+  if (rc != 0) return rc;
+  const int64_t B = d->B, S = d->S, D = d->D;
+  if (B == 0) return UNIRL_OK;
+  if (!d->noise_pred.ptr || !d->latents.ptr || !d->sigma || !d->sigma_next) return UNIRL_E_NULL;
+  const bool want_logp = (d->logp_out != nullptr) && !(d->eta < 1e-7);
+  if (want_logp && (!workspace || workspace_bytes < kWorkspaceBytes)) return UNIRL_E_WORKSPACE;
+  const int vec = P.vec;
+  const int items = (vec == 8) ? 2 : (vec == 4) ? 4 : 2;
+  const int64_t rows_all = B * S;
+  const unsigned int nblk = sde_blocks_per_sample(D / vec, items, rows_all);
+  // whole samples per launch, so that a launch's rows stay (sample, step) pairs
+  int64_t per_launch = sde_samples_per_launch(rows_all, nblk) / S;
+  if (per_launch < 1) return UNIRL_E_LIMIT;
+  const size_t sv = dtype_size(d->noise_pred.dtype), sx = dtype_size(d->latents.dtype);
+  const size_t smo = d->mean_out ? dtype_size(d->mean_dtype) : 4;
+  hipStream_t st = (hipStream_t)stream;
+  for (int64_t b0 = 0; b0 < B; b0 += per_launch) {
+    const int64_t nb = (B - b0 < per_launch) ? (B - b0) : per_launch;
+    SdeStepArgs A = {};
+    A.v = offset_ptr(d->noise_pred.ptr, b0 * P.stride_v, sv);
+    A.x = offset_ptr(d->latents.ptr, b0 * P.stride_x, sx);
+    A.third = A.x;  // the stored next latent lives in the same stack
+    A.stride_v = P.stride_v;
+    A.stride_x = P.stride_x;
+    A.stride_third = P.stride_x;
+    A.sigma = d->sigma;
+    A.sigma_next = d->sigma_next;
+    A.sigma_max_ptr = d->sigma_max_ptr;
+    A.sigma_max_val = d->sigma_max_val;
+    A.sigma_stride = 0;
+    A.sc = make_scalars(d->eta);
+    A.kind = d->kind;
+    A.want_logp = want_logp ? 1 : 0;
+    A.logp_sum = d->logp_sum;
+    A.D = D;
+    A.prev_out = nullptr;
+    A.mean_out = const_cast<void*>(offset_ptr(d->mean_out, b0 * S * D, smo));
+    A.prev_dtype = UNIRL_F32;
+    A.mean_dtype = d->mean_dtype;
+    A.stride_prev = D;
+    A.stride_mean = D;
+    A.logp_out = offset_f32(d->logp_out, b0 * S);
+    A.stride_logp = 1;
+    A.partials = ws_partials(workspace);
+    A.nblk = nblk;
+    A.items = items;
+    UNIRL_TRACE_SET(A, "sde_replay", nblk * (unsigned int)(nb * S));
+    rc = UNIRL_E_DTYPE;
+    switch (d->noise_pred.dtype) {
+      case UNIRL_F32: rc = launch_replay_x<float>(A, P.M, d->latents.dtype, nb * S, vec, st); break;
+      case UNIRL_BF16: rc = launch_replay_x<bf16_t>(A, P.M, d->latents.dtype, nb * S, vec, st); break;
+      case UNIRL_F16: rc = launch_replay_x<f16_t>(A, P.M, d->latents.dtype, nb * S, vec, st); break;
+    }
+    if (rc != 0) return rc;
+    if (want_logp && nblk > 1) {
+      const int per_block = kSdeThreads / kWave;
+      UNIRL_TRACE_SET(A, "sde_finalize", (unsigned int)((nb * S + per_block - 1) / per_block));
+      hipLaunchKernelGGL(sde_step_finalize_kernel, dim3((unsigned int)((nb * S + per_block - 1) / per_block)),
+                         dim3(kSdeThreads), 0, st, A, nb * S, nblk, (int)S);
+      rc = (int)hipGetLastError();
+      if (rc != 0) return rc;
+    }
+  }
+  return UNIRL_OK;
+}
+
+extern "C" int unirl_sde_replay_logp_bwd(const unirl_sde_replay_desc* d, const float* g_logp, const float* g_mean,
+                                         void* grad_v, int dtype_gv, void* stream) {
+  if (grad_v && !dtype_ok(dtype_gv)) return UNIRL_E_DTYPE;
+  ReplayPlan P;
+  int rc = plan_replay(d, g_mean, grad_v, grad_v ? dtype_size(dtype_gv) : 4, P);
+  if (rc != 0) return rc;
+  if (d->B == 0 || !grad_v) return UNIRL_OK;
+  if (!d->noise_pred.ptr || !d->latents.ptr || !d->sigma || !d->sigma_next) return UNIRL_E_NULL;
+  if (!aligned_to(g_logp, 4)) return UNIRL_E_ALIGN;
+  SdeBwdArgs A = {};
+  A.v = d->noise_pred.ptr;
+  A.x = d->latents.ptr;
+  A.third = d->latents.ptr;
+  A.sigma = d->sigma;
+  A.sigma_next = d->sigma_next;
+  A.sigma_max_ptr = d->sigma_max_ptr;
+  A.sigma_max_val = d->sigma_max_val;
+  A.sigma_stride = 0;
+  A.sc = make_scalars(d->eta);
+  A.kind = d->kind;
+  A.logp_sum = d->logp_sum;
+  A.D = d->D;
+  A.g_logp = (d->eta < 1e-7) ? nullptr : g_logp;
+  A.g_mean = g_mean;
+  A.g_prev = nullptr;
+  A.grad_v = grad_v;
+  A.grad_x = nullptr;
+  A.dtype_gv = dtype_gv;
+  A.dtype_gx = UNIRL_F32;
+  A.stride_v = P.stride_v;
+  A.stride_x = P.stride_x;
+  hipStream_t st = (hipStream_t)stream;
+  switch (d->noise_pred.dtype) {
+    case UNIRL_F32: return launch_replay_bwd_x<float>(A, P.M, d->latents.dtype, d->B * d->S, P.vec, st);
+    case UNIRL_BF16: return launch_replay_bwd_x<bf16_t>(A, P.M, d->latents.dtype, d->B * d->S, P.vec, st);
+    case UNIRL_F16: return launch_replay_bwd_x<f16_t>(A, P.M, d->latents.dtype, d->B * d->S, P.vec, st);
+  }
+  return UNIRL_E_DTYPE;
 }
 
 extern "C" int unirl_sde_step_logp(const void* noise_pred, int dtype_v, const void* sample, int dtype_x,

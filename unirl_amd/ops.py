@@ -246,6 +246,155 @@ def sde_step_logp_into(
     N.check(rc, "unirl_sde_step_logp_ex")
 
 
+def _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next, kind, eta, sigma_max, step_major):
+    """Checked operands and the filled ``unirl_sde_replay_desc`` of a batched replay; returns
+    ``(desc, keepalive, B, S, D, shape_tail)``."""
+    N.require_device(latents, "latents")
+    N.require_device(noise_pred, "noise_pred")
+    if latents.dim() < 3:
+        raise ValueError(f"latents must be a [B, K, ...] trajectory stack; got {tuple(latents.shape)}")
+    device = latents.device
+    B, K = int(latents.shape[0]), int(latents.shape[1])
+    tail = tuple(latents.shape[2:])
+    D = int(math.prod(tail))
+    slots_x, slots_p = [int(k) for k in slot_sample], [int(k) for k in slot_prev]
+    S = len(slots_x)
+    if S < 1 or len(slots_p) != S:
+        raise ValueError(f"slot_sample and slot_prev must name the same, non-zero number of steps; got {S} and {len(slots_p)}")
+    if S > N.MAX_ROLLOUT_STEPS:
+        raise ValueError(f"at most {N.MAX_ROLLOUT_STEPS} steps per replay call; got {S}")
+    for k in slots_x + slots_p:
+        if not 0 <= k < K:
+            raise ValueError(f"slot {k} is outside the stack's {K} slots")
+    want = ((S, B) if step_major else (B, S)) + tail
+    if tuple(noise_pred.shape) != want:
+        raise ValueError(f"noise_pred {tuple(noise_pred.shape)} != {want}")
+    v = noise_pred.detach()
+    if v.dtype not in N._DTYPE_CODE:
+        v = v.float()
+    x = latents.detach()
+    if x.dtype not in N._DTYPE_CODE:
+        x = x.float()
+    # every (sample, step) block must be one contiguous run of D elements.  The two leading strides
+    # are free, except that 0 means "dense" in the C ABI: a tensor broadcast over the samples or the
+    # steps is copied, as is a stack whose slots overlap
+    b_dim, s_dim = (1, 0) if step_major else (0, 1)
+    if B and not (v[0, 0].is_contiguous() and (B == 1 or v.stride(b_dim) >= 1) and (S == 1 or v.stride(s_dim) >= D)):
+        v = v.contiguous()
+    if B and not (x[0, 0].is_contiguous() and (B == 1 or x.stride(0) >= 1) and (K == 1 or x.stride(1) >= D)):
+        x = x.contiguous()
+
+    def steps_f32(t, name):
+        if not isinstance(t, torch.Tensor):
+            t = torch.tensor([float(a) for a in t], dtype=torch.float32)
+        t = t.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+        if t.numel() != S:
+            raise ValueError(f"{name} must hold one value per step ({S}); got {t.numel()}")
+        return t
+
+    sig, sig_n = steps_f32(sigma, "sigma"), steps_f32(sigma_next, "sigma_next")
+    smax_t, smax_v = _sigma_max_arg(sigma_max, device)
+    d = N.SdeReplayDesc()
+    d.noise_pred = N.SdeTensor(N.ptr(v), N.dtype_code(v.dtype), v.stride(b_dim) if B > 1 else S * D)
+    d.noise_pred_step_stride = v.stride(s_dim) if S > 1 else D
+    d.latents = N.SdeTensor(N.ptr(x), N.dtype_code(x.dtype), x.stride(0) if B > 1 else 0)
+    d.latents_slot_stride = x.stride(1) if K > 1 else 0
+    arr_x, arr_p = (ctypes.c_int64 * S)(*slots_x), (ctypes.c_int64 * S)(*slots_p)
+    d.K = K
+    d.slot_sample, d.slot_prev = arr_x, arr_p
+    d.sigma, d.sigma_next = N.ptr(sig), N.ptr(sig_n)
+    d.sigma_max_ptr, d.sigma_max_val = N.ptr(smax_t), smax_v
+    d.eta, d.kind = float(eta), SDE_KINDS[kind]
+    d.B, d.S, d.D = B, S, D
+    return d, (v, x, sig, sig_n, smax_t, arr_x, arr_p), B, S, D, tail
+
+
+def sde_replay_logp(
+    noise_pred: torch.Tensor,
+    latents: torch.Tensor,
+    slot_sample: Sequence[int],
+    slot_prev: Sequence[int],
+    sigma,
+    sigma_next,
+    *,
+    kind: str = "flow",
+    eta: float = 1.0,
+    sigma_max: Union[float, torch.Tensor] = 0.99,
+    step_major: bool = False,
+    want_means: bool = True,
+    means_dtype: Optional[torch.dtype] = None,
+    logp_sum: bool = False,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """The replay of ``S`` recorded steps of every sample in one launch: ``(log_probs [B, S] fp32 or
+    None when eta < 1e-7, means [B, S, ...] in means_dtype or None)``.
+
+    ``noise_pred`` is ``[B, S, ...]`` (``[S, B, ...]`` with ``step_major``); ``latents`` the
+    ``[B, K, ...]`` trajectory stack, read in place: step ``j`` starts from slot ``slot_sample[j]``
+    and its stored next latent is slot ``slot_prev[j]``; ``sigma`` / ``sigma_next`` hold one value
+    per step.  ``means_dtype`` defaults to the stack's dtype (the reference stores
+    ``stack(means).to(trajectory_dtype)``)."""
+    d, keep, B, S, D, tail = _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next, kind, eta,
+                                          sigma_max, step_major)
+    device = latents.device
+    x = keep[1]
+    mdt = means_dtype if means_dtype is not None else x.dtype
+    if want_means and mdt not in N._DTYPE_CODE:
+        raise TypeError(f"means_dtype {mdt} is not float32, bfloat16 or float16")
+    means = torch.empty((B, S) + tail, dtype=mdt, device=device) if want_means else None
+    logp = None if eta < 1e-7 else torch.empty((B, S), dtype=torch.float32, device=device)
+    if B == 0 or D == 0:
+        return logp, means
+    d.mean_out, d.mean_dtype = N.ptr(means), (N.dtype_code(mdt) if want_means else 0)
+    d.logp_out, d.logp_sum = N.ptr(logp), int(bool(logp_sum))
+    stream = N.current_stream(device)
+    ws, ws_bytes = N.workspace(device, stream)
+    with N.on_device(device):
+        rc = N.lib().unirl_sde_replay_logp(ctypes.byref(d), N.ptr(ws), ws_bytes, stream)
+    N.check(rc, "unirl_sde_replay_logp")
+    return logp, means
+
+
+def sde_replay_logp_bwd(
+    noise_pred: torch.Tensor,
+    latents: torch.Tensor,
+    slot_sample: Sequence[int],
+    slot_prev: Sequence[int],
+    sigma,
+    sigma_next,
+    *,
+    kind: str,
+    eta: float,
+    sigma_max,
+    step_major: bool,
+    g_logp: Optional[torch.Tensor],
+    g_mean: Optional[torch.Tensor],
+    logp_sum: bool = False,
+) -> torch.Tensor:
+    """Gradient of :func:`sde_replay_logp` with respect to ``noise_pred`` (same shape and dtype; the
+    latents are stored data and take no gradient)."""
+    d, keep, B, S, D, tail = _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next, kind, eta,
+                                          sigma_max, step_major)
+    device = latents.device
+    v = keep[0]
+    out_dtype = noise_pred.dtype if noise_pred.dtype in N._DTYPE_CODE else torch.float32
+    # the gradient takes the velocity's layout: same strides as the tensor the kernel reads
+    grad = torch.empty_strided(v.shape, v.stride(), dtype=out_dtype, device=device)
+    if B == 0 or D == 0:
+        return grad
+
+    def f32c(t, shape):  # the upstream gradients come in the outputs' [B, S, ...] layout
+        return None if t is None else t.detach().to(device=device, dtype=torch.float32).reshape(shape).contiguous()
+
+    gl = f32c(g_logp, (B, S))
+    gm = f32c(g_mean, (B, S, D))
+    d.logp_sum = int(bool(logp_sum))
+    with N.on_device(device):
+        rc = N.lib().unirl_sde_replay_logp_bwd(ctypes.byref(d), N.ptr(gl), N.ptr(gm), N.ptr(grad),
+                                               N.dtype_code(out_dtype), N.current_stream(device))
+    N.check(rc, "unirl_sde_replay_logp_bwd")
+    return grad if grad.dtype == noise_pred.dtype else grad.to(noise_pred.dtype)
+
+
 def sde_step_logp_bwd(
     noise_pred: torch.Tensor,
     sample: torch.Tensor,

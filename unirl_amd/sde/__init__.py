@@ -9,6 +9,7 @@ from .kernels import (
     SDEStrategy,
     StepStrategy,
     latents_at,
+    replay_slots,
     sde_rollout,
 )
 from .noise import generate_latents, generate_shared_noise, regen_initial_noise
@@ -28,5 +29,6 @@ __all__ = [
     "get_sigma_schedule",
     "latents_at",
     "regen_initial_noise",
+    "replay_slots",
     "sde_rollout",
 ]

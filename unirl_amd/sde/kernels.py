@@ -77,6 +77,38 @@ class _SdeStepFn(torch.autograd.Function):
         return grad_v, grad_x, None, None, None, None, None, None, None
 
 
+class _SdeReplayFn(torch.autograd.Function):
+    """Differentiable batched replay: gradients flow to ``noise_pred`` through the log-probs and the
+    means; the stored latents take none."""
+
+    @staticmethod
+    def forward(ctx, noise_pred, latents, sigma, sigma_next, sigma_max, eta, kind, slots, step_major, means_dtype):
+        logp, means = ops.sde_replay_logp(
+            noise_pred, latents, slots[0], slots[1], sigma, sigma_next, kind=kind, eta=eta, sigma_max=sigma_max,
+            step_major=step_major, means_dtype=means_dtype,
+        )
+        ctx.set_materialize_grads(False)
+        ctx.cfg = (kind, eta, sigma_max, slots, step_major)
+        ctx.has_logp = logp is not None
+        ctx.saved = (noise_pred.detach(), latents.detach(), sigma, sigma_next)
+        if logp is None:
+            logp = torch.empty(0, device=latents.device)
+            ctx.mark_non_differentiable(logp)
+        return logp, means
+
+    @staticmethod
+    def backward(ctx, g_logp, g_means):
+        if (g_logp is None or not ctx.has_logp) and g_means is None:
+            return (None,) * 10
+        v, latents, sigma, sigma_next = ctx.saved
+        kind, eta, sigma_max, slots, step_major = ctx.cfg
+        grad_v = ops.sde_replay_logp_bwd(
+            v, latents, slots[0], slots[1], sigma, sigma_next, kind=kind, eta=eta, sigma_max=sigma_max,
+            step_major=step_major, g_logp=g_logp if ctx.has_logp else None, g_mean=g_means,
+        )
+        return (grad_v,) + (None,) * 9
+
+
 class StepStrategy(ABC):
     """Base class of all sampling step strategies."""
 
@@ -197,6 +229,60 @@ class StepStrategy(ABC):
             noise=noise, sigma_max=sigma_max, prev_out=prev_out, mean_out=mean_out, logp_out=logp_out,
         )
         return not (eta < 1e-7)
+
+    def replay_steps(self, noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next, *, eta=1.0, sigma_max=0.99,
+                     step_major=False, means_dtype=None):
+        """The replay loop of a diffusion stage (``unirl/models/sd3/diffusion.py:467-497``) for velocities
+        that are all known, as ONE fused launch over the ``B * S`` (sample, step) transitions:
+        ``(log_probs [B, S] fp32, prev_sample_means [B, S, ...])``.
+
+        ``noise_pred``: ``[B, S, ...]`` (``[S, B, ...]`` with ``step_major``, the layout of a model pass
+        over the steps stacked into the batch); ``latents``: the segment's ``[B, K, ...]`` trajectory
+        stack, read in place -- step ``j`` starts from slot ``slot_sample[j]`` and is scored against
+        the stored latent in slot ``slot_prev[j]`` (see :func:`replay_slots`); ``sigma`` /
+        ``sigma_next``: one value per step.  The means come back in ``means_dtype`` (default: the
+        stack's dtype, i.e. ``stack(means, dim=1).to(trajectory_dtype)``).  Per row the arithmetic is
+        ``denoise(..., prev_sample=...)``'s.  Differentiable with respect to ``noise_pred``.
+        Raises ``RuntimeError`` when ``eta < 1e-7``: a replay needs a stochastic step, as in the
+        reference's loop."""
+        kind = self._kind
+        if kind is None:
+            raise NotImplementedError(f"{type(self).__name__} has no fused kernel")
+        if eta < 1e-7:
+            raise RuntimeError(
+                f"{type(self).__name__}.replay_steps: eta={eta} is a deterministic step (no log-prob); "
+                "replay requires a stochastic SDE strategy"
+            )
+        if not latents.is_cuda:
+            raise RuntimeError(
+                f"{type(self).__name__}.replay_steps: latents live on {latents.device}; the fused SDE kernel "
+                "runs on a HIP device only and there is no CPU fallback"
+            )
+        slots = ([int(k) for k in slot_sample], [int(k) for k in slot_prev])
+        if torch.is_grad_enabled() and noise_pred.requires_grad:
+            return _SdeReplayFn.apply(noise_pred, latents, sigma, sigma_next, sigma_max, float(eta), kind, slots,
+                                      bool(step_major), means_dtype)
+        return ops.sde_replay_logp(noise_pred, latents, slots[0], slots[1], sigma, sigma_next, kind=kind, eta=float(eta),
+                                   sigma_max=sigma_max, step_major=step_major, means_dtype=means_dtype)
+
+
+def replay_slots(indices, step_indices) -> Tuple[list, list]:
+    """Storage slots ``(of each step's latent, of its stored next latent)`` inside a trajectory stack
+    whose slot ``k`` holds the latent of step ``indices[k]`` (``LatentSegment.latents_at``,
+    ``unirl/types/segments/latent.py:82-97``, for ``step`` and ``step + 1``)."""
+    if indices is None:
+        raise RuntimeError("replay_slots: missing indices")
+    stored = [int(i) for i in (indices.tolist() if isinstance(indices, torch.Tensor) else indices)]
+    where = {}
+    for k, i in enumerate(stored):
+        where.setdefault(i, k)  # the first slot holding a step, as list.index finds it
+    out = ([], [])
+    for step in step_indices:
+        for offset, slots in zip((0, 1), out):
+            if int(step) + offset not in where:
+                raise KeyError(f"latents_at: step_idx={int(step) + offset} not in stored indices={stored}")
+            slots.append(where[int(step) + offset])
+    return out
 
 
 def latents_at(latents: Optional[torch.Tensor], indices: Optional[torch.Tensor], step_idx: int) -> torch.Tensor:
@@ -472,5 +558,6 @@ __all__ = [
     "STRATEGIES",
     "StepStrategy",
     "latents_at",
+    "replay_slots",
     "sde_rollout",
 ]
