@@ -369,3 +369,31 @@ def test_release_library_reads_no_environment_knobs(built_lib):
     names = set(re.findall(rb"UNIRL_[A-Z0-9_]{3,}", blob))
     assert not names, f"environment knob names in the release library: {sorted(names)}"
     assert b"getenv" not in blob or b"UNIRL_" not in blob
+
+
+def test_conforming_operands_are_handed_over_without_a_copy(monkeypatch):
+    """Tensors that already have the dtype, device and layout a kernel reads are passed as they
+    are -- no detach, cast or contiguous() hop, each of which costs more host time than the
+    whole argument check; anything else is converted once."""
+    from unirl_amd import _native as N
+    from unirl_amd import ops
+
+    monkeypatch.setattr(N, "require_device", lambda t, name: None)
+    cpu = torch.device("cpu")
+    new = torch.randn(4, 8, requires_grad=True)
+    old = torch.randn(4, 8)
+    adv = torch.randn(4)
+    lengths = torch.tensor([8, 4, 2, 1])
+    assert N.as_operand(new, torch.float32, cpu) is new          # requires grad: still no detach
+    assert N.as_operand(lengths, torch.int64, cpu) is lengths
+    half = N.as_operand(old.half(), torch.float32, cpu)
+    assert half.dtype == torch.float32 and half.is_contiguous()
+    strided = N.as_operand(old.t(), torch.float32, cpu)
+    assert strided.is_contiguous() and torch.equal(strided, old.t())
+    assert ops._flat2(new, "new") is new and ops._kernel_dtype(old) is old
+    assert ops._kernel_dtype(old.double()).dtype == torch.float32
+    plan = ops.RatioLossPlan(new, old, adv, kind=N.LOSS_GRPO, lengths=lengths)
+    assert plan.nw is new and plan.od is old and plan.adv is adv and plan.seq is lengths
+    # the sigma arguments of the SDE step: an fp32 scalar passes untouched
+    s = torch.tensor(0.5)
+    assert ops._sigma_arg(s, 4, cpu, "sigma")[0] is s

@@ -272,6 +272,20 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
+class _Functions:
+    """The library's entry points as plain attributes: the first use of a name loads the library
+    and binds the function; later uses are one attribute read (``lib().name`` costs a call and a
+    ctypes lookup every time, which shows on a path whose kernels run for ten microseconds)."""
+
+    def __getattr__(self, name: str):
+        fn = getattr(lib(), name)
+        setattr(self, name, fn)
+        return fn
+
+
+F = _Functions()
+
+
 def check(status: int, what: str) -> None:
     """Turn a C-ABI status into an exception: ValueError for argument errors,
     UnirlHipError for a failed launch."""
@@ -302,8 +316,29 @@ def ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
+# torch's raw accessors (no Stream / device objects built per call); the public API as a fallback
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
+def current_device_index() -> int:
+    return _raw_device() if _raw_device is not None else torch.cuda.current_device()
+
+
 def current_stream(device: torch.device) -> int:
-    return torch.cuda.current_stream(device).cuda_stream
+    """Raw handle of torch's current stream on ``device``."""
+    if _raw_stream is None:
+        return torch.cuda.current_stream(device).cuda_stream
+    index = device.index
+    return _raw_stream(current_device_index() if index is None else index)
+
+
+def as_operand(t: torch.Tensor, dtype: torch.dtype, device: torch.device) -> torch.Tensor:
+    """``t`` as a contiguous ``dtype`` tensor on ``device`` -- ``t`` itself (no detach, cast or copy:
+    only its address is taken) when it already is one."""
+    if t.dtype is dtype and t.device == device and t.is_contiguous():
+        return t
+    return t.detach().to(device=device, dtype=dtype).contiguous()
 
 
 class on_device:
@@ -315,7 +350,7 @@ class on_device:
 
     def __init__(self, device: torch.device) -> None:
         index = device.index
-        self._ctx = None if (index is None or index == torch.cuda.current_device()) else torch.cuda.device(index)
+        self._ctx = None if (index is None or index == current_device_index()) else torch.cuda.device(index)
 
     def __enter__(self):
         if self._ctx is not None:
@@ -335,7 +370,7 @@ def workspace(device: torch.device, stream: Optional[int] = None) -> Tuple[torch
     """Scratch for the reducing kernels (per-workgroup partial sums), one per (device, stream):
     calls on different streams may overlap and must not share it.  ``stream`` is the raw handle
     when the caller has already looked it up."""
-    index = device.index if device.index is not None else torch.cuda.current_device()
+    index = device.index if device.index is not None else current_device_index()
     key = (index, current_stream(device) if stream is None else stream)
     ws = _workspaces.get(key)
     if ws is None:

@@ -33,14 +33,16 @@ class _ScalarLossFn(torch.autograd.Function):
     def forward(ctx, new_logp: torch.Tensor, plan: RatioLossPlan):
         _, metrics = plan.forward(want_elem=False)
         ctx.plan = plan
-        ctx.n_valid = metrics[N.M_NUM_TOKENS : N.M_NUM_TOKENS + 1]
-        loss = metrics[N.M_LOSS].clone()
+        ctx.metrics = metrics  # slot M_NUM_TOKENS is the token-mean denominator of the backward
+        # a view, not a copy: a clone would be one more launch on a path of two
+        loss = metrics[N.M_LOSS]
         ctx.mark_non_differentiable(metrics)
         return loss, metrics
 
     @staticmethod
     def backward(ctx, g_loss, _g_metrics):
-        grad = ctx.plan.backward(g_scale=g_loss, g_elem=None, aggregate=True, n_valid=ctx.n_valid)
+        n_valid = ctx.metrics[N.M_NUM_TOKENS : N.M_NUM_TOKENS + 1]
+        grad = ctx.plan.backward(g_scale=g_loss, g_elem=None, aggregate=True, n_valid=n_valid)
         return grad, None
 
 
@@ -58,7 +60,7 @@ def scalar_loss(new_logp: torch.Tensor, plan: RatioLossPlan) -> Tuple[torch.Tens
     if torch.is_grad_enabled() and new_logp.requires_grad:
         return _ScalarLossFn.apply(new_logp, plan)
     _, metrics = plan.forward(want_elem=False)
-    return metrics[N.M_LOSS].clone(), metrics
+    return metrics[N.M_LOSS], metrics
 
 
 def fused_token_loss_backward(
@@ -127,7 +129,7 @@ ABSDIFF_METRICS: Dict[str, int] = {
 
 def metric_tensors(metrics: torch.Tensor, slots: Dict[str, int]) -> Dict[str, torch.Tensor]:
     """0-dim detached views into the metrics vector, keyed by the reference's metric names."""
-    m = metrics.detach()
+    m = metrics.detach().unbind(0)  # one call for the sixteen 0-dim views
     return {name: m[slot] for name, slot in slots.items()}
 
 

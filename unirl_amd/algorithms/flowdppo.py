@@ -95,6 +95,23 @@ class _MaskedRatioLossFn(torch.autograd.Function):
         return g_elem * elem, None, None, None, None
 
 
+class _MaskedRatioStepFn(torch.autograd.Function):
+    """The same loss with the KL over the means in the same call (``unirl_flowdppo_step``: the
+    streaming KL kernel plus one finishing workgroup -- two launches instead of three)."""
+
+    @staticmethod
+    def forward(ctx, new_logp, old_logp, new_means, old_means, advantages, sigma_t, threshold):
+        _, elem, metrics, _ = ops.flowdppo_step(new_logp, old_logp, new_means, old_means, advantages, sigma_t, threshold)
+        ctx.save_for_backward(elem)
+        ctx.mark_non_differentiable(metrics)
+        return elem, metrics
+
+    @staticmethod
+    def backward(ctx, g_elem, _g_metrics):
+        (elem,) = ctx.saved_tensors  # d(-A r)/d new_logp = -A r where kept, 0 where masked: the loss itself
+        return g_elem * elem, None, None, None, None, None, None
+
+
 def _flowdppo_kl_adv_loss(
     *,
     new_logp: torch.Tensor,
@@ -111,14 +128,24 @@ def _flowdppo_kl_adv_loss(
     axis = _sigma_axis(new_means, sigma_t)
     if axis not in (None, 1):
         raise ValueError(f"sigma_t {tuple(sigma_t.shape)} must be a scalar or vary along the step axis (dim 1)")
-    kl, _ = ops.gaussian_kl_mask(new_means, old_means, sigma_t, kl_mask_threshold, reduce_from_dim=2, want_mask=False)
-    if torch.is_grad_enabled() and new_logp.requires_grad:
-        elem, mvec = _MaskedRatioLossFn.apply(new_logp, old_logp, advantages, kl, float(kl_mask_threshold))
+    threshold = float(kl_mask_threshold)
+    needs_grad = torch.is_grad_enabled() and new_logp.requires_grad
+    rows = new_logp.numel()
+    if new_logp.dim() == 2 and tuple(new_means.shape[:2]) == tuple(new_logp.shape) and 0 < rows <= ops.FLOWDPPO_STEP_MAX_ROWS:
+        # the usual [B, S'] problem: KL, masks, loss and metrics as one call of two launches
+        if needs_grad:
+            elem, mvec = _MaskedRatioStepFn.apply(new_logp, old_logp, new_means, old_means, advantages, sigma_t, threshold)
+        else:
+            _, elem, mvec, _ = ops.flowdppo_step(new_logp, old_logp, new_means, old_means, advantages, sigma_t, threshold)
     else:
-        elem, mvec = ops.flowdppo_loss(new_logp, old_logp, advantages, kl, float(kl_mask_threshold))
+        kl, _ = ops.gaussian_kl_mask(new_means, old_means, sigma_t, threshold, reduce_from_dim=2, want_mask=False)
+        if needs_grad:
+            elem, mvec = _MaskedRatioLossFn.apply(new_logp, old_logp, advantages, kl, threshold)
+        else:
+            elem, mvec = ops.flowdppo_loss(new_logp, old_logp, advantages, kl, threshold)
     if elem.dtype != new_logp.dtype:
         elem = elem.to(new_logp.dtype)
-    m = mvec.detach()
+    m = mvec.detach().unbind(0)  # one call for the sixteen 0-dim views
     metrics = {name: m[slot] for name, slot in ops.FLOWDPPO_METRIC_SLOTS.items() if name != "loss_mean"}
     return elem, metrics
 

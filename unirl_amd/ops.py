@@ -19,8 +19,15 @@ SDE_KINDS = {"flow": N.SDE_FLOW, "dance": N.SDE_DANCE, "cps": N.SDE_CPS}
 
 
 def _flat2(t: torch.Tensor, name: str) -> torch.Tensor:
+    """``t`` itself when it is a contiguous device tensor (only its address is used, so a tensor
+    that requires grad needs no detach), else a contiguous copy."""
     N.require_device(t, name)
-    return t if t.is_contiguous() else t.contiguous()
+    return t if t.is_contiguous() else t.detach().contiguous()
+
+
+def _kernel_dtype(t: torch.Tensor) -> torch.Tensor:
+    """fp32 / bf16 / fp16 tensors pass; anything else (float64, ...) is cast to fp32."""
+    return t if t.dtype in N._DTYPE_CODE else t.detach().float()
 
 
 def _sigma_arg(sigma: torch.Tensor, B: int, device: torch.device, name: str) -> Tuple[torch.Tensor, int]:
@@ -43,6 +50,8 @@ def _sigma_max_arg(sigma_max, device: torch.device):
     """(device tensor or None, float value)."""
     if isinstance(sigma_max, torch.Tensor):
         if sigma_max.is_cuda:
+            if sigma_max.numel() == 1 and sigma_max.dtype is torch.float32 and sigma_max.device == device:
+                return sigma_max, 0.0  # one fp32 value on the device: its address is all that is needed
             t = sigma_max.detach().to(device=device, dtype=torch.float32).reshape(-1)[:1].contiguous()
             return t, 0.0
         return None, float(sigma_max)
@@ -76,12 +85,8 @@ def sde_step_logp(
     if noise_pred.shape != sample.shape:
         raise ValueError(f"noise_pred {tuple(noise_pred.shape)} != sample {tuple(sample.shape)}")
     device = sample.device
-    v = _flat2(noise_pred.detach(), "noise_pred")
-    x = _flat2(sample.detach(), "sample")
-    if v.dtype not in N._DTYPE_CODE:
-        v = v.float()
-    if x.dtype not in N._DTYPE_CODE:
-        x = x.float()
+    v = _kernel_dtype(_flat2(noise_pred, "noise_pred"))
+    x = _kernel_dtype(_flat2(sample, "sample"))
     B = x.shape[0]
     D = x.numel() // B if B else 0
     prev_in = None
@@ -89,12 +94,16 @@ def sde_step_logp(
         if prev_sample.shape != sample.shape:
             raise ValueError(f"prev_sample {tuple(prev_sample.shape)} != sample {tuple(sample.shape)}")
         # prev.float().to(x.dtype) == prev.to(x.dtype): casting here is the reference's round trip
-        prev_in = _flat2(prev_sample.detach(), "prev_sample").to(x.dtype)
+        prev_in = _flat2(prev_sample, "prev_sample")
+        if prev_in.dtype is not x.dtype:
+            prev_in = prev_in.detach().to(x.dtype)
     nz = None
     if noise is not None and prev_sample is None:
         if noise.shape != sample.shape:
             raise ValueError(f"noise {tuple(noise.shape)} != sample {tuple(sample.shape)}")
-        nz = _flat2(noise.detach(), "noise").float()
+        nz = _flat2(noise, "noise")
+        if nz.dtype is not torch.float32:
+            nz = nz.detach().float()
     sig, stride = _sigma_arg(sigma, B, device, "sigma")
     sig_n, stride_n = _sigma_arg(sigma_next, B, device, "sigma_next")
     if stride != stride_n:
@@ -115,7 +124,7 @@ def sde_step_logp(
     stream = N.current_stream(device)
     ws, ws_bytes = N.workspace(device, stream)
     with N.on_device(device):
-        rc = N.lib().unirl_sde_step_logp(
+        rc = N.F.unirl_sde_step_logp(
             N.ptr(v), N.dtype_code(v.dtype), N.ptr(x), N.dtype_code(x.dtype), N.ptr(prev_in), N.ptr(nz),
             N.ptr(sig), N.ptr(sig_n), stride, N.ptr(smax_t), smax_v, float(eta), SDE_KINDS[kind], B, D,
             N.ptr(prev_out), N.ptr(mean_out), N.ptr(logp_out), int(bool(logp_sum)), N.ptr(ws), ws_bytes,
@@ -242,7 +251,7 @@ def sde_step_logp_into(
     d.logp_out, d.logp_stride, d.logp_sum = N.ptr(lp), slp, int(bool(logp_sum))
     ws, ws_bytes = N.workspace(device)
     with N.on_device(device):
-        rc = N.lib().unirl_sde_step_logp_ex(ctypes.byref(d), N.ptr(ws), ws_bytes, N.current_stream(device))
+        rc = N.F.unirl_sde_step_logp_ex(ctypes.byref(d), N.ptr(ws), ws_bytes, N.current_stream(device))
     N.check(rc, "unirl_sde_step_logp_ex")
 
 
@@ -349,7 +358,7 @@ def sde_replay_logp(
     stream = N.current_stream(device)
     ws, ws_bytes = N.workspace(device, stream)
     with N.on_device(device):
-        rc = N.lib().unirl_sde_replay_logp(ctypes.byref(d), N.ptr(ws), ws_bytes, stream)
+        rc = N.F.unirl_sde_replay_logp(ctypes.byref(d), N.ptr(ws), ws_bytes, stream)
     N.check(rc, "unirl_sde_replay_logp")
     return logp, means
 
@@ -389,7 +398,7 @@ def sde_replay_logp_bwd(
     gm = f32c(g_mean, (B, S, D))
     d.logp_sum = int(bool(logp_sum))
     with N.on_device(device):
-        rc = N.lib().unirl_sde_replay_logp_bwd(ctypes.byref(d), N.ptr(gl), N.ptr(gm), N.ptr(grad),
+        rc = N.F.unirl_sde_replay_logp_bwd(ctypes.byref(d), N.ptr(gl), N.ptr(gm), N.ptr(grad),
                                                N.dtype_code(out_dtype), N.current_stream(device))
     N.check(rc, "unirl_sde_replay_logp_bwd")
     return grad if grad.dtype == noise_pred.dtype else grad.to(noise_pred.dtype)
@@ -446,7 +455,7 @@ def sde_step_logp_bwd(
     if gl is None and gm is None and gp is None:  # nothing flows back
         return (None if grad_v is None else grad_v.zero_()), (None if grad_x is None else grad_x.zero_())
     with N.on_device(device):
-        rc = N.lib().unirl_sde_step_logp_bwd(
+        rc = N.F.unirl_sde_step_logp_bwd(
             N.ptr(v), N.dtype_code(v.dtype), N.ptr(x), N.dtype_code(x.dtype), N.ptr(prev_in), N.ptr(nz),
             N.ptr(sig), N.ptr(sig_n), stride, N.ptr(smax_t), smax_v, float(eta), SDE_KINDS[kind], B, D,
             N.ptr(gl), N.ptr(gm), N.ptr(gp), int(bool(logp_sum)), N.ptr(grad_v), N.dtype_code(v.dtype),
@@ -527,7 +536,7 @@ def sde_rollout_logp(
     e_arr = (ctypes.c_double * S)(*[float(e) for e in etas])
     ws, ws_bytes = N.workspace(device)
     with N.on_device(device):
-        rc = N.lib().unirl_sde_rollout_logp(
+        rc = N.F.unirl_sde_rollout_logp(
             N.ptr(x), N.dtype_code(x.dtype), v_arr, N.dtype_code(vdtype), n_arr, N.ptr(sig), e_arr, S,
             N.ptr(smax_t), smax_v, SDE_KINDS[kind], B, D, N.ptr(x_out), N.ptr(traj), N.ptr(logp),
             int(bool(logp_sum)), N.ptr(ws), ws_bytes, N.current_stream(device),
@@ -569,7 +578,7 @@ def dpm2_step(
         raise ValueError("x0_out must not alias x0_prev")
     prev = torch.empty(sample.shape, dtype=torch.float32, device=device)
     with N.on_device(device):
-        rc = N.lib().unirl_dpm2_step(
+        rc = N.F.unirl_dpm2_step(
             N.ptr(v), N.dtype_code(v.dtype), N.ptr(x), N.dtype_code(x.dtype), N.ptr(m1), int(branch),
             ctypes.byref(coeffs), x.numel(), N.ptr(x0_out), N.ptr(prev), N.current_stream(device),
         )
@@ -596,14 +605,14 @@ def gaussian_kl_mask(
     if p.dim() <= reduce_from_dim:
         raise ValueError(f"need more than {reduce_from_dim} dims to reduce over; got {tuple(p.shape)}")
     device = p.device
-    pc = _flat2(p.detach(), "p")
-    qc = _flat2(q.detach(), "q").to(pc.dtype)
-    if pc.dtype not in N._DTYPE_CODE:
-        pc, qc = pc.float(), qc.float()
+    pc = _kernel_dtype(_flat2(p, "p"))
+    qc = _flat2(q, "q")
+    if qc.dtype is not pc.dtype:
+        qc = qc.detach().to(pc.dtype)
     lead = tuple(pc.shape[:reduce_from_dim])
     R = int(math.prod(lead))
     D = pc.numel() // R if R else 0
-    sig = sigma.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    sig = N.as_operand(sigma, torch.float32, device)  # the kernel reads it flat, whatever its shape
     if sig.numel() not in (1, lead[-1]):
         raise ValueError(f"sigma must hold 1 or {lead[-1]} values; got {tuple(sigma.shape)}")
     kl = torch.empty(lead, dtype=torch.float32, device=device)
@@ -613,7 +622,7 @@ def gaussian_kl_mask(
     stream = N.current_stream(device)
     ws, ws_bytes = N.workspace(device, stream)
     with N.on_device(device):
-        rc = N.lib().unirl_gaussian_kl_mask(
+        rc = N.F.unirl_gaussian_kl_mask(
             N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, float(threshold),
             N.ptr(kl), N.ptr(mask), N.ptr(ws), ws_bytes, stream,
         )
@@ -657,7 +666,7 @@ def flowdppo_loss(
     elem = torch.empty(shape, dtype=torch.float32, device=device)
     metrics = torch.empty(N.M_COUNT, dtype=torch.float32, device=device)
     with N.on_device(device):
-        rc = N.lib().unirl_flowdppo_loss(
+        rc = N.F.unirl_flowdppo_loss(
             N.ptr(nw), N.ptr(od), N.ptr(ad), N.ptr(klc), nw.numel(), float(threshold), N.ptr(elem),
             N.ptr(metrics), N.current_stream(device),
         )
@@ -699,30 +708,30 @@ def flowdppo_step(
     R = shape[0] * shape[1]
     if R == 0 or R > FLOWDPPO_STEP_MAX_ROWS:
         raise ValueError(f"flowdppo_step handles 1..{FLOWDPPO_STEP_MAX_ROWS} rows; got {R}")
-    pc = _flat2(new_means.detach(), "new_means")
-    qc = _flat2(old_means.detach(), "old_means").to(pc.dtype)
-    if pc.dtype not in N._DTYPE_CODE:
-        pc, qc = pc.float(), qc.float()
+    pc = _kernel_dtype(_flat2(new_means, "new_means"))
+    qc = _flat2(old_means, "old_means")
+    if qc.dtype is not pc.dtype:
+        qc = qc.detach().to(pc.dtype)
     D = pc.numel() // R
-    sig = sigma_t.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
+    sig = N.as_operand(sigma_t, torch.float32, device)  # read flat by the kernel
     if sig.numel() not in (1, shape[1]):
         raise ValueError(f"sigma_t must hold 1 or {shape[1]} values; got {tuple(sigma_t.shape)}")
 
     def f32c(t):
-        t = t.detach().to(device=device, dtype=torch.float32)
         if tuple(t.shape) != shape:
-            t = t.expand(shape)
-        return t.contiguous()
+            t = t.detach().expand(shape)
+        return N.as_operand(t, torch.float32, device)
 
     nw, od, ad = f32c(new_logp), f32c(old_logp), f32c(advantages)
-    kl = torch.empty(shape, dtype=torch.float32, device=device)
-    elem = torch.empty(shape, dtype=torch.float32, device=device)
-    grad = torch.empty(shape, dtype=torch.float32, device=device) if loss_scale is not None else None
+    # the three [B, S'] outputs are a few dozen floats that live and die together: one allocation
+    kl, elem, grad = torch.empty((3,) + shape, dtype=torch.float32, device=device).unbind(0)
+    if loss_scale is None:
+        grad = None
     metrics = torch.empty(N.M_COUNT, dtype=torch.float32, device=device)
     stream = N.current_stream(device)
     ws, ws_bytes = N.workspace(device, stream)
     with N.on_device(device):
-        rc = N.lib().unirl_flowdppo_step(
+        rc = N.F.unirl_flowdppo_step(
             N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, N.ptr(nw), N.ptr(od),
             N.ptr(ad), float(threshold), float(loss_scale or 0.0), N.ptr(kl), N.ptr(elem), N.ptr(grad),
             N.ptr(metrics), N.ptr(ws), ws_bytes, stream,
@@ -742,7 +751,7 @@ def expand_per_seq(values: torch.Tensor, cu_seqlens: torch.Tensor, n_tok: int) -
     out = torch.empty(int(n_tok), dtype=torch.float32, device=device)
     if n_tok:
         with N.on_device(device):
-            rc = N.lib().unirl_expand_per_seq(
+            rc = N.F.unirl_expand_per_seq(
                 N.ptr(v), N.ptr(cu), v.numel(), int(n_tok), N.ptr(out), N.current_stream(device)
             )
         N.check(rc, "unirl_expand_per_seq")
@@ -770,7 +779,7 @@ def gaussian_kl_elem(p: torch.Tensor, q: torch.Tensor, sigma: torch.Tensor, *, s
     if pc.numel() == 0:
         return out
     with N.on_device(device):
-        rc = N.lib().unirl_gaussian_kl_elem(
+        rc = N.F.unirl_gaussian_kl_elem(
             N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, N.ptr(out),
             N.current_stream(device),
         )
@@ -799,7 +808,7 @@ def gaussian_kl_elem_bwd(
     gq = torch.empty_like(pc) if need_q else None
     if pc.numel() and (need_p or need_q):
         with N.on_device(device):
-            rc = N.lib().unirl_gaussian_kl_elem_bwd(
+            rc = N.F.unirl_gaussian_kl_elem_bwd(
                 N.ptr(pc), N.ptr(qc), N.dtype_code(pc.dtype), N.ptr(sig), sig.numel(), R, D, N.ptr(g), N.ptr(gp),
                 N.ptr(gq), N.current_stream(device),
             )
@@ -823,16 +832,14 @@ def token_logp_entropy(
     device = logits.device
     V = logits.shape[-1]
     lead = tuple(logits.shape[:-1])
-    x = logits.detach()
-    if x.dtype not in N._DTYPE_CODE:
-        x = x.float()
+    x = _kernel_dtype(logits)
     idc = None
     if want_logp:
         if ids is None:
             raise ValueError("ids is required for the log-prob")
         if tuple(ids.shape) != lead:
             raise ValueError(f"ids {tuple(ids.shape)} does not match logits rows {lead}")
-        idc = ids.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
+        idc = N.as_operand(ids, torch.int64, device).reshape(-1)
     logp = torch.empty(lead, dtype=torch.float32, device=device) if want_logp else None
     ent = torch.empty(lead, dtype=torch.float32, device=device) if want_entropy else None
     lse = torch.empty(lead, dtype=torch.float32, device=device) if want_lse else None
@@ -846,6 +853,14 @@ def token_logp_entropy(
         return None if t is None else t.reshape(-1)
 
     stream = N.current_stream(device)
+    if x.is_contiguous():  # the usual case: one block, every tensor handed over whole
+        with N.on_device(device):
+            rc = N.F.unirl_token_logp_entropy(
+                x.data_ptr(), N.dtype_code(x.dtype), n_rows, V, V, N.ptr(idc), float(temperature), N.ptr(logp),
+                N.ptr(ent), N.ptr(lse), stream,
+            )
+        N.check(rc, "unirl_token_logp_entropy")
+        return logp, ent, lse
     # One launch per block of rows that share a row stride.  `[B, S, V][:, :-1]` (the shifted
     # logits of a training step) is B such blocks: reading it in place costs B launches, flattening
     # it would cost a copy of the logits.
@@ -858,7 +873,7 @@ def token_logp_entropy(
             def part(t):
                 return None if t is None else t[off : off + rows]
 
-            rc = N.lib().unirl_token_logp_entropy(
+            rc = N.F.unirl_token_logp_entropy(
                 N.ptr(x2), N.dtype_code(x2.dtype), rows, V, row_stride, N.ptr(part(idc)), float(temperature),
                 N.ptr(part(flat(logp))), N.ptr(part(flat(ent))), N.ptr(part(flat(lse))), stream,
             )
@@ -919,7 +934,7 @@ def token_logp_bwd(
         with N.on_device(device):
             for x2 in _row_blocks(x, V):  # sliced logits are read in place, block by block
                 rows = x2.shape[0]
-                rc = N.lib().unirl_token_logp_bwd(
+                rc = N.F.unirl_token_logp_bwd(
                     N.ptr(x2), N.dtype_code(x2.dtype), rows, V, x2.stride(0) if rows > 1 else V,
                     N.ptr(idc[off : off + rows]), float(temperature), N.ptr(lsec[off : off + rows]),
                     N.ptr(gc[off : off + rows]), N.ptr(grad[off : off + rows]), V, stream,
@@ -981,10 +996,10 @@ class RatioLossPlan:
         device = new_logp.device
         self.device = device
         self.shape = tuple(new_logp.shape)
-        self.nw = new_logp.detach().to(torch.float32).contiguous()
-        self.od = old_logp.detach().to(device=device, dtype=torch.float32).contiguous()
+        self.nw = N.as_operand(new_logp, torch.float32, device)
+        self.od = N.as_operand(old_logp, torch.float32, device)
         self.n_tok = self.nw.numel()
-        adv = advantages.detach().to(device=device, dtype=torch.float32).contiguous()
+        adv = N.as_operand(advantages, torch.float32, device)
         self.seq = None
         self.n_seq = 0
         self.seq_stride = 0
@@ -997,11 +1012,11 @@ class RatioLossPlan:
             self.n_seq, self.seq_stride = self.shape
             if lengths.device.type == "cpu":  # the token count is free on the host
                 self.n_valid_host = int(lengths.detach().reshape(-1).clamp(0, self.seq_stride).sum())
-            self.seq = lengths.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
+            self.seq = N.as_operand(lengths, torch.int64, device)  # read flat by the kernel
             if self.seq.numel() != self.n_seq:
                 raise ValueError(f"lengths has {self.seq.numel()} entries for {self.n_seq} sequences")
         elif cu_seqlens is not None:
-            self.seq = cu_seqlens.detach().to(device=device, dtype=torch.int64).reshape(-1).contiguous()
+            self.seq = N.as_operand(cu_seqlens, torch.int64, device)
             self.n_seq = self.seq.numel() - 1
             if self.n_seq < 0:
                 raise ValueError("cu_seqlens needs n_seq + 1 entries")
@@ -1022,7 +1037,7 @@ class RatioLossPlan:
         if loss_mask is not None:
             if loss_mask.numel() != self.n_tok:
                 raise ValueError(f"loss_mask {tuple(loss_mask.shape)} does not match tokens {self.shape}")
-            self.mask = loss_mask.detach().to(device=device, dtype=torch.float32).contiguous()
+            self.mask = N.as_operand(loss_mask, torch.float32, device)
         self.params = _ratio_params(
             kind, agg_mode, clip_low, clip_low if clip_high is None else clip_high, drpo_epsilon, mu_weighted,
             horizon, adv_per_token,
@@ -1040,7 +1055,7 @@ class RatioLossPlan:
         stream = N.current_stream(device)
         ws, ws_bytes = N.workspace(device, stream)
         with N.on_device(device):
-            rc = N.lib().unirl_ratio_loss_fwd(
+            rc = N.F.unirl_ratio_loss_fwd(
                 N.ptr(self.nw), N.ptr(self.od), N.ptr(self.adv), N.ptr(self.seq), N.ptr(self.mask), self.n_seq,
                 self.seq_stride, self.n_tok, ctypes.byref(self.params), N.ptr(elem), N.ptr(metrics), N.ptr(ws),
                 ws_bytes, stream,
@@ -1061,7 +1076,7 @@ class RatioLossPlan:
         stream = N.current_stream(device)
         ws, ws_bytes = N.workspace(device, stream)
         with N.on_device(device):
-            rc = N.lib().unirl_ratio_loss_fwd_bwd(
+            rc = N.F.unirl_ratio_loss_fwd_bwd(
                 N.ptr(self.nw), N.ptr(self.od), N.ptr(self.adv), N.ptr(self.seq), N.ptr(self.mask), self.n_seq,
                 self.seq_stride, self.n_tok, ctypes.byref(self.params), float(loss_scale), int(self.n_valid_host),
                 N.ptr(grad), N.ptr(metrics), N.ptr(ws), ws_bytes, stream,
@@ -1086,7 +1101,7 @@ class RatioLossPlan:
         ge = None if g_elem is None else g_elem.detach().to(device=device, dtype=torch.float32).contiguous()
         nv = None if n_valid is None else n_valid.detach().reshape(-1)[:1].contiguous()
         with N.on_device(device):
-            rc = N.lib().unirl_ratio_loss_bwd(
+            rc = N.F.unirl_ratio_loss_bwd(
                 N.ptr(self.nw), N.ptr(self.od), N.ptr(self.adv), N.ptr(self.seq), N.ptr(self.mask), self.n_seq,
                 self.seq_stride, self.n_tok, ctypes.byref(self.params), N.ptr(gs), N.ptr(ge),
                 int(bool(aggregate)), N.ptr(nv), N.ptr(grad), N.current_stream(device),
@@ -1116,7 +1131,7 @@ def group_advantages(
     if n_groups <= 0 or n % n_groups != 0:
         raise ValueError(f"non-uniform group sizes (n={n}, n_groups={n_groups})")
     with N.on_device(r.device):
-        rc = N.lib().unirl_group_advantages(
+        rc = N.F.unirl_group_advantages(
             N.ptr(r), n_groups, n // n_groups, int(bool(normalize)), float(eps), int(scope == "global"),
             int(bool(use_global_std)), N.ptr(out), N.current_stream(r.device),
         )
@@ -1154,7 +1169,7 @@ def normalize_grouped(
     mem_t = torch.tensor(members, dtype=torch.int64, device=device)
     off_t = torch.tensor(offsets, dtype=torch.int64, device=device)
     with N.on_device(device):
-        rc = N.lib().unirl_normalize_grouped(
+        rc = N.F.unirl_normalize_grouped(
             N.ptr(r), n, N.ptr(mem_t), N.ptr(off_t), n_groups, float(eps), float(trim_outliers_ratio),
             int(bool(use_global_std)), int(clip_max is not None), float(clip_max or 0.0), N.ptr(out),
             N.current_stream(device),
@@ -1172,7 +1187,7 @@ def calib_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
     if nbytes != dst.numel() * dst.element_size() or not (src.is_contiguous() and dst.is_contiguous()):
         raise ValueError("calib_copy needs two contiguous tensors of the same byte size")
     with N.on_device(src.device):
-        rc = N.lib().unirl_calib_copy(N.ptr(src), N.ptr(dst), nbytes, N.current_stream(src.device))
+        rc = N.F.unirl_calib_copy(N.ptr(src), N.ptr(dst), nbytes, N.current_stream(src.device))
     N.check(rc, "unirl_calib_copy")
 
 
@@ -1187,7 +1202,7 @@ def calib_stream(src: Optional[torch.Tensor], read_bytes: int, dst: Optional[tor
             if not t.is_contiguous() or t.numel() * t.element_size() < nbytes:
                 raise ValueError(f"{name} must be contiguous and hold at least {nbytes} bytes")
     with N.on_device(sink.device):
-        rc = N.lib().unirl_calib_stream(
+        rc = N.F.unirl_calib_stream(
             N.ptr(src) if read_bytes else None, int(read_bytes), N.ptr(dst) if write_bytes else None,
             int(write_bytes), int(bool(tail_launch)), N.ptr(sink), N.current_stream(sink.device),
         )
@@ -1206,7 +1221,7 @@ def calib_reduce(src: torch.Tensor, read_bytes: int, mode: int, n_workgroups: in
     if out.dtype != torch.float64 or out.numel() < 1:
         raise ValueError("out must be a float64 tensor")
     with N.on_device(src.device):
-        rc = N.lib().unirl_calib_reduce(N.ptr(src), int(read_bytes), int(mode), int(n_workgroups), N.ptr(scratch),
+        rc = N.F.unirl_calib_reduce(N.ptr(src), int(read_bytes), int(mode), int(n_workgroups), N.ptr(scratch),
                                         scratch.numel() * scratch.element_size(), N.ptr(out),
                                         N.current_stream(src.device))
     N.check(rc, "unirl_calib_reduce")
@@ -1230,7 +1245,7 @@ def gather_steps(tensor: torch.Tensor, positions: Sequence[int]) -> torch.Tensor
         return out
     pos_t = torch.tensor(pos, dtype=torch.int64, device=t.device)
     with N.on_device(t.device):
-        rc = N.lib().unirl_gather_steps(
+        rc = N.F.unirl_gather_steps(
             N.ptr(t), B, S, inner_bytes, N.ptr(pos_t), len(pos), N.ptr(out), N.current_stream(t.device)
         )
     N.check(rc, "unirl_gather_steps")
@@ -1253,7 +1268,7 @@ def expand_groups(unique: torch.Tensor, group_of: torch.Tensor, dtype: torch.dty
     if U == 0:
         raise ValueError("no noise groups to expand")
     with N.on_device(src.device):
-        rc = N.lib().unirl_expand_groups(
+        rc = N.F.unirl_expand_groups(
             N.ptr(src), U, D, N.ptr(idx), B, N.ptr(out), N.dtype_code(dtype), N.current_stream(src.device)
         )
     N.check(rc, "unirl_expand_groups")
