@@ -451,7 +451,8 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
     ref = timed(reference)
     out["reference_torch_checkpoint_chunk2048"] = ref[0]
     for name, kw in (("fused_recompute_chunk2048", dict(chunk=2048, keep_logits=False)),
-                     ("fused_recompute_chunk4096", dict(keep_logits=False)), ("fused_default", dict())):
+                     ("fused_recompute_chunk4096", dict(keep_logits=False)), ("fused_default", dict()),
+                     ("fused_head_chunk4096", dict(fused_head=True))):
         got = timed(lambda h: models.chunked_replay_logp(head, h, tokens, 1.0, **kw))
         got[0]["max_abs_logp_diff"] = float((got[1] - ref[1]).abs().max())
         got[0]["grad_hidden_rel"] = float((got[2] - ref[2]).norm() / ref[2].norm())
@@ -459,6 +460,65 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
         out[name] = got[0]
         log(f"replay {name}: {got[0]}")
     log(f"replay reference: {ref[0]}")
+    return out
+
+
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
+
+
+def head_probe(torch, dev, vocab: int, hidden: int = 2560):
+    """The fused lm_head + log-softmax kernel (`unirl_lmhead_logp`: the [rows, V] logits are never
+    written) against the library GEMM followed by the token kernel, forward only, for a bf16 head of
+    Qwen3-4B's size.  TFLOP/s count the GEMM's 2*rows*K*V flops over the whole call."""
+    from unirl_amd import ops
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    w = (torch.randn(vocab, hidden, generator=g, device=dev) * (3.0 / math.sqrt(hidden))).bfloat16()
+
+    def timed(fn, n=5):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / n
+
+    out = []
+    for rows in (64, 2048, 8192):
+        h = torch.randn(rows, hidden, generator=g, device=dev).bfloat16()
+        ids = torch.randint(0, vocab, (rows,), generator=g, device=dev)
+        flop = 2.0 * rows * hidden * vocab
+
+        def unfused():
+            logits = torch.nn.functional.linear(h, w)
+            return ops.token_logp_entropy(logits, ids, 1.0, want_lse=True)
+
+        torch.cuda.synchronize()
+        torch.cuda.reset_peak_memory_stats()
+        base = torch.cuda.memory_allocated()
+        t_f = timed(lambda: ops.lmhead_logp(h, w, None, ids, 1.0, want_entropy=True, want_lse=True))
+        mem_f = torch.cuda.max_memory_allocated() - base
+        torch.cuda.reset_peak_memory_stats()
+        t_u = timed(unfused)
+        mem_u = torch.cuda.max_memory_allocated() - base
+        t_g = timed(lambda: torch.nn.functional.linear(h, w))
+        lp_f = ops.lmhead_logp(h, w, None, ids, 1.0)[0]
+        lp_u = unfused()[0]
+        row = {
+            "rows": rows, "vocab": vocab, "hidden": hidden,
+            "fused_ms": round(t_f, 3), "fused_tflops": round(flop / t_f / 1e9, 0),
+            "fused_frac_of_mfma_peak": round(flop / t_f / 1e9 / MFMA_BF16_PEAK_TFLOPS, 3),
+            "library_gemm_plus_token_kernel_ms": round(t_u, 3), "library_gemm_alone_ms": round(t_g, 3),
+            "library_gemm_tflops": round(flop / t_g / 1e9, 0),
+            "fused_transient_mib": round(mem_f / 2**20, 1), "unfused_transient_mib": round(mem_u / 2**20, 1),
+            "logp_rows_differing_beyond_2e-3": int(((lp_f - lp_u).abs() > 2e-3 * lp_u.abs() + 2e-3).sum()),
+        }
+        log(f"head probe: {row}")
+        out.append(row)
     return out
 
 
@@ -616,6 +676,9 @@ def main() -> int:
                     help="device-side timeline (launch gaps, kernel bodies) of the small shapes inside the 64-launch "
                          "graph, from the measurement build's own clock readings; optional comma-separated shape "
                          "names; needs `python -m unirl_amd.build --tune`")
+    ap.add_argument("--head-probe", action="store_true",
+                    help="the fused lm_head + log-softmax kernel (logits never written) against the library GEMM + "
+                         "token kernel for a bf16 Linear(2560, --vocab) head at 64 / 2048 / 8192 rows, then exit")
     ap.add_argument("--tail-probe", action="store_true",
                     help="cost of finishing a grid-wide reduction after its streaming part: nothing, a second "
                          "launch, or polled inside the one launch (unirl_calib_reduce), then exit")
@@ -651,6 +714,10 @@ def main() -> int:
     if args.timeline is not None:
         names = [n for n in args.timeline.split(",") if n]
         print(json.dumps({"timeline": timeline_probe(torch, dev, names)}), flush=True)
+        return 0
+
+    if args.head_probe:
+        print(json.dumps({"head_probe": head_probe(torch, dev, args.vocab)}), flush=True)
         return 0
 
     if args.tail_probe:

@@ -37,7 +37,8 @@ extern "C" {
 
 /* 2: typed gradient outputs in unirl_sde_step_logp_bwd; unirl_ratio_loss_fwd_bwd and
  * unirl_flowdppo_step added.  3: unirl_dpm2_step added.  4: unirl_gaussian_kl_mask_static
- * added.  5: unirl_sde_replay_logp, unirl_sde_replay_logp_bwd, unirl_calib_reduce added. */
+ * added.  5: unirl_sde_replay_logp, unirl_sde_replay_logp_bwd, unirl_calib_reduce,
+ * unirl_lmhead_logp added. */
 #define UNIRL_ABI_VERSION 5
 
 enum unirl_dtype { UNIRL_F32 = 0, UNIRL_BF16 = 1, UNIRL_F16 = 2 };
@@ -380,6 +381,35 @@ int unirl_token_logp_bwd(const void* logits, int dtype, int64_t rows, int64_t V,
                          int64_t row_stride, const int64_t* ids, float temperature,
                          const float* lse, const float* g_logp, void* grad_logits,
                          int64_t grad_row_stride, void* stream);
+
+/* ------------------------------------------------------------------------
+ * The same three outputs straight from the hidden states: the lm_head GEMM with
+ * the log-softmax statistics reduced in its epilogue, so the [rows, V] logits
+ * of a replay chunk (unirl/models/qwen3/ar.py:82-99: `lm_head(h).float() / T`,
+ * gather, logsumexp) are never written.  bf16 only, for a head in nn.Linear's
+ * layout:
+ *   hidden  bf16 [rows, K], consecutive rows ld_hidden elements apart
+ *   weight  bf16 [V, K] (row v = the weights of vocabulary entry v), rows
+ *           ld_weight elements apart;  bias bf16 [V] or NULL
+ *   logits  = bf16(fp32 sum over K (+ bias)) -- one rounding to bf16, as a bf16
+ *           Linear produces them; the statistics are taken from those values
+ *   logits_out  NULL, or bf16 [rows, V] (rows ld_logits apart) to also receive
+ *           the logits (validation; it costs the write this entry point exists
+ *           to avoid)
+ *   logp_out / ent_out / lse_out, ids, temperature: as unirl_token_logp_entropy
+ * Requirements: K a multiple of 64; ld_hidden, ld_weight multiples of 8 and both
+ * bases 16-byte aligned (UNIRL_E_SHAPE / UNIRL_E_ALIGN otherwise: use the
+ * library GEMM and unirl_token_logp_entropy).  scratch: device memory of
+ * unirl_lmhead_logp_scratch_bytes(rows, V) bytes (16 bytes per row and 128
+ * columns), no initialisation needed, one call at a time.
+ * Non-finite logits give NaN outputs for their row.
+ * ---------------------------------------------------------------------- */
+size_t unirl_lmhead_logp_scratch_bytes(int64_t rows, int64_t V);
+int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
+                      const void* bias, int64_t rows, int64_t V, int64_t K, const int64_t* ids,
+                      float temperature, float* logp_out, float* ent_out, float* lse_out,
+                      void* logits_out, int64_t ld_logits, void* scratch, size_t scratch_bytes,
+                      void* stream);
 
 /* ------------------------------------------------------------------------
  * Token-level ratio losses with every metric reduction fused in.

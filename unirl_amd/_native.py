@@ -198,6 +198,12 @@ _SIGNATURES = {
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_void_p],
     ),
+    "unirl_lmhead_logp_scratch_bytes": (c_size_t, [c_int64, c_int64]),
+    "unirl_lmhead_logp": (
+        c_int,
+        [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p,
+         c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_size_t, c_void_p],
+    ),
     "unirl_token_logp_bwd": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int64,

@@ -1,0 +1,423 @@
+// Token log-prob + entropy straight from the hidden states: the lm_head GEMM with the
+// log-softmax statistics reduced in its epilogue, so the [rows, V] logits are never written.
+//
+// Replaces the forward of a replay chunk (unirl/models/qwen3/ar.py:82-99):
+//   lf   = lm_head(h).float() / T          bf16 Linear: fp32 accumulation, result rounded to bf16
+//   logp = lf[tok] - logsumexp(lf)
+// for a bf16 head W [V, K] (nn.Linear's layout, K contiguous) and bf16 hidden states H [rows, K]
+// (K contiguous): both operands are read along K, the layout MFMA fragments want.
+//
+// Kernel 1 (lmhead_tile_kernel): one workgroup of four wavefronts per 128 x 128 tile of the
+// logits.  K is walked in steps of 64 through two LDS stages (global -> registers -> LDS, the next
+// step's loads in flight while the current one is multiplied); each wavefront owns a 64 x 64
+// quarter as 2 x 2 blocks of v_mfma_f32_32x32x16_bf16.  Epilogue: accumulators (+ bias) are
+// rounded to bf16 -- the values the reference's logits hold -- and passed through LDS so that
+// every thread owns half a row of the tile; it reduces its 64 logits to (m, s, t): the maximum,
+// sum 2^a and sum 2^a * a with a = (x - m) * log2(e)/T.  One (m, s, t) per (row, column tile)
+// goes to scratch memory (16 bytes for 256 bytes of logits) and the tile that holds a row's
+// target column also stores that logit.
+// Kernel 2 (lmhead_merge_kernel): one wavefront per row merges the row's tile states in fp64 and
+// finishes logsumexp, log-prob and entropy.
+//
+// Tiles are dealt to the workgroups so that each XCD (workgroup id modulo 8) walks its own
+// contiguous range of column groups, row block by row block: the group's slice of W stays in
+// that XCD's L2 while the hidden states stream past it.
+
+#include "common.cuh"
+#include "unirl_internal.h"
+
+namespace unirl {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+constexpr int kHdThreads = 256;
+constexpr int kBM = 128, kBN = 128, kBK = 64;
+// LDS rows are padded by 16 bytes: the 16-byte fragment reads of 16 consecutive rows then
+// cover all 64 banks exactly once
+constexpr int kLdsRow = kBK + 8;             // bf16 elements per operand row
+constexpr int kOperandElems = kBM * kLdsRow;  // one operand, one stage
+constexpr int kOutRow = kBN + 8;              // bf16 elements per row of the epilogue tile
+constexpr int kXcds = 8;
+constexpr double kHdLn2 = 0.6931471805599453;
+
+struct HeadArgs {
+  const uint16_t* h;
+  const uint16_t* w;
+  const uint16_t* bias;
+  const int64_t* ids;
+  int64_t M, N, K, ldh, ldw;
+  float c;  // log2(e) / T
+  float4* state;  // [M][n_tiles]: (m, s, t, -)
+  float* xid;     // [M]: the target's logit, written by the tile that holds its column
+  uint16_t* logits_out;
+  int64_t ld_logits;
+  int n_tiles, m_blocks, group;
+  float* logp;
+  float* ent;
+  float* lse;
+  UNIRL_TRACE_FIELD
+};
+
+// Tile of workgroup `wg`: every XCD takes a contiguous range of the sequence
+//   for column group g: for row block mb: for column tile n of the group: (mb, g*group + n)
+__device__ __forceinline__ void head_tile_of(const HeadArgs& A, unsigned int wg, int& mb, int& nt) {
+  const long long total = (long long)A.m_blocks * A.n_tiles;
+  const long long per_xcd = (total + kXcds - 1) / kXcds;
+  const long long pos = (long long)(wg % kXcds) * per_xcd + wg / kXcds;
+  if (pos >= total) {
+    mb = -1;
+    nt = -1;
+    return;
+  }
+  const long long per_group = (long long)A.m_blocks * A.group;
+  const long long g = pos / per_group;
+  // the last group may hold fewer column tiles
+  const int g_cols = (int)((g + 1) * A.group <= A.n_tiles ? A.group : A.n_tiles - g * A.group);
+  const long long in_group = pos - g * per_group;
+  mb = (int)(in_group / g_cols);
+  nt = (int)(g * A.group + in_group % g_cols);
+}
+
+__device__ __forceinline__ bf16x8_t lds_frag(const uint16_t* p) {
+  return *reinterpret_cast<const bf16x8_t*>(p);
+}
+
+template <bool HAS_BIAS, bool WRITE_LOGITS>
+__global__ __launch_bounds__(kHdThreads, 2) void lmhead_tile_kernel(HeadArgs A) {
+  __shared__ __attribute__((aligned(16))) uint16_t lds[2 * 2 * kOperandElems];  // [stage][A | B][row][kLdsRow]
+  UNIRL_TRACE_T0();
+  int mb, nt;
+  head_tile_of(A, blockIdx.x, mb, nt);
+  if (mb < 0) return;  // the padding of the last XCD's range (whole workgroup)
+  const int64_t m0 = (int64_t)mb * kBM, n0 = (int64_t)nt * kBN;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // global -> LDS assignment: 16-byte chunk c = tid + 256*i covers row c/8, k-chunk c%8 of a tile
+  const uint16_t* pa[4];
+  const uint16_t* pb[4];
+  int lds_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int c = tid + kHdThreads * i;
+    const int row = c >> 3, kc = c & 7;
+    int64_t ra = m0 + row, rb = n0 + row;
+    ra = ra < A.M ? ra : A.M - 1;  // rows past the end repeat the last one; their results are dropped
+    rb = rb < A.N ? rb : A.N - 1;
+    pa[i] = A.h + ra * A.ldh + kc * 8;
+    pb[i] = A.w + rb * A.ldw + kc * 8;
+    lds_off[i] = row * kLdsRow + kc * 8;
+  }
+  // Two register sets stage the global loads two K steps ahead of the multiplication: a trip to
+  // L2 takes longer than one step's sixteen MFMAs, so the loads of step k+2 are issued before
+  // step k is multiplied and land in LDS one step later.
+  u32x4 ga[2][4], gb[2][4];
+  auto load_global = [&](int set, int64_t k0) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      ga[set][i] = *reinterpret_cast<const u32x4*>(pa[i] + k0);
+      gb[set][i] = *reinterpret_cast<const u32x4*>(pb[i] + k0);
+    }
+  };
+  auto store_lds = [&](int set, int stage) {
+    uint16_t* sa = lds + stage * 2 * kOperandElems;
+    uint16_t* sb = sa + kOperandElems;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      *reinterpret_cast<u32x4*>(sa + lds_off[i]) = ga[set][i];
+      *reinterpret_cast<u32x4*>(sb + lds_off[i]) = gb[set][i];
+    }
+  };
+
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int bi = 0; bi < 2; ++bi)
+#pragma unroll
+    for (int bj = 0; bj < 2; ++bj)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[bi][bj][i] = 0.0f;
+
+  // fragment addresses inside a stage: lane l reads row (l % 32) of a 32-row block, k = 8 * (l / 32) ..
+  const int frag_a = (wm * 64 + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
+  const int frag_b = (wn * 64 + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
+  auto multiply = [&](int stage) {
+    const uint16_t* sa = lds + stage * 2 * kOperandElems;
+    const uint16_t* sb = sa + kOperandElems;
+#pragma unroll
+    for (int ks = 0; ks < kBK / 16; ++ks) {
+      const bf16x8_t a0 = lds_frag(sa + frag_a + ks * 16);
+      const bf16x8_t a1 = lds_frag(sa + frag_a + 32 * kLdsRow + ks * 16);
+      const bf16x8_t b0 = lds_frag(sb + frag_b + ks * 16);
+      const bf16x8_t b1 = lds_frag(sb + frag_b + 32 * kLdsRow + ks * 16);
+      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[0][0], 0, 0, 0);
+      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
+      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
+      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[1][1], 0, 0, 0);
+    }
+  };
+
+  // Step k is multiplied from LDS stage k % 2; register set k % 2 carries step k from global
+  // memory to LDS.  One trip of the loop below does two steps so that the sets are fixed names.
+  // Every trip issues its loads and its LDS stores unconditionally (past the last step the
+  // loads repeat the last step's addresses and the stores fill a stage nobody reads any more):
+  // with a branch around them the compiler can no longer count which loads are outstanding at
+  // the stores and waits for all of them, the ones just issued included.
+  const int nk = (int)(A.K / kBK);
+  const int64_t k_last = (int64_t)(nk - 1) * kBK;
+  auto k_of = [&](int step) { return step < nk ? (int64_t)step * kBK : k_last; };
+  load_global(0, 0);
+  load_global(1, k_of(1));
+  store_lds(0, 0);
+  __syncthreads();
+  int kt = 0;
+  for (; kt + 1 < nk; kt += 2) {
+    // even step kt: set 0 is free (step kt sits in LDS), set 1 holds step kt+1
+    // (the scheduling barriers keep the compiler from sinking the loads below the multiplication,
+    // which would put them back to one step of lead)
+    load_global(0, k_of(kt + 2));
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(0);
+    __builtin_amdgcn_sched_barrier(0);
+    store_lds(1, 1);  // stage 1: every wavefront finished reading it one barrier ago
+    __syncthreads();
+    // odd step kt+1: set 1 is free, set 0 holds step kt+2
+    load_global(1, k_of(kt + 3));
+    __builtin_amdgcn_sched_barrier(0);
+    multiply(1);
+    __builtin_amdgcn_sched_barrier(0);
+    store_lds(0, 0);
+    __syncthreads();
+  }
+  if (kt < nk) {  // an odd number of steps: the last one sits in stage 0
+    multiply(0);
+    __syncthreads();
+  }
+  UNIRL_TRACE_MARK1();
+
+  // ---- epilogue: bf16 logits of the tile through LDS, then half a row per thread ----
+  uint16_t* out = lds;  // kBM * kOutRow bf16 (34 816 bytes), the operand stages are free now
+#pragma unroll
+  for (int bj = 0; bj < 2; ++bj) {
+    const int col = wn * 64 + bj * 32 + (lane & 31);
+    float bv = 0.0f;
+    if (HAS_BIAS) {
+      const int64_t gc = n0 + col;
+      bv = bf16_bits_to_f32(A.bias[gc < A.N ? gc : A.N - 1]);
+    }
+#pragma unroll
+    for (int bi = 0; bi < 2; ++bi) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int row = wm * 64 + bi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+        const float v = HAS_BIAS ? acc[bi][bj][i] + bv : acc[bi][bj][i];
+        out[row * kOutRow + col] = (uint16_t)f32_to_bf16_bits(v);
+      }
+    }
+  }
+  __syncthreads();
+
+  const int row = tid >> 1, half = tid & 1;
+  const int64_t grow = m0 + row;
+  const int64_t gcol0 = n0 + half * 64;
+  float x[64];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const u32x4 v = *reinterpret_cast<const u32x4*>(out + row * kOutRow + half * 64 + j * 8);
+    x[j * 8 + 0] = __uint_as_float(v.x << 16);
+    x[j * 8 + 1] = __uint_as_float(v.x & 0xffff0000u);
+    x[j * 8 + 2] = __uint_as_float(v.y << 16);
+    x[j * 8 + 3] = __uint_as_float(v.y & 0xffff0000u);
+    x[j * 8 + 4] = __uint_as_float(v.z << 16);
+    x[j * 8 + 5] = __uint_as_float(v.z & 0xffff0000u);
+    x[j * 8 + 6] = __uint_as_float(v.w << 16);
+    x[j * 8 + 7] = __uint_as_float(v.w & 0xffff0000u);
+  }
+  if (WRITE_LOGITS && grow < A.M) {
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (gcol0 + j * 8 + 8 <= A.N && (A.ld_logits % 8) == 0 && (reinterpret_cast<uintptr_t>(A.logits_out) & 15) == 0) {
+        *reinterpret_cast<u32x4*>(A.logits_out + grow * A.ld_logits + gcol0 + j * 8) =
+            *reinterpret_cast<const u32x4*>(out + row * kOutRow + half * 64 + j * 8);
+      } else {
+        for (int k = 0; k < 8; ++k)
+          if (gcol0 + j * 8 + k < A.N)
+            A.logits_out[grow * A.ld_logits + gcol0 + j * 8 + k] = out[row * kOutRow + half * 64 + j * 8 + k];
+      }
+    }
+  }
+  const int64_t n_valid = A.N - gcol0;  // columns of this half inside the vocabulary (may be <= 0)
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < 64; ++j) m = (j < n_valid) ? fmaxf(m, x[j]) : m;
+  float s = 0.0f, t = 0.0f;
+  const float c = A.c;
+#pragma unroll
+  for (int j = 0; j < 64; ++j) {
+    if (j < n_valid) {
+      const float a = (x[j] - m) * c;  // <= 0; the difference of two bf16 values is exact in fp32
+      const float e = __builtin_amdgcn_exp2f(a);
+      s += e;
+      t = fmaf(e, a, t);
+    }
+  }
+  if (grow < A.M && A.ids) {
+    const int64_t id = A.ids[grow];
+    const int64_t j = id - gcol0;
+    if (j >= 0 && j < 64 && id < A.N) {
+      float xv = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 64; ++k) xv = (k == j) ? x[k] : xv;
+      A.xid[grow] = xv;
+    }
+  }
+  // the two halves of a row sit in neighbouring lanes
+  const float m_o = __shfl_xor(m, 1, kWave), s_o = __shfl_xor(s, 1, kWave), t_o = __shfl_xor(t, 1, kWave);
+  const float mm = fmaxf(m, m_o);
+  float S = 0.0f, T = 0.0f;
+  if (m != -INFINITY) {
+    const float d = (mm - m) * c, f = __builtin_amdgcn_exp2f(-d);
+    S = f * s;
+    T = f * fmaf(-d, s, t);
+  }
+  if (m_o != -INFINITY) {
+    const float d = (mm - m_o) * c, f = __builtin_amdgcn_exp2f(-d);
+    S += f * s_o;
+    T += f * fmaf(-d, s_o, t_o);
+  }
+  if (half == 0 && grow < A.M) A.state[grow * A.n_tiles + nt] = make_float4(mm, S, T, 0.0f);
+  UNIRL_TRACE_END(A.trace);
+}
+
+struct HeadState {
+  double m, s, t;
+};
+
+// (m, s, t) of the union of two column sets; sums are relative to their own maximum
+__device__ __forceinline__ HeadState head_merge(const HeadState& p, const HeadState& q, double c) {
+  if (q.m == -INFINITY) return p;
+  if (p.m == -INFINITY) return q;
+  const double M = p.m > q.m ? p.m : q.m;
+  const double dp = (M - p.m) * c, dq = (M - q.m) * c;
+  const double fp = exp2(-dp), fq = exp2(-dq);
+  HeadState r;
+  r.m = (p.m != p.m || q.m != q.m) ? (p.m + q.m) : M;
+  r.s = fp * p.s + fq * q.s;
+  r.t = fp * (p.t - dp * p.s) + fq * (q.t - dq * q.s);
+  return r;
+}
+
+__device__ __forceinline__ double shfl_xor_f64(double v, int mask) {
+  const long long b = __double_as_longlong(v);
+  const unsigned int lo = (unsigned int)__shfl_xor((int)(unsigned int)b, mask, kWave);
+  const unsigned int hi = (unsigned int)__shfl_xor((int)(unsigned int)((unsigned long long)b >> 32), mask, kWave);
+  return __longlong_as_double((long long)(((unsigned long long)hi << 32) | lo));
+}
+
+// One wavefront per row: merge the row's tile states (index order per lane, then a butterfly)
+// and finish the three outputs.
+__global__ __launch_bounds__(kHdThreads) void lmhead_merge_kernel(HeadArgs A) {
+  const int64_t row = (int64_t)blockIdx.x * (kHdThreads / kWave) + threadIdx.x / kWave;
+  if (row >= A.M) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const double c = (double)A.c;
+  const float4* st = A.state + row * A.n_tiles;
+  HeadState acc{-(double)INFINITY, 0.0, 0.0};
+  for (int j = lane; j < A.n_tiles; j += kWave) {
+    const float4 v = st[j];
+    acc = head_merge(acc, HeadState{(double)v.x, (double)v.y, (double)v.z}, c);
+  }
+#pragma unroll
+  for (int mask = 1; mask < kWave; mask <<= 1) {
+    HeadState o{shfl_xor_f64(acc.m, mask), shfl_xor_f64(acc.s, mask), shfl_xor_f64(acc.t, mask)};
+    acc = head_merge(acc, o, c);
+  }
+  if (lane != 0) return;
+  // ln sum = ln2 * (m*c + log2 s);  H = ln s - ln2 * t / s;  logp = ln2 * (x_id - m) * c - ln s
+  const double ln_s = log(acc.s);
+  const double lse = kHdLn2 * (acc.m * c) + ln_s;
+  if (A.lse) A.lse[row] = (float)lse;
+  if (A.ent) {
+    const double h = ln_s - kHdLn2 * acc.t / acc.s;
+    A.ent[row] = (float)(h < 0.0 ? 0.0 : h);
+  }
+  if (A.logp) {
+    float out = quiet_nan();
+    const int64_t id = A.ids[row];
+    if (id >= 0 && id < A.N) out = (float)(kHdLn2 * (((double)A.xid[row] - acc.m) * c) - ln_s);
+    A.logp[row] = out;
+  }
+}
+
+}  // namespace unirl
+
+using namespace unirl;
+
+extern "C" size_t unirl_lmhead_logp_scratch_bytes(int64_t rows, int64_t V) {
+  if (rows <= 0 || V <= 0) return 0;
+  const int64_t n_tiles = (V + kBN - 1) / kBN;
+  return (size_t)rows * (size_t)n_tiles * sizeof(float4) + (size_t)rows * sizeof(float) + 256;
+}
+
+extern "C" int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
+                                 const void* bias, int64_t rows, int64_t V, int64_t K, const int64_t* ids,
+                                 float temperature, float* logp_out, float* ent_out, float* lse_out, void* logits_out,
+                                 int64_t ld_logits, void* scratch, size_t scratch_bytes, void* stream) {
+  if (rows < 0 || V <= 0 || K <= 0 || ld_hidden < K || ld_weight < K) return UNIRL_E_SHAPE;
+  if (K % kBK != 0 || ld_hidden % 8 != 0 || ld_weight % 8 != 0) return UNIRL_E_SHAPE;  // whole 64-wide K steps, 16-byte rows
+  if (logits_out && ld_logits < V) return UNIRL_E_SHAPE;
+  if (rows == 0) return UNIRL_OK;
+  if (!hidden || !weight || !scratch) return UNIRL_E_NULL;
+  if (logp_out && !ids) return UNIRL_E_NULL;
+  if (!aligned_to(hidden, 16) || !aligned_to(weight, 16) || !aligned_to(bias, 2) || !aligned_to(logits_out, 2) ||
+      !aligned_to(scratch, 16) || !aligned_to(ids, 8) || !aligned_to(logp_out, 4) || !aligned_to(ent_out, 4) ||
+      !aligned_to(lse_out, 4))
+    return UNIRL_E_ALIGN;
+  if (scratch_bytes < unirl_lmhead_logp_scratch_bytes(rows, V)) return UNIRL_E_WORKSPACE;
+  const int64_t n_tiles = (V + kBN - 1) / kBN, m_blocks = (rows + kBM - 1) / kBM;
+  if (n_tiles > 0x7fffffff || m_blocks > 0x7fffffff) return UNIRL_E_LIMIT;
+  const long long total = (long long)n_tiles * m_blocks;
+  const long long per_xcd = (total + kXcds - 1) / kXcds;
+  if (per_xcd * kXcds > 0x7fffffffLL) return UNIRL_E_LIMIT;
+  HeadArgs A = {};
+  A.h = reinterpret_cast<const uint16_t*>(hidden);
+  A.w = reinterpret_cast<const uint16_t*>(weight);
+  A.bias = reinterpret_cast<const uint16_t*>(bias);
+  A.ids = ids;
+  A.M = rows;
+  A.N = V;
+  A.K = K;
+  A.ldh = ld_hidden;
+  A.ldw = ld_weight;
+  const float T = temperature > 0.0f ? temperature : 1.0f;
+  A.c = (float)(1.4426950408889634 / (double)T);
+  A.state = reinterpret_cast<float4*>(scratch);
+  A.xid = reinterpret_cast<float*>(reinterpret_cast<char*>(scratch) + (size_t)rows * (size_t)n_tiles * sizeof(float4));
+  A.logits_out = reinterpret_cast<uint16_t*>(logits_out);
+  A.ld_logits = ld_logits;
+  A.n_tiles = (int)n_tiles;
+  A.m_blocks = (int)m_blocks;
+  A.group = (int)tune_int("UNIRL_HEAD_GROUP", 8);
+  A.logp = logp_out;
+  A.ent = ent_out;
+  A.lse = lse_out;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned int)(per_xcd * kXcds)), block(kHdThreads);
+  UNIRL_TRACE_SET(A, "lmhead_tile", grid.x);
+  if (bias) {
+    if (logits_out)
+      hipLaunchKernelGGL((lmhead_tile_kernel<true, true>), grid, block, 0, st, A);
+    else
+      hipLaunchKernelGGL((lmhead_tile_kernel<true, false>), grid, block, 0, st, A);
+  } else {
+    if (logits_out)
+      hipLaunchKernelGGL((lmhead_tile_kernel<false, true>), grid, block, 0, st, A);
+    else
+      hipLaunchKernelGGL((lmhead_tile_kernel<false, false>), grid, block, 0, st, A);
+  }
+  int rc = (int)hipGetLastError();
+  if (rc != 0) return rc;
+  const int per_block = kHdThreads / kWave;
+  hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned int)((rows + per_block - 1) / per_block)), block, 0, st, A);
+  return (int)hipGetLastError();
+}

@@ -88,14 +88,19 @@ class _RecomputedChunkFn(torch.autograd.Function):
     """
 
     @staticmethod
-    def forward(ctx, hidden: torch.Tensor, tokens: torch.Tensor, lm_head, temperature: float, *params):
+    def forward(ctx, hidden: torch.Tensor, tokens: torch.Tensor, lm_head, temperature: float, fused_head: bool, *params):
         del params  # listed only so autograd sees the head's parameters as inputs of this node
         ctx.autocast = (torch.is_autocast_enabled("cuda"), torch.get_autocast_dtype("cuda"))
         with torch.no_grad():
-            logits = lm_head(hidden)
-            logp, _, lse = ops.token_logp_entropy(
-                logits, tokens, temperature, want_logp=True, want_entropy=False, want_lse=True
-            )
+            if fused_head:
+                # the head's GEMM with the log-softmax statistics in its epilogue: no logits at all
+                logp, _, lse, _ = ops.lmhead_logp(hidden, lm_head.weight, lm_head.bias, tokens, temperature,
+                                                  want_lse=True)
+            else:
+                logits = lm_head(hidden)
+                logp, _, lse = ops.token_logp_entropy(
+                    logits, tokens, temperature, want_logp=True, want_entropy=False, want_lse=True
+                )
         ctx.save_for_backward(hidden, tokens, lse)
         ctx.lm_head, ctx.temperature = lm_head, temperature
         return logp
@@ -113,8 +118,8 @@ class _RecomputedChunkFn(torch.autograd.Function):
         )
         # parameter gradients accumulate into .grad here, as under a re-entrant checkpoint
         torch.autograd.backward(logits, d_logits)
-        n_params = len(ctx.needs_input_grad) - 4
-        return (h.grad, None, None, None) + (None,) * n_params
+        n_params = len(ctx.needs_input_grad) - 5
+        return (h.grad, None, None, None, None) + (None,) * n_params
 
 
 _KERNEL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
@@ -165,6 +170,7 @@ def chunked_replay_logp(
     temperature: float = 1.0,
     chunk: Optional[int] = None,
     keep_logits: Optional[bool] = None,
+    fused_head: bool = False,
 ) -> torch.Tensor:
     """Padded ``[B, T_max]`` fp32 log-probs of ``response_tokens`` under ``lm_head(resp_hidden)``.
 
@@ -185,6 +191,14 @@ def chunked_replay_logp(
     of ``8192 // B`` rows.  The recomputing path is taken when ``resp_hidden`` or a parameter of
     an ``nn.Module`` head requires grad; a bare callable whose captured weights alone require
     grad keeps its logits.
+
+    ``fused_head=True`` (a plain bf16 ``nn.Linear`` head, bf16 hidden states, hidden size a
+    multiple of 64, outside autocast) computes the forward with ``unirl_lmhead_logp``: the head's
+    GEMM with the log-softmax statistics reduced in its epilogue, so no logits exist in the
+    forward at all (the backward rebuilds each chunk's logits with ``lm_head`` as above).  It
+    trades time for memory -- the hand-written GEMM runs at about 0.6 of the library's speed --
+    and is off by default.  Its bf16 logits differ from the library GEMM's in about 0.02 % of the
+    entries by one bf16 ulp (a different fp32 summation order), as two library versions would.
     """
     bsz, t_max = int(resp_hidden.size(0)), int(response_tokens.size(1))
     if t_max == 0:
@@ -194,6 +208,14 @@ def chunked_replay_logp(
             _is_plain_linear(lm_head)
             and bsz * t_max * lm_head.out_features * lm_head.weight.element_size() <= KEEP_LOGITS_BYTES
         )
+    if fused_head:
+        if not (_is_plain_linear(lm_head) and ops.lmhead_logp_supported(resp_hidden, lm_head.weight, lm_head.bias)
+                and not torch.is_autocast_enabled("cuda")):
+            raise ValueError(
+                "fused_head needs a plain bf16 nn.Linear head, bf16 hidden states on the same HIP device, a hidden "
+                "size that is a multiple of 64, and no autocast"
+            )
+        keep_logits = False
     rows_per_chunk = 8192 if keep_logits else 4096
     step = int(chunk) if chunk is not None else max(64, rows_per_chunk // max(1, bsz))
     T = float(temperature) if float(temperature) > 0.0 else 1.0
@@ -206,7 +228,9 @@ def chunked_replay_logp(
     for s in range(0, t_max, step):
         h, tok = resp_hidden[:, s : s + step, :], response_tokens[:, s : s + step]
         if recompute:
-            parts.append(_RecomputedChunkFn.apply(h, tok, lm_head, T, *params))
+            parts.append(_RecomputedChunkFn.apply(h, tok, lm_head, T, fused_head, *params))
+        elif fused_head:
+            parts.append(ops.lmhead_logp(h, lm_head.weight, lm_head.bias, tok, T)[0])
         else:
             logits = lm_head(h)
             if _is_plain_linear(lm_head) and torch.is_grad_enabled() and logits.requires_grad:

@@ -882,6 +882,74 @@ def token_logp_entropy(
     return logp, ent, lse
 
 
+def lmhead_logp_supported(hidden: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> bool:
+    """Whether :func:`lmhead_logp` takes these operands as they are: bf16 on one HIP device, the
+    hidden size a multiple of 64, rows contiguous and 16-byte aligned."""
+    if not (hidden.is_cuda and weight.is_cuda and hidden.device == weight.device):
+        return False
+    if hidden.dtype is not torch.bfloat16 or weight.dtype is not torch.bfloat16 or weight.dim() != 2:
+        return False
+    K = weight.shape[1]
+    if hidden.dim() < 1 or hidden.shape[-1] != K or K % 64 != 0 or weight.stride(1) != 1 or weight.stride(0) % 8 != 0:
+        return False
+    if bias is not None and (bias.dtype is not torch.bfloat16 or bias.numel() != weight.shape[0] or not bias.is_cuda):
+        return False
+    return weight.data_ptr() % 16 == 0
+
+
+def lmhead_logp(
+    hidden: torch.Tensor,
+    weight: torch.Tensor,
+    bias: Optional[torch.Tensor],
+    ids: Optional[torch.Tensor],
+    temperature: float = 1.0,
+    *,
+    want_logp: bool = True,
+    want_entropy: bool = False,
+    want_lse: bool = False,
+    want_logits: bool = False,
+) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """``(logp, entropy, logsumexp, logits)`` of ``F.linear(hidden, weight, bias)`` per row, without
+    writing the logits (``want_logits`` writes them as well, for validation).  bf16 ``hidden [..., K]``
+    and ``weight [V, K]``; the statistics are fp32 ``[...]``."""
+    if not lmhead_logp_supported(hidden, weight, bias):
+        raise ValueError(
+            "lmhead_logp needs bf16 hidden states [..., K] and a bf16 weight [V, K] on one HIP device, K a multiple "
+            f"of 64, 16-byte aligned rows; got {hidden.dtype} {tuple(hidden.shape)} and {weight.dtype} {tuple(weight.shape)}"
+        )
+    device = hidden.device
+    V, K = int(weight.shape[0]), int(weight.shape[1])
+    lead = tuple(hidden.shape[:-1])
+    h2 = hidden.detach().reshape(-1, K)
+    if h2.shape[0] and (h2.stride(1) != 1 or h2.stride(0) % 8 != 0 or h2.data_ptr() % 16 != 0):
+        h2 = h2.contiguous()
+    rows = int(h2.shape[0])
+    idc = None
+    if want_logp:
+        if ids is None:
+            raise ValueError("ids is required for the log-prob")
+        if tuple(ids.shape) != lead:
+            raise ValueError(f"ids {tuple(ids.shape)} does not match the hidden-state rows {lead}")
+        idc = N.as_operand(ids, torch.int64, device).reshape(-1)
+    logp = torch.empty(lead, dtype=torch.float32, device=device) if want_logp else None
+    ent = torch.empty(lead, dtype=torch.float32, device=device) if want_entropy else None
+    lse = torch.empty(lead, dtype=torch.float32, device=device) if want_lse else None
+    logits = torch.empty(lead + (V,), dtype=torch.bfloat16, device=device) if want_logits else None
+    if rows == 0:
+        return logp, ent, lse, logits
+    nbytes = int(N.F.unirl_lmhead_logp_scratch_bytes(rows, V))
+    scratch = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    b = None if bias is None else bias.detach().contiguous()
+    with N.on_device(device):
+        rc = N.F.unirl_lmhead_logp(
+            h2.data_ptr(), h2.stride(0) if rows > 1 else K, weight.data_ptr(), weight.stride(0), N.ptr(b), rows, V, K,
+            N.ptr(idc), float(temperature), N.ptr(logp), N.ptr(ent), N.ptr(lse), N.ptr(logits), V, scratch.data_ptr(),
+            nbytes, N.current_stream(device),
+        )
+    N.check(rc, "unirl_lmhead_logp")
+    return logp, ent, lse, logits
+
+
 def _row_blocks(x: torch.Tensor, V: int):
     """``x [..., V]`` as a sequence of 2-D ``[rows, V]`` views, in row-major order of the leading
     dimensions, each with unit element stride and one row stride >= V.  A tensor that is one such
