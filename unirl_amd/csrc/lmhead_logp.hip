@@ -7,15 +7,17 @@
 // for a bf16 head W [V, K] (nn.Linear's layout, K contiguous) and bf16 hidden states H [rows, K]
 // (K contiguous): both operands are read along K, the layout MFMA fragments want.
 //
-// Kernel 1 (lmhead_tile_kernel): one workgroup of four wavefronts per 128 x 128 tile of the
-// logits.  K is walked in steps of 64 through two LDS stages (global -> registers -> LDS, the next
-// step's loads in flight while the current one is multiplied); each wavefront owns a 64 x 64
-// quarter as 2 x 2 blocks of v_mfma_f32_32x32x16_bf16.  Epilogue: accumulators (+ bias) are
-// rounded to bf16 -- the values the reference's logits hold -- and passed through LDS so that
-// every thread owns half a row of the tile; it reduces its 64 logits to (m, s, t): the maximum,
-// sum 2^a and sum 2^a * a with a = (x - m) * log2(e)/T.  One (m, s, t) per (row, column tile)
-// goes to scratch memory (16 bytes for 256 bytes of logits) and the tile that holds a row's
-// target column also stores that logit.
+// Kernel 1 (lmhead_tile_kernel): one workgroup of four wavefronts (2 x 2) per tile of the logits,
+// 256 x 256 once a call has 1024 rows (one workgroup per compute unit, accumulators in AGPRs), 128
+// x 128 below (two per compute unit).  K is walked in steps of 64 through two LDS stages (global
+// -> registers -> LDS, later steps' loads in flight while the current one is multiplied); each
+// wavefront owns a quarter of the tile as blocks of v_mfma_f32_32x32x16_bf16.  Epilogue:
+// accumulators (+ bias) are rounded to bf16 -- the values the reference's logits hold -- and
+// passed through LDS so that every thread owns a row of the tile (half a row at 128 x 128); it
+// reduces its logits, 64 at a time, to (m, s, t): the maximum, sum 2^a and sum 2^a * a with
+// a = (x - m) * log2(e)/T.  One (m, s, t) per (row, column tile) goes to scratch memory (16 bytes
+// for 256 or 512 bytes of logits) and the tile that holds a row's target column also stores that
+// logit.
 // Kernel 2 (lmhead_merge_kernel): one wavefront per row merges the row's tile states in fp64 and
 // finishes logsumexp, log-prob and entropy.
 //
@@ -32,12 +34,10 @@ typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kHdThreads = 256;
-constexpr int kBM = 128, kBN = 128, kBK = 64;
+constexpr int kBK = 64;
 // LDS rows are padded by 16 bytes: the 16-byte fragment reads of 16 consecutive rows then
 // cover all 64 banks exactly once
-constexpr int kLdsRow = kBK + 8;             // bf16 elements per operand row
-constexpr int kOperandElems = kBM * kLdsRow;  // one operand, one stage
-constexpr int kOutRow = kBN + 8;              // bf16 elements per row of the epilogue tile
+constexpr int kLdsRow = kBK + 8;  // bf16 elements per operand row
 constexpr int kXcds = 8;
 constexpr double kHdLn2 = 0.6931471805599453;
 
@@ -83,111 +83,129 @@ __device__ __forceinline__ bf16x8_t lds_frag(const uint16_t* p) {
   return *reinterpret_cast<const bf16x8_t*>(p);
 }
 
-template <bool HAS_BIAS, bool WRITE_LOGITS>
-__global__ __launch_bounds__(kHdThreads, 2) void lmhead_tile_kernel(HeadArgs A) {
-  __shared__ __attribute__((aligned(16))) uint16_t lds[2 * 2 * kOperandElems];  // [stage][A | B][row][kLdsRow]
+// BM x BN: the workgroup's tile of the logits; its four wavefronts sit 2 x 2, each on a
+// (BM/2) x (BN/2) quarter of BI x BJ MFMA blocks.  SETS: register sets staging the global loads
+// (2 = loads run two K steps ahead of the multiplication, 1 = one step).
+template <int BM, int BN, int SETS, bool HAS_BIAS, bool WRITE_LOGITS>
+__global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmhead_tile_kernel(HeadArgs A) {
+  constexpr int WM = BM / 2, WN = BN / 2, BI = WM / 32, BJ = WN / 32;
+  constexpr int kAElems = BM * kLdsRow, kBElems = BN * kLdsRow, kStage = kAElems + kBElems;
+  constexpr int CA = BM * 8 / kHdThreads, CB = BN * 8 / kHdThreads;  // 16-byte chunks per thread and step
+  constexpr int kOutRow = BN + 8;  // bf16 elements per row of the epilogue tile
+  static_assert(BM * kOutRow <= 2 * kStage, "the epilogue tile reuses the operand stages");
+  __shared__ __attribute__((aligned(16))) uint16_t lds[2 * kStage];  // [stage][A rows | B rows][kLdsRow]
   UNIRL_TRACE_T0();
   int mb, nt;
   head_tile_of(A, blockIdx.x, mb, nt);
   if (mb < 0) return;  // the padding of the last XCD's range (whole workgroup)
-  const int64_t m0 = (int64_t)mb * kBM, n0 = (int64_t)nt * kBN;
+  const int64_t m0 = (int64_t)mb * BM, n0 = (int64_t)nt * BN;
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int wm = wave >> 1, wn = wave & 1;
 
   // global -> LDS assignment: 16-byte chunk c = tid + 256*i covers row c/8, k-chunk c%8 of a tile
-  const uint16_t* pa[4];
-  const uint16_t* pb[4];
-  int lds_off[4];
+  const int kc = tid & 7, row0 = tid >> 3;
+  const uint16_t* pa[CA];
+  const uint16_t* pb[CB];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int c = tid + kHdThreads * i;
-    const int row = c >> 3, kc = c & 7;
-    int64_t ra = m0 + row, rb = n0 + row;
-    ra = ra < A.M ? ra : A.M - 1;  // rows past the end repeat the last one; their results are dropped
-    rb = rb < A.N ? rb : A.N - 1;
-    pa[i] = A.h + ra * A.ldh + kc * 8;
-    pb[i] = A.w + rb * A.ldw + kc * 8;
-    lds_off[i] = row * kLdsRow + kc * 8;
+  for (int i = 0; i < CA; ++i) {
+    int64_t r = m0 + row0 + 32 * i;
+    r = r < A.M ? r : A.M - 1;  // rows past the end repeat the last one; their results are dropped
+    pa[i] = A.h + r * A.ldh + kc * 8;
   }
-  // Two register sets stage the global loads two K steps ahead of the multiplication: a trip to
-  // L2 takes longer than one step's sixteen MFMAs, so the loads of step k+2 are issued before
-  // step k is multiplied and land in LDS one step later.
-  u32x4 ga[2][4], gb[2][4];
+#pragma unroll
+  for (int i = 0; i < CB; ++i) {
+    int64_t r = n0 + row0 + 32 * i;
+    r = r < A.N ? r : A.N - 1;
+    pb[i] = A.w + r * A.ldw + kc * 8;
+  }
+  const int lds_off0 = row0 * kLdsRow + kc * 8;  // chunk i sits 32 rows further down
+  u32x4 ga[SETS][CA], gb[SETS][CB];
   auto load_global = [&](int set, int64_t k0) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      ga[set][i] = *reinterpret_cast<const u32x4*>(pa[i] + k0);
-      gb[set][i] = *reinterpret_cast<const u32x4*>(pb[i] + k0);
-    }
+    for (int i = 0; i < CA; ++i) ga[set][i] = *reinterpret_cast<const u32x4*>(pa[i] + k0);
+#pragma unroll
+    for (int i = 0; i < CB; ++i) gb[set][i] = *reinterpret_cast<const u32x4*>(pb[i] + k0);
   };
   auto store_lds = [&](int set, int stage) {
-    uint16_t* sa = lds + stage * 2 * kOperandElems;
-    uint16_t* sb = sa + kOperandElems;
+    uint16_t* sa = lds + stage * kStage;
+    uint16_t* sb = sa + kAElems;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      *reinterpret_cast<u32x4*>(sa + lds_off[i]) = ga[set][i];
-      *reinterpret_cast<u32x4*>(sb + lds_off[i]) = gb[set][i];
-    }
+    for (int i = 0; i < CA; ++i) *reinterpret_cast<u32x4*>(sa + lds_off0 + i * 32 * kLdsRow) = ga[set][i];
+#pragma unroll
+    for (int i = 0; i < CB; ++i) *reinterpret_cast<u32x4*>(sb + lds_off0 + i * 32 * kLdsRow) = gb[set][i];
   };
 
-  f32x16_t acc[2][2];
+  f32x16_t acc[BI][BJ];
 #pragma unroll
-  for (int bi = 0; bi < 2; ++bi)
+  for (int bi = 0; bi < BI; ++bi)
 #pragma unroll
-    for (int bj = 0; bj < 2; ++bj)
+    for (int bj = 0; bj < BJ; ++bj)
 #pragma unroll
       for (int i = 0; i < 16; ++i) acc[bi][bj][i] = 0.0f;
 
   // fragment addresses inside a stage: lane l reads row (l % 32) of a 32-row block, k = 8 * (l / 32) ..
-  const int frag_a = (wm * 64 + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
-  const int frag_b = (wn * 64 + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
+  const int frag_a = (wm * WM + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
+  const int frag_b = (wn * WN + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
   auto multiply = [&](int stage) {
-    const uint16_t* sa = lds + stage * 2 * kOperandElems;
-    const uint16_t* sb = sa + kOperandElems;
+    const uint16_t* sa = lds + stage * kStage;
+    const uint16_t* sb = sa + kAElems;
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
-      const bf16x8_t a0 = lds_frag(sa + frag_a + ks * 16);
-      const bf16x8_t a1 = lds_frag(sa + frag_a + 32 * kLdsRow + ks * 16);
-      const bf16x8_t b0 = lds_frag(sb + frag_b + ks * 16);
-      const bf16x8_t b1 = lds_frag(sb + frag_b + 32 * kLdsRow + ks * 16);
-      acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc[0][0], 0, 0, 0);
-      acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b1, acc[0][1], 0, 0, 0);
-      acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b0, acc[1][0], 0, 0, 0);
-      acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc[1][1], 0, 0, 0);
+      bf16x8_t a[BI], b[BJ];
+#pragma unroll
+      for (int bi = 0; bi < BI; ++bi) a[bi] = lds_frag(sa + frag_a + bi * 32 * kLdsRow + ks * 16);
+#pragma unroll
+      for (int bj = 0; bj < BJ; ++bj) b[bj] = lds_frag(sb + frag_b + bj * 32 * kLdsRow + ks * 16);
+#pragma unroll
+      for (int bi = 0; bi < BI; ++bi)
+#pragma unroll
+        for (int bj = 0; bj < BJ; ++bj)
+          acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[bi], b[bj], acc[bi][bj], 0, 0, 0);
     }
   };
 
-  // Step k is multiplied from LDS stage k % 2; register set k % 2 carries step k from global
-  // memory to LDS.  One trip of the loop below does two steps so that the sets are fixed names.
-  // Every trip issues its loads and its LDS stores unconditionally (past the last step the
-  // loads repeat the last step's addresses and the stores fill a stage nobody reads any more):
-  // with a branch around them the compiler can no longer count which loads are outstanding at
-  // the stores and waits for all of them, the ones just issued included.
+  // Step k is multiplied from LDS stage k % 2.  Every trip issues its loads and its LDS stores
+  // unconditionally (past the last step the loads repeat the last step's addresses and the
+  // stores fill a stage nobody reads any more): with a branch around them the compiler can no
+  // longer count which loads are outstanding at the stores and waits for all of them.  The
+  // scheduling barriers keep it from sinking the loads below the multiplication.
   const int nk = (int)(A.K / kBK);
   const int64_t k_last = (int64_t)(nk - 1) * kBK;
   auto k_of = [&](int step) { return step < nk ? (int64_t)step * kBK : k_last; };
   load_global(0, 0);
-  load_global(1, k_of(1));
+  if (SETS == 2) load_global(SETS - 1, k_of(1));
   store_lds(0, 0);
   __syncthreads();
   int kt = 0;
   for (; kt + 1 < nk; kt += 2) {
-    // even step kt: set 0 is free (step kt sits in LDS), set 1 holds step kt+1
-    // (the scheduling barriers keep the compiler from sinking the loads below the multiplication,
-    // which would put them back to one step of lead)
-    load_global(0, k_of(kt + 2));
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(0);
-    __builtin_amdgcn_sched_barrier(0);
-    store_lds(1, 1);  // stage 1: every wavefront finished reading it one barrier ago
-    __syncthreads();
-    // odd step kt+1: set 1 is free, set 0 holds step kt+2
-    load_global(1, k_of(kt + 3));
-    __builtin_amdgcn_sched_barrier(0);
-    multiply(1);
-    __builtin_amdgcn_sched_barrier(0);
-    store_lds(0, 0);
-    __syncthreads();
+    if (SETS == 2) {
+      // register set k % 2 carries step k; even step kt: set 0 is free, set 1 holds step kt+1
+      load_global(0, k_of(kt + 2));
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(0);
+      __builtin_amdgcn_sched_barrier(0);
+      store_lds(SETS - 1, 1);  // stage 1: every wavefront finished reading it one barrier ago
+      __syncthreads();
+      load_global(SETS - 1, k_of(kt + 3));
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(1);
+      __builtin_amdgcn_sched_barrier(0);
+      store_lds(0, 0);
+      __syncthreads();
+    } else {
+      load_global(0, k_of(kt + 1));
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(0);
+      __builtin_amdgcn_sched_barrier(0);
+      store_lds(0, 1);
+      __syncthreads();
+      load_global(0, k_of(kt + 2));
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(1);
+      __builtin_amdgcn_sched_barrier(0);
+      store_lds(0, 0);
+      __syncthreads();
+    }
   }
   if (kt < nk) {  // an odd number of steps: the last one sits in stage 0
     multiply(0);
@@ -195,21 +213,21 @@ __global__ __launch_bounds__(kHdThreads, 2) void lmhead_tile_kernel(HeadArgs A) 
   }
   UNIRL_TRACE_MARK1();
 
-  // ---- epilogue: bf16 logits of the tile through LDS, then half a row per thread ----
-  uint16_t* out = lds;  // kBM * kOutRow bf16 (34 816 bytes), the operand stages are free now
+  // ---- epilogue: bf16 logits of the tile through LDS, then a row (or half a row) per thread ----
+  uint16_t* out = lds;  // BM * kOutRow bf16; the operand stages are free now
 #pragma unroll
-  for (int bj = 0; bj < 2; ++bj) {
-    const int col = wn * 64 + bj * 32 + (lane & 31);
+  for (int bj = 0; bj < BJ; ++bj) {
+    const int col = wn * WN + bj * 32 + (lane & 31);
     float bv = 0.0f;
     if (HAS_BIAS) {
       const int64_t gc = n0 + col;
       bv = bf16_bits_to_f32(A.bias[gc < A.N ? gc : A.N - 1]);
     }
 #pragma unroll
-    for (int bi = 0; bi < 2; ++bi) {
+    for (int bi = 0; bi < BI; ++bi) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const int row = wm * 64 + bi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+        const int row = wm * WM + bi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
         const float v = HAS_BIAS ? acc[bi][bj][i] + bv : acc[bi][bj][i];
         out[row * kOutRow + col] = (uint16_t)f32_to_bf16_bits(v);
       }
@@ -217,75 +235,94 @@ __global__ __launch_bounds__(kHdThreads, 2) void lmhead_tile_kernel(HeadArgs A) 
   }
   __syncthreads();
 
-  const int row = tid >> 1, half = tid & 1;
+  constexpr int PARTS = kHdThreads / BM;  // threads that share a row of the tile (2 or 1)
+  constexpr int COLS = BN / PARTS;        // columns each of them reduces, 64 at a time
+  const int row = tid / PARTS, part = tid % PARTS;
   const int64_t grow = m0 + row;
-  const int64_t gcol0 = n0 + half * 64;
-  float x[64];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    const u32x4 v = *reinterpret_cast<const u32x4*>(out + row * kOutRow + half * 64 + j * 8);
-    x[j * 8 + 0] = __uint_as_float(v.x << 16);
-    x[j * 8 + 1] = __uint_as_float(v.x & 0xffff0000u);
-    x[j * 8 + 2] = __uint_as_float(v.y << 16);
-    x[j * 8 + 3] = __uint_as_float(v.y & 0xffff0000u);
-    x[j * 8 + 4] = __uint_as_float(v.z << 16);
-    x[j * 8 + 5] = __uint_as_float(v.z & 0xffff0000u);
-    x[j * 8 + 6] = __uint_as_float(v.w << 16);
-    x[j * 8 + 7] = __uint_as_float(v.w & 0xffff0000u);
-  }
-  if (WRITE_LOGITS && grow < A.M) {
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      if (gcol0 + j * 8 + 8 <= A.N && (A.ld_logits % 8) == 0 && (reinterpret_cast<uintptr_t>(A.logits_out) & 15) == 0) {
-        *reinterpret_cast<u32x4*>(A.logits_out + grow * A.ld_logits + gcol0 + j * 8) =
-            *reinterpret_cast<const u32x4*>(out + row * kOutRow + half * 64 + j * 8);
-      } else {
-        for (int k = 0; k < 8; ++k)
-          if (gcol0 + j * 8 + k < A.N)
-            A.logits_out[grow * A.ld_logits + gcol0 + j * 8 + k] = out[row * kOutRow + half * 64 + j * 8 + k];
-      }
-    }
-  }
-  const int64_t n_valid = A.N - gcol0;  // columns of this half inside the vocabulary (may be <= 0)
-  float m = -INFINITY;
-#pragma unroll
-  for (int j = 0; j < 64; ++j) m = (j < n_valid) ? fmaxf(m, x[j]) : m;
-  float s = 0.0f, t = 0.0f;
   const float c = A.c;
-#pragma unroll
-  for (int j = 0; j < 64; ++j) {
-    if (j < n_valid) {
-      const float a = (x[j] - m) * c;  // <= 0; the difference of two bf16 values is exact in fp32
-      const float e = __builtin_amdgcn_exp2f(a);
-      s += e;
-      t = fmaf(e, a, t);
-    }
-  }
+  int64_t id_col = -1;  // the target's column relative to this thread's first one
   if (grow < A.M && A.ids) {
     const int64_t id = A.ids[grow];
-    const int64_t j = id - gcol0;
-    if (j >= 0 && j < 64 && id < A.N) {
+    if (id >= 0 && id < A.N) id_col = id - (n0 + part * COLS);
+  }
+  float m = -INFINITY, s = 0.0f, t = 0.0f;
+  for (int p0 = 0; p0 < COLS; p0 += 64) {
+    const uint16_t* src = out + row * kOutRow + part * COLS + p0;
+    const int64_t gcol0 = n0 + part * COLS + p0;
+    float x[64];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const u32x4 v = *reinterpret_cast<const u32x4*>(src + j * 8);
+      x[j * 8 + 0] = __uint_as_float(v.x << 16);
+      x[j * 8 + 1] = __uint_as_float(v.x & 0xffff0000u);
+      x[j * 8 + 2] = __uint_as_float(v.y << 16);
+      x[j * 8 + 3] = __uint_as_float(v.y & 0xffff0000u);
+      x[j * 8 + 4] = __uint_as_float(v.z << 16);
+      x[j * 8 + 5] = __uint_as_float(v.z & 0xffff0000u);
+      x[j * 8 + 6] = __uint_as_float(v.w << 16);
+      x[j * 8 + 7] = __uint_as_float(v.w & 0xffff0000u);
+    }
+    if (WRITE_LOGITS && grow < A.M) {
+      const bool vec_ok = (A.ld_logits % 8) == 0 && (reinterpret_cast<uintptr_t>(A.logits_out) & 15) == 0;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (vec_ok && gcol0 + j * 8 + 8 <= A.N) {
+          *reinterpret_cast<u32x4*>(A.logits_out + grow * A.ld_logits + gcol0 + j * 8) =
+              *reinterpret_cast<const u32x4*>(src + j * 8);
+        } else {
+          for (int k = 0; k < 8; ++k)
+            if (gcol0 + j * 8 + k < A.N) A.logits_out[grow * A.ld_logits + gcol0 + j * 8 + k] = src[j * 8 + k];
+        }
+      }
+    }
+    const int64_t n_valid = A.N - gcol0;  // columns of this piece inside the vocabulary (may be <= 0)
+    float pm = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 64; ++j) pm = (j < n_valid) ? fmaxf(pm, x[j]) : pm;
+    if (pm > m) {  // raise the reference of what has been summed so far
+      if (m != -INFINITY) {
+        const float d = (pm - m) * c, f = __builtin_amdgcn_exp2f(-d);
+        t = f * fmaf(-d, s, t);
+        s = f * s;
+      }
+      m = pm;
+    }
+#pragma unroll
+    for (int j = 0; j < 64; ++j) {
+      if (j < n_valid) {
+        const float a = (x[j] - m) * c;  // <= 0; the difference of two bf16 values is exact in fp32
+        const float e = __builtin_amdgcn_exp2f(a);
+        s += e;
+        t = fmaf(e, a, t);
+      }
+    }
+    const int64_t j_id = id_col - p0;
+    if (j_id >= 0 && j_id < 64) {
       float xv = 0.0f;
 #pragma unroll
-      for (int k = 0; k < 64; ++k) xv = (k == j) ? x[k] : xv;
+      for (int k = 0; k < 64; ++k) xv = (k == j_id) ? x[k] : xv;
       A.xid[grow] = xv;
     }
   }
-  // the two halves of a row sit in neighbouring lanes
-  const float m_o = __shfl_xor(m, 1, kWave), s_o = __shfl_xor(s, 1, kWave), t_o = __shfl_xor(t, 1, kWave);
-  const float mm = fmaxf(m, m_o);
-  float S = 0.0f, T = 0.0f;
-  if (m != -INFINITY) {
-    const float d = (mm - m) * c, f = __builtin_amdgcn_exp2f(-d);
-    S = f * s;
-    T = f * fmaf(-d, s, t);
+  if (PARTS == 2) {  // the two halves of a row sit in neighbouring lanes
+    const float m_o = __shfl_xor(m, 1, kWave), s_o = __shfl_xor(s, 1, kWave), t_o = __shfl_xor(t, 1, kWave);
+    const float mm = fmaxf(m, m_o);
+    float S = 0.0f, T = 0.0f;
+    if (m != -INFINITY) {
+      const float d = (mm - m) * c, f = __builtin_amdgcn_exp2f(-d);
+      S = f * s;
+      T = f * fmaf(-d, s, t);
+    }
+    if (m_o != -INFINITY) {
+      const float d = (mm - m_o) * c, f = __builtin_amdgcn_exp2f(-d);
+      S += f * s_o;
+      T += f * fmaf(-d, s_o, t_o);
+    }
+    m = mm;
+    s = S;
+    t = T;
   }
-  if (m_o != -INFINITY) {
-    const float d = (mm - m_o) * c, f = __builtin_amdgcn_exp2f(-d);
-    S += f * s_o;
-    T += f * fmaf(-d, s_o, t_o);
-  }
-  if (half == 0 && grow < A.M) A.state[grow * A.n_tiles + nt] = make_float4(mm, S, T, 0.0f);
+  if (part == 0 && grow < A.M) A.state[grow * A.n_tiles + nt] = make_float4(m, s, t, 0.0f);
   UNIRL_TRACE_END(A.trace);
 }
 
@@ -353,10 +390,31 @@ __global__ __launch_bounds__(kHdThreads) void lmhead_merge_kernel(HeadArgs A) {
 
 using namespace unirl;
 
+// Tile edge of a call: 256 x 256 tiles (one workgroup per compute unit, the fewest LDS reads per
+// MFMA) once there are enough rows to fill them, 128 x 128 below.
+static int head_tile_edge(int64_t rows) { return rows >= (int64_t)tune_int("UNIRL_HEAD_BIG_ROWS", 1024) ? 256 : 128; }
+
 extern "C" size_t unirl_lmhead_logp_scratch_bytes(int64_t rows, int64_t V) {
   if (rows <= 0 || V <= 0) return 0;
-  const int64_t n_tiles = (V + kBN - 1) / kBN;
+  const int64_t n_tiles = (V + 127) / 128;  // the finer of the two tilings
   return (size_t)rows * (size_t)n_tiles * sizeof(float4) + (size_t)rows * sizeof(float) + 256;
+}
+
+template <int EDGE, int SETS>
+static int launch_head_tiles(const HeadArgs& A, dim3 grid, hipStream_t st) {
+  dim3 block(kHdThreads);
+  if (A.bias) {
+    if (A.logits_out)
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, SETS, true, true>), grid, block, 0, st, A);
+    else
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, SETS, true, false>), grid, block, 0, st, A);
+  } else {
+    if (A.logits_out)
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, SETS, false, true>), grid, block, 0, st, A);
+    else
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, SETS, false, false>), grid, block, 0, st, A);
+  }
+  return (int)hipGetLastError();
 }
 
 extern "C" int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
@@ -374,7 +432,8 @@ extern "C" int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const vo
       !aligned_to(lse_out, 4))
     return UNIRL_E_ALIGN;
   if (scratch_bytes < unirl_lmhead_logp_scratch_bytes(rows, V)) return UNIRL_E_WORKSPACE;
-  const int64_t n_tiles = (V + kBN - 1) / kBN, m_blocks = (rows + kBM - 1) / kBM;
+  const int edge = head_tile_edge(rows);
+  const int64_t n_tiles = (V + edge - 1) / edge, m_blocks = (rows + edge - 1) / edge;
   if (n_tiles > 0x7fffffff || m_blocks > 0x7fffffff) return UNIRL_E_LIMIT;
   const long long total = (long long)n_tiles * m_blocks;
   const long long per_xcd = (total + kXcds - 1) / kXcds;
@@ -402,22 +461,12 @@ extern "C" int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const vo
   A.ent = ent_out;
   A.lse = lse_out;
   hipStream_t st = (hipStream_t)stream;
-  dim3 grid((unsigned int)(per_xcd * kXcds)), block(kHdThreads);
+  dim3 grid((unsigned int)(per_xcd * kXcds));
   UNIRL_TRACE_SET(A, "lmhead_tile", grid.x);
-  if (bias) {
-    if (logits_out)
-      hipLaunchKernelGGL((lmhead_tile_kernel<true, true>), grid, block, 0, st, A);
-    else
-      hipLaunchKernelGGL((lmhead_tile_kernel<true, false>), grid, block, 0, st, A);
-  } else {
-    if (logits_out)
-      hipLaunchKernelGGL((lmhead_tile_kernel<false, true>), grid, block, 0, st, A);
-    else
-      hipLaunchKernelGGL((lmhead_tile_kernel<false, false>), grid, block, 0, st, A);
-  }
-  int rc = (int)hipGetLastError();
+  int rc = (edge == 256) ? launch_head_tiles<256, 1>(A, grid, st) : launch_head_tiles<128, 2>(A, grid, st);
   if (rc != 0) return rc;
   const int per_block = kHdThreads / kWave;
-  hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned int)((rows + per_block - 1) / per_block)), block, 0, st, A);
+  hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned int)((rows + per_block - 1) / per_block)), dim3(kHdThreads), 0,
+                     st, A);
   return (int)hipGetLastError();
 }
