@@ -848,6 +848,22 @@ def main() -> int:
                 del floor_run
             except Exception as exc:
                 log(f"{sh['name']}: floor measurement failed ({type(exc).__name__}: {exc})")
+            if sh["write_bytes"] == 0:
+                # a read-only reducing shape: the plainest reduction of the same bytes (one fp64 partial per
+                # workgroup, then a dependent launch that adds them) in the same harness -- what the
+                # two-launch scheme itself costs before any of the shape's arithmetic
+                try:
+                    rb = (sh["read_bytes"] + 15) // 16 * 16
+                    srcs = [torch.ones(rb, dtype=torch.uint8, device=dev) for _ in range(sh["sets"])]
+                    scratch = torch.zeros(16 + 16 * 512, dtype=torch.uint8, device=dev)
+                    sink = torch.zeros(1, dtype=torch.float64, device=dev)
+                    red_us = time_in_graph(
+                        torch, lambda i: ops.calib_reduce(srcs[i % len(srcs)], rb, 1, 512, scratch, sink), sh["sets"])
+                    row["plain_reduction_us"] = round(red_us, 2)
+                    row["frac_of_plain_reduction"] = round(red_us / us, 4)
+                    del srcs
+                except Exception as exc:
+                    log(f"{sh['name']}: plain-reduction measurement failed ({type(exc).__name__}: {exc})")
             if not args.skip_cpu and "cpu" in sh:
                 cms = time_cpu(sh["cpu"], reps=sh.get("cpu_reps", 5), warmup=1)
                 row["cpu_ms"] = round(cms, 2)
