@@ -207,3 +207,45 @@ def test_replay_steps_argument_errors(dev):
     # zero samples: empty outputs, no launch
     lp, means = st.replay_steps(v[:0], stack[:0], [0, 1], [1, 2], s2, s2, eta=0.7)
     assert tuple(lp.shape) == (0, 2) and tuple(means.shape) == (0, 2, 8, 8)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("traj_dtype", [torch.float32, torch.bfloat16])
+def test_replay_steps_odd_extents_and_offset_views(dev, kind, traj_dtype):
+    """D not a multiple of 4 (element-wise path), a stack and velocities that are offset slices of larger
+    buffers (bases off the 16-byte grid, sample strides larger than the data), one sample, one step."""
+    from unirl_amd import sde
+
+    st = strategy(kind)
+    stored = [0, 1, 2, 3]
+    for B, tail, steps in ((3, (3, 5, 7), [1, 0]), (1, (2, 9), [2]), (2, (8, 8), [0, 1, 2])):
+        stack, v = make_case(B, len(stored), tail, steps, stored, traj_dtype, traj_dtype, 40 + B)
+        ref_lp, ref_means = oracle_replay(kind, stack, v, steps, stored, SIG, traj_dtype)
+        slot_x, slot_p = sde.replay_slots(stored, steps)
+        # device copies inside larger buffers: one leading element of padding, one extra slot / step
+        big_stack = torch.zeros((B, len(stored) + 1) + tail, dtype=traj_dtype, device=dev)
+        flat = torch.zeros(big_stack.numel() + 1, dtype=traj_dtype, device=dev)
+        stack_view = flat[1:].view(big_stack.shape)[:, : len(stored)]
+        stack_view.copy_(stack.to(dev))
+        big_v = torch.zeros((B, len(steps) + 2) + tail, dtype=traj_dtype, device=dev)
+        v_view = big_v[:, 1 : 1 + len(steps)]
+        v_view.copy_(v.to(dev))
+        assert B == 1 or not (stack_view.is_contiguous() or v_view.is_contiguous())
+        sig = [float(SIG[i]) for i in steps]
+        sig_n = [float(SIG[i + 1]) for i in steps]
+        lp, means = st.replay_steps(v_view, stack_view, slot_x, slot_p, sig, sig_n, eta=0.7, sigma_max=float(SIG[1]))
+        assert torch.equal(means.cpu(), ref_means), (B, tail)
+        rtol = FP32_RTOL if traj_dtype == torch.float32 else BF16_RTOL
+        assert_close(lp, ref_lp, rtol, 2e-6, f"log-probs B={B} tail={tail}")
+        # the gradient takes the velocities' (strided) layout
+        vg = v_view.detach().clone().requires_grad_(True)
+        lp_g, _ = st.replay_steps(vg, stack_view, slot_x, slot_p, sig, sig_n, eta=0.7, sigma_max=float(SIG[1]))
+        lp_g.sum().backward()
+        v_ref = v.float().clone().requires_grad_(True)
+        tot = 0.0
+        for j, i in enumerate(steps):
+            tot = tot + osde.sde_denoise(kind, v_ref[:, j], stack[:, i], SIG[i], SIG[i + 1], eta=0.7,
+                                         prev_sample=stack[:, i + 1], sigma_max=SIG[1])[1].sum()
+        tot.backward()
+        gtol = 1e-4 if traj_dtype == torch.float32 else 1e-2
+        assert_close(vg.grad.float(), v_ref.grad, gtol, gtol * float(v_ref.grad.abs().max()), "grad, strided velocities")
