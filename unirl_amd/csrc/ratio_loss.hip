@@ -80,6 +80,9 @@ struct RatioArgs {
   int64_t n_valid_host;  // token-mean denominator when the host knows it, else < 0
   int64_t per_wave;      // packed kernel: vectors in a wavefront's run (a multiple of 64)
   UNIRL_TRACE_FIELD
+#ifdef UNIRL_TUNE
+  int synth_len;  // timing experiment: row lengths from a hash of the row instead of the load
+#endif
 };
 
 // exp(x) for fp32 within ~1.5 ulp: 2^(x*log2(e)) on the hardware exp2, with the rounding error
@@ -439,28 +442,37 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
   const bool adv_tok = (FLAGS < 0) ? (C.adv_per_token != 0) : ((FLAGS & 2) != 0);
 
   // global factor of the gradient; the token-mean denominator is the number of valid tokens,
-  // which is the sum of the (clamped) lengths when the host did not pass it
+  // which is the sum of the (clamped) lengths when the host did not pass it.  That sum is only
+  // needed once the first data has arrived: its loads go out here, and the sum itself (a
+  // workgroup reduction) is taken by every wavefront after it has issued its first pass of
+  // loads -- or after the row loop, for a wavefront without a pass.  Every wavefront of the
+  // workgroup takes it exactly once, so the barriers inside pair up.
   float gfac = 0.0f;
+  bool sum_pending = false;
+  int64_t len_first = 0;
   if (GRAD) {
     if (C.agg_mode == UNIRL_AGG_TOKEN_MEAN) {
-      double nv = (double)A.n_valid_host;
       if (A.n_valid_host < 0) {
-        double s = 0.0;  // exact: lengths are far below 2^53
-        for (int64_t i = threadIdx.x; i < A.n_seq; i += kRlThreads) {
-          int64_t len = A.seq[i];
-          len = len < 0 ? 0 : (len > A.seq_stride ? A.seq_stride : len);
-          s += (double)len;
-        }
-        nv = block_sum(s, &lds_v[0][0]);
-        __syncthreads();  // lds_v is reused below
+        sum_pending = true;
+        if ((int64_t)threadIdx.x < A.n_seq) len_first = A.seq[threadIdx.x];
+      } else {
+        gfac = A.loss_scale / (float)(double)A.n_valid_host;
       }
-      gfac = A.loss_scale / (float)nv;
     } else if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_SUM) {
       gfac = (A.loss_scale / (float)A.n_seq) / C.horizon;
     } else {
       gfac = A.loss_scale / (float)A.n_seq;
     }
   }
+  auto finish_token_count = [&]() {
+    auto clamped = [&](int64_t len) { return len < 0 ? 0 : (len > A.seq_stride ? A.seq_stride : len); };
+    double s = (double)clamped(len_first);  // exact: lengths are far below 2^53
+    for (int64_t i = (int64_t)threadIdx.x + kRlThreads; i < A.n_seq; i += kRlThreads) s += (double)clamped(A.seq[i]);
+    const double nv = block_sum(s, &lds_v[0][0]);
+    __syncthreads();  // lds_v is reused at the end
+    gfac = A.loss_scale / (float)nv;
+    sum_pending = false;
+  };
 
   Acc acc;
   WaveCounts wc;
@@ -479,7 +491,14 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
     // tokens [base, base+count) are valid; whole vectors may be loaded up to base+row_end
     int64_t base = 0, count = A.n_tok, row_end = A.n_tok;
     if (padded) {
-      int64_t len = A.seq[r];
+      int64_t len;
+#ifdef UNIRL_TUNE
+      // measurement build only: what the kernel would cost if a row's length needed no trip to
+      // memory (the results are those of other lengths; a timing experiment)
+      if (A.synth_len) len = 512 + (int64_t)(((unsigned int)r * 2654435761u) >> 8) % (A.seq_stride - 511);
+      else
+#endif
+      len = A.seq[r];
       len = len < 0 ? 0 : (len > A.seq_stride ? A.seq_stride : len);
       base = r * A.seq_stride;
       count = len;
@@ -507,6 +526,7 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
         if (has_mask) Vec<float, VEC>::load(A.mask + base + ic * VEC, mk[it]);
         else fill_ones(mk[it]);
       }
+      if (GRAD && sum_pending) finish_token_count();
 #pragma unroll
       for (int it = 0; it < ITEMS; ++it) {
         const int64_t wv = w0 + it * stride;  // the wavefront's first vector of this item
@@ -527,7 +547,7 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
     }
     // a row whose length is not a multiple of VEC ends in one vector that cannot be loaded whole;
     // one lane of the grid takes it token by token
-    if (nvec > nvec_full && first == nvec_full % stride) {
+    if (nvec > nvec_full && first == nvec_full % stride) {  // (flat layout only: no pending sum there)
       const int64_t t0 = nvec_full * VEC;
       float nw[VEC], od[VEC], ad[VEC], mk[VEC], out[VEC], gr[VEC];
 #pragma unroll
@@ -565,6 +585,7 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
       }
     }
   }
+  if (GRAD && sum_pending) finish_token_count();
   UNIRL_TRACE_MARK1();
   store_block_partials(A, acc, wc, lds_v);
   UNIRL_TRACE_END(A.trace);
@@ -1049,6 +1070,9 @@ static int check_common(const float* new_logp, const float* old_logp, const floa
   A.n_seq = n_seq;
   A.seq_stride = seq_stride;
   A.n_tok = n_tok;
+#ifdef UNIRL_TUNE
+  A.synth_len = (int)tune_int("UNIRL_RATIO_SYNTH_LEN", 0);
+#endif
   return UNIRL_OK;
 }
 
