@@ -450,9 +450,10 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
     out = {"rows": rows, "vocab": vocab, "hidden": hidden}
     ref = timed(reference)
     out["reference_torch_checkpoint_chunk2048"] = ref[0]
-    for name, kw in (("fused_recompute_chunk2048", dict(chunk=2048, keep_logits=False)),
-                     ("fused_recompute_chunk4096", dict(keep_logits=False)), ("fused_default", dict()),
-                     ("fused_head_chunk4096", dict(fused_head=True))):
+    for name, kw in (("fused_recompute_chunk2048", dict(chunk=2048, keep_logits=False, transposed_head=False)),
+                     ("fused_recompute_chunk4096", dict(keep_logits=False, transposed_head=False)),
+                     ("fused_keep_logits", dict(transposed_head=False)), ("fused_default", dict()),
+                     ("fused_head_chunk4096", dict(fused_head=True, transposed_head=False))):
         got = timed(lambda h: models.chunked_replay_logp(head, h, tokens, 1.0, **kw))
         got[0]["max_abs_logp_diff"] = float((got[1] - ref[1]).abs().max())
         got[0]["grad_hidden_rel"] = float((got[2] - ref[2]).norm() / ref[2].norm())
@@ -460,6 +461,18 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
         out[name] = got[0]
         log(f"replay {name}: {got[0]}")
     log(f"replay reference: {ref[0]}")
+    # what the default's transposed copy of the weight costs, once per weight version
+    from unirl_amd.models import ar_logp
+
+    ar_logp._TRANSPOSED.clear()
+    torch.cuda.synchronize()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    ar_logp._transposed_weight(head.weight)
+    b.record()
+    torch.cuda.synchronize()
+    out["weight_transposition_ms"] = round(a.elapsed_time(b), 2)
+    log(f"replay: transposing the weight once takes {out['weight_transposition_ms']} ms")
     return out
 
 

@@ -412,6 +412,19 @@ int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const void* weight,
                       void* stream);
 
 /* ------------------------------------------------------------------------
+ * dst[c][r] = src[r][c] for a [rows, cols] matrix of 2- or 4-byte elements
+ * (rows ld_src elements apart; destination rows ld_dst apart).  Replaces the
+ * `weight.t().contiguous()` a caller makes to hand the GEMM library the head's
+ * weight as [K, V]: the gradient of the hidden states in the backward of
+ * `lm_head` (unirl/models/qwen3/ar.py:82-99 under autograd), dL [rows, V] @ W
+ * [V, K], runs 1.2 - 1.5 times faster on that layout.  16-byte accesses when
+ * bases and leading dimensions allow them, element-wise otherwise.  Limit:
+ * rows <= 4 194 240 (UNIRL_E_LIMIT).
+ * ---------------------------------------------------------------------- */
+int unirl_transpose_2d(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, int64_t rows,
+                       int64_t cols, int elem_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
  * Token-level ratio losses with every metric reduction fused in.
  * Replaces _grpo_clip_loss (unirl/algorithms/base.py:115-157), _drpo_loss
  * (unirl/algorithms/drpo.py:97-159), rollout_replay_logp_absdiff

@@ -201,3 +201,39 @@ def test_chunked_replay_with_the_fused_head(dev):
     assert torch.equal(out_ng, out_f)
     with pytest.raises(ValueError, match="fused_head"):
         models.chunked_replay_logp(head.float(), hidden.float(), toks, T, fused_head=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32, torch.int16, torch.int32])
+def test_transpose_2d_is_exact(dev, dtype):
+    """unirl_transpose_2d: bit-exact against torch's transposed copy for whole tiles, ragged edges, one
+    row / one column, strided source rows and a base off the 16-byte grid (element-wise path)."""
+    from unirl_amd import ops
+
+    g = torch.Generator().manual_seed(30)
+    for rows, cols in ((64, 64), (128, 192), (1, 1), (1, 300), (300, 1), (65, 127), (200, 72), (7, 1000), (513, 66)):
+        if dtype.is_floating_point:
+            src = torch.randn(rows, cols, generator=g).to(dtype).to(dev)
+        else:
+            src = torch.randint(-30000, 30000, (rows, cols), generator=g).to(dtype).to(dev)
+        out = ops.transpose_2d(src)
+        assert out.shape == (cols, rows) and out.is_contiguous()
+        assert torch.equal(out, src.t().contiguous()), (rows, cols)
+        # rows of a wider buffer, starting one element in: a leading dimension and a base that rule out
+        # 16-byte loads
+        wide = torch.zeros(rows, cols + 3, dtype=dtype, device=dev)
+        view = wide[:, 1 : 1 + cols]
+        view.copy_(src)
+        assert torch.equal(ops.transpose_2d(view), src.t().contiguous()), (rows, cols, "strided")
+    with pytest.raises(ValueError):
+        ops.transpose_2d(torch.zeros(4, 4, dtype=torch.float64, device=dev))
+    with pytest.raises(ValueError):
+        ops.transpose_2d(torch.zeros(4, 4, 4, device=dev))
+
+
+def test_transpose_2d_head_sized(dev):
+    """The Qwen3-4B head's weight, [151936, 2560] bf16 (778 MB)."""
+    from unirl_amd import ops
+
+    w = torch.randn(151936, 2560, device=dev, dtype=torch.bfloat16)
+    wt = ops.transpose_2d(w)
+    assert torch.equal(wt, w.t().contiguous())

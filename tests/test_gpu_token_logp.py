@@ -312,7 +312,7 @@ def test_chunked_replay_recomputes_logits_in_backward(dev, dtype):
         hd.weight.copy_(head.weight)
         hd.bias.copy_(head.bias)
     out = models.chunked_replay_logp(hd, hidden.to(dev), toks.to(dev), temperature=T, chunk=64, keep_logits=False)
-    assert "RecomputedChunk" in type(out.grad_fn.next_functions[0][0]).__name__
+    assert "LinearHeadChunk" in type(out.grad_fn.next_functions[0][0]).__name__
     (out * upstream.to(dev)).sum().backward()
     assert_close(hd.weight.grad.cpu(), ref_grads[1], 1e-4, 1e-5 * float(ref_grads[1].abs().max()), "weight grad only")
 
@@ -367,8 +367,69 @@ def test_chunked_replay_keeps_logits_only_within_its_budget(dev, monkeypatch):
         again = torch.nn.functional.linear(h[:, :16].detach(), hooked.weight, hooked.bias)
     assert torch.allclose(captured, again), "a hooked head's captured logits were overwritten"
 
+    def keeps(lm_head):
+        """Whether the replay kept (and so consumed) its logits: then a second backward raises."""
+        h = torch.randn(B, T_max, H, generator=g).to(dev).requires_grad_(True)
+        out = models.chunked_replay_logp(lm_head, h, toks, chunk=16)
+        out.sum().backward(retain_graph=True)
+        try:
+            out.sum().backward()
+        except RuntimeError as e:
+            assert "overwritten by their gradient" in str(e)
+            return True
+        return False
+
     assert B * T_max * V * 4 < ar_logp.KEEP_LOGITS_BYTES
-    assert not any("RecomputedChunk" in n for n in path(head))
+    assert all("LinearHeadChunk" in n for n in path(head))  # a plain Linear: head and backward in one node
+    assert keeps(head)
     monkeypatch.setattr(ar_logp, "KEEP_LOGITS_BYTES", B * T_max * V * 4 - 1)
-    assert all("RecomputedChunk" in n for n in path(head))
+    assert all("LinearHeadChunk" in n for n in path(head))
+    assert not keeps(head)
     assert all("RecomputedChunk" in n for n in path(lambda h: h @ head.weight.t()))
+    assert all("RecomputedChunk" in n for n in path(sub))
+
+
+def test_chunked_replay_transposed_head_gradient(dev):
+    """The hidden states' gradient computed on the cached transposed copy of the weight equals the
+    plain product (another summation order), and the copy follows the weight: after an in-place
+    update (what an optimizer step is) the next replay sees the new values."""
+    from unirl_amd import models
+    from unirl_amd.models import ar_logp
+
+    B, T_max, H, V = 2, 48, 32, 700
+    g = torch.Generator().manual_seed(13)
+    head = torch.nn.Linear(H, V).to(dev)
+    toks = torch.randint(0, V, (B, T_max), generator=g).to(dev)
+    hidden = torch.randn(B, T_max, H, generator=g).to(dev)
+    up = torch.randn(B, T_max, generator=g).to(dev)
+
+    def grads(transposed):
+        head.zero_grad(set_to_none=True)
+        h = hidden.clone().requires_grad_(True)
+        out = models.chunked_replay_logp(head, h, toks, 0.9, chunk=16, transposed_head=transposed)
+        (out * up).sum().backward()
+        return out.detach(), h.grad, head.weight.grad.clone(), head.bias.grad.clone()
+
+    def reference():
+        h = hidden.clone().requires_grad_(True)
+        lf = torch.nn.functional.linear(h, head.weight.detach(), head.bias.detach()).float() / 0.9
+        ref = lf.gather(-1, toks.unsqueeze(-1)).squeeze(-1) - torch.logsumexp(lf, dim=-1)
+        (ref * up).sum().backward()
+        return h.grad
+
+    for _ in range(2):
+        out_t, gh_t, gw_t, gb_t = grads(True)
+        out_p, gh_p, gw_p, gb_p = grads(False)
+        assert torch.equal(out_t, out_p) and torch.equal(gw_t, gw_p) and torch.equal(gb_t, gb_p)
+        assert_close(gh_t, gh_p, 1e-5, 1e-6 * float(gh_p.abs().max()), "hidden grad, transposed copy vs plain")
+        assert_close(gh_t, reference(), 1e-4, 1e-5 * float(gh_p.abs().max()), "hidden grad vs autograd of the chain")
+        cached = ar_logp._TRANSPOSED[id(head.weight)]
+        assert torch.equal(cached[3], head.weight.detach().t())
+        with torch.no_grad():  # an optimizer step: in place, the version moves on
+            head.weight.add_(0.05 * torch.randn(V, H, generator=g).to(dev))
+        assert cached[1] != head.weight._version
+    # by default small replays do not pay for the copy
+    ar_logp._TRANSPOSED.clear()
+    h = hidden.clone().requires_grad_(True)
+    models.chunked_replay_logp(head, h, toks, 0.9, chunk=16).sum().backward()
+    assert id(head.weight) not in ar_logp._TRANSPOSED and B * T_max < ar_logp.TRANSPOSED_HEAD_MIN_ROWS

@@ -204,6 +204,7 @@ _SIGNATURES = {
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p,
          c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_size_t, c_void_p],
     ),
+    "unirl_transpose_2d": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "unirl_token_logp_bwd": (
         c_int,
         [c_void_p, c_int, c_int64, c_int64, c_int64, c_void_p, c_float, c_void_p, c_void_p, c_void_p, c_int64,

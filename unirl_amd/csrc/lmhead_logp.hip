@@ -386,6 +386,121 @@ __global__ __launch_bounds__(kHdThreads) void lmhead_merge_kernel(HeadArgs A) {
   }
 }
 
+
+// ---- transposed copy of a 2-D matrix of 2- or 4-byte elements --------------------------------
+// dst[c][r] = src[r][c].  One workgroup per 64 x 64 tile: 16-byte loads along the source rows,
+// the tile through LDS as 32-bit words (rows padded by one word so that a walk down a column
+// meets every bank once), 16-byte stores along the destination rows; eight (2-byte elements) or
+// sixteen (4-byte) neighbouring lanes write one whole 128- or 256-byte run of a destination row.
+constexpr int kTrTile = 64;
+constexpr int kTrThreads = 256;
+
+struct TransposeArgs {
+  const void* src;
+  void* dst;
+  int64_t rows, cols, ld_src, ld_dst;
+  int vec_src, vec_dst;  // 16-byte accesses allowed on that side (alignment of base and leading dimension)
+};
+
+template <typename T>
+__global__ __launch_bounds__(kTrThreads) void transpose_tile_kernel(TransposeArgs A) {
+  constexpr int VE = 16 / (int)sizeof(T);          // elements per 16-byte vector
+  constexpr int WPR = kTrTile * (int)sizeof(T) / 4;  // 32-bit words per tile row
+  constexpr int TPR = kTrTile / VE;                // threads covering a tile row with one vector each
+  constexpr int RPP = kTrThreads / TPR;            // tile rows per pass
+  __shared__ uint32_t lds[kTrTile][WPR + 1];
+  const T* src = reinterpret_cast<const T*>(A.src);
+  T* dst = reinterpret_cast<T*>(A.dst);
+  const int64_t r0 = (int64_t)blockIdx.y * kTrTile, c0 = (int64_t)blockIdx.x * kTrTile;
+  const int tid = threadIdx.x;
+
+  // load: thread (row tid / TPR, vector tid % TPR) of each pass
+#pragma unroll
+  for (int p = 0; p < kTrTile / RPP; ++p) {
+    const int lr = p * RPP + tid / TPR, lv = tid % TPR;
+    const int64_t r = r0 + lr, c = c0 + (int64_t)lv * VE;
+    u32x4 v = {0u, 0u, 0u, 0u};
+    if (r < A.rows) {
+      if (A.vec_src && c + VE <= A.cols) {
+        v = *reinterpret_cast<const u32x4*>(src + r * A.ld_src + c);
+      } else {
+        T e[VE];
+#pragma unroll
+        for (int k = 0; k < VE; ++k) e[k] = (c + k < A.cols) ? src[r * A.ld_src + c + k] : (T)0;
+        if (sizeof(T) == 2) {
+          v.x = (uint32_t)e[0] | ((uint32_t)e[1 % VE] << 16);
+          v.y = (uint32_t)e[2 % VE] | ((uint32_t)e[3 % VE] << 16);
+          v.z = (uint32_t)e[4 % VE] | ((uint32_t)e[5 % VE] << 16);
+          v.w = (uint32_t)e[6 % VE] | ((uint32_t)e[7 % VE] << 16);
+        } else {
+          v.x = (uint32_t)e[0];
+          v.y = (uint32_t)e[1 % VE];
+          v.z = (uint32_t)e[2 % VE];
+          v.w = (uint32_t)e[3 % VE];
+        }
+      }
+    }
+    uint32_t* w = &lds[lr][lv * 4];
+    w[0] = v.x;
+    w[1] = v.y;
+    w[2] = v.z;
+    w[3] = v.w;
+  }
+  __syncthreads();
+
+  if (sizeof(T) == 2) {
+    // thread (source rows 8*rg .. +7, source column pair cp): two destination rows, 16 bytes each
+    const int rg = tid % 8, cp = tid / 8;
+    uint32_t w[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w[j] = lds[8 * rg + j][cp];
+    u32x4 lo, hi;
+    lo.x = (w[0] & 0xffffu) | (w[1] << 16);
+    lo.y = (w[2] & 0xffffu) | (w[3] << 16);
+    lo.z = (w[4] & 0xffffu) | (w[5] << 16);
+    lo.w = (w[6] & 0xffffu) | (w[7] << 16);
+    hi.x = (w[0] >> 16) | (w[1] & 0xffff0000u);
+    hi.y = (w[2] >> 16) | (w[3] & 0xffff0000u);
+    hi.z = (w[4] >> 16) | (w[5] & 0xffff0000u);
+    hi.w = (w[6] >> 16) | (w[7] & 0xffff0000u);
+    const int64_t dr = c0 + 2 * cp, dc = r0 + 8 * rg;  // destination row (= source column), first column
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+      const u32x4 v = e ? hi : lo;
+      if (dr + e >= A.cols) continue;
+      if (A.vec_dst && dc + 8 <= A.rows) {
+        *reinterpret_cast<u32x4*>(dst + (dr + e) * A.ld_dst + dc) = v;
+      } else {
+        const uint32_t q[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+          if (dc + k < A.rows) dst[(dr + e) * A.ld_dst + dc + k] = (T)((q[k / 2] >> (16 * (k % 2))) & 0xffffu);
+      }
+    }
+  } else {
+    // thread (source rows 4*rg .. +3, source column c) of each of four passes
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int rg = tid % 16, c = p * 16 + tid / 16;
+      u32x4 v;
+      v.x = lds[4 * rg + 0][c];
+      v.y = lds[4 * rg + 1][c];
+      v.z = lds[4 * rg + 2][c];
+      v.w = lds[4 * rg + 3][c];
+      const int64_t dr = c0 + c, dc = r0 + 4 * rg;
+      if (dr >= A.cols) continue;
+      if (A.vec_dst && dc + 4 <= A.rows) {
+        *reinterpret_cast<u32x4*>(dst + dr * A.ld_dst + dc) = v;
+      } else {
+        const uint32_t q[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+          if (dc + k < A.rows) dst[dr * A.ld_dst + dc + k] = (T)q[k];
+      }
+    }
+  }
+}
+
 }  // namespace unirl
 
 using namespace unirl;
@@ -468,5 +583,31 @@ extern "C" int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const vo
   const int per_block = kHdThreads / kWave;
   hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned int)((rows + per_block - 1) / per_block)), dim3(kHdThreads), 0,
                      st, A);
+  return (int)hipGetLastError();
+}
+
+extern "C" int unirl_transpose_2d(const void* src, int64_t ld_src, void* dst, int64_t ld_dst, int64_t rows,
+                                  int64_t cols, int elem_bytes, void* stream) {
+  if (rows < 0 || cols < 0) return UNIRL_E_SHAPE;
+  if (rows == 0 || cols == 0) return UNIRL_OK;
+  if (!src || !dst) return UNIRL_E_NULL;
+  if (elem_bytes != 2 && elem_bytes != 4) return UNIRL_E_DTYPE;
+  if (ld_src < cols || ld_dst < rows) return UNIRL_E_SHAPE;
+  if (!aligned_to(src, elem_bytes) || !aligned_to(dst, elem_bytes)) return UNIRL_E_ALIGN;
+  const int64_t tiles_x = (cols + kTrTile - 1) / kTrTile, tiles_y = (rows + kTrTile - 1) / kTrTile;
+  if (tiles_x > 0x7fffffffLL || tiles_y > 65535) return UNIRL_E_LIMIT;  // grid extents (y: 4 M source rows)
+  TransposeArgs A;
+  A.src = src;
+  A.dst = dst;
+  A.rows = rows;
+  A.cols = cols;
+  A.ld_src = ld_src;
+  A.ld_dst = ld_dst;
+  const int64_t ve = 16 / elem_bytes;
+  A.vec_src = (aligned_to(src, 16) && ld_src % ve == 0) ? 1 : 0;
+  A.vec_dst = (aligned_to(dst, 16) && ld_dst % ve == 0) ? 1 : 0;
+  const dim3 grid((unsigned int)tiles_x, (unsigned int)tiles_y), block(kTrThreads);
+  if (elem_bytes == 2) hipLaunchKernelGGL(transpose_tile_kernel<uint16_t>, grid, block, 0, (hipStream_t)stream, A);
+  else hipLaunchKernelGGL(transpose_tile_kernel<uint32_t>, grid, block, 0, (hipStream_t)stream, A);
   return (int)hipGetLastError();
 }

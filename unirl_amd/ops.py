@@ -882,6 +882,30 @@ def token_logp_entropy(
     return logp, ent, lse
 
 
+def transpose_2d(src: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """A contiguous ``[cols, rows]`` transposed copy of a 2-D tensor of 2- or 4-byte elements whose
+    rows are dense (``src.stride(1) == 1``; the row stride is free)."""
+    if src.dim() != 2 or not src.is_cuda or src.element_size() not in (2, 4):
+        raise ValueError(f"transpose_2d needs a 2-D HIP tensor of 2- or 4-byte elements, got {src.dtype} {tuple(src.shape)}")
+    rows, cols = int(src.shape[0]), int(src.shape[1])
+    s = src.detach()
+    if rows > 1 and cols > 0 and (s.stride(1) != 1 or s.stride(0) < cols):
+        s = s.contiguous()
+    if out is None:
+        out = torch.empty((cols, rows), dtype=src.dtype, device=src.device)
+    elif tuple(out.shape) != (cols, rows) or out.dtype != src.dtype or out.device != src.device or not out.is_contiguous():
+        raise ValueError("transpose_2d: out must be a contiguous [cols, rows] tensor of the source's dtype and device")
+    if rows == 0 or cols == 0:
+        return out
+    with N.on_device(src.device):
+        N.check(
+            N.F.unirl_transpose_2d(s.data_ptr(), int(s.stride(0)) if rows > 1 else cols, out.data_ptr(), rows, rows, cols,
+                                   src.element_size(), N.current_stream(src.device)),
+            "unirl_transpose_2d",
+        )
+    return out
+
+
 def lmhead_logp_supported(hidden: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> bool:
     """Whether :func:`lmhead_logp` takes these operands as they are: bf16 on one HIP device, the
     hidden size a multiple of 64, rows contiguous and 16-byte aligned."""
