@@ -83,10 +83,26 @@ __device__ __forceinline__ bf16x8_t lds_frag(const uint16_t* p) {
   return *reinterpret_cast<const bf16x8_t*>(p);
 }
 
+// Scheduling pattern of one slice of NM matrix instructions: before the m-th of them go its share
+// of the slice's NR LDS reads, NW LDS writes and NL global loads.
+template <int MASK, int N>
+__device__ __forceinline__ void sched_group() {
+  if constexpr (N > 0) __builtin_amdgcn_sched_group_barrier(MASK, N, 0);
+}
+template <int NM, int NR, int NW, int NL, int M = 0>
+__device__ __forceinline__ void sched_slice() {
+  if constexpr (M < NM) {
+    sched_group<0x100, (M + 1) * NR / NM - M * NR / NM>();  // LDS reads
+    sched_group<0x020, (M + 1) * NL / NM - M * NL / NM>();  // global loads
+    sched_group<0x200, (M + 1) * NW / NM - M * NW / NM>();  // LDS writes
+    sched_group<0x008, 1>();                                // one MFMA
+    sched_slice<NM, NR, NW, NL, M + 1>();
+  }
+}
+
 // BM x BN: the workgroup's tile of the logits; its four wavefronts sit 2 x 2, each on a
-// (BM/2) x (BN/2) quarter of BI x BJ MFMA blocks.  SETS: register sets staging the global loads
-// (2 = loads run two K steps ahead of the multiplication, 1 = one step).
-template <int BM, int BN, int SETS, bool HAS_BIAS, bool WRITE_LOGITS>
+// (BM/2) x (BN/2) quarter of BI x BJ MFMA blocks.
+template <int BM, int BN, bool HAS_BIAS, bool WRITE_LOGITS>
 __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmhead_tile_kernel(HeadArgs A) {
   constexpr int WM = BM / 2, WN = BN / 2, BI = WM / 32, BJ = WN / 32;
   constexpr int kAElems = BM * kLdsRow, kBElems = BN * kLdsRow, kStage = kAElems + kBElems;
@@ -95,6 +111,9 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   static_assert(BM * kOutRow <= 2 * kStage, "the epilogue tile reuses the operand stages");
   __shared__ __attribute__((aligned(16))) uint16_t lds[2 * kStage];  // [stage][A rows | B rows][kLdsRow]
   UNIRL_TRACE_T0();
+#ifdef UNIRL_TRACE
+  const long long trace_c0_ = clock64();  // shader clock: with the 100 MHz marks it gives the clock rate under load
+#endif
   int mb, nt;
   head_tile_of(A, blockIdx.x, mb, nt);
   if (mb < 0) return;  // the padding of the last XCD's range (whole workgroup)
@@ -102,37 +121,40 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
   const int wm = wave >> 1, wn = wave & 1;
 
-  // global -> LDS assignment: 16-byte chunk c = tid + 256*i covers row c/8, k-chunk c%8 of a tile
+  // global -> LDS assignment: 16-byte chunk c = tid + 256*i covers row c/8, k-chunk c%8 of a tile.
+  // The operands are read through buffer descriptors based at the tile's first row: a lane keeps
+  // one 32-bit offset per operand (row and k-chunk; the K step travels in the scalar offset), and
+  // rows past the end of the matrix fall outside the descriptor's range and read as zeros.
   const int kc = tid & 7, row0 = tid >> 3;
-  const uint16_t* pa[CA];
-  const uint16_t* pb[CB];
-#pragma unroll
-  for (int i = 0; i < CA; ++i) {
-    int64_t r = m0 + row0 + 32 * i;
-    r = r < A.M ? r : A.M - 1;  // rows past the end repeat the last one; their results are dropped
-    pa[i] = A.h + r * A.ldh + kc * 8;
-  }
-#pragma unroll
-  for (int i = 0; i < CB; ++i) {
-    int64_t r = n0 + row0 + 32 * i;
-    r = r < A.N ? r : A.N - 1;
-    pb[i] = A.w + r * A.ldw + kc * 8;
-  }
-  const int lds_off0 = row0 * kLdsRow + kc * 8;  // chunk i sits 32 rows further down
-  u32x4 ga[SETS][CA], gb[SETS][CB];
-  auto load_global = [&](int set, int64_t k0) {
-#pragma unroll
-    for (int i = 0; i < CA; ++i) ga[set][i] = *reinterpret_cast<const u32x4*>(pa[i] + k0);
-#pragma unroll
-    for (int i = 0; i < CB; ++i) gb[set][i] = *reinterpret_cast<const u32x4*>(pb[i] + k0);
+  auto tile_rsrc = [](const uint16_t* base, int64_t rows_left, int64_t ld, int64_t K) {
+    const int64_t bytes = rows_left > 0 ? ((rows_left - 1) * ld + K) * 2 : 0;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint16_t*>(base), 0,
+                                             bytes > 0xffffffffLL ? (int)0xffffffffu : (int)(uint32_t)bytes, 0x00020000);
   };
-  auto store_lds = [&](int set, int stage) {
+  const __amdgpu_buffer_rsrc_t ra = tile_rsrc(A.h + m0 * A.ldh, A.M - m0, A.ldh, A.K);
+  const __amdgpu_buffer_rsrc_t rb = tile_rsrc(A.w + n0 * A.ldw, A.N - n0, A.ldw, A.K);
+  const int va0 = (int)((row0 * A.ldh + kc * 8) * 2), vb0 = (int)((row0 * A.ldw + kc * 8) * 2);
+  const int va_step = (int)(32 * A.ldh * 2), vb_step = (int)(32 * A.ldw * 2);  // chunk i sits 32 rows further down
+  const int lds_off0 = row0 * kLdsRow + kc * 8;
+  // Two register sets stage the operands of two K steps between global memory and LDS.  A step's
+  // CA + CB loads (and, a step later, its stores to LDS) are issued a quarter at a time, one
+  // quarter under each 16-wide slice of the multiplication.
+  constexpr int NW = CA + CB, NQ = NW / 4;
+  static_assert(NW % 4 == 0 && CA % NQ == 0, "a quarter of a step's chunks lies inside one operand");
+  u32x4 gs[2][NW];  // [set][chunk]: chunks 0 .. CA-1 of the hidden states, CA .. of the weight
+  auto load_quarter = [&](int set, int64_t k0, int q) {
+    const int sk = (int)(k0 * 2);
+#pragma unroll
+    for (int j = q * NQ; j < (q + 1) * NQ; ++j)
+      gs[set][j] = (j < CA) ? __builtin_amdgcn_raw_buffer_load_b128(ra, va0 + j * va_step, sk, 0)
+                            : __builtin_amdgcn_raw_buffer_load_b128(rb, vb0 + (j - CA) * vb_step, sk, 0);
+  };
+  auto store_quarter = [&](int set, int stage, int q) {
     uint16_t* sa = lds + stage * kStage;
     uint16_t* sb = sa + kAElems;
 #pragma unroll
-    for (int i = 0; i < CA; ++i) *reinterpret_cast<u32x4*>(sa + lds_off0 + i * 32 * kLdsRow) = ga[set][i];
-#pragma unroll
-    for (int i = 0; i < CB; ++i) *reinterpret_cast<u32x4*>(sb + lds_off0 + i * 32 * kLdsRow) = gb[set][i];
+    for (int j = q * NQ; j < (q + 1) * NQ; ++j)
+      *reinterpret_cast<u32x4*>((j < CA ? sa + j * 32 * kLdsRow : sb + (j - CA) * 32 * kLdsRow) + lds_off0) = gs[set][j];
   };
 
   f32x16_t acc[BI][BJ];
@@ -146,72 +168,87 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   // fragment addresses inside a stage: lane l reads row (l % 32) of a 32-row block, k = 8 * (l / 32) ..
   const int frag_a = (wm * WM + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
   const int frag_b = (wn * WN + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
-  auto multiply = [&](int stage) {
+  bf16x8_t fa[2][BI], fb[2][BJ];  // the fragments of two consecutive 16-wide K slices
+  auto read_frags = [&](int stage, int ks, bf16x8_t(&a)[BI], bf16x8_t(&b)[BJ]) {
     const uint16_t* sa = lds + stage * kStage;
     const uint16_t* sb = sa + kAElems;
 #pragma unroll
+    for (int bi = 0; bi < BI; ++bi) a[bi] = lds_frag(sa + frag_a + bi * 32 * kLdsRow + ks * 16);
+#pragma unroll
+    for (int bj = 0; bj < BJ; ++bj) b[bj] = lds_frag(sb + frag_b + bj * 32 * kLdsRow + ks * 16);
+  };
+  constexpr int NR = BI + BJ, NM = BI * BJ;  // LDS reads and MFMAs per K slice
+  // One K step out of LDS stage `stage`.  Under it travel, a quarter per slice: the loads of step
+  // k + 2 into register set `stage` (which held this step's operands until they were stored a step
+  // ago) and the stores of step k + 1's operands (register set stage ^ 1, loaded a step ago) into
+  // the other LDS stage, which every wavefront finished reading one barrier ago.  The fragments of
+  // slice ks + 1 are read while slice ks is multiplied.  So every memory instruction is issued
+  // between matrix instructions: a wavefront issues in order, and a burst of sixteen loads or
+  // stores holds up the MFMAs behind it for as long as the memory pipeline takes to accept them
+  // (measured: the bursts cost 0.9 us of a 1.8 us step).  The scheduling fences keep each slice's
+  // instructions together; inside a slice sched_slice deals them out among the MFMAs.
+  auto multiply = [&](int stage, int64_t k_load) {
+    read_frags(stage, 0, fa[0], fb[0]);
+#pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
-      bf16x8_t a[BI], b[BJ];
-#pragma unroll
-      for (int bi = 0; bi < BI; ++bi) a[bi] = lds_frag(sa + frag_a + bi * 32 * kLdsRow + ks * 16);
-#pragma unroll
-      for (int bj = 0; bj < BJ; ++bj) b[bj] = lds_frag(sb + frag_b + bj * 32 * kLdsRow + ks * 16);
+      const int cur = ks & 1;
+      if (ks + 1 < kBK / 16) read_frags(stage, ks + 1, fa[cur ^ 1], fb[cur ^ 1]);
+      load_quarter(stage, k_load, ks);
+      store_quarter(stage ^ 1, stage ^ 1, ks);
 #pragma unroll
       for (int bi = 0; bi < BI; ++bi)
 #pragma unroll
         for (int bj = 0; bj < BJ; ++bj)
-          acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[bi], b[bj], acc[bi][bj], 0, 0, 0);
+          acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][bi], fb[cur][bj], acc[bi][bj], 0, 0, 0);
+      if (ks + 1 < kBK / 16) sched_slice<NM, NR, NQ, NQ>();
+      else sched_slice<NM, 0, NQ, NQ>();
+      __builtin_amdgcn_sched_barrier(0);
     }
   };
 
-  // Step k is multiplied from LDS stage k % 2.  Every trip issues its loads and its LDS stores
-  // unconditionally (past the last step the loads repeat the last step's addresses and the
-  // stores fill a stage nobody reads any more): with a branch around them the compiler can no
-  // longer count which loads are outstanding at the stores and waits for all of them.  The
-  // scheduling barriers keep it from sinking the loads below the multiplication.
+  // Step k sits in LDS stage k % 2 and came through register set k % 2.  Every trip issues its
+  // loads and stores unconditionally (past the last step the loads repeat the last step's
+  // addresses and the stores fill a stage nobody reads any more): with a branch around them the
+  // compiler can no longer count which loads are outstanding at the stores and waits for all of
+  // them.
   const int nk = (int)(A.K / kBK);
   const int64_t k_last = (int64_t)(nk - 1) * kBK;
   auto k_of = [&](int step) { return step < nk ? (int64_t)step * kBK : k_last; };
-  load_global(0, 0);
-  if (SETS == 2) load_global(SETS - 1, k_of(1));
-  store_lds(0, 0);
+#ifdef UNIRL_TRACE
+  long long trace_bar_ = 0;  // shader cycles this wavefront spent waiting at the step barriers
+#define UNIRL_HEAD_STEP_BARRIER()              \
+  do {                                         \
+    const long long b0_ = clock64();           \
+    __syncthreads();                           \
+    trace_bar_ += clock64() - b0_;             \
+  } while (0)
+#else
+#define UNIRL_HEAD_STEP_BARRIER() __syncthreads()
+#endif
+#pragma unroll
+  for (int q = 0; q < 4; ++q) load_quarter(0, 0, q);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) load_quarter(1, k_of(1), q);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) store_quarter(0, 0, q);
   __syncthreads();
   int kt = 0;
   for (; kt + 1 < nk; kt += 2) {
-    if (SETS == 2) {
-      // register set k % 2 carries step k; even step kt: set 0 is free, set 1 holds step kt+1
-      load_global(0, k_of(kt + 2));
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(0);
-      __builtin_amdgcn_sched_barrier(0);
-      store_lds(SETS - 1, 1);  // stage 1: every wavefront finished reading it one barrier ago
-      __syncthreads();
-      load_global(SETS - 1, k_of(kt + 3));
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(1);
-      __builtin_amdgcn_sched_barrier(0);
-      store_lds(0, 0);
-      __syncthreads();
-    } else {
-      load_global(0, k_of(kt + 1));
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(0);
-      __builtin_amdgcn_sched_barrier(0);
-      store_lds(0, 1);
-      __syncthreads();
-      load_global(0, k_of(kt + 2));
-      __builtin_amdgcn_sched_barrier(0);
-      multiply(1);
-      __builtin_amdgcn_sched_barrier(0);
-      store_lds(0, 0);
-      __syncthreads();
-    }
+    multiply(0, k_of(kt + 2));
+    UNIRL_HEAD_STEP_BARRIER();
+    multiply(1, k_of(kt + 3));
+    UNIRL_HEAD_STEP_BARRIER();
   }
   if (kt < nk) {  // an odd number of steps: the last one sits in stage 0
-    multiply(0);
-    __syncthreads();
+    multiply(0, k_last);
+    UNIRL_HEAD_STEP_BARRIER();
   }
+#undef UNIRL_HEAD_STEP_BARRIER
   UNIRL_TRACE_MARK1();
+#ifdef UNIRL_TRACE
+  // slot 2 of the record: shader cycles of the K loop (low half) and of its barrier waits (high half)
+  trace_m2_ = ((unsigned long long)(clock64() - trace_c0_) & 0xffffffffull) | ((unsigned long long)trace_bar_ << 32);
+#endif
 
   // ---- epilogue: bf16 logits of the tile through LDS, then a row (or half a row) per thread ----
   uint16_t* out = lds;  // BM * kOutRow bf16; the operand stages are free now
@@ -515,19 +552,19 @@ extern "C" size_t unirl_lmhead_logp_scratch_bytes(int64_t rows, int64_t V) {
   return (size_t)rows * (size_t)n_tiles * sizeof(float4) + (size_t)rows * sizeof(float) + 256;
 }
 
-template <int EDGE, int SETS>
+template <int EDGE>
 static int launch_head_tiles(const HeadArgs& A, dim3 grid, hipStream_t st) {
   dim3 block(kHdThreads);
   if (A.bias) {
     if (A.logits_out)
-      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, SETS, true, true>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, true, true>), grid, block, 0, st, A);
     else
-      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, SETS, true, false>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, true, false>), grid, block, 0, st, A);
   } else {
     if (A.logits_out)
-      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, SETS, false, true>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, false, true>), grid, block, 0, st, A);
     else
-      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, SETS, false, false>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, false, false>), grid, block, 0, st, A);
   }
   return (int)hipGetLastError();
 }
@@ -538,6 +575,7 @@ extern "C" int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const vo
                                  int64_t ld_logits, void* scratch, size_t scratch_bytes, void* stream) {
   if (rows < 0 || V <= 0 || K <= 0 || ld_hidden < K || ld_weight < K) return UNIRL_E_SHAPE;
   if (K % kBK != 0 || ld_hidden % 8 != 0 || ld_weight % 8 != 0) return UNIRL_E_SHAPE;  // whole 64-wide K steps, 16-byte rows
+  if (ld_hidden > (1 << 22) || ld_weight > (1 << 22)) return UNIRL_E_LIMIT;  // 32-bit byte offsets inside a 256-row tile
   if (logits_out && ld_logits < V) return UNIRL_E_SHAPE;
   if (rows == 0) return UNIRL_OK;
   if (!hidden || !weight || !scratch) return UNIRL_E_NULL;
@@ -578,7 +616,7 @@ extern "C" int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const vo
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned int)(per_xcd * kXcds));
   UNIRL_TRACE_SET(A, "lmhead_tile", grid.x);
-  int rc = (edge == 256) ? launch_head_tiles<256, 1>(A, grid, st) : launch_head_tiles<128, 2>(A, grid, st);
+  int rc = (edge == 256) ? launch_head_tiles<256>(A, grid, st) : launch_head_tiles<128>(A, grid, st);
   if (rc != 0) return rc;
   const int per_block = kHdThreads / kWave;
   hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned int)((rows + per_block - 1) / per_block)), dim3(kHdThreads), 0,
