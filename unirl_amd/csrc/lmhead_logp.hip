@@ -9,21 +9,23 @@
 //
 // Kernel 1 (lmhead_tile_kernel): one workgroup of four wavefronts (2 x 2) per tile of the logits,
 // 256 x 256 once a call has 1024 rows (one workgroup per compute unit, accumulators in AGPRs), 128
-// x 128 below (two per compute unit).  K is walked in steps of 64 through two LDS stages (global
-// -> registers -> LDS, later steps' loads in flight while the current one is multiplied); each
-// wavefront owns a quarter of the tile as blocks of v_mfma_f32_32x32x16_bf16.  Epilogue:
-// accumulators (+ bias) are rounded to bf16 -- the values the reference's logits hold -- and
-// passed through LDS so that every thread owns a row of the tile (half a row at 128 x 128); it
-// reduces its logits, 64 at a time, to (m, s, t): the maximum, sum 2^a and sum 2^a * a with
-// a = (x - m) * log2(e)/T.  One (m, s, t) per (row, column tile) goes to scratch memory (16 bytes
-// for 256 or 512 bytes of logits) and the tile that holds a row's target column also stores that
-// logit.
+// x 128 below (two per compute unit).  K is walked in steps of 64 through two LDS stages: buffer
+// loads into two register sets run two steps ahead, the stores to LDS one step ahead, and every
+// memory instruction is issued between the step's MFMAs; each wavefront owns a quarter of the tile
+// as blocks of v_mfma_f32_32x32x16_bf16.  Epilogue: accumulators (+ bias) are rounded to bf16 --
+// the values the reference's logits hold -- and passed through LDS transposed, so that a thread
+// owns four rows over a part of the tile's columns; it reduces them to (m, s, t) per row: the
+// maximum, sum 2^a and sum 2^a * a with a = (x - m) * log2(e)/T, and the parts of a row are
+// merged.  One (m, s, t) per (row, column tile) goes to scratch memory (16 bytes for 256 or 512
+// bytes of logits) and the tile that holds a row's target column also stores that logit.
 // Kernel 2 (lmhead_merge_kernel): one wavefront per row merges the row's tile states in fp64 and
 // finishes logsumexp, log-prob and entropy.
 //
 // Tiles are dealt to the workgroups so that each XCD (workgroup id modulo 8) walks its own
 // contiguous range of column groups, row block by row block: the group's slice of W stays in
 // that XCD's L2 while the hidden states stream past it.
+
+#include <type_traits>
 
 #include "common.cuh"
 #include "unirl_internal.h"
@@ -107,8 +109,11 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   constexpr int WM = BM / 2, WN = BN / 2, BI = WM / 32, BJ = WN / 32;
   constexpr int kAElems = BM * kLdsRow, kBElems = BN * kLdsRow, kStage = kAElems + kBElems;
   constexpr int CA = BM * 8 / kHdThreads, CB = BN * 8 / kHdThreads;  // 16-byte chunks per thread and step
-  constexpr int kOutRow = BN + 8;  // bf16 elements per row of the epilogue tile
-  static_assert(BM * kOutRow <= 2 * kStage, "the epilogue tile reuses the operand stages");
+  // epilogue: the tile's bf16 logits transposed, [BN][kOutPitch]; the pitch (BM * 2 + 8 bytes, 2 mod 32
+  // words) spreads the 8-byte stores of 32 lanes on 32 columns over all banks
+  constexpr int kOutPitch = BM + 4;
+  static_assert(BN * kOutPitch * 2 + (kHdThreads / (BM / 4)) * BM * 12 <= 2 * kStage * 2,
+                "the epilogue tile and the partial states reuse the operand stages");
   __shared__ __attribute__((aligned(16))) uint16_t lds[2 * kStage];  // [stage][A rows | B rows][kLdsRow]
   UNIRL_TRACE_T0();
 #ifdef UNIRL_TRACE
@@ -250,8 +255,14 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   trace_m2_ = ((unsigned long long)(clock64() - trace_c0_) & 0xffffffffull) | ((unsigned long long)trace_bar_ << 32);
 #endif
 
-  // ---- epilogue: bf16 logits of the tile through LDS, then a row (or half a row) per thread ----
-  uint16_t* out = lds;  // BM * kOutRow bf16; the operand stages are free now
+  // ---- epilogue ----
+  // The tile's logits -- accumulators (+ bias) rounded to bf16, the values the reference's logits
+  // hold -- go through LDS transposed, tile column by tile column: a lane's four consecutive
+  // accumulators are four consecutive rows of one column, 8 bytes.  Then thread (row quad q,
+  // column part cq) reduces rows 4q .. 4q+3 over the COLS columns of its part: one 8-byte read
+  // per column, consecutive lanes on consecutive row quads (one contiguous run of LDS per
+  // wavefront read).  Per logit: unpack, max, fma, exp2, add, fma.
+  uint16_t* out = lds;  // [BN][kOutPitch] bf16; the operand stages are free now
 #pragma unroll
   for (int bj = 0; bj < BJ; ++bj) {
     const int col = wn * WN + bj * 32 + (lane & 31);
@@ -263,103 +274,126 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
 #pragma unroll
     for (int bi = 0; bi < BI; ++bi) {
 #pragma unroll
-      for (int i = 0; i < 16; ++i) {
-        const int row = wm * WM + bi * 32 + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
-        const float v = HAS_BIAS ? acc[bi][bj][i] + bv : acc[bi][bj][i];
-        out[row * kOutRow + col] = (uint16_t)f32_to_bf16_bits(v);
+      for (int g4 = 0; g4 < 4; ++g4) {
+        const int row = wm * WM + bi * 32 + 8 * g4 + 4 * (lane >> 5);
+        uint32_t b[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) b[k] = f32_to_bf16_bits(HAS_BIAS ? acc[bi][bj][g4 * 4 + k] + bv : acc[bi][bj][g4 * 4 + k]);
+        u32x2 pk;
+        pk.x = b[0] | (b[1] << 16);
+        pk.y = b[2] | (b[3] << 16);
+        *reinterpret_cast<u32x2*>(out + col * kOutPitch + row) = pk;
       }
     }
   }
   __syncthreads();
 
-  constexpr int PARTS = kHdThreads / BM;  // threads that share a row of the tile (2 or 1)
-  constexpr int COLS = BN / PARTS;        // columns each of them reduces, 64 at a time
-  const int row = tid / PARTS, part = tid % PARTS;
-  const int64_t grow = m0 + row;
+  constexpr int NQUAD = BM / 4;              // row quads of the tile
+  constexpr int PARTS = kHdThreads / NQUAD;  // column parts (4 or 8)
+  constexpr int COLS = BN / PARTS;           // columns of a part (64 or 16)
+  constexpr int PIECE = 16;                  // columns between two updates of the running maxima
+  static_assert(COLS % PIECE == 0, "whole pieces");
+  const int q = tid % NQUAD, cq = tid / NQUAD;
   const float c = A.c;
-  int64_t id_col = -1;  // the target's column relative to this thread's first one
-  if (grow < A.M && A.ids) {
-    const int64_t id = A.ids[grow];
-    if (id >= 0 && id < A.N) id_col = id - (n0 + part * COLS);
+  float m[4], sum[4], tsum[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    m[r] = -INFINITY;
+    sum[r] = 0.0f;
+    tsum[r] = 0.0f;
   }
-  float m = -INFINITY, s = 0.0f, t = 0.0f;
-  for (int p0 = 0; p0 < COLS; p0 += 64) {
-    const uint16_t* src = out + row * kOutRow + part * COLS + p0;
-    const int64_t gcol0 = n0 + part * COLS + p0;
-    float x[64];
+  const int64_t gcol0 = n0 + (int64_t)cq * COLS;  // this thread's first column in the vocabulary
+  auto reduce_columns = [&](auto full_tag) {
+    constexpr bool FULL = decltype(full_tag)::value;  // every column of the tile lies inside the vocabulary
+    const uint16_t* src = out + (cq * COLS) * kOutPitch + 4 * q;
+#pragma unroll 1
+    for (int p0 = 0; p0 < COLS; p0 += PIECE) {
+      float x[4][PIECE];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const u32x4 v = *reinterpret_cast<const u32x4*>(src + j * 8);
-      x[j * 8 + 0] = __uint_as_float(v.x << 16);
-      x[j * 8 + 1] = __uint_as_float(v.x & 0xffff0000u);
-      x[j * 8 + 2] = __uint_as_float(v.y << 16);
-      x[j * 8 + 3] = __uint_as_float(v.y & 0xffff0000u);
-      x[j * 8 + 4] = __uint_as_float(v.z << 16);
-      x[j * 8 + 5] = __uint_as_float(v.z & 0xffff0000u);
-      x[j * 8 + 6] = __uint_as_float(v.w << 16);
-      x[j * 8 + 7] = __uint_as_float(v.w & 0xffff0000u);
-    }
-    if (WRITE_LOGITS && grow < A.M) {
-      const bool vec_ok = (A.ld_logits % 8) == 0 && (reinterpret_cast<uintptr_t>(A.logits_out) & 15) == 0;
+      for (int j = 0; j < PIECE; ++j) {
+        const u32x2 v = *reinterpret_cast<const u32x2*>(src + (p0 + j) * kOutPitch);
+        const bool ok = FULL || (gcol0 + p0 + j < A.N);
+        x[0][j] = ok ? __uint_as_float(v.x << 16) : -INFINITY;
+        x[1][j] = ok ? __uint_as_float(v.x & 0xffff0000u) : -INFINITY;
+        x[2][j] = ok ? __uint_as_float(v.y << 16) : -INFINITY;
+        x[3][j] = ok ? __uint_as_float(v.y & 0xffff0000u) : -INFINITY;
+      }
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        if (vec_ok && gcol0 + j * 8 + 8 <= A.N) {
-          *reinterpret_cast<u32x4*>(A.logits_out + grow * A.ld_logits + gcol0 + j * 8) =
-              *reinterpret_cast<const u32x4*>(src + j * 8);
-        } else {
-          for (int k = 0; k < 8; ++k)
-            if (gcol0 + j * 8 + k < A.N) A.logits_out[grow * A.ld_logits + gcol0 + j * 8 + k] = src[j * 8 + k];
+      for (int r = 0; r < 4; ++r) {
+        float pm = x[r][0];
+#pragma unroll
+        for (int j = 1; j < PIECE; ++j) pm = fmaxf(pm, x[r][j]);
+        const float mn = fmaxf(m[r], pm);
+        // raise the reference of what has been summed so far (nothing yet: the sums are zero)
+        const float d = (mn - m[r]) * c;
+        const float f = __builtin_amdgcn_exp2f(-d);
+        const bool had = m[r] != -INFINITY;
+        tsum[r] = had ? f * fmaf(-d, sum[r], tsum[r]) : 0.0f;
+        sum[r] = had ? f * sum[r] : 0.0f;
+        m[r] = mn;
+        if (!FULL && mn == -INFINITY) continue;  // nothing but columns outside the vocabulary so far
+        const float mc = -mn * c;
+#pragma unroll
+        for (int j = 0; j < PIECE; ++j) {
+          // a = (x - m) * c <= 0; a column outside the vocabulary is -inf: e = 0 and e * a must be 0, not NaN
+          const float a = fmaf(x[r][j], c, mc);
+          const float e = __builtin_amdgcn_exp2f(a);
+          sum[r] += e;
+          tsum[r] = (FULL || x[r][j] != -INFINITY) ? fmaf(e, a, tsum[r]) : tsum[r];
         }
       }
     }
-    const int64_t n_valid = A.N - gcol0;  // columns of this piece inside the vocabulary (may be <= 0)
-    float pm = -INFINITY;
+  };
+  if (n0 + BN <= A.N) reduce_columns(std::true_type{});
+  else reduce_columns(std::false_type{});
+
+  // the PARTS partial states of a row meet in LDS above the logits; thread `row` merges them in part order
+  float* part_state = reinterpret_cast<float*>(lds + BN * kOutPitch);  // [PARTS][BM][3]
 #pragma unroll
-    for (int j = 0; j < 64; ++j) pm = (j < n_valid) ? fmaxf(pm, x[j]) : pm;
-    if (pm > m) {  // raise the reference of what has been summed so far
-      if (m != -INFINITY) {
-        const float d = (pm - m) * c, f = __builtin_amdgcn_exp2f(-d);
-        t = f * fmaf(-d, s, t);
-        s = f * s;
+  for (int r = 0; r < 4; ++r) {
+    float* ps = part_state + ((size_t)cq * BM + 4 * q + r) * 3;
+    ps[0] = m[r];
+    ps[1] = sum[r];
+    ps[2] = tsum[r];
+  }
+  __syncthreads();
+  if (tid < BM) {
+    const int row = tid;
+    const int64_t grow = m0 + row;
+    float M = -INFINITY, S = 0.0f, T = 0.0f;
+#pragma unroll
+    for (int p = 0; p < PARTS; ++p) {
+      const float* ps = part_state + ((size_t)p * BM + row) * 3;
+      const float pm = ps[0], psum = ps[1], pt = ps[2];
+      if (pm == -INFINITY) continue;  // a part wholly outside the vocabulary
+      if (M == -INFINITY) {
+        M = pm;
+        S = psum;
+        T = pt;
+        continue;
       }
-      m = pm;
+      const float mm = fmaxf(M, pm);
+      const float d0 = (mm - M) * c, f0 = __builtin_amdgcn_exp2f(-d0);
+      const float d1 = (mm - pm) * c, f1 = __builtin_amdgcn_exp2f(-d1);
+      T = f0 * fmaf(-d0, S, T) + f1 * fmaf(-d1, psum, pt);
+      S = f0 * S + f1 * psum;
+      M = (M != M || pm != pm) ? (M + pm) : mm;
     }
-#pragma unroll
-    for (int j = 0; j < 64; ++j) {
-      if (j < n_valid) {
-        const float a = (x[j] - m) * c;  // <= 0; the difference of two bf16 values is exact in fp32
-        const float e = __builtin_amdgcn_exp2f(a);
-        s += e;
-        t = fmaf(e, a, t);
+    if (grow < A.M) {
+      A.state[grow * A.n_tiles + nt] = make_float4(M, S, T, 0.0f);
+      if (A.ids) {  // the tile that holds the row's target column stores that logit
+        const int64_t id = A.ids[grow];
+        if (id >= n0 && id < n0 + BN && id < A.N) A.xid[grow] = bf16_bits_to_f32(out[(id - n0) * kOutPitch + row]);
       }
-    }
-    const int64_t j_id = id_col - p0;
-    if (j_id >= 0 && j_id < 64) {
-      float xv = 0.0f;
-#pragma unroll
-      for (int k = 0; k < 64; ++k) xv = (k == j_id) ? x[k] : xv;
-      A.xid[grow] = xv;
     }
   }
-  if (PARTS == 2) {  // the two halves of a row sit in neighbouring lanes
-    const float m_o = __shfl_xor(m, 1, kWave), s_o = __shfl_xor(s, 1, kWave), t_o = __shfl_xor(t, 1, kWave);
-    const float mm = fmaxf(m, m_o);
-    float S = 0.0f, T = 0.0f;
-    if (m != -INFINITY) {
-      const float d = (mm - m) * c, f = __builtin_amdgcn_exp2f(-d);
-      S = f * s;
-      T = f * fmaf(-d, s, t);
+  if (WRITE_LOGITS) {  // validation: the tile's logits, row by row
+    for (int idx = tid; idx < BM * BN; idx += kHdThreads) {
+      const int row = idx / BN, col = idx % BN;
+      const int64_t grow = m0 + row, gcol = n0 + col;
+      if (grow < A.M && gcol < A.N) A.logits_out[grow * A.ld_logits + gcol] = out[col * kOutPitch + row];
     }
-    if (m_o != -INFINITY) {
-      const float d = (mm - m_o) * c, f = __builtin_amdgcn_exp2f(-d);
-      S += f * s_o;
-      T += f * fmaf(-d, s_o, t_o);
-    }
-    m = mm;
-    s = S;
-    t = T;
   }
-  if (part == 0 && grow < A.M) A.state[grow * A.n_tiles + nt] = make_float4(m, s, t, 0.0f);
   UNIRL_TRACE_END(A.trace);
 }
 
