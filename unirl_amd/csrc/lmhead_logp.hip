@@ -142,23 +142,24 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   const int va_step = (int)(32 * A.ldh * 2), vb_step = (int)(32 * A.ldw * 2);  // chunk i sits 32 rows further down
   const int lds_off0 = row0 * kLdsRow + kc * 8;
   // Two register sets stage the operands of two K steps between global memory and LDS.  A step's
-  // CA + CB loads (and, a step later, its stores to LDS) are issued a quarter at a time, one
-  // quarter under each 16-wide slice of the multiplication.
+  // CA + CB loads go out a quarter under each 16-wide slice of the multiplication and, a step
+  // later, its stores to LDS a third under each of the first three slices.
   constexpr int NW = CA + CB, NQ = NW / 4;
-  static_assert(NW % 4 == 0 && CA % NQ == 0, "a quarter of a step's chunks lies inside one operand");
+  static_assert(NW % 4 == 0, "a quarter of a step's chunks per slice");
+  constexpr int W0 = (NW + 2) / 3, W1 = (NW - W0 + 1) / 2;  // stores under slices 0 and 1; the rest under slice 2
   u32x4 gs[2][NW];  // [set][chunk]: chunks 0 .. CA-1 of the hidden states, CA .. of the weight
-  auto load_quarter = [&](int set, int64_t k0, int q) {
+  auto load_range = [&](int set, int64_t k0, int j0, int j1) {
     const int sk = (int)(k0 * 2);
 #pragma unroll
-    for (int j = q * NQ; j < (q + 1) * NQ; ++j)
+    for (int j = j0; j < j1; ++j)
       gs[set][j] = (j < CA) ? __builtin_amdgcn_raw_buffer_load_b128(ra, va0 + j * va_step, sk, 0)
                             : __builtin_amdgcn_raw_buffer_load_b128(rb, vb0 + (j - CA) * vb_step, sk, 0);
   };
-  auto store_quarter = [&](int set, int stage, int q) {
+  auto store_range = [&](int set, int stage, int j0, int j1) {
     uint16_t* sa = lds + stage * kStage;
     uint16_t* sb = sa + kAElems;
 #pragma unroll
-    for (int j = q * NQ; j < (q + 1) * NQ; ++j)
+    for (int j = j0; j < j1; ++j)
       *reinterpret_cast<u32x4*>((j < CA ? sa + j * 32 * kLdsRow : sb + (j - CA) * 32 * kLdsRow) + lds_off0) = gs[set][j];
   };
 
@@ -183,42 +184,19 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
     for (int bj = 0; bj < BJ; ++bj) b[bj] = lds_frag(sb + frag_b + bj * 32 * kLdsRow + ks * 16);
   };
   constexpr int NR = BI + BJ, NM = BI * BJ;  // LDS reads and MFMAs per K slice
-  // One K step out of LDS stage `stage`.  Under it travel, a quarter per slice: the loads of step
-  // k + 2 into register set `stage` (which held this step's operands until they were stored a step
-  // ago) and the stores of step k + 1's operands (register set stage ^ 1, loaded a step ago) into
-  // the other LDS stage, which every wavefront finished reading one barrier ago.  The fragments of
-  // slice ks + 1 are read while slice ks is multiplied.  So every memory instruction is issued
-  // between matrix instructions: a wavefront issues in order, and a burst of sixteen loads or
-  // stores holds up the MFMAs behind it for as long as the memory pipeline takes to accept them
-  // (measured: the bursts cost 0.9 us of a 1.8 us step).  The scheduling fences keep each slice's
-  // instructions together; inside a slice sched_slice deals them out among the MFMAs.
-  auto multiply = [&](int stage, int64_t k_load) {
-    read_frags(stage, 0, fa[0], fb[0]);
-#pragma unroll
-    for (int ks = 0; ks < kBK / 16; ++ks) {
-      const int cur = ks & 1;
-      if (ks + 1 < kBK / 16) read_frags(stage, ks + 1, fa[cur ^ 1], fb[cur ^ 1]);
-      load_quarter(stage, k_load, ks);
-      store_quarter(stage ^ 1, stage ^ 1, ks);
-#pragma unroll
-      for (int bi = 0; bi < BI; ++bi)
-#pragma unroll
-        for (int bj = 0; bj < BJ; ++bj)
-          acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][bi], fb[cur][bj], acc[bi][bj], 0, 0, 0);
-      if (ks + 1 < kBK / 16) sched_slice<NM, NR, NQ, NQ>();
-      else sched_slice<NM, 0, NQ, NQ>();
-      __builtin_amdgcn_sched_barrier(0);
-    }
-  };
-
-  // Step k sits in LDS stage k % 2 and came through register set k % 2.  Every trip issues its
-  // loads and stores unconditionally (past the last step the loads repeat the last step's
-  // addresses and the stores fill a stage nobody reads any more): with a branch around them the
-  // compiler can no longer count which loads are outstanding at the stores and waits for all of
-  // them.
-  const int nk = (int)(A.K / kBK);
-  const int64_t k_last = (int64_t)(nk - 1) * kBK;
-  auto k_of = [&](int step) { return step < nk ? (int64_t)step * kBK : k_last; };
+  // One K step out of LDS stage `stage`, as four slices of NM matrix instructions.  Under them
+  // travel: the loads of step k + 2 into register set `stage` (which held this step's operands
+  // until they were stored a step ago), a quarter per slice; the stores of step k + 1's operands
+  // (register set stage ^ 1, loaded a step ago) into the other LDS stage, under slices 0 - 2; and
+  // the fragment reads of the next slice.  The step's barrier stands before its LAST slice: by
+  // then every wavefront has read this stage's last fragments and stored its share of the next
+  // stage, so the last slice already reads the next step's first fragments and no slice waits for
+  // LDS behind a barrier.  (The next step's stores go to this stage, which nobody reads any more.)
+  // Every memory instruction is issued between matrix instructions: a wavefront issues in order,
+  // and a burst of sixteen loads or stores holds up the MFMAs behind it for as long as the memory
+  // pipeline takes to accept them (measured: the bursts cost 0.9 us of a 1.8 us step).  The
+  // scheduling fences keep each slice's instructions together; inside a slice sched_slice deals
+  // them out among the MFMAs.
 #ifdef UNIRL_TRACE
   long long trace_bar_ = 0;  // shader cycles this wavefront spent waiting at the step barriers
 #define UNIRL_HEAD_STEP_BARRIER()              \
@@ -230,25 +208,65 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
 #else
 #define UNIRL_HEAD_STEP_BARRIER() __syncthreads()
 #endif
+  // (With two workgroups on a compute unit -- the 128 x 128 tile -- the other workgroup fills such
+  // waits, and the plain arrangement measures faster: barrier at the end of the step, the stores a
+  // quarter under each slice, the step's first fragments read after the barrier.)
+  constexpr bool kEarlyBarrier = BM * BN > 128 * 128;
+  auto multiply = [&](int stage, int64_t k_load) {
+    if (!kEarlyBarrier) read_frags(stage, 0, fa[0], fb[0]);
 #pragma unroll
-  for (int q = 0; q < 4; ++q) load_quarter(0, 0, q);
+    for (int ks = 0; ks < kBK / 16; ++ks) {
+      const int cur = ks & 1;
+      if (ks + 1 < kBK / 16) read_frags(stage, ks + 1, fa[cur ^ 1], fb[cur ^ 1]);
+      else if (kEarlyBarrier) read_frags(stage ^ 1, 0, fa[cur ^ 1], fb[cur ^ 1]);  // the next step's first slice
+      load_range(stage, k_load, ks * NQ, (ks + 1) * NQ);
+      if (kEarlyBarrier) {
+        if (ks == 0) store_range(stage ^ 1, stage ^ 1, 0, W0);
+        if (ks == 1) store_range(stage ^ 1, stage ^ 1, W0, W0 + W1);
+        if (ks == 2) store_range(stage ^ 1, stage ^ 1, W0 + W1, NW);
+      } else {
+        store_range(stage ^ 1, stage ^ 1, ks * NQ, (ks + 1) * NQ);
+      }
 #pragma unroll
-  for (int q = 0; q < 4; ++q) load_quarter(1, k_of(1), q);
+      for (int bi = 0; bi < BI; ++bi)
 #pragma unroll
-  for (int q = 0; q < 4; ++q) store_quarter(0, 0, q);
+        for (int bj = 0; bj < BJ; ++bj)
+          acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][bi], fb[cur][bj], acc[bi][bj], 0, 0, 0);
+      if (kEarlyBarrier) {
+        if (ks == 0) sched_slice<NM, NR, W0, NQ>();
+        if (ks == 1) sched_slice<NM, NR, W1, NQ>();
+        if (ks == 2) sched_slice<NM, NR, NW - W0 - W1, NQ>();
+        if (ks == 3) sched_slice<NM, NR, 0, NQ>();
+      } else {
+        if (ks + 1 < kBK / 16) sched_slice<NM, NR, NQ, NQ>();
+        else sched_slice<NM, 0, NQ, NQ>();
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (ks == (kEarlyBarrier ? 2 : 3)) UNIRL_HEAD_STEP_BARRIER();
+    }
+  };
+
+  // Step k sits in LDS stage k % 2 and came through register set k % 2.  Every trip issues its
+  // loads and stores unconditionally (past the last step the loads repeat the last step's
+  // addresses and the stores fill a stage nobody multiplies any more): with a branch around them
+  // the compiler can no longer count which loads are outstanding at the stores and waits for all
+  // of them.
+  const int nk = (int)(A.K / kBK);
+  const int64_t k_last = (int64_t)(nk - 1) * kBK;
+  auto k_of = [&](int step) { return step < nk ? (int64_t)step * kBK : k_last; };
+  load_range(0, 0, 0, NW);
+  load_range(1, k_of(1), 0, NW);
+  store_range(0, 0, 0, NW);
   __syncthreads();
+  if (kEarlyBarrier) read_frags(0, 0, fa[0], fb[0]);
   int kt = 0;
   for (; kt + 1 < nk; kt += 2) {
     multiply(0, k_of(kt + 2));
-    UNIRL_HEAD_STEP_BARRIER();
     multiply(1, k_of(kt + 3));
-    UNIRL_HEAD_STEP_BARRIER();
   }
-  if (kt < nk) {  // an odd number of steps: the last one sits in stage 0
-    multiply(0, k_last);
-    UNIRL_HEAD_STEP_BARRIER();
-  }
+  if (kt < nk) multiply(0, k_last);  // an odd number of steps: the last one sits in stage 0
 #undef UNIRL_HEAD_STEP_BARRIER
+  if (kEarlyBarrier) __syncthreads();  // the last slice's reads of the other stage are done before the epilogue writes over it
   UNIRL_TRACE_MARK1();
 #ifdef UNIRL_TRACE
   // slot 2 of the record: shader cycles of the K loop (low half) and of its barrier waits (high half)
