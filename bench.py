@@ -488,10 +488,14 @@ def head_probe(torch, dev, vocab: int, hidden: int = 2560):
     g = torch.Generator(device=dev).manual_seed(0)
     w = (torch.randn(vocab, hidden, generator=g, device=dev) * (3.0 / math.sqrt(hidden))).bfloat16()
 
-    def timed(fn, n=5):
-        for _ in range(2):
-            fn()
-        torch.cuda.synchronize()
+    def timed(fn, n=10):
+        # a quarter of a second of the same calls first: the clocks of an idle device ramp over the
+        # first few hundred milliseconds of work (a 1.5 ms call measured cold reads 20 % slow)
+        t_end = time.perf_counter() + 0.25
+        while time.perf_counter() < t_end:
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
         for _ in range(n):
@@ -501,7 +505,7 @@ def head_probe(torch, dev, vocab: int, hidden: int = 2560):
         return a.elapsed_time(b) / n
 
     out = []
-    for rows in (64, 2048, 8192):
+    for rows in (64, 256, 1024, 2048, 8192):
         h = torch.randn(rows, hidden, generator=g, device=dev).bfloat16()
         ids = torch.randint(0, vocab, (rows,), generator=g, device=dev)
         flop = 2.0 * rows * hidden * vocab
