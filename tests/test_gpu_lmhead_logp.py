@@ -68,7 +68,10 @@ def check_against_oracle(dev, h, w, b, ids, T, what):
 
 
 @pytest.mark.parametrize("rows,K,V,bias", [(64, 256, 1024, False), (130, 128, 300, True), (1, 64, 129, False),
-                                           (257, 192, 1000, True), (128, 2560, 640, False)])
+                                           (257, 192, 1000, True), (128, 2560, 640, False),
+                                           # the 256 x 256 tile: exact fit, ragged rows and columns, one K step
+                                           (512, 64, 256, False), (300, 128, 700, True), (1000, 320, 513, True),
+                                           (255, 128, 257, False), (256, 64, 1, False)])
 @pytest.mark.parametrize("T", [1.0, 0.7])
 def test_small_heads_match_oracle(dev, rows, K, V, bias, T):
     h, w, b, ids = make(rows, K, V, seed=rows + K + V, bias=bias, scale=4.0)
