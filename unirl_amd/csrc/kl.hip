@@ -256,10 +256,10 @@ struct DppoAcc {
 };
 
 // Element i of the [B,S'] problem: ratio, the two removal masks, the kept loss (and its gradient).
-__device__ __forceinline__ void dppo_elem(const DppoArgs& A, int64_t i, float kl, DppoAcc& s) {
-  const float ld = A.nw[i] - A.od[i];
+__device__ __forceinline__ void dppo_elem_of(const DppoArgs& A, int64_t i, float nw, float od, float a, float kl,
+                                             DppoAcc& s) {
+  const float ld = nw - od;
   const float r = expf(ld);
-  const float a = A.adv[i];
   const bool low_kl = kl < A.threshold;
   const bool pos = !low_kl && (r > 1.0f) && (a > 0.0f);
   const bool neg = !low_kl && (r < 1.0f) && (a < 0.0f);
@@ -279,6 +279,10 @@ __device__ __forceinline__ void dppo_elem(const DppoArgs& A, int64_t i, float kl
   s.rmin = fminf(s.rmin, r);
   s.rmax = fmaxf(s.rmax, r);
   s.klmax = fmaxf(s.klmax, kl);
+}
+
+__device__ __forceinline__ void dppo_elem(const DppoArgs& A, int64_t i, float kl, DppoAcc& s) {
+  dppo_elem_of(A, i, A.nw[i], A.od[i], A.adv[i], kl, s);
 }
 
 // The twelve metrics from the totals; one thread.
@@ -314,10 +318,16 @@ __device__ __forceinline__ void dppo_metrics(const DppoArgs& A, const double (&t
 
 // The whole [B,S'] problem on one wavefront (it is a few dozen elements): no barriers, the
 // reductions are DPP only.  `kl` points at global or LDS memory.  Every lane must call.
-__device__ __forceinline__ void dppo_on_one_wave(const DppoArgs& A, const float* kl) {
+// `first`: the lane's first element (new, old, advantage), already loaded by the caller, or null.
+__device__ __forceinline__ void dppo_on_one_wave(const DppoArgs& A, const float* kl, const float* first = nullptr) {
   const int lane = threadIdx.x & (kWave - 1);
   DppoAcc s;
-  for (int64_t i = lane; i < A.n; i += kWave) dppo_elem(A, i, kl[i], s);
+  int64_t i = lane;
+  if (first && i < A.n) {
+    dppo_elem_of(A, i, first[0], first[1], first[2], kl[i], s);
+    i += kWave;
+  }
+  for (; i < A.n; i += kWave) dppo_elem(A, i, kl[i], s);
   double tot[D_SUMS];
 #pragma unroll
   for (int v = 0; v < D_SUMS; ++v) tot[v] = wave_sum(s.acc[v]);
@@ -352,6 +362,13 @@ __global__ __launch_bounds__(kKlThreads) void flowdppo_finish_kernel(KlArgs K, D
   UNIRL_TRACE_T0();
   const int wave = threadIdx.x / kWave;
   const int64_t R = A.n;
+  // the first wavefront's share of the [B,S'] problem is loaded now, with the partials, not after them
+  float first[3] = {0.0f, 0.0f, 0.0f};
+  if (wave == 0 && (int64_t)threadIdx.x < A.n) {
+    first[0] = A.nw[threadIdx.x];
+    first[1] = A.od[threadIdx.x];
+    first[2] = A.adv[threadIdx.x];
+  }
   for (int64_t row = wave; row < R; row += kKlThreads / kWave) {
     const float den = kl_den(K, row);  // issued with the partial loads, not after them
     const double q = wave_ordered_sum(K.partials + row * nblk, nblk);
@@ -364,7 +381,7 @@ __global__ __launch_bounds__(kKlThreads) void flowdppo_finish_kernel(KlArgs K, D
   }
   UNIRL_TRACE_MARK1();
   __syncthreads();
-  if (wave == 0) dppo_on_one_wave(A, lds_kl);
+  if (wave == 0) dppo_on_one_wave(A, lds_kl, first);
   UNIRL_TRACE_END(K.trace);
 }
 
