@@ -23,7 +23,7 @@ def stub_namespace():
 
     text = (ROOT / "INTEGRATION.md").read_text()
     blocks = re.findall(r"```python\n(.*?)```", text, flags=re.S)
-    code = [b for b in blocks if "predict_noise(...)" not in b]  # the loop sketch is not runnable on its own
+    code = [b for b in blocks if "self.strategy." not in b]  # the two loop sketches are not runnable on their own
     assert len(code) == 4, "stub, denoise_hip, logp_chunk_hip, kl_mask_hip"
     source = "\n".join(code).replace('ctypes.CDLL("libunirl_hip.so")', f'ctypes.CDLL("{N.LIB_PATH}")')
     ns = {}
