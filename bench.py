@@ -114,6 +114,21 @@ def wrapper_latency_us(torch, fn, reps: int = 20):
     return statistics.median(out)
 
 
+def host_issue_us(torch, fn, reps: int = 300):
+    """Python time per call when nothing waits for the device: `reps` calls issued back to back (the
+    device queue is far deeper), microseconds per call.  This is what the wrapper itself costs."""
+    best = float("inf")
+    for _ in range(3):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(reps):
+            fn(i)
+        t1 = time.perf_counter()
+        torch.cuda.synchronize()
+        best = min(best, (t1 - t0) * 1e6 / reps)
+    return best
+
+
 # ----------------------------------------------------------------------------------------------
 # the five synthetic shapes of BASELINE.json
 # ----------------------------------------------------------------------------------------------
@@ -849,13 +864,14 @@ def main() -> int:
                 _, ms = time_steps(torch, sh["run"], 200, 20)
                 us, method = ms * 1e3, "hip events over 200 stream-ordered launches (launch-bound)"
             lat = wrapper_latency_us(torch, sh["run"])
+            host = host_issue_us(torch, sh["run"])
             gbps = sh["bytes"] / (us * 1e-6) / 1e9
             row = {
                 "name": sh["name"], "config": sh["config"], "shape": sh["shape"], "algorithmic_bytes": sh["bytes"],
                 "elements": sh["elements"], "kernel_us": round(us, 2), "gbps": round(gbps, 1),
                 "frac_of_peak": round(gbps / HBM_PEAK_GBPS, 4),
                 "elements_per_s": round(sh["elements"] / (us * 1e-6), 0), "wrapper_latency_us": round(lat, 1),
-                "timing": method,
+                "host_issue_us": round(host, 1), "timing": method,
             }
             if "bytes_padded" in sh:
                 row["gbps_padded_bytes"] = round(sh["bytes_padded"] / (us * 1e-6) / 1e9, 1)
@@ -889,7 +905,7 @@ def main() -> int:
                 row["cpu_gbps"] = round(sh["cpu_bytes"] / (cms * 1e-3) / 1e9, 3)
                 row["cpu_cores"] = torch.get_num_threads()
             log(f"{sh['name']}: {us:.2f} us/launch, {gbps:.0f} GB/s = {gbps / HBM_PEAK_GBPS:.1%} of peak, "
-                f"floor {row.get('floor_us', float('nan')):.2f} us, wrapper {lat:.0f} us")
+                f"floor {row.get('floor_us', float('nan')):.2f} us, call + sync {lat:.0f} us, host {host:.0f} us")
             shapes_out.append(row)
 
     # HBM bytes per launch from hardware counters.  Counter runs cannot be made from inside the bench,

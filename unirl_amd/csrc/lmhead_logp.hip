@@ -8,16 +8,20 @@
 // (K contiguous): both operands are read along K, the layout MFMA fragments want.
 //
 // Kernel 1 (lmhead_tile_kernel): one workgroup of four wavefronts (2 x 2) per tile of the logits,
-// 256 x 256 once a call has 1024 rows (one workgroup per compute unit, accumulators in AGPRs), 128
-// x 128 below (two per compute unit).  K is walked in steps of 64 through two LDS stages: buffer
-// loads into two register sets run two steps ahead, the stores to LDS one step ahead, and every
-// memory instruction is issued between the step's MFMAs; each wavefront owns a quarter of the tile
-// as blocks of v_mfma_f32_32x32x16_bf16.  Epilogue: accumulators (+ bias) are rounded to bf16 --
-// the values the reference's logits hold -- and passed through LDS transposed, so that a thread
-// owns four rows over a part of the tile's columns; it reduces them to (m, s, t) per row: the
-// maximum, sum 2^a and sum 2^a * a with a = (x - m) * log2(e)/T, and the parts of a row are
-// merged.  One (m, s, t) per (row, column tile) goes to scratch memory (16 bytes for 256 or 512
-// bytes of logits) and the tile that holds a row's target column also stores that logit.
+// 256 x 256 from 256 rows (one workgroup per compute unit, accumulators in AGPRs), 128 x 128 below
+// (two per compute unit).  K is walked in steps of 64 through two LDS stages; each wavefront owns
+// a quarter of the tile as blocks of v_mfma_f32_32x32x16_bf16, its fragments double-buffered in
+// registers, and every memory instruction is issued between the step's MFMAs.  The operands reach
+// LDS in one of two ways: from 512 rows straight from global memory (buffer loads with the LDS
+// as destination, unpadded rows, bank conflicts avoided by an XOR swizzle applied on the global
+// side), half a step's loads under the step's first slice and half under the previous step's
+// last; below, through two register sets, loads two steps ahead and stores to LDS one step
+// ahead.  Epilogue: accumulators (+ bias) are rounded to bf16 -- the values the reference's
+// logits hold -- and passed through LDS transposed, so that a thread owns four rows over a part
+// of the tile's columns; it reduces them to (m, s, t) per row: the maximum, sum 2^a and sum
+// 2^a * a with a = (x - m) * log2(e)/T, and the parts of a row are merged.  One (m, s, t) per (row,
+// column tile) goes to scratch memory (16 bytes for 256 or 512 bytes of logits) and the tile that
+// holds a row's target column also stores that logit.
 // Kernel 2 (lmhead_merge_kernel): one wavefront per row merges the row's tile states in fp64 and
 // finishes logsumexp, log-prob and entropy.
 //
@@ -104,7 +108,7 @@ __device__ __forceinline__ void sched_slice() {
 
 // BM x BN: the workgroup's tile of the logits; its four wavefronts sit 2 x 2, each on a
 // (BM/2) x (BN/2) quarter of BI x BJ MFMA blocks.
-template <int BM, int BN, bool HAS_BIAS, bool WRITE_LOGITS>
+template <int BM, int BN, bool HAS_BIAS, bool WRITE_LOGITS, bool DMA = false>
 __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmhead_tile_kernel(HeadArgs A) {
   constexpr int WM = BM / 2, WN = BN / 2, BI = WM / 32, BJ = WN / 32;
   constexpr int kAElems = BM * kLdsRow, kBElems = BN * kLdsRow, kStage = kAElems + kBElems;
@@ -141,6 +145,24 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   const int va0 = (int)((row0 * A.ldh + kc * 8) * 2), vb0 = (int)((row0 * A.ldw + kc * 8) * 2);
   const int va_step = (int)(32 * A.ldh * 2), vb_step = (int)(32 * A.ldw * 2);  // chunk i sits 32 rows further down
   const int lds_off0 = row0 * kLdsRow + kc * 8;
+  // DMA: global -> LDS without registers.  One instruction of a wavefront fills 1 KB of LDS, lane by
+  // lane: 8 operand rows of 128 bytes, unpadded.  Bank conflicts are avoided by an XOR swizzle on
+  // the global side: the lane that fills slot (row r, chunk c) fetches chunk c ^ (r % 8).  Stage =
+  // [BM + BN rows][64]; instruction i = 4 j + wave covers rows 8 i .. 8 i + 7 of (hidden rows, weight rows).
+  constexpr int kStageD = (BM + BN) * kBK;
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  const int dr = lane >> 3, dc = (lane & 7) ^ (lane >> 3);
+  const int da0 = (int)((((int64_t)wave_u * 8 + dr) * A.ldh + dc * 8) * 2);
+  const int db0 = (int)((((int64_t)wave_u * 8 + dr) * A.ldw + dc * 8) * 2);
+  auto dma_range = [&](int stage, int64_t k0, int j0, int j1) {
+    const int sk = (int)(k0 * 2);
+#pragma unroll
+    for (int j = j0; j < j1; ++j) {
+      auto* dst = (__attribute__((address_space(3))) void*)(lds + stage * kStageD + (j * 4 + wave_u) * 512);
+      if (j < CA) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, dst, 16, da0 + j * va_step, sk, 0, 0);
+      else __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, dst, 16, db0 + (j - CA) * vb_step, sk, 0, 0);
+    }
+  };
   // Two register sets stage the operands of two K steps between global memory and LDS.  A step's
   // CA + CB loads go out a quarter under each 16-wide slice of the multiplication and, a step
   // later, its stores to LDS a third under each of the first three slices.
@@ -175,13 +197,31 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   const int frag_a = (wm * WM + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
   const int frag_b = (wn * WN + (lane & 31)) * kLdsRow + 8 * (lane >> 5);
   bf16x8_t fa[2][BI], fb[2][BJ];  // the fragments of two consecutive 16-wide K slices
+  // DMA layout: slot of (row, chunk kc) is chunk kc ^ (row % 8); row % 8 = lane % 8 for every block
+  int fsw[kBK / 16];
+#pragma unroll
+  for (int ks = 0; ks < kBK / 16; ++ks) fsw[ks] = (lane & 31) * kBK + (((2 * ks + (lane >> 5)) ^ (lane & 7)) * 8);
   auto read_frags = [&](int stage, int ks, bf16x8_t(&a)[BI], bf16x8_t(&b)[BJ]) {
+    if (DMA) {
+      const uint16_t* sa = lds + stage * kStageD + (wm * WM) * kBK + fsw[ks];
+      const uint16_t* sb = lds + stage * kStageD + (BM + wn * WN) * kBK + fsw[ks];
+#pragma unroll
+      for (int bi = 0; bi < BI; ++bi) a[bi] = lds_frag(sa + bi * 32 * kBK);
+#pragma unroll
+      for (int bj = 0; bj < BJ; ++bj) b[bj] = lds_frag(sb + bj * 32 * kBK);
+      return;
+    }
     const uint16_t* sa = lds + stage * kStage;
     const uint16_t* sb = sa + kAElems;
 #pragma unroll
     for (int bi = 0; bi < BI; ++bi) a[bi] = lds_frag(sa + frag_a + bi * 32 * kLdsRow + ks * 16);
 #pragma unroll
     for (int bj = 0; bj < BJ; ++bj) b[bj] = lds_frag(sb + frag_b + bj * 32 * kLdsRow + ks * 16);
+  };
+  // DMA mode, one fragment: index < BI of the hidden-state blocks, else of the weight blocks
+  auto read_one = [&](int stage, int ks, int idx, bf16x8_t(&a)[BI], bf16x8_t(&b)[BJ]) {
+    if (idx < BI) a[idx] = lds_frag(lds + stage * kStageD + (wm * WM + idx * 32) * kBK + fsw[ks]);
+    else b[idx - BI] = lds_frag(lds + stage * kStageD + (BM + wn * WN + (idx - BI) * 32) * kBK + fsw[ks]);
   };
   constexpr int NR = BI + BJ, NM = BI * BJ;  // LDS reads and MFMAs per K slice
   // One K step out of LDS stage `stage`, as four slices of NM matrix instructions.  Under them
@@ -211,16 +251,32 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   // (With two workgroups on a compute unit -- the 128 x 128 tile -- the other workgroup fills such
   // waits, and the plain arrangement measures faster: barrier at the end of the step, the stores a
   // quarter under each slice, the step's first fragments read after the barrier.)
-  constexpr bool kEarlyBarrier = BM * BN > 128 * 128;
-  auto multiply = [&](int stage, int64_t k_load) {
+  constexpr bool kEarlyBarrier = DMA || BM * BN > 128 * 128;
+  auto multiply = [&](int stage, int64_t k_load, int64_t k_load2) {
     if (!kEarlyBarrier) read_frags(stage, 0, fa[0], fb[0]);
 #pragma unroll
     for (int ks = 0; ks < kBK / 16; ++ks) {
       const int cur = ks & 1;
-      if (ks + 1 < kBK / 16) read_frags(stage, ks + 1, fa[cur ^ 1], fb[cur ^ 1]);
-      else if (kEarlyBarrier) read_frags(stage ^ 1, 0, fa[cur ^ 1], fb[cur ^ 1]);  // the next step's first slice
-      load_range(stage, k_load, ks * NQ, (ks + 1) * NQ);
-      if (kEarlyBarrier) {
+      if (DMA) {
+        // the other stage is free from the previous step's barrier to this step's: the second half
+        // of step k + 1 goes into it now, the first half went under the previous step's last slice;
+        // after this step's barrier this stage is free and takes the first half of step k + 2.
+        // Loads into LDS and reads of LDS keep their program order, so they alternate here.
+        static_assert(NW / 2 <= NR, "at most one load per fragment read");
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+          if (ks + 1 < kBK / 16) read_one(stage, ks + 1, i, fa[cur ^ 1], fb[cur ^ 1]);
+          else read_one(stage ^ 1, 0, i, fa[cur ^ 1], fb[cur ^ 1]);
+          if (ks == 0 && i < NW / 2) dma_range(stage ^ 1, k_load, NW / 2 + i, NW / 2 + i + 1);
+          if (ks == 3 && i < NW / 2) dma_range(stage, k_load2, i, i + 1);
+        }
+      } else {
+        if (ks + 1 < kBK / 16) read_frags(stage, ks + 1, fa[cur ^ 1], fb[cur ^ 1]);
+        else if (kEarlyBarrier) read_frags(stage ^ 1, 0, fa[cur ^ 1], fb[cur ^ 1]);  // the next step's first slice
+        load_range(stage, k_load, ks * NQ, (ks + 1) * NQ);
+      }
+      if (DMA) {
+      } else if (kEarlyBarrier) {
         if (ks == 0) store_range(stage ^ 1, stage ^ 1, 0, W0);
         if (ks == 1) store_range(stage ^ 1, stage ^ 1, W0, W0 + W1);
         if (ks == 2) store_range(stage ^ 1, stage ^ 1, W0 + W1, NW);
@@ -232,7 +288,10 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
 #pragma unroll
         for (int bj = 0; bj < BJ; ++bj)
           acc[bi][bj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][bi], fb[cur][bj], acc[bi][bj], 0, 0, 0);
-      if (kEarlyBarrier) {
+      if (DMA) {
+        if (ks == 0 || ks == 3) sched_slice<NM, NR, 0, NW / 2>();
+        else sched_slice<NM, NR, 0, 0>();
+      } else if (kEarlyBarrier) {
         if (ks == 0) sched_slice<NM, NR, W0, NQ>();
         if (ks == 1) sched_slice<NM, NR, W1, NQ>();
         if (ks == 2) sched_slice<NM, NR, NW - W0 - W1, NQ>();
@@ -254,17 +313,23 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
   const int nk = (int)(A.K / kBK);
   const int64_t k_last = (int64_t)(nk - 1) * kBK;
   auto k_of = [&](int step) { return step < nk ? (int64_t)step * kBK : k_last; };
-  load_range(0, 0, 0, NW);
-  load_range(1, k_of(1), 0, NW);
-  store_range(0, 0, 0, NW);
-  __syncthreads();
+  if (DMA) {
+    dma_range(0, 0, 0, NW);
+    __syncthreads();
+    dma_range(1, k_of(1), 0, NW / 2);
+  } else {
+    load_range(0, 0, 0, NW);
+    load_range(1, k_of(1), 0, NW);
+    store_range(0, 0, 0, NW);
+    __syncthreads();
+  }
   if (kEarlyBarrier) read_frags(0, 0, fa[0], fb[0]);
   int kt = 0;
   for (; kt + 1 < nk; kt += 2) {
-    multiply(0, k_of(kt + 2));
-    multiply(1, k_of(kt + 3));
+    multiply(0, DMA ? k_of(kt + 1) : k_of(kt + 2), k_of(kt + 2));
+    multiply(1, DMA ? k_of(kt + 2) : k_of(kt + 3), k_of(kt + 3));
   }
-  if (kt < nk) multiply(0, k_last);  // an odd number of steps: the last one sits in stage 0
+  if (kt < nk) multiply(0, k_last, k_last);  // an odd number of steps: the last one sits in stage 0
 #undef UNIRL_HEAD_STEP_BARRIER
   if (kEarlyBarrier) __syncthreads();  // the last slice's reads of the other stage are done before the epilogue writes over it
   UNIRL_TRACE_MARK1();
@@ -605,19 +670,19 @@ extern "C" size_t unirl_lmhead_logp_scratch_bytes(int64_t rows, int64_t V) {
   return (size_t)rows * (size_t)n_tiles * sizeof(float4) + (size_t)rows * sizeof(float) + 256;
 }
 
-template <int EDGE>
+template <int EDGE, bool DMA>
 static int launch_head_tiles(const HeadArgs& A, dim3 grid, hipStream_t st) {
   dim3 block(kHdThreads);
   if (A.bias) {
     if (A.logits_out)
-      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, true, true>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, true, true, DMA>), grid, block, 0, st, A);
     else
-      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, true, false>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, true, false, DMA>), grid, block, 0, st, A);
   } else {
     if (A.logits_out)
-      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, false, true>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, false, true, DMA>), grid, block, 0, st, A);
     else
-      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, false, false>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((lmhead_tile_kernel<EDGE, EDGE, false, false, DMA>), grid, block, 0, st, A);
   }
   return (int)hipGetLastError();
 }
@@ -669,7 +734,10 @@ extern "C" int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const vo
   hipStream_t st = (hipStream_t)stream;
   dim3 grid((unsigned int)(per_xcd * kXcds));
   UNIRL_TRACE_SET(A, "lmhead_tile", grid.x);
-  int rc = (edge == 256) ? launch_head_tiles<256>(A, grid, st) : launch_head_tiles<128>(A, grid, st);
+  // from 512 rows the operands of the 256 x 256 tile travel global memory -> LDS directly
+  const bool dma = edge == 256 && rows >= (int64_t)tune_int("UNIRL_HEAD_DMA_ROWS", 512);
+  int rc = (edge == 256) ? (dma ? launch_head_tiles<256, true>(A, grid, st) : launch_head_tiles<256, false>(A, grid, st))
+                         : launch_head_tiles<128, false>(A, grid, st);
   if (rc != 0) return rc;
   const int per_block = kHdThreads / kWave;
   hipLaunchKernelGGL(lmhead_merge_kernel, dim3((unsigned int)((rows + per_block - 1) / per_block)), dim3(kHdThreads), 0,
