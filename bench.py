@@ -465,12 +465,12 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
     out = {"rows": rows, "vocab": vocab, "hidden": hidden}
     ref = timed(reference)
     out["reference_torch_checkpoint_chunk2048"] = ref[0]
-    for name, kw in (("fused_recompute_chunk2048", dict(chunk=2048, keep_logits=False, transposed_head=False)),
-                     ("fused_recompute_chunk4096", dict(keep_logits=False, transposed_head=False)),
+    for name, kw in (("fused_recompute_chunk2048", dict(chunk=2048, keep_logits=False, transposed_head=False, fused_head=False)),
+                     ("fused_recompute_chunk4096", dict(keep_logits=False, transposed_head=False, fused_head=False)),
                      ("fused_keep_logits", dict(transposed_head=False)), ("fused_default", dict()),
-                     ("fused_head_chunk4096", dict(fused_head=True, transposed_head=False)),
-                     ("fused_head_chunk2048_transposed", dict(fused_head=True, chunk=2048)),
-                     ("fused_recompute_chunk2048_transposed", dict(chunk=2048, keep_logits=False))):
+                     ("fused_head_chunk4096", dict(keep_logits=False, transposed_head=False)),
+                     ("fused_head_chunk2048_transposed", dict(keep_logits=False, chunk=2048)),
+                     ("fused_recompute_chunk2048_transposed", dict(chunk=2048, keep_logits=False, fused_head=False))):
         got = timed(lambda h: models.chunked_replay_logp(head, h, tokens, 1.0, **kw))
         got[0]["max_abs_logp_diff"] = float((got[1] - ref[1]).abs().max())
         got[0]["grad_hidden_rel"] = float((got[2] - ref[2]).norm() / ref[2].norm())

@@ -240,3 +240,34 @@ def test_transpose_2d_head_sized(dev):
     w = torch.randn(151936, 2560, device=dev, dtype=torch.bfloat16)
     wt = ops.transpose_2d(w)
     assert torch.equal(wt, w.t().contiguous())
+
+
+def test_chunked_replay_picks_the_fused_head_where_no_logits_are_kept(dev):
+    """Left to itself, the replay of a plain bf16 head runs the fused kernel without autograd and on the
+    recomputing path, and the library GEMM where it keeps the logits for the backward."""
+    from unirl_amd import models, ops
+
+    B, T_max, H, V = 2, 40, 64, 500
+    g = torch.Generator().manual_seed(22)
+    head = torch.nn.Linear(H, V, bias=False).to(dev).to(torch.bfloat16)
+    hidden = torch.randn(B, T_max, H, generator=g).bfloat16().to(dev)
+    toks = torch.randint(0, V, (B, T_max), generator=g).to(dev)
+    fused = ops.lmhead_logp(hidden, head.weight, None, toks, 1.0)[0]
+    with torch.no_grad():
+        assert torch.equal(models.chunked_replay_logp(head, hidden, toks), fused)
+        unfused = models.chunked_replay_logp(head, hidden, toks, fused_head=False)
+    h = hidden.clone().requires_grad_(True)
+    kept = models.chunked_replay_logp(head, h, toks)                       # fits the budget: logits kept, library GEMM
+    assert torch.equal(kept.detach(), unfused)
+    dropped = models.chunked_replay_logp(head, h, toks, keep_logits=False)  # nothing kept: fused forward
+    assert torch.equal(dropped.detach(), fused)
+    dropped.sum().backward()
+    g_fused = h.grad.clone()
+    h.grad = None
+    kept.sum().backward()
+    assert float((g_fused.float() - h.grad.float()).norm() / h.grad.float().norm()) < 2e-2
+    # a head the fused kernel does not take (fp32) falls back silently when left to itself
+    head32 = torch.nn.Linear(H, V).to(dev)
+    with torch.no_grad():
+        out32 = models.chunked_replay_logp(head32, hidden.float(), toks)
+    assert out32.dtype == torch.float32 and bool(torch.isfinite(out32).all())

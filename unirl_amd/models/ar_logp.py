@@ -246,7 +246,7 @@ def chunked_replay_logp(
     temperature: float = 1.0,
     chunk: Optional[int] = None,
     keep_logits: Optional[bool] = None,
-    fused_head: bool = False,
+    fused_head: Optional[bool] = None,
     transposed_head: Optional[bool] = None,
 ) -> torch.Tensor:
     """Padded ``[B, T_max]`` fp32 log-probs of ``response_tokens`` under ``lm_head(resp_hidden)``.
@@ -269,14 +269,16 @@ def chunked_replay_logp(
     an ``nn.Module`` head requires grad; a bare callable whose captured weights alone require
     grad keeps its logits.
 
-    ``fused_head=True`` (a plain bf16 ``nn.Linear`` head, bf16 hidden states, hidden size a
-    multiple of 64, outside autocast) computes the forward with ``unirl_lmhead_logp``: the head's
-    GEMM with the log-softmax statistics reduced in its epilogue, so no logits exist in the
-    forward at all (the backward rebuilds each chunk's logits with ``lm_head`` as above).  Measured
-    on the MI355X with Qwen3-4B's head it is faster than the library GEMM plus the token kernel up
-    to 1024 rows per chunk, level at 2048 and 9 % slower at 8192; it is off by default because
-    the default keeps the logits for the backward.  Its bf16 logits differ from the library GEMM's in about 0.02 % of the
-    entries by one bf16 ulp (a different fp32 summation order), as two library versions would.
+    ``fused_head`` computes the forward with ``unirl_lmhead_logp``: the head's GEMM with the
+    log-softmax statistics reduced in its epilogue, so no logits exist in the forward at all (the
+    backward rebuilds each chunk's logits with ``lm_head`` as above).  It needs a plain bf16
+    ``nn.Linear`` head, bf16 hidden states on the same device, a hidden size that is a multiple
+    of 64 and no autocast (``True`` raises otherwise).  Measured on the MI355X with Qwen3-4B's head
+    it is faster than the library GEMM plus the token kernel from 64 to 8192 rows per chunk and
+    holds 6 % of the transient memory.  Left at ``None`` it is used wherever it applies and the
+    logits are not kept: without autograd (scoring a rollout) and on the recomputing path.  Its
+    bf16 logits differ from the library GEMM's in about 0.02 % of the entries by one bf16 ulp (a
+    different fp32 summation order), as two library versions would.
 
     For a plain ``nn.Linear`` head on hidden states of its own dtype (no autocast) the head and
     its backward run inside one autograd node, which issues the gradient GEMMs itself.
@@ -293,9 +295,17 @@ def chunked_replay_logp(
             _is_plain_linear(lm_head)
             and bsz * t_max * lm_head.out_features * lm_head.weight.element_size() <= KEEP_LOGITS_BYTES
         )
+    fused_ok = (
+        _is_plain_linear(lm_head) and ops.lmhead_logp_supported(resp_hidden, lm_head.weight, lm_head.bias)
+        and not torch.is_autocast_enabled("cuda")
+    )
+    if fused_head is None:
+        # kept logits come from the library GEMM; everywhere else nothing needs them in the forward
+        trains = fused_ok and torch.is_grad_enabled() and (
+            resp_hidden.requires_grad or any(p.requires_grad for p in lm_head.parameters()))
+        fused_head = fused_ok and not (trains and keep_logits)
     if fused_head:
-        if not (_is_plain_linear(lm_head) and ops.lmhead_logp_supported(resp_hidden, lm_head.weight, lm_head.bias)
-                and not torch.is_autocast_enabled("cuda")):
+        if not fused_ok:
             raise ValueError(
                 "fused_head needs a plain bf16 nn.Linear head, bf16 hidden states on the same HIP device, a hidden "
                 "size that is a multiple of 64, and no autocast"
