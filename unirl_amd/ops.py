@@ -8,6 +8,7 @@ API (``unirl_amd.sde``, ``unirl_amd.algorithms``, ...) is built on these.
 from __future__ import annotations
 
 import ctypes
+import functools
 import math
 from typing import Dict, List, Optional, Sequence, Tuple, Union
 
@@ -141,7 +142,7 @@ def _per_sample_view(t: torch.Tensor, name: str, *, writable: bool = False) -> T
     N.require_device(t, name)
     B = t.shape[0]
     D = t.numel() // B if B else 0
-    inner_ok = B == 0 or t[0].is_contiguous()
+    inner_ok = B == 0 or _dense_from(t, 1)
     # A sample stride of 0 means "densely packed" in the C ABI, so a tensor broadcast over the
     # samples (expand(B, ...), stride 0) cannot be handed over as it is: it is copied.
     if inner_ok and (B <= 1 or t.stride(0) >= (D if writable else 1)):
@@ -255,6 +256,32 @@ def sde_step_logp_into(
     N.check(rc, "unirl_sde_step_logp_ex")
 
 
+def _dense_from(t: torch.Tensor, first_dim: int) -> bool:
+    """Whether dimensions ``first_dim ..`` of ``t`` form one contiguous run (``t[0, .., 0].is_contiguous()``
+    without making the view)."""
+    shape, strides, expect = t.shape, t.stride(), 1
+    for k in range(t.dim() - 1, first_dim - 1, -1):
+        if shape[k] != 1 and strides[k] != expect:
+            return False
+        expect *= shape[k]
+    return True
+
+
+@functools.lru_cache(maxsize=256)
+def _replay_slot_arrays(slots_x: tuple, slots_p: tuple, K: int):
+    """The two checked slot tables of a replay as C arrays (the same few tuples come back call after call)."""
+    slots_x, slots_p = [int(k) for k in slots_x], [int(k) for k in slots_p]
+    S = len(slots_x)
+    if S < 1 or len(slots_p) != S:
+        raise ValueError(f"slot_sample and slot_prev must name the same, non-zero number of steps; got {S} and {len(slots_p)}")
+    if S > N.MAX_ROLLOUT_STEPS:
+        raise ValueError(f"at most {N.MAX_ROLLOUT_STEPS} steps per replay call; got {S}")
+    for k in slots_x + slots_p:
+        if not 0 <= k < K:
+            raise ValueError(f"slot {k} is outside the stack's {K} slots")
+    return (ctypes.c_int64 * S)(*slots_x), (ctypes.c_int64 * S)(*slots_p), S
+
+
 def _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next, kind, eta, sigma_max, step_major):
     """Checked operands and the filled ``unirl_sde_replay_desc`` of a batched replay; returns
     ``(desc, keepalive, B, S, D, shape_tail)``."""
@@ -266,15 +293,7 @@ def _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next,
     B, K = int(latents.shape[0]), int(latents.shape[1])
     tail = tuple(latents.shape[2:])
     D = int(math.prod(tail))
-    slots_x, slots_p = [int(k) for k in slot_sample], [int(k) for k in slot_prev]
-    S = len(slots_x)
-    if S < 1 or len(slots_p) != S:
-        raise ValueError(f"slot_sample and slot_prev must name the same, non-zero number of steps; got {S} and {len(slots_p)}")
-    if S > N.MAX_ROLLOUT_STEPS:
-        raise ValueError(f"at most {N.MAX_ROLLOUT_STEPS} steps per replay call; got {S}")
-    for k in slots_x + slots_p:
-        if not 0 <= k < K:
-            raise ValueError(f"slot {k} is outside the stack's {K} slots")
+    arr_x, arr_p, S = _replay_slot_arrays(tuple(slot_sample), tuple(slot_prev), K)
     want = ((S, B) if step_major else (B, S)) + tail
     if tuple(noise_pred.shape) != want:
         raise ValueError(f"noise_pred {tuple(noise_pred.shape)} != {want}")
@@ -288,12 +307,15 @@ def _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next,
     # are free, except that 0 means "dense" in the C ABI: a tensor broadcast over the samples or the
     # steps is copied, as is a stack whose slots overlap
     b_dim, s_dim = (1, 0) if step_major else (0, 1)
-    if B and not (v[0, 0].is_contiguous() and (B == 1 or v.stride(b_dim) >= 1) and (S == 1 or v.stride(s_dim) >= D)):
+    if B and not (_dense_from(v, 2) and (B == 1 or v.stride(b_dim) >= 1) and (S == 1 or v.stride(s_dim) >= D)):
         v = v.contiguous()
-    if B and not (x[0, 0].is_contiguous() and (B == 1 or x.stride(0) >= 1) and (K == 1 or x.stride(1) >= D)):
+    if B and not (_dense_from(x, 2) and (B == 1 or x.stride(0) >= 1) and (K == 1 or x.stride(1) >= D)):
         x = x.contiguous()
 
     def steps_f32(t, name):
+        if (isinstance(t, torch.Tensor) and t.dtype is torch.float32 and t.device == device and t.dim() == 1
+                and t.shape[0] == S and t.stride(0) == 1 and not t.requires_grad):
+            return t  # already what the kernel reads
         if not isinstance(t, torch.Tensor):
             t = torch.tensor([float(a) for a in t], dtype=torch.float32)
         t = t.detach().to(device=device, dtype=torch.float32).reshape(-1).contiguous()
@@ -304,11 +326,13 @@ def _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next,
     sig, sig_n = steps_f32(sigma, "sigma"), steps_f32(sigma_next, "sigma_next")
     smax_t, smax_v = _sigma_max_arg(sigma_max, device)
     d = N.SdeReplayDesc()
-    d.noise_pred = N.SdeTensor(N.ptr(v), N.dtype_code(v.dtype), v.stride(b_dim) if B > 1 else S * D)
-    d.noise_pred_step_stride = v.stride(s_dim) if S > 1 else D
-    d.latents = N.SdeTensor(N.ptr(x), N.dtype_code(x.dtype), x.stride(0) if B > 1 else 0)
-    d.latents_slot_stride = x.stride(1) if K > 1 else 0
-    arr_x, arr_p = (ctypes.c_int64 * S)(*slots_x), (ctypes.c_int64 * S)(*slots_p)
+    vs, xs = v.stride(), x.stride()
+    t = d.noise_pred
+    t.ptr, t.dtype, t.sample_stride = v.data_ptr(), N.dtype_code(v.dtype), (vs[b_dim] if B > 1 else S * D)
+    d.noise_pred_step_stride = vs[s_dim] if S > 1 else D
+    t = d.latents
+    t.ptr, t.dtype, t.sample_stride = x.data_ptr(), N.dtype_code(x.dtype), (xs[0] if B > 1 else 0)
+    d.latents_slot_stride = xs[1] if K > 1 else 0
     d.K = K
     d.slot_sample, d.slot_prev = arr_x, arr_p
     d.sigma, d.sigma_next = N.ptr(sig), N.ptr(sig_n)
