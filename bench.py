@@ -496,7 +496,7 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published peak
 
 
-def head_probe(torch, dev, vocab: int, hidden: int = 2560):
+def head_probe(torch, dev, vocab: int, hidden: int = 2560, row_counts=(64, 256, 1024, 2048, 8192)):
     """The fused lm_head + log-softmax kernel (`unirl_lmhead_logp`: the [rows, V] logits are never
     written) against the library GEMM followed by the token kernel, forward only, for a bf16 head of
     Qwen3-4B's size.  TFLOP/s count the GEMM's 2*rows*K*V flops over the whole call."""
@@ -522,7 +522,7 @@ def head_probe(torch, dev, vocab: int, hidden: int = 2560):
         return a.elapsed_time(b) / n
 
     out = []
-    for rows in (64, 256, 1024, 2048, 8192):
+    for rows in row_counts:
         h = torch.randn(rows, hidden, generator=g, device=dev).bfloat16()
         ids = torch.randint(0, vocab, (rows,), generator=g, device=dev)
         flop = 2.0 * rows * hidden * vocab
@@ -926,6 +926,17 @@ def main() -> int:
         except (ValueError, OSError, KeyError):
             traffic = None
 
+    # the one matrix-core kernel of the path: lm_head with the log-softmax statistics in its epilogue
+    # (logits never written), Qwen3-4B's head, against the library GEMM followed by the token kernel
+    lmhead_out = []
+    if not args.skip_shapes:
+        try:
+            for r in head_probe(torch, dev, args.vocab, row_counts=(2048, 8192)):
+                r["roofline"] = {"bound": "mfma", "achieved": r["fused_tflops"], "peak": MFMA_BF16_PEAK_TFLOPS,
+                                 "unit": "TFLOP/s", "frac": r["fused_frac_of_mfma_peak"]}
+                lmhead_out.append(r)
+        except Exception as exc:
+            log(f"lmhead probe failed ({type(exc).__name__}: {exc})")
     result = {
         "metric": "fused-kernel HBM GB/s (token log-prob + entropy)",
         "value": round(value, 1),
@@ -954,6 +965,7 @@ def main() -> int:
         "cpu_baseline": cpu_baseline,
         "parity": parity,
         "shapes": shapes_out,
+        "lmhead": lmhead_out,
         "device": torch.cuda.get_device_name(0),
     }
     print(json.dumps(result), flush=True)
