@@ -224,14 +224,19 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
     else b[idx - BI] = lds_frag(lds + stage * kStageD + (BM + wn * WN + (idx - BI) * 32) * kBK + fsw[ks]);
   };
   constexpr int NR = BI + BJ, NM = BI * BJ;  // LDS reads and MFMAs per K slice
-  // One K step out of LDS stage `stage`, as four slices of NM matrix instructions.  Under them
-  // travel: the loads of step k + 2 into register set `stage` (which held this step's operands
-  // until they were stored a step ago), a quarter per slice; the stores of step k + 1's operands
-  // (register set stage ^ 1, loaded a step ago) into the other LDS stage, under slices 0 - 2; and
-  // the fragment reads of the next slice.  The step's barrier stands before its LAST slice: by
-  // then every wavefront has read this stage's last fragments and stored its share of the next
-  // stage, so the last slice already reads the next step's first fragments and no slice waits for
-  // LDS behind a barrier.  (The next step's stores go to this stage, which nobody reads any more.)
+  // One K step out of LDS stage `stage`, as four slices of NM matrix instructions, each with the
+  // fragment reads of the next slice under it.  The next step's operands travel under them too.
+  // Register-staged: the loads of step k + 2 go into register set `stage` (which held this step's
+  // operands until they were stored a step ago), a quarter per slice, and the stores of step
+  // k + 1's operands (register set stage ^ 1, loaded a step ago) into the other LDS stage, under
+  // slices 0 - 2.  DMA: the other stage is free from the previous step's barrier to this step's;
+  // half of step k + 1's loads into it went out under the previous step's last slice, the other
+  // half goes out under this step's first slice.
+  // The step's barrier stands before its LAST slice: by then every wavefront has read this
+  // stage's last fragments and the other stage is complete (stores issued, or loads into LDS
+  // waited for), so the last slice already reads the next step's first fragments and no slice
+  // waits for LDS behind a barrier.  (What the next step writes goes to this stage, which nobody
+  // reads any more.)
   // Every memory instruction is issued between matrix instructions: a wavefront issues in order,
   // and a burst of sixteen loads or stores holds up the MFMAs behind it for as long as the memory
   // pipeline takes to accept them (measured: the bursts cost 0.9 us of a 1.8 us step).  The
@@ -275,12 +280,11 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
         else if (kEarlyBarrier) read_frags(stage ^ 1, 0, fa[cur ^ 1], fb[cur ^ 1]);  // the next step's first slice
         load_range(stage, k_load, ks * NQ, (ks + 1) * NQ);
       }
-      if (DMA) {
-      } else if (kEarlyBarrier) {
+      if (!DMA && kEarlyBarrier) {
         if (ks == 0) store_range(stage ^ 1, stage ^ 1, 0, W0);
         if (ks == 1) store_range(stage ^ 1, stage ^ 1, W0, W0 + W1);
         if (ks == 2) store_range(stage ^ 1, stage ^ 1, W0 + W1, NW);
-      } else {
+      } else if (!DMA) {
         store_range(stage ^ 1, stage ^ 1, ks * NQ, (ks + 1) * NQ);
       }
 #pragma unroll
@@ -305,7 +309,7 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
     }
   };
 
-  // Step k sits in LDS stage k % 2 and came through register set k % 2.  Every trip issues its
+  // Step k sits in LDS stage k % 2 (and came through register set k % 2).  Every trip issues its
   // loads and stores unconditionally (past the last step the loads repeat the last step's
   // addresses and the stores fill a stage nobody multiplies any more): with a branch around them
   // the compiler can no longer count which loads are outstanding at the stores and waits for all
