@@ -397,3 +397,31 @@ def test_conforming_operands_are_handed_over_without_a_copy(monkeypatch):
     # the sigma arguments of the SDE step: an fp32 scalar passes untouched
     s = torch.tensor(0.5)
     assert ops._sigma_arg(s, 4, cpu, "sigma")[0] is s
+
+
+def test_dense_from_agrees_with_torch_on_strided_views():
+    """`_dense_from(t, k)` is `t[0, .., 0].is_contiguous()` (k leading indices) without making the view."""
+    from unirl_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    base = torch.zeros(6, 5, 4, 3, 2)
+    views = [base, base[:, 1], base[:, :, ::2], base.transpose(1, 2), base.transpose(3, 4), base[..., 0],
+             base[:, :, :, :, :1], base.permute(1, 0, 2, 3, 4), base[:, :, 1:3], base.expand(6, 5, 4, 3, 2),
+             torch.zeros(3, 1, 4).expand(3, 7, 4), torch.zeros(4, 4)[:, :1], torch.zeros(2, 3, 1, 5).transpose(1, 2)]
+    for t in views:
+        for k in range(0, t.dim()):
+            idx = (0,) * k
+            assert ops._dense_from(t, k) == t[idx].is_contiguous(), (tuple(t.shape), t.stride(), k)
+
+
+def test_replay_slot_tables_are_checked_and_cached():
+    from unirl_amd import ops
+
+    a = ops._replay_slot_arrays((0, 2, 3), (1, 3, 4), 5)
+    assert list(a[0]) == [0, 2, 3] and list(a[1]) == [1, 3, 4] and a[2] == 3
+    assert ops._replay_slot_arrays((0, 2, 3), (1, 3, 4), 5) is a
+    for bad in (((0, 5), (1, 2)), ((0,), (1, 2)), ((), ()), ((-1,), (0,))):
+        with pytest.raises(ValueError):
+            ops._replay_slot_arrays(bad[0], bad[1], 5)
+    with pytest.raises(ValueError):
+        ops._replay_slot_arrays(tuple(range(65)), tuple(range(65)), 100)
