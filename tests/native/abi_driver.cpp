@@ -311,6 +311,129 @@ void check_advantages(hipStream_t st) {
   std::printf("group advantages: checked %lld rewards\n", (long long)(G * b));
 }
 
+// The replay loop of a diffusion stage as one call (unirl/models/sd3/diffusion.py:467-497): every
+// (sample, step) transition reads its latent and its stored next latent from the trajectory stack.
+// Checked against the single-step entry point called once per step on copies of the slots.
+void check_sde_replay(hipStream_t st, void* ws, size_t ws_bytes) {
+  const int64_t B = 2, K = 4, S = 2, D = 520;
+  const double eta = 0.7, sigma_max = 0.98780483;
+  Rng rng(15);
+  std::vector<float> stack(B * K * D), v(B * S * D);
+  for (auto& e : stack) e = (float)rng.normal();
+  for (auto& e : v) e = (float)rng.normal();
+  const std::vector<float> sg = {0.84375006f, 0.5f}, sn = {0.82258058f, 0.4f};
+  const int64_t slot_x[2] = {2, 0}, slot_p[2] = {3, 1};
+  DevBuf<float> dstack(stack), dv(v), dsg(sg), dsn(sn), dmean(B * S * D), dlp(B * S);
+  unirl_sde_replay_desc d;
+  std::memset(&d, 0, sizeof(d));
+  d.noise_pred = {dv.p, UNIRL_F32, S * D};
+  d.noise_pred_step_stride = D;
+  d.latents = {dstack.p, UNIRL_F32, K * D};
+  d.latents_slot_stride = D;
+  d.K = K;
+  d.slot_sample = slot_x;
+  d.slot_prev = slot_p;
+  d.sigma = dsg.p;
+  d.sigma_next = dsn.p;
+  d.sigma_max_ptr = nullptr;
+  d.sigma_max_val = (float)sigma_max;
+  d.eta = eta;
+  d.kind = UNIRL_SDE_FLOW;
+  d.B = B;
+  d.S = S;
+  d.D = D;
+  d.mean_out = dmean.p;
+  d.mean_dtype = UNIRL_F32;
+  d.logp_out = dlp.p;
+  d.logp_sum = 0;
+  expect_status("unirl_sde_replay_logp", unirl_sde_replay_logp(&d, ws, ws_bytes, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto mean = dmean.host(), lp = dlp.host();
+  for (int64_t j = 0; j < S; ++j) {
+    // the same step through the single-step entry point, on dense copies of the two slots
+    std::vector<float> x(B * D), prev(B * D), vj(B * D);
+    for (int64_t b = 0; b < B; ++b)
+      for (int64_t i = 0; i < D; ++i) {
+        x[b * D + i] = stack[(b * K + slot_x[j]) * D + i];
+        prev[b * D + i] = stack[(b * K + slot_p[j]) * D + i];
+        vj[b * D + i] = v[(b * S + j) * D + i];
+      }
+    DevBuf<float> dx(x), dprev(prev), dvj(vj), dm1(B * D), dl1(B);
+    expect_status("unirl_sde_step_logp (one step of the replay)",
+                  unirl_sde_step_logp(dvj.p, UNIRL_F32, dx.p, UNIRL_F32, dprev.p, nullptr, dsg.p + j, dsn.p + j, 0,
+                                      nullptr, (float)sigma_max, eta, UNIRL_SDE_FLOW, B, D, nullptr, dm1.p, dl1.p, 0,
+                                      ws, ws_bytes, st));
+    HIP_OK(hipStreamSynchronize(st));
+    const auto m1 = dm1.host(), l1 = dl1.host();
+    for (int64_t b = 0; b < B; ++b) {
+      expect_close("replay log-prob vs single step", lp[b * S + j], l1[b], 1e-6, 1e-7);
+      for (int64_t i = 0; i < D; ++i)
+        if (mean[(b * S + j) * D + i] != m1[b * D + i]) {
+          std::printf("FAIL replay mean differs from the single step at (%lld,%lld,%lld)\n", (long long)b, (long long)j,
+                      (long long)i);
+          ++g_failures;
+          break;
+        }
+    }
+  }
+  std::printf("batched replay: %lld x %lld transitions equal the single-step calls\n", (long long)B, (long long)S);
+}
+
+// lm_head + log-softmax with the logits never written (unirl/models/qwen3/ar.py:82-99), and the
+// transposed copy of the weight used by its backward: against a float64 product of the same bf16
+// operands rounded to bf16 (a logit one bf16 ulp off moves a log-prob by that ulp at most).
+void check_lmhead(hipStream_t st) {
+  const int64_t rows = 70, K = 128, V = 300;
+  Rng rng(16);
+  std::vector<uint16_t> h(rows * K), w(V * K);
+  for (auto& e : h) e = to_bf16((float)rng.normal());
+  for (auto& e : w) e = to_bf16((float)(0.2 * rng.normal()));
+  std::vector<int64_t> ids(rows);
+  for (auto& e : ids) e = (int64_t)(rng.uniform() * (double)V) % V;
+  const float T = 0.8f;
+  DevBuf<uint16_t> dh(h), dw(w), dwt(V * K);
+  DevBuf<int64_t> dids(ids);
+  DevBuf<float> dlp(rows), dent(rows), dlse(rows);
+  const size_t sb = unirl_lmhead_logp_scratch_bytes(rows, V);
+  DevBuf<unsigned char> scratch(sb);
+  expect_status("unirl_lmhead_logp", unirl_lmhead_logp(dh.p, K, dw.p, K, nullptr, rows, V, K, dids.p, T, dlp.p, dent.p,
+                                                       dlse.p, nullptr, 0, scratch.p, sb, st));
+  expect_status("unirl_transpose_2d", unirl_transpose_2d(dw.p, K, dwt.p, V, V, K, 2, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto lp = dlp.host(), ent = dent.host(), lse = dlse.host();
+  const auto wt = dwt.host();
+  for (int64_t v = 0; v < V; ++v)
+    for (int64_t k = 0; k < K; ++k)
+      if (wt[k * V + v] != w[v * K + k]) {
+        std::printf("FAIL transpose at (%lld,%lld)\n", (long long)v, (long long)k);
+        ++g_failures;
+        v = V;
+        break;
+      }
+  for (int64_t r = 0; r < rows; ++r) {
+    std::vector<double> x(V);
+    double m = -1e300;
+    for (int64_t v = 0; v < V; ++v) {
+      double acc = 0.0;
+      for (int64_t k = 0; k < K; ++k) acc += (double)from_bf16(h[r * K + k]) * (double)from_bf16(w[v * K + k]);
+      x[v] = (double)from_bf16(to_bf16((float)acc)) / (double)T;
+      m = x[v] > m ? x[v] : m;
+    }
+    double sum = 0.0, tsum = 0.0;
+    for (int64_t v = 0; v < V; ++v) {
+      const double e = std::exp(x[v] - m);
+      sum += e;
+      tsum += e * x[v];
+    }
+    const double ref_lse = m + std::log(sum);
+    expect_close("lm_head log-sum-exp", lse[r], ref_lse, 2e-3, 2e-3);
+    expect_close("lm_head log-prob", lp[r], x[ids[r]] - ref_lse, 2e-3, 2.5e-2);  // + one bf16 ulp of a logit of <= 4
+    expect_close("lm_head entropy", ent[r], ref_lse - tsum / sum, 2e-3, 2e-3);
+  }
+  std::printf("fused lm_head: checked %lld rows of %lld logits; transpose %lld x %lld exact\n", (long long)rows,
+              (long long)V, (long long)V, (long long)K);
+}
+
 }  // namespace
 
 int main() {
@@ -334,6 +457,8 @@ int main() {
   check_kl(st, ws, ws_bytes);
   check_grpo(st, ws, ws_bytes);
   check_advantages(st);
+  check_sde_replay(st, ws, ws_bytes);
+  check_lmhead(st);
   HIP_OK(hipStreamSynchronize(st));
   HIP_OK(hipFree(ws));
   HIP_OK(hipStreamDestroy(st));
