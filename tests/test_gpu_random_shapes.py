@@ -240,3 +240,87 @@ def test_misaligned_base_pointers(dev, seed):
                                          step_index=step)
             assert torch.equal(got.cpu(), want), f"dpm2 step {step}, offsets {k}"
             xs = want.to(dtype)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_sde_replay_random(dev, seed):
+    """The batched replay on random stacks, step lists, dtypes and velocity layouts against the
+    oracle's single steps: means bit-exact, log-probs to the dtype's tolerance."""
+    from unirl_amd import sde
+
+    rng = random.Random(5000 + seed)
+    for _ in range(5):
+        shape = rand_shape(rng, max_elems=3000)
+        B, tail = shape[0], shape[1:]
+        kind = rng.choice(("flow", "dance", "cps"))
+        dtype, vdtype = rng.choice(DTYPES), rng.choice(DTYPES)
+        n_stored = rng.randint(2, 7)
+        stored = sorted(rng.sample(range(0, 12), n_stored))
+        # trained steps: those whose successor is stored as well; make sure there is at least one
+        if not any(s + 1 in stored for s in stored):
+            stored = sorted(set(stored) | {stored[0] + 1})
+        can = [s for s in stored if s + 1 in stored]
+        steps = [rng.choice(can) for _ in range(rng.randint(1, 4))]
+        eta = rng.choice((0.3, 0.7, 1.0))
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        stack = torch.randn((B, len(stored)) + tail, generator=g).to(dtype)
+        step_major = rng.random() < 0.4
+        v = torch.randn((B, len(steps)) + tail, generator=g).to(vdtype)
+        what = f"{kind} B={B} tail={tail} {dtype}/{vdtype} stored={stored} steps={steps} eta={eta} step_major={step_major}"
+        refs = [osde.sde_denoise(kind, v[:, j], stack[:, stored.index(s)], SIG[s], SIG[s + 1], eta=eta,
+                                 prev_sample=stack[:, stored.index(s + 1)], sigma_max=SIG[1], ieee_sqrt=True)
+                for j, s in enumerate(steps)]
+        slot_x, slot_p = sde.replay_slots(stored, steps)
+        v_dev = v.transpose(0, 1).contiguous().to(dev) if step_major else v.to(dev)
+        lp, means = sde.STRATEGIES[kind]().replay_steps(
+            v_dev, stack.to(dev), slot_x, slot_p, [float(SIG[s]) for s in steps], [float(SIG[s + 1]) for s in steps],
+            eta=eta, sigma_max=float(SIG[1]), step_major=step_major)
+        assert torch.equal(means.cpu(), torch.stack([r[2] for r in refs], 1).to(dtype)), what
+        rtol = FP32_RTOL if dtype == torch.float32 and vdtype == torch.float32 else BF16_RTOL
+        assert_close(lp, torch.stack([r[1] for r in refs], 1), rtol, 2e-6, what)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_lmhead_logp_random(dev, seed):
+    """The fused lm_head kernel on random (rows, K, V), with and without bias, at the row counts that
+    select each of its three code paths: logits within one bf16 ulp of the float64 product, statistics
+    against the oracle on the kernel's own logits."""
+    from unirl_amd import ops
+
+    rng = random.Random(6000 + seed)
+    for _ in range(3):
+        rows = rng.choice((rng.randint(1, 255), rng.randint(256, 511), rng.randint(512, 1100)))
+        K = 64 * rng.randint(1, 6)
+        V = rng.choice((rng.randint(1, 300), rng.randint(300, 1500)))
+        bias, T = rng.random() < 0.5, rng.choice((1.0, 0.7, 1.3))
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        h = torch.randn(rows, K, generator=g).bfloat16()
+        w = (torch.randn(V, K, generator=g) * (3.0 / K ** 0.5)).bfloat16()
+        b = torch.randn(V, generator=g).bfloat16() if bias else None
+        ids = torch.randint(0, V, (rows,), generator=g)
+        what = f"rows={rows} K={K} V={V} bias={bias} T={T}"
+        lp, ent, lse, logits = ops.lmhead_logp(h.to(dev), w.to(dev), None if b is None else b.to(dev), ids.to(dev), T,
+                                               want_entropy=True, want_lse=True, want_logits=True)
+        exact = h.double() @ w.double().T + (0 if b is None else b.double())
+        mag = h.double().abs() @ w.double().abs().T + (0 if b is None else b.double().abs())
+        ulp = torch.maximum(exact.abs(), torch.tensor(2.0 ** -126, dtype=torch.float64)).log2().floor().exp2() * 2.0 ** -7
+        assert bool(((logits.cpu().double() - exact).abs() <= ulp + mag * 2.0 ** -20).all()), what
+        own = logits.cpu()
+        assert_close(lp, otok.token_logp(own, ids, T), 1e-5, 2e-6, what + " log-prob")
+        assert_close(lse, torch.logsumexp(own.double() / T, dim=-1).float(), 1e-5, 2e-6, what + " lse")
+        assert_close(ent, otok.token_entropy(own, T), 1e-5, 2e-6, what + " entropy")
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_transpose_random(dev, seed):
+    from unirl_amd import ops
+
+    rng = random.Random(7000 + seed)
+    for _ in range(8):
+        rows, cols = rng.randint(1, 400), rng.randint(1, 400)
+        dtype = rng.choice((torch.bfloat16, torch.float16, torch.float32))
+        pad, off = rng.randint(0, 9), rng.randint(0, 3)
+        g = torch.Generator().manual_seed(rng.randint(0, 10**6))
+        wide = torch.randn(rows, cols + pad + off, generator=g).to(dtype).to(dev)
+        src = wide[:, off : off + cols]
+        assert torch.equal(ops.transpose_2d(src), src.t().contiguous()), (rows, cols, dtype, pad, off)
