@@ -785,6 +785,16 @@ def main() -> int:
                     sh["run"](i)
                 torch.cuda.synchronize()
                 probe[sh["name"] + "_algorithmic_bytes"] = sh.get("bytes_padded", sh["bytes"])
+            # the fused lm_head kernel at 8192 rows: operands once, the tile states written and read once
+            hd_rows, hd_k = 8192, 2560
+            hw = torch.randn(args.vocab, hd_k, device=dev).bfloat16()
+            hh = torch.randn(hd_rows, hd_k, device=dev).bfloat16()
+            hid = torch.randint(0, args.vocab, (hd_rows,), device=dev)
+            for _ in range(3):
+                ops.lmhead_logp(hh, hw, None, hid, 1.0, want_lse=True)
+            torch.cuda.synchronize()
+            n_tiles = (args.vocab + 255) // 256
+            probe["lmhead_logp_8192_algorithmic_bytes"] = (hw.numel() + hh.numel()) * 2 + 2 * hd_rows * n_tiles * 16
         print(json.dumps({"traffic_probe": probe}), flush=True)
         return 0
 
