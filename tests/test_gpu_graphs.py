@@ -111,3 +111,50 @@ def test_two_streams_keep_their_own_scratch(dev):
         for got, want in ((got_a, alone_a), (got_b, alone_b)):
             for u, w in zip(got, want):
                 assert torch.equal(u.view(torch.uint8), w.view(torch.uint8)), f"overlapping call {rep} differs"
+
+
+def test_graph_replays_of_the_batched_replay_and_the_fused_head(dev):
+    """The batched SDE replay, the fused lm_head kernel (register-staged below 512 rows, loads straight
+    into LDS from 512) and the transposition under capture: several replays with fresh inputs and
+    eager calls in between, each bit-identical to the eager result."""
+    from unirl_amd import ops, sde
+
+    g = torch.Generator(device=dev).manual_seed(6)
+    stack = torch.randn(3, 5, 4, 24, 24, device=dev, generator=g).bfloat16()
+    vel = torch.randn(3, 2, 4, 24, 24, device=dev, generator=g).bfloat16()
+    slot_x, slot_p = sde.replay_slots([0, 1, 2, 3, 4], [1, 3])
+    sg = torch.stack([SIG[1], SIG[3]]).to(dev)
+    sn = torch.stack([SIG[2], SIG[4]]).to(dev)
+    smax = SIG[1].to(dev)
+    w = (0.1 * torch.randn(700, 192, device=dev, generator=g)).bfloat16()
+    h_small = torch.randn(300, 192, device=dev, generator=g).bfloat16()
+    h_big = torch.randn(600, 192, device=dev, generator=g).bfloat16()
+    ids_small = torch.randint(0, 700, (300,), device=dev, generator=g)
+    ids_big = torch.randint(0, 700, (600,), device=dev, generator=g)
+
+    def run_all():
+        lp, means = ops.sde_replay_logp(vel, stack, slot_x, slot_p, sg, sn, kind="flow", eta=0.7, sigma_max=smax)
+        a = ops.lmhead_logp(h_small, w, None, ids_small, 0.9, want_entropy=True, want_lse=True)[:3]
+        b = ops.lmhead_logp(h_big, w, None, ids_big, 0.9, want_entropy=True, want_lse=True)[:3]
+        wt = ops.transpose_2d(w)
+        return (lp, means) + tuple(a) + tuple(b) + (wt,)
+
+    run_all()  # scratch buffers of the head are torch allocations: let the caching allocator have them
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        outs = run_all()
+    torch.cuda.synchronize()
+    for rep in range(4):
+        for t in (stack, vel, w, h_small, h_big):
+            t.copy_((torch.randn(t.shape, device=dev, generator=g) * (0.1 if t is w else 1.0)).bfloat16())
+        ops.lmhead_logp(h_small[:64], w, None, ids_small[:64], 1.0)  # eager work of the library between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        want = run_all()
+        torch.cuda.synchronize()
+        for k, (a, b) in enumerate(zip(got, want)):
+            assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), f"replay {rep}, output {k} differs from eager"
