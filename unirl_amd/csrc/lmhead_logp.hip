@@ -363,12 +363,12 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
 #pragma unroll
       for (int g4 = 0; g4 < 4; ++g4) {
         const int row = wm * WM + bi * 32 + 8 * g4 + 4 * (lane >> 5);
-        uint32_t b[4];
+        float f[4];
 #pragma unroll
-        for (int k = 0; k < 4; ++k) b[k] = f32_to_bf16_bits(HAS_BIAS ? acc[bi][bj][g4 * 4 + k] + bv : acc[bi][bj][g4 * 4 + k]);
-        u32x2 pk;
-        pk.x = b[0] | (b[1] << 16);
-        pk.y = b[2] | (b[3] << 16);
+        for (int k = 0; k < 4; ++k) f[k] = HAS_BIAS ? acc[bi][bj][g4 * 4 + k] + bv : acc[bi][bj][g4 * 4 + k];
+        u32x2 pk;  // two values per conversion instruction
+        pk.x = f32x2_to_bf16x2_bits(f[0], f[1]);
+        pk.y = f32x2_to_bf16x2_bits(f[2], f[3]);
         *reinterpret_cast<u32x2*>(out + col * kOutPitch + row) = pk;
       }
     }
@@ -390,8 +390,9 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
     tsum[r] = 0.0f;
   }
   const int64_t gcol0 = n0 + (int64_t)cq * COLS;  // this thread's first column in the vocabulary
-  auto reduce_columns = [&](auto full_tag) {
+  auto reduce_columns = [&](auto full_tag, auto ent_tag) {
     constexpr bool FULL = decltype(full_tag)::value;  // every column of the tile lies inside the vocabulary
+    constexpr bool ENT = decltype(ent_tag)::value;    // the entropy is asked for: sum 2^a * a is needed
     const uint16_t* src = out + (cq * COLS) * kOutPitch + 4 * q;
 #pragma unroll 1
     for (int p0 = 0; p0 < COLS; p0 += PIECE) {
@@ -415,7 +416,7 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
         const float d = (mn - m[r]) * c;
         const float f = __builtin_amdgcn_exp2f(-d);
         const bool had = m[r] != -INFINITY;
-        tsum[r] = had ? f * fmaf(-d, sum[r], tsum[r]) : 0.0f;
+        if (ENT) tsum[r] = had ? f * fmaf(-d, sum[r], tsum[r]) : 0.0f;
         sum[r] = had ? f * sum[r] : 0.0f;
         m[r] = mn;
         if (!FULL && mn == -INFINITY) continue;  // nothing but columns outside the vocabulary so far
@@ -426,13 +427,18 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
           const float a = fmaf(x[r][j], c, mc);
           const float e = __builtin_amdgcn_exp2f(a);
           sum[r] += e;
-          tsum[r] = (FULL || x[r][j] != -INFINITY) ? fmaf(e, a, tsum[r]) : tsum[r];
+          if (ENT) tsum[r] = (FULL || x[r][j] != -INFINITY) ? fmaf(e, a, tsum[r]) : tsum[r];
         }
       }
     }
   };
-  if (n0 + BN <= A.N) reduce_columns(std::true_type{});
-  else reduce_columns(std::false_type{});
+  if (A.ent) {
+    if (n0 + BN <= A.N) reduce_columns(std::true_type{}, std::true_type{});
+    else reduce_columns(std::false_type{}, std::true_type{});
+  } else {
+    if (n0 + BN <= A.N) reduce_columns(std::true_type{}, std::false_type{});
+    else reduce_columns(std::false_type{}, std::false_type{});
+  }
 
   // the PARTS partial states of a row meet in LDS above the logits; thread `row` merges them in part order
   float* part_state = reinterpret_cast<float*>(lds + BN * kOutPitch);  // [PARTS][BM][3]
