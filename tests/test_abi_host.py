@@ -425,3 +425,21 @@ def test_replay_slot_tables_are_checked_and_cached():
             ops._replay_slot_arrays(bad[0], bad[1], 5)
     with pytest.raises(ValueError):
         ops._replay_slot_arrays(tuple(range(65)), tuple(range(65)), 100)
+
+
+def test_replay_slots_follow_latents_at_on_the_host():
+    """`replay_slots` is `LatentSegment.latents_at` (unirl/types/segments/latent.py:82-97) for a step and
+    its successor: the first slot that holds the step, KeyError with the stored indices when it is not
+    stored, RuntimeError without indices."""
+    from unirl_amd import sde
+
+    stored = torch.tensor([0, 3, 4, 4, 7, 8])
+    assert sde.replay_slots(stored, [3, 7]) == ([1, 4], [2, 5])
+    assert sde.replay_slots([5, 1, 2], [1]) == ([1], [2])          # unsorted storage
+    assert sde.replay_slots(stored, []) == ([], [])
+    with pytest.raises(KeyError, match=r"step_idx=5 not in stored indices=\[0, 3, 4, 4, 7, 8\]"):
+        sde.replay_slots(stored, [4])                              # step 4 is stored, its successor is not
+    with pytest.raises(KeyError, match="step_idx=1 "):
+        sde.replay_slots(stored, [1])
+    with pytest.raises(RuntimeError, match="missing indices"):
+        sde.replay_slots(None, [0])
