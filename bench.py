@@ -292,7 +292,7 @@ def make_shapes(torch, dev):
             shape=f"fp32 [256,8192] padded, {n_valid} valid tokens: loss + metrics + grad_new in one pass",
             bytes=bytes3_step, read_bytes=bytes3_valid, write_bytes=new.numel() * 4, elements=n_valid,
             run=(lambda i, k=kind: plans[k][i % ns3].forward_backward(1.0)), sets=ns3,
-            cpu=(lambda k=kind, o=okw: cpu_step(k, o)), cpu_bytes=bytes3_step,
+            cpu=(lambda k=kind, o=okw: cpu_step(k, o)), cpu_bytes=bytes3_step, plain_reduction=True,
         ))
 
     # the same tokens in the packed layout the AR algorithms use ([total_tokens] + cu_seqlens)
@@ -308,7 +308,7 @@ def make_shapes(torch, dev):
             name=f"ratio_step_{kind}_packed", config=3,
             shape=f"fp32 packed [{n_valid}] + cu_seqlens[257]: loss + metrics + grad_new in one pass",
             bytes=3 * n_valid * 4, read_bytes=bytes3_valid, write_bytes=n_valid * 4, elements=n_valid,
-            run=(lambda i, k=kind: pplans[k][i % ns3p].forward_backward(1.0)), sets=ns3p,
+            run=(lambda i, k=kind: pplans[k][i % ns3p].forward_backward(1.0)), sets=ns3p, plain_reduction=True,
         ))
 
     # -- config 4: Flow-DPPO KL mask, WAN bf16 [2,16,21,60,104] -----------------------------------
@@ -381,7 +381,7 @@ def make_shapes(torch, dev):
 def make_floor(torch, dev, read_bytes: int, write_bytes: int, n_sets: int, tail_launch: bool):
     """The launch floor of a shape: a kernel that only moves the shape's bytes (same read / write
     split, rotating buffers), plus the minimal dependent second launch of a two-launch reduction."""
-    from unirl_amd import ops
+    from unirl_amd import _tune
 
     rb, wb = (read_bytes + 15) // 16 * 16, (write_bytes + 15) // 16 * 16
     srcs = [torch.ones(max(rb, 16), dtype=torch.uint8, device=dev) for _ in range(n_sets)]
@@ -389,7 +389,7 @@ def make_floor(torch, dev, read_bytes: int, write_bytes: int, n_sets: int, tail_
     sink = torch.zeros(4, dtype=torch.int32, device=dev)
 
     def run(i):
-        ops.calib_stream(srcs[i % n_sets], rb, dsts[i % n_sets], wb, sink, tail_launch=tail_launch)
+        _tune.calib_stream(srcs[i % n_sets], rb, dsts[i % n_sets], wb, sink, tail_launch=tail_launch)
 
     return run
 
@@ -399,7 +399,7 @@ def kernel_source_sha256() -> str:
     import hashlib
 
     h = hashlib.sha256()
-    for name in ("token_logp.hip", "common.cuh"):
+    for name in ("token_logp.hip", "common_hip.h"):
         h.update((ROOT / "unirl_amd" / "csrc" / name).read_bytes())
     return h.hexdigest()
 
@@ -562,7 +562,7 @@ def tail_probe(torch, dev):
     library's scheme), and finished inside the one launch by a polling workgroup
     (`unirl_calib_reduce` modes 0 / 1 / 2), each as 64 back-to-back calls in a HIP graph over
     rotating inputs."""
-    from unirl_amd import ops
+    from unirl_amd import _tune
 
     pool = torch.ones(160 * 2**20, dtype=torch.float32, device=dev)  # 640 MiB: beyond L2 + last-level cache
     out = torch.zeros(1, dtype=torch.float64, device=dev)
@@ -576,18 +576,18 @@ def tail_probe(torch, dev):
             got = {}
             for mode in (1, 2):  # same sum both ways, also on a second call that meets the first one's tags
                 for _ in range(2):
-                    ops.calib_reduce(views[0], nbytes, mode, nwg, scratch, out)
+                    _tune.calib_reduce(views[0], nbytes, mode, nwg, scratch, out)
                 torch.cuda.synchronize()
                 got[mode] = float(out.item())
             row = {"shape": label, "bytes": nbytes, "workgroups": nwg, "results_agree": got[1] == got[2]}
             for mode, key in ((0, "stream_only_us"), (1, "two_launches_us"), (2, "one_launch_polled_us")):
-                row[key] = round(time_in_graph(torch, lambda i, m=mode: ops.calib_reduce(views[i % n_sets], nbytes, m, nwg,
+                row[key] = round(time_in_graph(torch, lambda i, m=mode: _tune.calib_reduce(views[i % n_sets], nbytes, m, nwg,
                                                                                          scratch, out), n_sets), 2)
             log(f"tail probe: {row}")
             rows.append(row)
     empty = torch.zeros(4, dtype=torch.int32, device=dev)
     rows.append({"shape": "one-wavefront kernel with one store, alone",
-                 "us": round(time_in_graph(torch, lambda i: ops.calib_stream(None, 0, None, 0, empty, tail_launch=True), 2), 2)})
+                 "us": round(time_in_graph(torch, lambda i: _tune.calib_stream(None, 0, None, 0, empty, tail_launch=True), 2), 2)})
     return rows
 
 
@@ -607,11 +607,10 @@ def timeline_probe(torch, dev, names):
 
     if not TUNE_LIB_PATH.exists():
         raise SystemExit(f"bench.py --timeline needs {TUNE_LIB_PATH}: build it with `python -m unirl_amd.build --tune`")
-    N.LIB_PATH = TUNE_LIB_PATH  # before the first call binds the library
-    lib = N.lib()
-    lib.unirl_trace_begin.argtypes = [ctypes.c_void_p, ctypes.c_size_t]
-    lib.unirl_trace_entry.restype = ctypes.c_char_p
-    lib.unirl_trace_entry.argtypes = [ctypes.c_int, ctypes.POINTER(ctypes.c_uint), ctypes.POINTER(ctypes.c_size_t)]
+    N.LIB_PATH = TUNE_LIB_PATH  # before the first call binds the library: every product call runs the traced kernels
+    from unirl_amd import _tune
+
+    lib = _tune.lib()
     tick_ns = 10.0
     buf = torch.zeros(8 * 2**20, dtype=torch.int64, device=dev)
     spin = torch.randn(64 * 2**20, device=dev)
@@ -770,10 +769,12 @@ def main() -> int:
         return ops.token_logp_entropy(x, ids, 1.0, want_logp=True, want_entropy=True)
 
     if args.traffic_probe:
+        from unirl_amd import _tune  # the calibration copy is a kernel of the measurement build
+
         src = torch.empty(2**30, dtype=torch.uint8, device=dev).fill_(7)
         dst = torch.empty_like(src)
         for _ in range(3):
-            ops.calib_copy(src, dst)
+            _tune.calib_copy(src, dst)
         for i in range(3):
             step(i)
         torch.cuda.synchronize()
@@ -865,6 +866,11 @@ def main() -> int:
             "elements_per_s": round(x.numel() / (bwd_ms * 1e-3), 0), "timing": "hip events over the timed steps",
         })
         del lse, g_lp
+        from unirl_amd import _tune
+
+        have_tune = _tune.available()
+        if not have_tune:
+            log("measurement build absent (python -m unirl_amd.build --tune): floors and plain reductions are null")
         for sh in make_shapes(torch, dev):
             try:
                 us = time_in_graph(torch, sh["run"], sh["sets"])
@@ -885,37 +891,46 @@ def main() -> int:
             }
             if "bytes_padded" in sh:
                 row["gbps_padded_bytes"] = round(sh["bytes_padded"] / (us * 1e-6) / 1e9, 1)
-            try:  # what a kernel that only moves these bytes costs in the same harness
-                floor_run = make_floor(torch, dev, sh["read_bytes"], sh["write_bytes"], sh["sets"], True)
-                floor_us = time_in_graph(torch, floor_run, sh["sets"])
-                row["floor_us"] = round(floor_us, 2)
-                row["frac_of_floor"] = round(floor_us / us, 4)
-                del floor_run
-            except Exception as exc:
-                log(f"{sh['name']}: floor measurement failed ({type(exc).__name__}: {exc})")
-            if sh["write_bytes"] == 0:
-                # a read-only reducing shape: the plainest reduction of the same bytes (one fp64 partial per
-                # workgroup, then a dependent launch that adds them) in the same harness -- what the
-                # two-launch scheme itself costs before any of the shape's arithmetic
+            # Yardsticks, timed in the same harness (kernels of the measurement build; null without it).
+            # floor: a kernel that only moves the shape's bytes, plus a one-wavefront dependent launch.
+            # plain reduction: the plainest two-launch reduction of the shape's READ bytes (one fp64
+            # partial per workgroup, a dependent launch that adds them) -- what the scheme costs before
+            # any of the shape's arithmetic; for a shape that also writes (the one-pass training steps)
+            # it prices the reads only.
+            row["floor_us"] = row["frac_of_floor"] = None
+            if sh["write_bytes"] == 0 or sh.get("plain_reduction"):
+                row["plain_reduction_us"] = row["frac_of_plain_reduction"] = None
+            if have_tune:
                 try:
-                    rb = (sh["read_bytes"] + 15) // 16 * 16
-                    srcs = [torch.ones(rb, dtype=torch.uint8, device=dev) for _ in range(sh["sets"])]
-                    scratch = torch.zeros(16 + 16 * 512, dtype=torch.uint8, device=dev)
-                    sink = torch.zeros(1, dtype=torch.float64, device=dev)
-                    red_us = time_in_graph(
-                        torch, lambda i: ops.calib_reduce(srcs[i % len(srcs)], rb, 1, 512, scratch, sink), sh["sets"])
-                    row["plain_reduction_us"] = round(red_us, 2)
-                    row["frac_of_plain_reduction"] = round(red_us / us, 4)
-                    del srcs
+                    floor_run = make_floor(torch, dev, sh["read_bytes"], sh["write_bytes"], sh["sets"], True)
+                    floor_us = time_in_graph(torch, floor_run, sh["sets"])
+                    row["floor_us"] = round(floor_us, 2)
+                    row["frac_of_floor"] = round(floor_us / us, 4)
+                    del floor_run
                 except Exception as exc:
-                    log(f"{sh['name']}: plain-reduction measurement failed ({type(exc).__name__}: {exc})")
+                    log(f"{sh['name']}: floor measurement failed ({type(exc).__name__}: {exc})")
+                if "plain_reduction_us" in row:
+                    try:
+                        rb = (sh["read_bytes"] + 15) // 16 * 16
+                        srcs = [torch.ones(rb, dtype=torch.uint8, device=dev) for _ in range(sh["sets"])]
+                        scratch = torch.zeros(16 + 16 * 512, dtype=torch.uint8, device=dev)
+                        sink = torch.zeros(1, dtype=torch.float64, device=dev)
+                        red_us = time_in_graph(
+                            torch, lambda i: _tune.calib_reduce(srcs[i % len(srcs)], rb, 1, 512, scratch, sink),
+                            sh["sets"])
+                        row["plain_reduction_us"] = round(red_us, 2)
+                        row["frac_of_plain_reduction"] = round(red_us / us, 4)
+                        del srcs
+                    except Exception as exc:
+                        log(f"{sh['name']}: plain-reduction measurement failed ({type(exc).__name__}: {exc})")
             if not args.skip_cpu and "cpu" in sh:
                 cms = time_cpu(sh["cpu"], reps=sh.get("cpu_reps", 5), warmup=1)
                 row["cpu_ms"] = round(cms, 2)
                 row["cpu_gbps"] = round(sh["cpu_bytes"] / (cms * 1e-3) / 1e9, 3)
                 row["cpu_cores"] = torch.get_num_threads()
             log(f"{sh['name']}: {us:.2f} us/launch, {gbps:.0f} GB/s = {gbps / HBM_PEAK_GBPS:.1%} of peak, "
-                f"floor {row.get('floor_us', float('nan')):.2f} us, call + sync {lat:.0f} us, host {host:.0f} us")
+                f"floor {row['floor_us']} us, plain reduction {row.get('plain_reduction_us')} us, "
+                f"call + sync {lat:.0f} us, host {host:.0f} us")
             shapes_out.append(row)
 
     # HBM bytes per launch from hardware counters.  Counter runs cannot be made from inside the bench,
@@ -956,7 +971,7 @@ def main() -> int:
         "warmup": args.warmup,
         "ms_per_step": round(wall_ms, 4),
         "higher_is_better": True,
-        "scaling": "weak",
+        "scaling": None,  # one GPU: there is no scaling regime to name
         "vs_baseline": None,
         "dtype": "f32",
         "storage_dtype": "bf16",

@@ -37,9 +37,9 @@ extern "C" {
 
 /* 2: typed gradient outputs in unirl_sde_step_logp_bwd; unirl_ratio_loss_fwd_bwd and
  * unirl_flowdppo_step added.  3: unirl_dpm2_step added.  4: unirl_gaussian_kl_mask_static
- * added.  5: unirl_sde_replay_logp, unirl_sde_replay_logp_bwd, unirl_calib_reduce,
- * unirl_lmhead_logp added. */
-#define UNIRL_ABI_VERSION 5
+ * added.  5: unirl_sde_replay_logp, unirl_sde_replay_logp_bwd, unirl_lmhead_logp added.
+ * 6: the unirl_calib_* measurement aids left the library (they live in the measurement build). */
+#define UNIRL_ABI_VERSION 6
 
 enum unirl_dtype { UNIRL_F32 = 0, UNIRL_BF16 = 1, UNIRL_F16 = 2 };
 
@@ -65,36 +65,6 @@ const char* unirl_status_string(int status);
 size_t unirl_workspace_bytes(void);
 /* Optional: zero-fill a workspace (a fill kernel on `stream`); no entry point needs it. */
 int unirl_workspace_init(void* workspace, size_t workspace_bytes, void* stream);
-
-/* Measurement aid, no counterpart in the reference: a plain streaming copy of
- * `bytes` (a multiple of 16, both pointers 16-byte aligned).  Hardware byte
- * counters read for this kernel calibrate the ones read for the kernels below. */
-int unirl_calib_copy(const void* src, void* dst, size_t bytes, void* stream);
-
-/* Measurement aid, no counterpart in the reference: the launch floor of a
- * streaming kernel.  One kernel reads `read_bytes` from src and writes
- * `write_bytes` to dst (multiples of 16, 16-byte aligned; the two streams are
- * independent and no arithmetic is done), followed, when tail_launch != 0, by
- * a one-wavefront kernel -- the shape of a fused kernel plus its finalize
- * launch.  Timing it for the byte counts of a fused kernel gives the time no
- * kernel of that traffic can beat on the device.  sink: 16 writable bytes. */
-int unirl_calib_stream(const void* src, size_t read_bytes, void* dst, size_t write_bytes,
-                       int tail_launch, void* sink, void* stream);
-
-/* Measurement aid, no counterpart in the reference: what finishing a grid-wide reduction costs.
- * Sums the `read_bytes / 4` floats at src (a multiple of 16 bytes, 16-byte aligned) over
- * n_workgroups workgroups of 256 threads and finishes in one of three ways:
- *   mode 0  the streaming kernel only (per-workgroup partials stored, *out untouched);
- *   mode 1  plus a dependent second launch that adds the partials -- the scheme of every
- *           reducing entry point of this library;
- *   mode 2  a single launch: the partials are published as self-validating tagged 8-byte units
- *           (relaxed device-scope atomics) and polled by the last workgroup, bounded by a
- *           one-second clock budget (*out is NaN if it ever runs out).
- * scratch: at least 16 + 16 * n_workgroups bytes, zero-filled ONCE before its first use with
- * mode 2 (its first word carries the call tag from call to call) and used by one call at a
- * time.  Modes 1 and 2 return the same bits in *out. */
-int unirl_calib_reduce(const void* src, size_t read_bytes, int mode, unsigned int n_workgroups,
-                       void* scratch, size_t scratch_bytes, double* out, void* stream);
 
 /* ------------------------------------------------------------------------
  * One SDE transition + per-sample Gaussian log-prob.
@@ -212,7 +182,9 @@ struct unirl_sde_replay_desc {
 int unirl_sde_replay_logp(const struct unirl_sde_replay_desc* desc /* host */, void* workspace,
                           size_t workspace_bytes, void* stream);
 
-/* Its backward with respect to the velocities (the latents are stored data): g_logp f32 [B,S]
+/* Its backward with respect to the velocities (the latents are stored data) -- the gradient
+ * autograd carries from `new_logp` into the model through the replay loop of
+ * unirl/models/sd3/diffusion.py:467-497 and unirl/sde/kernels.py:200-228: g_logp f32 [B,S]
  * (NULL = 0), g_mean f32 [B,S,D] dense (NULL = 0; the Flow-DPPO loss sends none, its KL mask is
  * detached); grad_v in dtype_gv, laid out like noise_pred (same strides).  mean_out / logp_out
  * of the descriptor are ignored. */
@@ -220,8 +192,8 @@ int unirl_sde_replay_logp_bwd(const struct unirl_sde_replay_desc* desc /* host *
                               const float* g_mean, void* grad_v, int dtype_gv, void* stream);
 
 /* Backward of unirl_sde_step_logp with respect to noise_pred and sample, for
- * the autograd graph the reference builds through kernels.py:225-228 and
- * :200-204 (prev_sample is detached there).  Inputs as in the forward call;
+ * the autograd graph the reference builds through unirl/sde/kernels.py:225-228
+ * and :200-204 (prev_sample is detached there).  Inputs as in the forward call;
  * g_logp [B] f32 (NULL = 0), g_mean [B,D] f32 (NULL = 0), g_prev [B,D] f32
  * (sampling only, NULL = 0).  Outputs grad_v / grad_x are [B,D] in the dtype
  * given for each (autograd hands a gradient back in its input's dtype, so a
@@ -319,7 +291,7 @@ int unirl_gaussian_kl_mask_static(const void* p, const void* q, int dtype, const
                                   int64_t n_sigma, int64_t R, int64_t D, float threshold,
                                   float* kl_out, uint8_t* mask_out, void* stream);
 
-/* The [B,S'] part of _flowdppo_kl_adv_loss (flowdppo.py:86-137) given the row
+/* The [B,S'] part of _flowdppo_kl_adv_loss (unirl/algorithms/flowdppo.py:86-137) given the row
  * KLs from unirl_gaussian_kl_mask: ratio, the KL / advantage-sign masks,
  * loss_elem = where(keep, -A*ratio, 0) and the logged metrics.  All arrays are
  * f32 [n].  metrics [16] f32: 0 ratio_mean, 1 ratio_std, 2 ratio_min,
@@ -332,7 +304,8 @@ int unirl_flowdppo_loss(const float* new_logp, const float* old_logp, const floa
                         float* metrics, void* stream);
 
 /* unirl_gaussian_kl_mask and unirl_flowdppo_loss as one call of two launches for
- * the loss step of FlowDPPO.compute_loss_and_backward (flowdppo.py:309-320):
+ * the loss step of FlowDPPO.compute_loss_and_backward
+ * (unirl/algorithms/flowdppo.py:309-320):
  * the streaming KL kernel, then one workgroup that adds its partials row by
  * row and runs the [B,S'] problem on the result.  R = B*S' rows of D elements
  * in p / q; new_logp, old_logp, advantages, kl_out, loss_elem are f32 [R].
@@ -346,14 +319,14 @@ int unirl_flowdppo_step(const void* p, const void* q, int dtype, const float* si
                         float* metrics /* [16] f32, as unirl_flowdppo_loss */, void* workspace,
                         size_t workspace_bytes, void* stream);
 
-/* Element-wise form of the same quantity (flowdppo.py:51), f32 output [R,D]. */
+/* Element-wise form of the same quantity (unirl/algorithms/flowdppo.py:51), f32 output [R,D]. */
 int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, const float* sigma,
                            int64_t n_sigma, int64_t R, int64_t D, float* out, void* stream);
 
 /* Its backward, for callers that differentiate _gaussian_kl_div (the reference's function is
  * plain torch and therefore differentiable; its own loss detaches the result).  g_out f32 [R,D];
  * grad_p / grad_q in the means' dtype, either may be NULL.  Follows autograd's chain through
- * the 16-bit subtraction and square (flowdppo.py:51). */
+ * the 16-bit subtraction and square (unirl/algorithms/flowdppo.py:51). */
 int unirl_gaussian_kl_elem_bwd(const void* p, const void* q, int dtype, const float* sigma,
                                int64_t n_sigma, int64_t R, int64_t D, const float* g_out,
                                void* grad_p, void* grad_q, void* stream);
@@ -376,7 +349,7 @@ int unirl_token_logp_entropy(const void* logits, int dtype, int64_t rows, int64_
                              float* logp_out, float* ent_out, float* lse_out, void* stream);
 
 /* grad_logits[r, j] = g_logp[r] * (1[j == ids[r]] - softmax(x)[r, j]) / T in
- * `dtype`, the gradient autograd gives through qwen3/ar.py:83-85. */
+ * `dtype`, the gradient autograd gives through unirl/models/qwen3/ar.py:83-85. */
 int unirl_token_logp_bwd(const void* logits, int dtype, int64_t rows, int64_t V,
                          int64_t row_stride, const int64_t* ids, float temperature,
                          const float* lse, const float* g_logp, void* grad_logits,
@@ -404,12 +377,13 @@ int unirl_token_logp_bwd(const void* logits, int dtype, int64_t rows, int64_t V,
  * columns), no initialisation needed, one call at a time.
  * Non-finite logits give NaN outputs for their row.
  * ---------------------------------------------------------------------- */
-size_t unirl_lmhead_logp_scratch_bytes(int64_t rows, int64_t V);
 int unirl_lmhead_logp(const void* hidden, int64_t ld_hidden, const void* weight, int64_t ld_weight,
                       const void* bias, int64_t rows, int64_t V, int64_t K, const int64_t* ids,
                       float temperature, float* logp_out, float* ent_out, float* lse_out,
                       void* logits_out, int64_t ld_logits, void* scratch, size_t scratch_bytes,
                       void* stream);
+/* Bytes of `scratch` unirl_lmhead_logp needs for this many rows and vocabulary entries. */
+size_t unirl_lmhead_logp_scratch_bytes(int64_t rows, int64_t V);
 
 /* ------------------------------------------------------------------------
  * dst[c][r] = src[r][c] for a [rows, cols] matrix of 2- or 4-byte elements
@@ -487,7 +461,10 @@ int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp, const flo
                          float* metrics /* [UNIRL_M_COUNT] f32 */, void* workspace,
                          size_t workspace_bytes, void* stream);
 
-/* grad_new = g_scale * w_tok * dloss/dnew, where w_tok is the aggregation
+/* Backward of unirl_ratio_loss_fwd: what `(loss * loss_scale).backward()` leaves in new_logp
+ * (unirl/algorithms/grpo.py:156, unirl/algorithms/drpo.py:331) through the token arithmetic of
+ * unirl/algorithms/base.py:133-157 / unirl/algorithms/drpo.py:131-159.
+ * grad_new = g_scale * w_tok * dloss/dnew, where w_tok is the aggregation
  * weight of the token (1/N, 1/(n_seq*horizon) or 1/(n_seq*len)), times
  * g_elem per token when that is not NULL (the caller reduced loss_per_elem
  * itself).  Padded slots past a sequence's length receive 0. */

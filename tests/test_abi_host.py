@@ -33,11 +33,45 @@ def test_header_symbols_are_exported_and_bound(built_lib):
     assert sorted(_native.EXPORTED_SYMBOLS) == names, "ctypes signature table and header disagree"
 
 
+def test_shipped_library_exports_exactly_the_declared_entry_points(built_lib):
+    """The dynamic symbol table of the shipped library holds the header's entry points and no other
+    `unirl_*` name: no yardstick kernel, timeline hook or other measurement aid is exported.  Every
+    declaration in the header cites the reference lines it replaces, except the one allocation-free
+    entry point, whose comment says that it has no counterpart there."""
+    import shutil
+    import subprocess
+
+    nm = shutil.which("nm") or shutil.which("llvm-nm", path="/opt/rocm/llvm/bin")
+    if nm is None:
+        pytest.skip("no nm on this host")
+    out = subprocess.run([nm, "-D", "--defined-only", str(built_lib)], check=True, capture_output=True, text=True).stdout
+    exported = sorted({line.split()[-1] for line in out.splitlines() if re.search(r"\bunirl_[a-z0-9_]+$", line)})
+    assert exported == declared_symbols()
+    assert not [n for n in exported if "calib" in n or "trace" in n]
+    # each entry point's comment names the reference (a path under unirl/ with a line), the library-level
+    # calls (version, status text, workspace size and fill, scratch size) aside
+    text = HEADER.read_text()
+    library_level = {"unirl_abi_version", "unirl_status_string", "unirl_workspace_bytes", "unirl_workspace_init",
+                     "unirl_lmhead_logp_scratch_bytes"}
+    missing = []
+    starts = sorted((re.search(r"^(?:int|size_t|const char\*) " + n + r"\(", text, flags=re.M).start(), n) for n in exported)
+    for k, (decl, name) in enumerate(starts):
+        if name in library_level:
+            continue
+        comment = text[(starts[k - 1][0] if k else 0):decl]  # everything since the previous declaration
+        comment = re.sub(r"\s*\n\s*\*?\s*", " ", comment)  # undo the comment's line breaks
+        if name == "unirl_gaussian_kl_mask_static" or name.endswith("_noalloc"):
+            assert "no counterpart in the reference" in comment, name
+        elif not re.search(r"unirl/[a-z0-9_/]+\.py:\d+", comment):
+            missing.append(name)
+    assert not missing, f"declarations whose comment cites no reference line: {missing}"
+
+
 def test_version_status_strings_and_workspace(built_lib):
     from unirl_amd import _native as N
 
     L = N.lib()
-    assert L.unirl_abi_version() == N.ABI_VERSION == 5
+    assert L.unirl_abi_version() == N.ABI_VERSION == 6
     assert f"#define UNIRL_ABI_VERSION {N.ABI_VERSION}" in (ROOT / "include" / "unirl_hip.h").read_text()
     assert L.unirl_workspace_bytes() >= 64 * 1024
     assert L.unirl_status_string(0) == b"ok"

@@ -130,16 +130,13 @@ class Dpm2Coeffs(Structure):
 
 
 # UNIRL_ABI_VERSION of include/unirl_hip.h that the signatures below describe
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _SIGNATURES = {
     "unirl_abi_version": (c_int, []),
     "unirl_status_string": (c_char_p, [c_int]),
     "unirl_workspace_bytes": (c_size_t, []),
     "unirl_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
-    "unirl_calib_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
-    "unirl_calib_stream": (c_int, [c_void_p, c_size_t, c_void_p, c_size_t, c_int, c_void_p, c_void_p]),
-    "unirl_calib_reduce": (c_int, [c_void_p, c_size_t, c_int, ctypes.c_uint, c_void_p, c_size_t, c_void_p, c_void_p]),
     "unirl_sde_step_logp": (
         c_int,
         [c_void_p, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_float,

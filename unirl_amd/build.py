@@ -62,8 +62,12 @@ def _run(cmd: List[str]) -> None:
         print(out, file=sys.stderr)
 
 
-def sources() -> List[Path]:
-    return sorted(CSRC_DIR.glob("*.hip"))
+# sources of the measurement build only (yardstick kernels, the timeline's host side)
+TUNE_ONLY = ("calib_tune.hip",)
+
+
+def sources(tune: bool = False) -> List[Path]:
+    return sorted(p for p in CSRC_DIR.glob("*.hip") if tune or p.name not in TUNE_ONLY)
 
 
 def build(verbose: bool = True, jobs: int | None = None, *, tune: bool = False, out: Path | None = None,
@@ -71,8 +75,9 @@ def build(verbose: bool = True, jobs: int | None = None, *, tune: bool = False, 
     """Compile every kernel source and link the shared library. Always recompiles.
 
     ``tune=True`` makes a measurement build (``-DUNIRL_TUNE -DUNIRL_TRACE``: launch-shape knobs read
-    from the environment, device-side timeline marks); it must be given its own ``out`` path and is
-    never the library the package loads.
+    from the environment, device-side timeline marks, plus the yardstick kernels of
+    ``calib_tune.hip``); it must be given its own ``out`` path and is never the library the
+    package loads.
     """
     hipcc = _hipcc()
     if tune and out is None:
@@ -80,7 +85,7 @@ def build(verbose: bool = True, jobs: int | None = None, *, tune: bool = False, 
     lib_path = Path(out) if out is not None else LIB_PATH
     obj_dir = OBJ_DIR if out is None else lib_path.parent / (lib_path.stem + "_obj")
     obj_dir.mkdir(parents=True, exist_ok=True)
-    srcs = sources()
+    srcs = sources(tune)
     if not srcs:
         raise RuntimeError(f"no .hip sources under {CSRC_DIR}")
     objs = [obj_dir / (s.stem + ".o") for s in srcs]

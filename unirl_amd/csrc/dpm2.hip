@@ -15,7 +15,7 @@
 // HBM traffic: model_output and sample read once (+ x0_prev for the second order), x0 and prev
 // written once: 16 (20) bytes per element for fp32 inputs.
 
-#include "common.cuh"
+#include "common_hip.h"
 #include "unirl_internal.h"
 
 namespace unirl {

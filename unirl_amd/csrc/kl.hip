@@ -13,7 +13,7 @@
 
 #include <mutex>
 
-#include "common.cuh"
+#include "common_hip.h"
 #include "unirl_internal.h"
 
 namespace unirl {

@@ -31,7 +31,7 @@
 
 #include <type_traits>
 
-#include "common.cuh"
+#include "common_hip.h"
 #include "unirl_internal.h"
 
 namespace unirl {

@@ -1,7 +1,7 @@
 // Small kernels around the hot path: group-normalised advantages and the
 // step gather.
 
-#include "common.cuh"
+#include "common_hip.h"
 #include "unirl_internal.h"
 
 namespace unirl {

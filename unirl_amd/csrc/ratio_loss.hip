@@ -23,7 +23,7 @@
 // HBM traffic: 8 bytes read per valid token (+4 with a mask, +4 with per-token
 // advantages), +4 written per slot when loss_per_elem or grad_new is requested.
 
-#include "common.cuh"
+#include "common_hip.h"
 #include "unirl_internal.h"
 
 namespace unirl {

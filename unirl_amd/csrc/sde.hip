@@ -16,7 +16,7 @@
 // HBM traffic per element (fp32, sampling): read v, x, noise; write prev, mean
 // = 20 bytes; replay with the mean kept: read v, x, prev; write mean = 16.
 
-#include "common.cuh"
+#include "common_hip.h"
 #include "unirl_internal.h"
 
 namespace unirl {

@@ -35,7 +35,7 @@
 
 #include <float.h>
 
-#include "common.cuh"
+#include "common_hip.h"
 #include "unirl_internal.h"
 
 namespace unirl {

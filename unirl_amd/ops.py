@@ -1294,55 +1294,6 @@ def normalize_grouped(
     return out
 
 
-def calib_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
-    """Plain streaming copy of ``src`` into ``dst`` (same byte size, a multiple of 16): the
-    reference kernel for calibrating hardware byte counters."""
-    N.require_device(src, "src")
-    N.require_device(dst, "dst")
-    nbytes = src.numel() * src.element_size()
-    if nbytes != dst.numel() * dst.element_size() or not (src.is_contiguous() and dst.is_contiguous()):
-        raise ValueError("calib_copy needs two contiguous tensors of the same byte size")
-    with N.on_device(src.device):
-        rc = N.F.unirl_calib_copy(N.ptr(src), N.ptr(dst), nbytes, N.current_stream(src.device))
-    N.check(rc, "unirl_calib_copy")
-
-
-def calib_stream(src: Optional[torch.Tensor], read_bytes: int, dst: Optional[torch.Tensor], write_bytes: int,
-                 sink: torch.Tensor, *, tail_launch: bool = False) -> None:
-    """Launch-floor yardstick: one kernel that reads ``read_bytes`` of ``src`` and writes
-    ``write_bytes`` of ``dst`` with no arithmetic, then (``tail_launch``) a one-wavefront kernel."""
-    N.require_device(sink, "sink")
-    for t, nbytes, name in ((src, read_bytes, "src"), (dst, write_bytes, "dst")):
-        if nbytes:
-            N.require_device(t, name)
-            if not t.is_contiguous() or t.numel() * t.element_size() < nbytes:
-                raise ValueError(f"{name} must be contiguous and hold at least {nbytes} bytes")
-    with N.on_device(sink.device):
-        rc = N.F.unirl_calib_stream(
-            N.ptr(src) if read_bytes else None, int(read_bytes), N.ptr(dst) if write_bytes else None,
-            int(write_bytes), int(bool(tail_launch)), N.ptr(sink), N.current_stream(sink.device),
-        )
-    N.check(rc, "unirl_calib_stream")
-
-
-def calib_reduce(src: torch.Tensor, read_bytes: int, mode: int, n_workgroups: int, scratch: torch.Tensor,
-                 out: torch.Tensor) -> None:
-    """Measurement aid: the sum of ``read_bytes // 4`` floats of ``src``, finished by nothing (mode 0),
-    a second launch (mode 1) or inside the one kernel by polling tagged partials (mode 2).
-    ``scratch``: zero-filled once, at least ``16 + 16 * n_workgroups`` bytes; ``out``: float64 [1]."""
-    for t, name in ((src, "src"), (scratch, "scratch"), (out, "out")):
-        N.require_device(t, name)
-    if not src.is_contiguous() or src.numel() * src.element_size() < read_bytes:
-        raise ValueError(f"src must be contiguous and hold at least {read_bytes} bytes")
-    if out.dtype != torch.float64 or out.numel() < 1:
-        raise ValueError("out must be a float64 tensor")
-    with N.on_device(src.device):
-        rc = N.F.unirl_calib_reduce(N.ptr(src), int(read_bytes), int(mode), int(n_workgroups), N.ptr(scratch),
-                                        scratch.numel() * scratch.element_size(), N.ptr(out),
-                                        N.current_stream(src.device))
-    N.check(rc, "unirl_calib_reduce")
-
-
 def gather_steps(tensor: torch.Tensor, positions: Sequence[int]) -> torch.Tensor:
     """``tensor[:, positions]`` for a ``[B, S, ...]`` tensor, as one gather kernel."""
     N.require_device(tensor, "tensor")
