@@ -348,6 +348,21 @@ __device__ __forceinline__ double row_max_last(double v) {
   return v;
 }
 
+__device__ __forceinline__ unsigned int row_sum_last(unsigned int v) {
+  v += dpp_u32_or_zero<0x111, 0xf>(v);
+  v += dpp_u32_or_zero<0x112, 0xf>(v);
+  v += dpp_u32_or_zero<0x114, 0xf>(v);
+  v += dpp_u32_or_zero<0x118, 0xf>(v);
+  return v;
+}
+__device__ __forceinline__ float row_max_last(float v) {
+  v = fmaxf(v, dpp_f32_or_self<0x111, 0xf>(v));
+  v = fmaxf(v, dpp_f32_or_self<0x112, 0xf>(v));
+  v = fmaxf(v, dpp_f32_or_self<0x114, 0xf>(v));
+  v = fmaxf(v, dpp_f32_or_self<0x118, 0xf>(v));
+  return v;
+}
+
 // Wave-uniform results.
 __device__ __forceinline__ float wave_sum(float v) {
   UNIRL_DPP_REDUCE(v, op_add, dpp_f32_or_zero)
@@ -444,12 +459,39 @@ __device__ __forceinline__ float block_min(float v, float* lds) {
 // arrival finalises" tickets serialise at ~90 ns per same-address atomic,
 // which exceeds the ~2 us cost of the second launch beyond ~25 workgroups.
 // ---------------------------------------------------------------------------
-// Sum of `n` partials at `p`, added in a fixed order by one wavefront; valid in every lane.
-__device__ __forceinline__ double wave_ordered_sum(const double* __restrict__ p, int64_t n) {
+// Fixed-order sums of `n` partials at `p` by one wavefront.  Lane l adds p[first + l],
+// p[first + l + 64], ... in that order.  The loads go out in batches of kBatch before the first is
+// used -- a plain `for (j) q += p[j]` makes one trip to memory per iteration, each waiting for the
+// one before -- and a lane past the end loads the last partial and adds zero instead (a load
+// behind a condition would be waited for before the next is issued).
+template <int kBatch>
+__device__ __forceinline__ double lane_ordered_sum_batched(const double* __restrict__ p, int64_t n, int64_t first) {
   const int lane = threadIdx.x & (kWave - 1);
   double q = 0.0;
-  for (int64_t j = lane; j < n; j += kWave) q += p[j];
-  return wave_sum(q);
+  for (int64_t j0 = first + lane; j0 - lane < n; j0 += kWave * kBatch) {
+    double y[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int64_t j = j0 + b * kWave;
+      y[b] = p[j < n ? j : n - 1];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) q += (j0 + b * kWave < n) ? y[b] : 0.0;
+  }
+  return q;
+}
+// The batch follows the count (wave-uniform): surplus loads of a short row cost more than they hide.
+__device__ __forceinline__ double lane_ordered_sum(const double* __restrict__ p, int64_t n, int64_t first) {
+  const int64_t rem = n - first;
+  if (rem <= kWave) return lane_ordered_sum_batched<1>(p, n, first);
+  if (rem <= 2 * kWave) return lane_ordered_sum_batched<2>(p, n, first);
+  if (rem <= 4 * kWave) return lane_ordered_sum_batched<4>(p, n, first);
+  return lane_ordered_sum_batched<8>(p, n, first);
+}
+// The whole sum, valid in every lane.
+__device__ __forceinline__ double wave_ordered_sum(const double* __restrict__ p, int64_t n) {
+  return wave_sum(lane_ordered_sum(p, n, 0));
 }
 
 }  // namespace unirl

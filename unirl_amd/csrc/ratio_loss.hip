@@ -29,20 +29,48 @@
 namespace unirl {
 
 constexpr int kRlThreads = 256;
-constexpr int kRlVals = 16;  // partial values per workgroup
+constexpr int kRlVals = 16;  // slots of the workgroup reduction (13 in use)
 
 enum { LAYOUT_FLAT = 0, LAYOUT_PADDED = 1, LAYOUT_PACKED = 2 };
 
-// Slots of the per-workgroup partial vector.  Slots below kFirstMax are sums, the rest maxima
-// (the ratio minimum travels negated); the reductions handle four consecutive slots per
-// wavefront, so this order keeps the two kinds in different wavefronts.  10, 11, 15 are unused.
+// Slots of the workgroup reduction: six fp64 sums, four token counters, three fp32 maxima (the
+// ratio minimum travels negated).  The reductions handle four consecutive slots per wavefront,
+// so this order gives every wavefront one type and one operation.  6, 7 and 15 are unused.
 enum {
-  P_SR = 0, P_SR2, P_LOSS, P_KL, P_PEN, P_ABS, P_CNT, P_CHI, P_CLO, P_CANY,
+  P_SR = 0, P_SR2, P_LOSS, P_KL, P_PEN, P_ABS,
+  P_CNT = 8, P_CHI, P_CLO, P_CANY,
   P_NRMIN = 12, P_RMAX = 13, P_AMAX = 14
 };
-constexpr int kFirstMax = 12;
+constexpr int kNumSums = 6, kFirstCnt = 8, kNumCnt = 4, kFirstMax = 12, kNumMax = 3;
 constexpr int kRlParts = 16;  // threads that share one slot in the reductions below
 static_assert(kRlParts * 16 == 256, "reductions assume 256 threads = 16 slots x 16 parts");
+
+// What a workgroup hands to the finalize kernel: 76 bytes in five 16-byte chunks -- sums 0-1,
+// 2-3, 4-5, the four counters (they fit 32 bits: a workgroup sees far fewer than 2^32 tokens),
+// the three extrema (fp32 values).  The chunks are stored chunk-major, so that each finalize
+// wavefront reads one contiguous array, and inside a chunk array the workgroups are ordered by
+// (j mod 8, j / 8): consecutive workgroups run on different XCDs (dispatch deals them out in
+// turn), each behind its own L2, and a 128-byte line written piecewise from eight L2s costs the
+// reader far more than one written from a single L2 -- this order makes every line of the arrays
+// the work of one XCD.  (Only speed depends on that dispatch order, never a result.)
+constexpr int kRlChunks = 5;
+constexpr unsigned int kXcds = 8;
+__host__ __device__ __forceinline__ unsigned int partial_per_xcd(unsigned int nblk) { return (nblk + kXcds - 1) / kXcds; }
+__device__ __forceinline__ char* partial_slot(char* base, unsigned int nblk, unsigned int blk, int v) {
+  int chunk, off;
+  if (v < kNumSums) {
+    chunk = v >> 1;
+    off = (v & 1) * 8;
+  } else if (v < kFirstMax) {
+    chunk = 3;
+    off = (v - kFirstCnt) * 4;
+  } else {
+    chunk = 4;
+    off = (v - kFirstMax) * 4;
+  }
+  const unsigned int per = partial_per_xcd(nblk);
+  return base + ((size_t)chunk * (per * kXcds) + (blk % kXcds) * per + blk / kXcds) * 16 + off;
+}
 
 struct RatioConsts {
   int kind;
@@ -55,6 +83,10 @@ struct RatioConsts {
   float drpo_two_eps;        // (float)(2.0 * epsilon)
   float inv_two_eps;         // 1 / drpo_two_eps, correctly rounded
   float horizon;
+  // DRPO, token-adaptive boundary: with epsilon >= 1 a token with mu <= 1 and r <= fast_hi =
+  // fl(1 + epsilon) can be on neither side of its trust region (see drpo_flags_provably_clear)
+  int fast_ok;
+  float fast_hi;
 };
 
 struct RatioArgs {
@@ -68,7 +100,7 @@ struct RatioArgs {
   RatioConsts C;
   float* loss_elem;
   float* metrics;
-  double* partials;
+  char* partials;  // kRlChunks * n_workgroups 16-byte units, see partial_slot
   // backward only
   const float* g_scale;
   const float* g_elem;
@@ -218,12 +250,32 @@ struct WaveCounts {
 //   1 - r = -(r - 1)                  -- rounding is symmetric, so the lower clip test reuses r-1.
 // With GRAD the derivative of the token's loss with respect to new_logp is left in `dl` (the
 // expressions of ratio_token, which the stand-alone backward kernel uses).
-template <int KIND, bool GRAD>
+// DRPO's two boundary flags of one token: ratio beyond 1 +- epsilon_t with epsilon_t = epsilon / mu
+// (torch evaluates scalar / tensor as reciprocal(tensor) * scalar; infinity where mu == 0).
+__device__ __forceinline__ void drpo_flags(float r, float mu, const RatioConsts& C, bool& hi, bool& lo) {
+  float aeps = C.drpo_eps;
+  if (C.mu_weighted) aeps = (mu > 0.0f) ? recip_pos(mu) * C.drpo_eps : INFINITY;
+  hi = r > (1.0f + aeps);
+  lo = r < (1.0f - aeps);
+}
+// True when both flags are false without evaluating them (C.fast_ok: mu-weighted, epsilon >= 1).
+// mu <= 1 gives fl(1/mu) >= 1, so epsilon_t = fl(fl(1/mu) * epsilon) >= epsilon and, rounding
+// being monotone, fl(1 + epsilon_t) >= fl(1 + epsilon) = fast_hi >= r: not above.  And
+// fl(1 - epsilon_t) <= fl(1 - epsilon) <= 0 < r (r = exp of a clamped value): not below.  A NaN in
+// mu or r fails the comparisons and sends the token to drpo_flags.
+__device__ __forceinline__ bool drpo_flags_provably_clear(float r, float mu, const RatioConsts& C) {
+  return (mu <= 1.0f) && (r <= C.fast_hi);
+}
+
+// FLAGS = false (DRPO only): the boundary flags are left to the caller, who gets r and mu.
+template <int KIND, bool GRAD, bool FLAGS = true>
 __device__ __forceinline__ float accumulate_token(float nw, float od, float A, float lw, const RatioConsts& C,
-                                                  Acc& acc, bool& hi, bool& lo, float& dl) {
+                                                  Acc& acc, bool& hi, bool& lo, float& dl, float& r_out,
+                                                  float& mu_out) {
   const float d0 = nw - od;
   float r, loss;
   dl = 0.0f;
+  mu_out = 0.0f;
   if (KIND == UNIRL_LOSS_GRPO) {
     r = exp_f32(d0);
     const float nA = -A;
@@ -252,10 +304,9 @@ __device__ __forceinline__ float accumulate_token(float nw, float od, float A, f
     const float w = C.mu_weighted ? mu : 1.0f;
     const float pen = div_by_const((fabsf(A) * w) * (d * d), C.drpo_two_eps, C.inv_two_eps);
     loss = (-A) * r + pen;
-    float aeps = C.drpo_eps;
-    if (C.mu_weighted) aeps = (mu > 0.0f) ? recip_pos(mu) * C.drpo_eps : INFINITY;
-    hi = r > (1.0f + aeps);
-    lo = r < (1.0f - aeps);
+    if (FLAGS) drpo_flags(r, mu, C, hi, lo);
+    else hi = lo = false;
+    mu_out = mu;
     acc.s1 += d;
     acc.s2 = fmaf(d, d, acc.s2);
     acc.kl += d - ld;
@@ -272,7 +323,14 @@ __device__ __forceinline__ float accumulate_token(float nw, float od, float A, f
   const unsigned int rb = __float_as_uint(r);
   acc.rmin = rb < acc.rmin ? rb : acc.rmin;
   acc.rmax = rb > acc.rmax ? rb : acc.rmax;
+  r_out = r;
   return loss;
+}
+template <int KIND, bool GRAD>
+__device__ __forceinline__ float accumulate_token(float nw, float od, float A, float lw, const RatioConsts& C,
+                                                  Acc& acc, bool& hi, bool& lo, float& dl) {
+  float r, mu;
+  return accumulate_token<KIND, GRAD, true>(nw, od, A, lw, C, acc, hi, lo, dl, r, mu);
 }
 
 // sequence lookup for the packed layout: largest s with cu[s] <= tok
@@ -360,6 +418,32 @@ __device__ __forceinline__ void ratio_vec_wave(const RatioConsts& C, const float
                                                const float (&mk)[VEC], bool adv_tok, float gfac, const SeqCtx& sq,
                                                Acc& acc, WaveCounts& wc, float (&out)[VEC], float (&gr)[VEC]) {
   const float grow = gfac * sq.w;
+  if (KIND == UNIRL_LOSS_DRPO && C.fast_ok) {
+    // The boundary flags cost a reciprocal and two comparisons per token and are almost never set:
+    // evaluate them only when some token of the wavefront's vector is not provably clear of both.
+    float r[VEC], mu[VEC];
+    bool slow = false;
+#pragma unroll
+    for (int k = 0; k < VEC; ++k) {
+      const float a = adv_tok ? ad[k] : sq.adv;
+      bool hi, lo;
+      float dl;
+      out[k] = accumulate_token<KIND, GRAD, false>(nw[k], od[k], a, WTOK ? mk[k] * sq.w : mk[k], C, acc, hi, lo, dl,
+                                                   r[k], mu[k]);
+      gr[k] = (grow * mk[k]) * dl;
+      slow = slow || !drpo_flags_provably_clear(r[k], mu[k], C);
+    }
+    if (__builtin_amdgcn_ballot_w64(slow) != 0ull) {
+#pragma unroll
+      for (int k = 0; k < VEC; ++k) {
+        bool hi, lo;
+        drpo_flags(r[k], mu[k], C, hi, lo);
+        wc.add(hi, lo);
+      }
+    }
+    acc.cnt += VEC;
+    return;
+  }
 #pragma unroll
   for (int k = 0; k < VEC; ++k) {
     const float a = adv_tok ? ad[k] : sq.adv;
@@ -372,50 +456,79 @@ __device__ __forceinline__ void ratio_vec_wave(const RatioConsts& C, const float
   acc.cnt += VEC;
 }
 
-__device__ __forceinline__ bool slot_used(int v) { return v <= P_CANY || (v >= P_NRMIN && v <= P_AMAX); }
+__device__ __forceinline__ bool slot_used(int v) {
+  return v < kNumSums || (v >= kFirstCnt && v < kFirstCnt + kNumCnt) || (v >= kFirstMax && v < kFirstMax + kNumMax);
+}
+
+// LDS of the workgroup reduction, each value in its own type: [slot][thread].
+struct RlLds {
+  double sums[kNumSums][kRlThreads];
+  unsigned int cnts[kNumCnt][kRlThreads];
+  float exts[kNumMax][kRlThreads];
+};
 
 // Workgroup partial vector -> A.partials[workgroup].  Every thread must call.
 // Through LDS rather than thirteen wavefront reductions: every thread stores its values as
 // [slot][thread] (consecutive lanes, consecutive words), then thread (slot, part) = (tid / 16,
 // tid % 16) combines the sixteen entries part, part + 16, ... of its slot and four row shifts
 // finish each 16-lane row.  Fixed order, one barrier.
-__device__ __forceinline__ void store_block_partials(const RatioArgs& A, Acc& acc, const WaveCounts& wc,
-                                                     double (*lds_v)[kRlThreads]) {
+__device__ __forceinline__ void store_block_partials(const RatioArgs& A, Acc& acc, const WaveCounts& wc, RlLds& lds) {
   const int t = threadIdx.x;
   const bool lead = (t & (kWave - 1)) == 0;  // carries the wavefront's own counters
-  lds_v[P_SR][t] = acc.t_s1;
-  lds_v[P_SR2][t] = acc.t_s2;
-  lds_v[P_LOSS][t] = acc.t_loss;
-  lds_v[P_KL][t] = acc.t_kl;
-  lds_v[P_PEN][t] = acc.t_pen;
-  lds_v[P_ABS][t] = acc.t_ab;
-  lds_v[P_CNT][t] = (double)acc.cnt;
-  lds_v[P_CHI][t] = (double)(acc.chi + (lead ? wc.hi : 0u));
-  lds_v[P_CLO][t] = (double)(acc.clo + (lead ? wc.lo : 0u));
-  lds_v[P_CANY][t] = (double)(acc.cany + (lead ? wc.any : 0u));
+  lds.sums[P_SR][t] = acc.t_s1;
+  lds.sums[P_SR2][t] = acc.t_s2;
+  lds.sums[P_LOSS][t] = acc.t_loss;
+  lds.sums[P_KL][t] = acc.t_kl;
+  lds.sums[P_PEN][t] = acc.t_pen;
+  lds.sums[P_ABS][t] = acc.t_ab;
+  lds.cnts[P_CNT - kFirstCnt][t] = acc.cnt;
+  lds.cnts[P_CHI - kFirstCnt][t] = acc.chi + (lead ? wc.hi : 0u);
+  lds.cnts[P_CLO - kFirstCnt][t] = acc.clo + (lead ? wc.lo : 0u);
+  lds.cnts[P_CANY - kFirstCnt][t] = acc.cany + (lead ? wc.any : 0u);
   // NaN ratios drop out of the maxima below; the finalize kernel restores NaN from the sums
-  lds_v[P_NRMIN][t] = -(double)__uint_as_float(acc.rmin);
-  lds_v[P_RMAX][t] = acc.cnt ? (double)__uint_as_float(acc.rmax) : -(double)INFINITY;
-  lds_v[P_AMAX][t] = acc.cnt ? (double)acc.amax : -(double)INFINITY;
+  lds.exts[P_NRMIN - kFirstMax][t] = -__uint_as_float(acc.rmin);
+  lds.exts[P_RMAX - kFirstMax][t] = acc.cnt ? __uint_as_float(acc.rmax) : -INFINITY;
+  lds.exts[P_AMAX - kFirstMax][t] = acc.cnt ? acc.amax : -INFINITY;
   __syncthreads();
+  constexpr int kPer = kRlThreads / kRlParts;
   const int v = t / kRlParts, part = t % kRlParts;
-  double x = 0.0;
-  if (slot_used(v)) {
-    double y[kRlThreads / kRlParts];
-#pragma unroll
-    for (int j = 0; j < kRlThreads / kRlParts; ++j) y[j] = lds_v[v][j * kRlParts + part];
-    x = y[0];
-    if (v < kFirstMax) {
-#pragma unroll
-      for (int j = 1; j < kRlThreads / kRlParts; ++j) x += y[j];
-    } else {
-#pragma unroll
-      for (int j = 1; j < kRlThreads / kRlParts; ++j) x = fmax(x, y[j]);
+  const unsigned int blk = blockIdx.y * gridDim.x + blockIdx.x, nblk = gridDim.x * gridDim.y;
+  char* out = partial_slot(A.partials, nblk, blk, v);  // reduced by ratio_loss_finalize_kernel
+  // The chunk arrays hold 8 * ceil(nblk / 8) positions; when nblk is not a multiple of 8 the last
+  // position of the XCDs nblk % 8 ... 7 belongs to no workgroup: workgroup 0 stores the identity there.
+  if (blk == 0 && (nblk % kXcds) != 0 && t < kRlChunks * (int)kXcds) {
+    const unsigned int chunk = t / kXcds, x = t % kXcds, per = partial_per_xcd(nblk);
+    if (x >= nblk % kXcds) {
+      const unsigned int w = (chunk == 4) ? 0xff800000u : 0u;  // -inf for the maxima, 0 for sums and counters
+      const u32x4 ident = {w, w, w, w};
+      reinterpret_cast<u32x4*>(A.partials)[(size_t)chunk * (per * kXcds) + x * per + per - 1] = ident;
     }
   }
-  x = (v < kFirstMax) ? row_sum_last(x) : row_max_last(x);
-  const unsigned int blk = blockIdx.y * gridDim.x + blockIdx.x;
-  if (part == kRlParts - 1) A.partials[(int64_t)blk * kRlVals + v] = x;  // reduced by ratio_loss_finalize_kernel
+  if (v < kNumSums) {
+    double y[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) y[j] = lds.sums[v][j * kRlParts + part];
+    double x = y[0];
+#pragma unroll
+    for (int j = 1; j < kPer; ++j) x += y[j];
+    x = row_sum_last(x);
+    if (part == kRlParts - 1) *reinterpret_cast<double*>(out) = x;
+  } else if (v >= kFirstCnt && v < kFirstCnt + kNumCnt) {
+    unsigned int x = 0;
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) x += lds.cnts[v - kFirstCnt][j * kRlParts + part];
+    x = row_sum_last(x);
+    if (part == kRlParts - 1) *reinterpret_cast<unsigned int*>(out) = x;
+  } else if (v >= kFirstMax && v < kFirstMax + kNumMax) {
+    float y[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) y[j] = lds.exts[v - kFirstMax][j * kRlParts + part];
+    float x = y[0];
+#pragma unroll
+    for (int j = 1; j < kPer; ++j) x = fmaxf(x, y[j]);
+    x = row_max_last(x);
+    if (part == kRlParts - 1) *reinterpret_cast<float*>(out) = x;
+  }
 }
 
 template <int VEC>
@@ -435,7 +548,7 @@ __device__ __forceinline__ void fill_ones(float (&m)[VEC]) {
 // most of the kernel (9.2 -> 8.7 us on 1.1 M tokens in 256 ragged rows).
 template <int KIND, int VEC, bool PACKED, int FLAGS, bool GRAD, int ITEMS = 2>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A) {
-  __shared__ double lds_v[kRlVals][kRlThreads];
+  __shared__ RlLds lds_v;
   UNIRL_TRACE_T0();
   const RatioConsts C = A.C;
   const bool has_mask = (FLAGS < 0) ? (A.mask != nullptr) : ((FLAGS & 1) != 0);
@@ -468,7 +581,7 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
     auto clamped = [&](int64_t len) { return len < 0 ? 0 : (len > A.seq_stride ? A.seq_stride : len); };
     double s = (double)clamped(len_first);  // exact: lengths are far below 2^53
     for (int64_t i = (int64_t)threadIdx.x + kRlThreads; i < A.n_seq; i += kRlThreads) s += (double)clamped(A.seq[i]);
-    const double nv = block_sum(s, &lds_v[0][0]);
+    const double nv = block_sum(s, &lds_v.sums[0][0]);
     __syncthreads();  // lds_v is reused at the end
     gfac = A.loss_scale / (float)nv;
     sum_pending = false;
@@ -626,7 +739,7 @@ __device__ __forceinline__ int64_t wave_find_seq(const CU& cu, int64_t n_seq, in
 template <int KIND, int FLAGS, bool GRAD, int ITEMS>
 __global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs A) {
   constexpr int VEC = 4;
-  __shared__ double lds_v[kRlVals][kRlThreads];
+  __shared__ RlLds lds_v;
   UNIRL_TRACE_T0();
   const RatioConsts C = A.C;
   const bool has_mask = (FLAGS & 1) != 0;
@@ -797,56 +910,93 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs
   UNIRL_TRACE_END(A.trace);
 }
 
-// One workgroup of T threads (256, or 1024 when there are more than 512 partial vectors, so that
-// every load of a thread is still in flight at once): fixed-order reduction of every
-// workgroup's partial vector, then the metrics.
-template <int T>
-__global__ __launch_bounds__(T) void ratio_loss_finalize_kernel(RatioArgs A, unsigned int nblk) {
-  constexpr int kSlices = T / kRlVals;  // 16 or 64
-  static_assert(kSlices == kRlParts || kSlices == kWave, "a slot's slices fill a 16-lane row or a wavefront");
-  __shared__ double lds_t[T];
+// One workgroup of five wavefronts: wavefront c reads the c-th 16-byte chunk of every workgroup's
+// partial vector (two sums; two sums; two sums; the four counters; the three extrema),
+// lane l the vectors l, l + 64, ... in that order, every load of a lane in flight at once; one
+// wavefront reduction per value then leaves the thirteen totals in LDS and sixteen lanes turn them
+// into the metrics.  Fixed order throughout.
+constexpr int kFinThreads = 5 * kWave;
+__global__ __launch_bounds__(kFinThreads) void ratio_loss_finalize_kernel(RatioArgs A, unsigned int nblk) {
   __shared__ double lds_tot[kRlVals];
   UNIRL_TRACE_T0();
   const RatioConsts C = A.C;
   const int t = threadIdx.x;
   {
-    // thread = (slot v, slice j0): the slices walk the workgroups' vectors (a wavefront reads
-    // four whole vectors per load), kBatch loads in flight each
-    const int v = t % kRlVals;
-    const int j0 = t / kRlVals;
-    constexpr int kBatch = 32;
-    const double ident = (v < kFirstMax) ? 0.0 : -(double)INFINITY;
-    double x = ident;
-    for (unsigned int j = j0; j < nblk; j += kSlices * kBatch) {
-      double y[kBatch];
+    const int lane = t & (kWave - 1);
+    const int chunk = __builtin_amdgcn_readfirstlane(t) / kWave;  // wave-uniform
+    const unsigned int per = partial_per_xcd(nblk), npos = per * kXcds;
+    const u32x4* src = reinterpret_cast<const u32x4*>(A.partials) + (size_t)chunk * npos;
+    constexpr int kBatch = 16;
+    const unsigned int idw = (chunk == 4) ? 0xff800000u : 0u;  // -inf for the maxima, 0 for the sums
+    const u32x4 ident = {idw, idw, idw, idw};
+    double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
+    float m0 = -INFINITY, m1 = -INFINITY, m2 = -INFINITY;
+    for (unsigned int j0 = 0; j0 < npos; j0 += kWave * kBatch) {
+      u32x4 y[kBatch];
 #pragma unroll
       for (int b = 0; b < kBatch; ++b) {
-        const unsigned int jj = j + b * kSlices;
-        y[b] = (jj < nblk) ? A.partials[(int64_t)jj * kRlVals + v] : ident;
+        // Every position below npos holds a workgroup's chunk or the identity (store_block_partials).
+        // A lane past the end loads the last position and discards it: a load behind a condition
+        // would make the compiler wait for each one before issuing the next.
+        const unsigned int pos = j0 + b * kWave + lane;
+        y[b] = src[pos < npos ? pos : npos - 1];
       }
-      // one kind of operation per lane, chosen once per batch rather than per element
-      if (v < kFirstMax) {
+      __builtin_amdgcn_sched_barrier(0);  // every load issued before the first value is touched
 #pragma unroll
-        for (int b = 0; b < kBatch; ++b) x += y[b];
+      for (int b = 0; b < kBatch; ++b)
+        if (j0 + b * kWave + lane >= npos) y[b] = ident;
+      if (chunk < 3) {
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+          a0 += __longlong_as_double((long long)(((unsigned long long)y[b].y << 32) | y[b].x));
+          a1 += __longlong_as_double((long long)(((unsigned long long)y[b].w << 32) | y[b].z));
+        }
+      } else if (chunk == 3) {
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+          a0 += (double)y[b].x;
+          a1 += (double)y[b].y;
+          a2 += (double)y[b].z;
+          a3 += (double)y[b].w;
+        }
       } else {
 #pragma unroll
-        for (int b = 0; b < kBatch; ++b) x = fmax(x, y[b]);
+        for (int b = 0; b < kBatch; ++b) {
+          m0 = fmaxf(m0, __uint_as_float(y[b].x));
+          m1 = fmaxf(m1, __uint_as_float(y[b].y));
+          m2 = fmaxf(m2, __uint_as_float(y[b].z));
+        }
       }
     }
-    lds_t[v * kSlices + j0] = x;  // transposed: the slices of a slot side by side
-  }
-  UNIRL_TRACE_MARK1();
-  __syncthreads();
-  {
-    // thread = (slot, slice) again, now with a slot's slices in one 16-lane row / one wavefront
-    const int v = t / kSlices;
-    double z = lds_t[t];
-    if (kSlices == kRlParts) {
-      z = (v < kFirstMax) ? row_sum_last(z) : row_max_last(z);
-      if (t % kRlParts == kRlParts - 1) lds_tot[v] = z;
+    UNIRL_TRACE_MARK1();
+    if (chunk < 3) {
+      a0 = wave_sum(a0);
+      a1 = wave_sum(a1);
+      if (lane == 0) {
+        lds_tot[2 * chunk] = a0;
+        lds_tot[2 * chunk + 1] = a1;
+      }
+    } else if (chunk == 3) {
+      a0 = wave_sum(a0);
+      a1 = wave_sum(a1);
+      a2 = wave_sum(a2);
+      a3 = wave_sum(a3);
+      if (lane == 0) {
+        lds_tot[kFirstCnt] = a0;
+        lds_tot[kFirstCnt + 1] = a1;
+        lds_tot[kFirstCnt + 2] = a2;
+        lds_tot[kFirstCnt + 3] = a3;
+      }
     } else {
-      z = (v < kFirstMax) ? wave_sum(z) : wave_max(z);
-      if (t % kWave == 0) lds_tot[v] = z;
+      m0 = wave_max(m0);
+      m1 = wave_max(m1);
+      m2 = wave_max(m2);
+      if (lane == 0) {
+        lds_tot[kFirstMax] = (double)m0;
+        lds_tot[kFirstMax + 1] = (double)m1;
+        lds_tot[kFirstMax + 2] = (double)m2;
+        lds_tot[6] = lds_tot[7] = lds_tot[15] = 0.0;
+      }
     }
   }
   __syncthreads();
@@ -891,7 +1041,7 @@ __global__ __launch_bounds__(T) void ratio_loss_finalize_kernel(RatioArgs A, uns
       ((unsigned long long)UNIRL_M_ABSDIFF_MEAN << (4 * P_ABS)) |
       ((unsigned long long)UNIRL_M_NUM_TOKENS << (4 * P_CNT)) | ((unsigned long long)UNIRL_M_CLIPFRAC_HI << (4 * P_CHI)) |
       ((unsigned long long)UNIRL_M_CLIPFRAC_LO << (4 * P_CLO)) |
-      ((unsigned long long)UNIRL_M_CLIP_FRACTION << (4 * P_CANY)) | (13ull << (4 * 10)) | (14ull << (4 * 11)) |
+      ((unsigned long long)UNIRL_M_CLIP_FRACTION << (4 * P_CANY)) | (13ull << (4 * 6)) | (14ull << (4 * 7)) |
       ((unsigned long long)UNIRL_M_RATIO_MIN << (4 * P_NRMIN)) | ((unsigned long long)UNIRL_M_RATIO_MAX << (4 * P_RMAX)) |
       ((unsigned long long)UNIRL_M_ABSDIFF_MAX << (4 * P_AMAX)) | (15ull << (4 * 15));
   A.metrics[(kMetricOf >> (4 * v)) & 15u] = (float)y;
@@ -1004,6 +1154,8 @@ static int fill_consts(const unirl_ratio_loss_params* p, RatioConsts& C) {
   C.drpo_two_eps = (float)(2.0 * p->drpo_epsilon);
   C.inv_two_eps = (float)(1.0 / (double)C.drpo_two_eps);
   C.horizon = (float)p->horizon;
+  C.fast_ok = (p->kind == UNIRL_LOSS_DRPO && p->mu_weighted && C.drpo_eps >= 1.0f) ? 1 : 0;
+  C.fast_hi = 1.0f + C.drpo_eps;  // fp32, as the kernel would form it
   return UNIRL_OK;
 }
 
@@ -1080,7 +1232,7 @@ static int check_common(const float* new_logp, const float* old_logp, const floa
 static int launch_forward(RatioArgs& A, hipStream_t st) {
   RatioShape S;
   plan(A, false, S);
-  if ((int64_t)S.grid.x * S.grid.y * kRlVals > kPartialCapacity) return UNIRL_E_LIMIT;
+  if (((size_t)S.grid.x * S.grid.y + kXcds) * kRlChunks * 16 > kWorkspaceBytes) return UNIRL_E_LIMIT;
   dim3 block(kRlThreads);
   const bool packed = (A.layout == LAYOUT_PACKED);
   const bool grad = (A.grad_new != nullptr);
@@ -1157,10 +1309,7 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
   if (launch_rc != 0 || !A.metrics) return launch_rc;
   const unsigned int nblk = S.grid.x * S.grid.y;
   UNIRL_TRACE_SET(A, "ratio_finalize", 1);
-  if (nblk <= 512)
-    hipLaunchKernelGGL(ratio_loss_finalize_kernel<256>, dim3(1), dim3(256), 0, st, A, nblk);
-  else
-    hipLaunchKernelGGL(ratio_loss_finalize_kernel<1024>, dim3(1), dim3(1024), 0, st, A, nblk);
+  hipLaunchKernelGGL(ratio_loss_finalize_kernel, dim3(1), dim3(kFinThreads), 0, st, A, nblk);
   return (int)hipGetLastError();
 }
 
@@ -1174,10 +1323,11 @@ extern "C" int unirl_ratio_loss_fwd(const float* new_logp, const float* old_logp
   if (rc != 0) return rc;
   if (!metrics) return UNIRL_E_NULL;
   if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
+  if (!aligned_to(workspace, 16)) return UNIRL_E_ALIGN;
   A.mask = loss_mask;
   A.loss_elem = loss_per_elem;
   A.metrics = metrics;
-  A.partials = ws_partials(workspace);
+  A.partials = reinterpret_cast<char*>(workspace);
   return launch_forward(A, (hipStream_t)stream);
 }
 
@@ -1192,9 +1342,10 @@ extern "C" int unirl_ratio_loss_fwd_bwd(const float* new_logp, const float* old_
   if (!metrics || !grad_new) return UNIRL_E_NULL;
   if (!aligned_to(grad_new, 4)) return UNIRL_E_ALIGN;
   if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
+  if (!aligned_to(workspace, 16)) return UNIRL_E_ALIGN;
   A.mask = loss_mask;
   A.metrics = metrics;
-  A.partials = ws_partials(workspace);
+  A.partials = reinterpret_cast<char*>(workspace);
   A.grad_new = grad_new;
   A.loss_scale = loss_scale;
   // the token-mean denominator counts every valid token (masked ones too): all tokens outside

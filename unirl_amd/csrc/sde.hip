@@ -269,6 +269,9 @@ __global__ __launch_bounds__(kSdeThreads) void sde_replay_kernel(SdeStepArgs A, 
 // One wavefront per row: adds the workgroup partials in index order and finishes the log-prob.
 // sigma_mod: rows per sample of a batched replay (sigma is then indexed by the step, row modulo
 // sigma_mod), 0 for the plain step (sigma indexed by the sample through sigma_stride).
+// kBatch: partial loads a lane has in flight, chosen by the host from nblk (1, 2, 4 or 8 cover 64,
+// 128, 256 and more partials per row: surplus loads of a short row cost more than they hide).
+template <int kBatch>
 __global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepArgs A, int64_t B, unsigned int nblk,
                                                                        int sigma_mod) {
   UNIRL_TRACE_T0();
@@ -277,13 +280,22 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepA
   // the partial loads are issued first; the coefficients are worked out while they are in flight
   const int lane = threadIdx.x & (kWave - 1);
   const double* __restrict__ pp = A.partials + b * nblk;
-  double q = (lane < (int)nblk) ? pp[lane] : 0.0;
+  double y[kBatch];  // lane l adds partials l, l + 64, ... in that order
+#pragma unroll
+  for (int k = 0; k < kBatch; ++k) {
+    const unsigned int j = lane + k * kWave;
+    y[k] = pp[j < nblk ? j : nblk - 1];  // past the end: a harmless repeat, discarded below
+  }
   const int64_t sig_idx = sigma_mod ? b % sigma_mod : b * A.sigma_stride;
   const float s = A.sigma[sig_idx];
   const float sn = A.sigma_next[sig_idx];
   const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
+  __builtin_amdgcn_sched_barrier(0);  // all of the above in flight before the first value is used
   const SdeCoef c = sde_coef(A.kind, s, sn, smax, A.sc);
-  for (int64_t j = lane + kWave; j < nblk; j += kWave) q += pp[j];
+  double q = 0.0;
+#pragma unroll
+  for (int k = 0; k < kBatch; ++k) q += (lane + k * kWave < (int)nblk) ? y[k] : 0.0;
+  if (nblk > kBatch * kWave) q += lane_ordered_sum(pp, nblk, kBatch * kWave);
   q = wave_sum(q);
   UNIRL_TRACE_MARK1();
   if (lane != 0) return;
@@ -579,6 +591,21 @@ static int64_t sde_samples_per_launch(int64_t B, int64_t partials_per_sample) {
   if (nb > 32768) nb = 32768;
   if (nb > B) nb = B;
   return nb < 1 ? 1 : nb;
+}
+
+// Finalize launch of a step / replay call: one wavefront per row, the in-flight batch picked from nblk.
+static int launch_step_finalize(const SdeStepArgs& A, int64_t rows, unsigned int nblk, int sigma_mod, hipStream_t st) {
+  const int per_block = kSdeThreads / kWave;
+  const dim3 grid((unsigned int)((rows + per_block - 1) / per_block)), block(kSdeThreads);
+  if (nblk <= kWave)
+    hipLaunchKernelGGL(sde_step_finalize_kernel<1>, grid, block, 0, st, A, rows, nblk, sigma_mod);
+  else if (nblk <= 2 * kWave)
+    hipLaunchKernelGGL(sde_step_finalize_kernel<2>, grid, block, 0, st, A, rows, nblk, sigma_mod);
+  else if (nblk <= 4 * kWave)
+    hipLaunchKernelGGL(sde_step_finalize_kernel<4>, grid, block, 0, st, A, rows, nblk, sigma_mod);
+  else
+    hipLaunchKernelGGL(sde_step_finalize_kernel<8>, grid, block, 0, st, A, rows, nblk, sigma_mod);
+  return (int)hipGetLastError();
 }
 
 template <typename TV, typename TX, bool SAMPLING>
@@ -913,11 +940,8 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
     }
     if (rc != 0) return rc;
     if (want_logp && nblk > 1) {
-      const int per_block = kSdeThreads / kWave;
-      UNIRL_TRACE_SET(A, "sde_finalize", (unsigned int)((nb + per_block - 1) / per_block));
-      hipLaunchKernelGGL(sde_step_finalize_kernel, dim3((unsigned int)((nb + per_block - 1) / per_block)),
-                         dim3(kSdeThreads), 0, st, A, nb, nblk, 0);
-      rc = (int)hipGetLastError();
+      UNIRL_TRACE_SET(A, "sde_finalize", (unsigned int)((nb + kSdeThreads / kWave - 1) / (kSdeThreads / kWave)));
+      rc = launch_step_finalize(A, nb, nblk, 0, st);
       if (rc != 0) return rc;
     }
   }
@@ -985,11 +1009,8 @@ extern "C" int unirl_sde_replay_logp(const unirl_sde_replay_desc* d, void* works
     }
     if (rc != 0) return rc;
     if (want_logp && nblk > 1) {
-      const int per_block = kSdeThreads / kWave;
-      UNIRL_TRACE_SET(A, "sde_finalize", (unsigned int)((nb * S + per_block - 1) / per_block));
-      hipLaunchKernelGGL(sde_step_finalize_kernel, dim3((unsigned int)((nb * S + per_block - 1) / per_block)),
-                         dim3(kSdeThreads), 0, st, A, nb * S, nblk, (int)S);
-      rc = (int)hipGetLastError();
+      UNIRL_TRACE_SET(A, "sde_finalize", (unsigned int)((nb * S + kSdeThreads / kWave - 1) / (kSdeThreads / kWave)));
+      rc = launch_step_finalize(A, nb * S, nblk, (int)S, st);
       if (rc != 0) return rc;
     }
   }
