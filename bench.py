@@ -478,14 +478,13 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
         out[name] = got[0]
         log(f"replay {name}: {got[0]}")
     log(f"replay reference: {ref[0]}")
-    # what the default's transposed copy of the weight costs, once per weight version
+    # what the default's transposed copy of the weight costs, once per replay (inside the times above)
     from unirl_amd.models import ar_logp
 
-    ar_logp._TRANSPOSED.clear()
     torch.cuda.synchronize()
     a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     a.record()
-    ar_logp._transposed_weight(head.weight)
+    ar_logp.transpose_weight(head.weight)
     b.record()
     torch.cuda.synchronize()
     out["weight_transposition_ms"] = round(a.elapsed_time(b), 2)

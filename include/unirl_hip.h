@@ -282,7 +282,9 @@ int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, const float*
  * per-workgroup partials go to a static device array inside the library (256 KiB, held by every
  * GPU the library runs on until the process ends) instead of a caller-owned workspace; its
  * address is looked up once per device, on the first call made with that device current, which
- * is best made outside a graph capture.  Same kernels, same launch shape and bit-identical
+ * is best made outside a graph capture (make one call on each GPU at set-up).  The current
+ * device must be the one that owns `stream`, p and q, as for any launch.  Same kernels, same
+ * launch shape and bit-identical
  * results as unirl_gaussian_kl_mask.  Limit: R <= UNIRL_KL_STATIC_MAX_ROWS (UNIRL_E_LIMIT
  * beyond).  Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU
  * (different streams or threads) race; calls ordered on one stream do not. */

@@ -396,6 +396,21 @@ def test_per_sample_view_never_hands_stride_zero_for_several_samples(monkeypatch
         ops._per_sample_view(one.expand(3, 3, 4), "prev_out", writable=True)
 
 
+def test_replay_velocity_blocks_must_be_disjoint():
+    """The batched replay writes the velocities' gradient in the velocities' own layout: a view whose
+    (sample, step) blocks overlap is copied first (overlapping rows would be written concurrently
+    where autograd expects their sum)."""
+    from unirl_amd.ops import _blocks_disjoint as disjoint
+
+    assert disjoint(12 * 5, 4, 5, 12, 5)        # dense [B=4, S=12, D=5]
+    assert disjoint(5, 4, 20, 12, 5)            # step-major dense [S=12, B=4, D=5]
+    assert disjoint(70, 4, 5, 12, 5)            # padded samples
+    assert not disjoint(1, 4, 5, 12, 5)         # samples one element apart
+    assert not disjoint(60, 4, 4, 12, 5)        # steps closer than a block
+    assert not disjoint(30, 4, 5, 12, 5)        # a sample starts inside the previous sample's steps
+    assert disjoint(1, 1, 5, 12, 5) and disjoint(100, 4, 3, 1, 5)  # an extent of 1 leaves its stride free
+
+
 def test_release_library_reads_no_environment_knobs(built_lib):
     """The launch-shape knobs of the measurement build (UNIRL_* environment variables) must not
     exist in the shipped library: an exported variable must never change a production launch."""

@@ -229,7 +229,14 @@ def f64_denoise(v, x, s, sn, *, eta, prev_sample, sigma_max):
     return prev, lp.mean(dim=tuple(range(1, lp.ndim))), mean
 
 
-def no_worse_than_fp32(got, fp32_ref, f64_ref, what, scale=None, slack=2.0):
+# every comparison of a micro-step test with the fp32 oracle: (what, relative to the value, relative to
+# the magnitude of the summed terms).  The second is bounded by TERMS_RTOL: a mean of n terms of
+# magnitude s, each carrying fp32 rounding, moves by a few ulps of s between two correct evaluations.
+REL_TO_FP32_ORACLE = []
+TERMS_RTOL = 1e-5
+
+
+def no_worse_than_fp32(got, fp32_ref, f64_ref, what, scale=None, slack=2.0, terms_scale=None):
     """`got` (the kernels) must be as close to the float64 value as the reference's own fp32
     evaluation is (within `slack`), or within one fp32 ulp (2^-23) of `scale`, the typical magnitude
     of the terms the value is a mean of (default: the value itself) -- a mean of cancelling terms
@@ -238,6 +245,14 @@ def no_worse_than_fp32(got, fp32_ref, f64_ref, what, scale=None, slack=2.0):
     got, fp32_ref, f64_ref = float(got), float(fp32_ref), float(f64_ref)
     scale = abs(f64_ref) if scale is None else float(scale)
     err, ref_err = abs(got - f64_ref), abs(fp32_ref - f64_ref)
+    # the plain difference to the fp32 oracle, printed (pytest -s / -rP) and bounded: relative to the
+    # value, and relative to the magnitude of the terms the value is a mean of
+    rel_value = abs(got - fp32_ref) / max(abs(fp32_ref), 1e-30)
+    rel_terms = abs(got - fp32_ref) / max(scale if terms_scale is None else float(terms_scale), 1e-30)
+    print(f"[vs fp32 oracle] {what}: kernel {got:.9g}, oracle {fp32_ref:.9g}, float64 {f64_ref:.9g}; "
+          f"|kernel - oracle| = {rel_value:.2e} of the value, {rel_terms:.2e} of the terms' magnitude")
+    REL_TO_FP32_ORACLE.append((what, rel_value, rel_terms))
+    assert rel_terms <= TERMS_RTOL, f"{what}: {rel_terms:.3e} of the terms' magnitude from the fp32 oracle"
     assert err <= slack * ref_err + 2.0 ** -23 * scale + 1e-12, (
         f"{what}: kernel {got!r} is {err:.3e} from the float64 value {f64_ref!r}, "
         f"the fp32 reference {fp32_ref!r} only {ref_err:.3e} (scale {scale:.3e})")
@@ -303,8 +318,13 @@ def test_flowdppo_micro_step(dev):
     # fp32 rounding, so two correct fp32 evaluations differ by more than 1e-5 of it.  The bound is
     # therefore the reference's own distance from the float64 value.
     no_worse_than_fp32(res.loss, ref_loss, loss64, "loss", scale=elem64.abs().mean())
+    # magnitude of the terms behind each metric, for the plain bound against the fp32 oracle: the ratio
+    # statistics are built from ratios of magnitude 1 (their std is a small difference of those), and
+    # approx_kl = mean(ld^2 / 2) moves by ld * ulp(log-prob) when a log-prob moves by an ulp
+    terms = {k: 1.0 for k in ("ratio_mean", "ratio_std", "ratio_min", "ratio_max")}
+    terms["approx_kl"] = float((new.log_probs - anchor.log_probs).abs().mean() * new.log_probs.abs().mean())
     for k, v in ref_m.items():
-        no_worse_than_fp32(res.metrics[k], v, m64[k], k)
+        no_worse_than_fp32(res.metrics[k], v, m64[k], k, terms_scale=terms.get(k))
     assert 0.0 < res.metrics["kl_mask_fraction"] < 1.0
     no_worse_than_fp32(stage.w.grad, cpu.w.grad, f64.w.grad, "d loss / d w through the SDE backward kernel",
                        scale=grad_scale64)

@@ -93,6 +93,33 @@ def test_without_logits_gives_the_same_statistics(dev):
     assert tuple(lp3.shape) == (4, 50) and torch.equal(lp3.reshape(-1), c[0])
 
 
+@pytest.mark.parametrize("rows,V", [(300, 1024), (64, 700)])
+def test_masked_vocabulary_entries_stay_finite(dev, rows, V):
+    """A -inf bias masks vocabulary entries.  The reference's logsumexp and the token kernel give finite
+    log-probs and entropies for the other entries (0 * log 0 = 0); so must the fused head, in whole
+    tiles (V = 1024: every 16-column piece of the first tile is masked before any finite logit is met)
+    and in the ragged last tile."""
+    from unirl_amd import ops
+
+    h, w, _, ids = make(rows, 128, V, 77)
+    b = torch.zeros(V).bfloat16()
+    b[:300] = float("-inf")          # whole 16-column pieces, and more than one 256-column tile's first half
+    b[517::7] = float("-inf")        # scattered single entries
+    ids = torch.where(torch.isinf(b.float()[ids]), torch.full_like(ids, 301), ids)  # targets on live entries
+    lp, ent, lse, logits = ops.lmhead_logp(h.to(dev), w.to(dev), b.to(dev), ids.to(dev), 0.9, want_entropy=True,
+                                           want_lse=True, want_logits=True)
+    got = logits.cpu()
+    assert bool(torch.isinf(got.float()[:, :300]).all())
+    assert bool(torch.isfinite(lp).all()) and bool(torch.isfinite(ent).all()) and bool(torch.isfinite(lse).all())
+    assert_close(lp, otok.token_logp(got, ids, 0.9), 1e-5, 2e-6, "log-prob with masked entries")
+    assert_close(lse, torch.logsumexp(got.float() / 0.9, dim=-1), 1e-5, 2e-6, "logsumexp with masked entries")
+    assert_close(ent, otok.token_entropy(got, 0.9), 1e-5, 1e-6, "entropy with masked entries")
+    # and the two paths chunked_replay_logp may take agree
+    lp2, ent2, _ = ops.token_logp_entropy(logits, ids.to(dev), 0.9, want_logp=True, want_entropy=True)
+    assert_close(lp, lp2.cpu(), 1e-5, 2e-6, "fused head vs token kernel on the same logits")
+    assert_close(ent, ent2.cpu(), 1e-5, 1e-6, "fused head vs token kernel: entropy")
+
+
 def test_out_of_range_id_and_argument_errors(dev):
     from unirl_amd import ops
 

@@ -390,9 +390,11 @@ def test_chunked_replay_keeps_logits_only_within_its_budget(dev, monkeypatch):
 
 
 def test_chunked_replay_transposed_head_gradient(dev):
-    """The hidden states' gradient computed on the cached transposed copy of the weight equals the
-    plain product (another summation order), and the copy follows the weight: after an in-place
-    update (what an optimizer step is) the next replay sees the new values."""
+    """The hidden states' gradient computed on the transposed copy of the weight equals the plain
+    product (another summation order), and the copy can never be stale: it is made inside each
+    replay's backward and dropped with it, so the next replay reads the weight afresh however it was
+    written in between -- in place (an optimizer step, which moves the version counter) or through
+    `.data` (EMA, weight sync, parameter injection: neither the version nor the address changes)."""
     from unirl_amd import models
     from unirl_amd.models import ar_logp
 
@@ -417,19 +419,41 @@ def test_chunked_replay_transposed_head_gradient(dev):
         (ref * up).sum().backward()
         return h.grad
 
-    for _ in range(2):
+    writes = ("in place", ".data", "none")
+    for how in writes:
+        version, address = head.weight._version, head.weight.data_ptr()
         out_t, gh_t, gw_t, gb_t = grads(True)
         out_p, gh_p, gw_p, gb_p = grads(False)
         assert torch.equal(out_t, out_p) and torch.equal(gw_t, gw_p) and torch.equal(gb_t, gb_p)
-        assert_close(gh_t, gh_p, 1e-5, 1e-6 * float(gh_p.abs().max()), "hidden grad, transposed copy vs plain")
+        assert_close(gh_t, gh_p, 1e-5, 1e-6 * float(gh_p.abs().max()), f"hidden grad, transposed copy vs plain ({how})")
         assert_close(gh_t, reference(), 1e-4, 1e-5 * float(gh_p.abs().max()), "hidden grad vs autograd of the chain")
-        cached = ar_logp._TRANSPOSED[id(head.weight)]
-        assert torch.equal(cached[3], head.weight.detach().t())
-        with torch.no_grad():  # an optimizer step: in place, the version moves on
-            head.weight.add_(0.05 * torch.randn(V, H, generator=g).to(dev))
-        assert cached[1] != head.weight._version
-    # by default small replays do not pay for the copy
-    ar_logp._TRANSPOSED.clear()
+        fresh = 0.05 * torch.randn(V, H, generator=g).to(dev)
+        if how == "in place":  # an optimizer step: the version moves on
+            with torch.no_grad():
+                head.weight.add_(fresh)
+            assert head.weight._version != version
+        elif how == ".data":   # invisible to a version / address check
+            head.weight.data.copy_(head.weight.data + 8.0 * fresh)
+            assert head.weight._version == version and head.weight.data_ptr() == address
+    # a retained graph: the second backward meets a weight written in place in between and remakes the copy
     h = hidden.clone().requires_grad_(True)
-    models.chunked_replay_logp(head, h, toks, 0.9, chunk=16).sum().backward()
-    assert id(head.weight) not in ar_logp._TRANSPOSED and B * T_max < ar_logp.TRANSPOSED_HEAD_MIN_ROWS
+    out = models.chunked_replay_logp(head, h, toks, 0.9, chunk=16, transposed_head=True, keep_logits=False)
+    (out * up).sum().backward(retain_graph=True)
+    first = h.grad.clone()
+    h.grad = None
+    (out * up).sum().backward()
+    assert torch.equal(h.grad, first)
+    # nothing is cached between replays, and by default small replays do not use the copy at all
+    assert not hasattr(ar_logp, "_TRANSPOSED")
+    calls = []
+    real = ar_logp.transpose_weight
+    ar_logp.transpose_weight = lambda w: (calls.append(1), real(w))[1]
+    try:
+        h = hidden.clone().requires_grad_(True)
+        models.chunked_replay_logp(head, h, toks, 0.9, chunk=16).sum().backward()
+        assert not calls and B * T_max < ar_logp.TRANSPOSED_HEAD_MIN_ROWS
+        h = hidden.clone().requires_grad_(True)
+        models.chunked_replay_logp(head, h, toks, 0.9, chunk=16, transposed_head=True).sum().backward()
+        assert len(calls) == 1, "one transposition per replay, shared by its chunks"
+    finally:
+        ar_logp.transpose_weight = real

@@ -184,6 +184,37 @@ def test_drpo_backward_closed_form_clamp_and_gradcheck():
     )
 
 
+def test_drpo_stationary_point_is_the_trust_region_boundary():
+    """What the mathematics fixes about the penalty's scale, with no formula retyped: for A > 0 the
+    per-token loss -A r + |A| mu (r-1)^2 / (2 eps) is stationary in r exactly at r* = 1 + eps/mu, the
+    boundary `clipfrac_upper` counts against (for A < 0 at 1 - eps/mu, the one `clipfrac_lower`
+    uses).  A penalty of |A| mu (r-1)^2 / eps -- the 2 dropped -- would be stationary at
+    1 + eps/(2 mu) and fail here; so would a penalty without mu, or with the wrong sign."""
+    for eps, mu, sign in ((0.4, 0.5, 1.0), (12.5, 0.9, 1.0), (5.0, 0.75, 1.0), (0.3, 0.6, -1.0), (0.05, 0.25, -1.0)):
+        r_star = 1.0 + sign * eps / mu
+        assert r_star > 0.0
+        old = torch.tensor([mu], dtype=torch.float64).log()
+        adv = torch.tensor([sign * 1.7], dtype=torch.float64)
+
+        def grad_at(r):
+            new = (old + torch.tensor([r], dtype=torch.float64).log()).requires_grad_(True)
+            loss, m = olos.drpo_loss(new, old, adv, eps, True)
+            loss.sum().backward()
+            return float(new.grad), m
+
+        g0, _ = grad_at(r_star)
+        assert abs(g0) < 1e-12 * abs(float(adv)) * r_star, (eps, mu, sign, g0)
+        g_in, m_in = grad_at(1.0 + sign * (eps / mu) * (1 - 1e-3))    # inside the trust region: still descending
+        g_out, m_out = grad_at(1.0 + sign * (eps / mu) * (1 + 1e-3))  # outside: the penalty has taken over
+        # d loss / d new_logp = r * d loss / d r; moving r away from 1 lowers the loss inside, raises it outside
+        assert sign * g_in < 0.0 < sign * g_out
+        key = "clipfrac_upper" if sign > 0 else "clipfrac_lower"
+        assert float(m_in[key]) == 0.0 and float(m_out[key]) == 1.0
+        # the wrong scale's stationary point is not one
+        g_half, _ = grad_at(1.0 + sign * eps / (2 * mu))
+        assert abs(g_half) > 0.1 * abs(float(adv))
+
+
 # ---------------------------------------------------------------- expansion / aggregation
 def test_expand_and_aggregate():
     adv = torch.tensor([1.0, -2.0, 3.0, 0.5])

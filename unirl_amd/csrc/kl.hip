@@ -481,6 +481,9 @@ extern "C" int unirl_gaussian_kl_mask(const void* p, const void* q, int dtype, c
 // at its own address, looked up once per device; host code only ever uses that address, never
 // the array's name.  The kernels overwrite every partial they read back, so nothing needs
 // clearing between calls; calls that overlap on one GPU share the array and race.
+// The address used is the CURRENT device's (hipGetDevice): as for every launch, the current device
+// must be the one that owns `stream` and the pointers -- a stream of another GPU is refused by the
+// launch itself (invalid resource handle), so a foreign array address is never dereferenced.
 // ---------------------------------------------------------------------------
 static __device__ __align__(256) double scratch[kKlStaticRows];
 
@@ -512,7 +515,7 @@ extern "C" int unirl_gaussian_kl_mask_static(const void* p, const void* q, int d
                                              uint8_t* mask_out, void* stream) {
   if (!dtype_ok(dtype)) return UNIRL_E_DTYPE;
   if (R < 0 || D <= 0 || n_sigma <= 0) return UNIRL_E_SHAPE;
-  if (R > kKlStaticRows) return UNIRL_E_LIMIT;  // one launch pair, partials within the static array
+  if (R > kKlStaticRows) return UNIRL_E_LIMIT;  // the partials of every launch of the call fit the static array
   if (R == 0) return UNIRL_OK;
   if (!p || !q || !sigma || !kl_out) return UNIRL_E_NULL;
   double* partials = nullptr;

@@ -419,15 +419,17 @@ __global__ __launch_bounds__(kHdThreads, (BM * BN > 128 * 128) ? 1 : 2) void lmh
         if (ENT) tsum[r] = had ? f * fmaf(-d, sum[r], tsum[r]) : 0.0f;
         sum[r] = had ? f * sum[r] : 0.0f;
         m[r] = mn;
-        if (!FULL && mn == -INFINITY) continue;  // nothing but columns outside the vocabulary so far
+        // nothing but -inf so far (columns outside the vocabulary, or masked entries: a -inf bias)
+        if (mn == -INFINITY) continue;
         const float mc = -mn * c;
 #pragma unroll
         for (int j = 0; j < PIECE; ++j) {
-          // a = (x - m) * c <= 0; a column outside the vocabulary is -inf: e = 0 and e * a must be 0, not NaN
+          // a = (x - m) * c <= 0.  A -inf logit (outside the vocabulary, or masked) has e = 0 and must
+          // add 0 to the entropy sum, not 0 * -inf: the product is taken with a held at a large finite value
           const float a = fmaf(x[r][j], c, mc);
           const float e = __builtin_amdgcn_exp2f(a);
           sum[r] += e;
-          if (ENT) tsum[r] = (FULL || x[r][j] != -INFINITY) ? fmaf(e, a, tsum[r]) : tsum[r];
+          if (ENT) tsum[r] = fmaf(e, fmaxf(a, -65536.0f), tsum[r]);
         }
       }
     }

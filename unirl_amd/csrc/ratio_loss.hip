@@ -624,6 +624,11 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_fwd_kernel(RatioArgs A)
     const int64_t nvec_full = row_end / VEC;       // vectors that can be loaded whole
     const int64_t nload = nvec < nvec_full ? nvec : nvec_full;
 
+    // INVARIANT: finish_token_count() holds the only workgroup barriers before store_block_partials,
+    // and every wavefront takes it exactly once -- inside this loop (its first pass) or after the row
+    // loop.  The wavefronts therefore reach those barriers at different program points, which pairs up
+    // only because s_barrier counts arrivals and this loop's bounds are wave-uniform.  No other barrier
+    // may be placed inside the row loop, and no loop bound here may become lane-dependent.
     for (int64_t w0 = wave_first; w0 < nload; w0 += stride * ITEMS) {
       float nw[ITEMS][VEC], od[ITEMS][VEC], ad[ITEMS][VEC], mk[ITEMS][VEC];
       // Every item loads: past the end the index falls back to the row's last loadable vector

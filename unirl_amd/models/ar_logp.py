@@ -18,7 +18,6 @@ in the logits' dtype, so the chunk needs no activation checkpoint of an fp32 cop
 
 from __future__ import annotations
 
-import weakref
 from typing import Callable, Dict, List, Optional, Tuple
 
 import torch
@@ -126,30 +125,42 @@ class _RecomputedChunkFn(torch.autograd.Function):
 
 _KERNEL_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
 
-# id(weight) -> (weak reference, version, data pointer, transposed copy)
-_TRANSPOSED: Dict[int, Tuple["weakref.ref", int, int, torch.Tensor]] = {}
+def transpose_weight(weight: torch.Tensor) -> torch.Tensor:
+    """A contiguous ``[K, V]`` copy of a head's ``[V, K]`` weight (``unirl_transpose_2d``: 0.3 ms for
+    the Qwen3-4B head where torch's strided copy takes 6 ms)."""
+    if weight.dim() == 2 and weight.is_cuda and weight.element_size() in (2, 4) and weight.stride(1) == 1:
+        return ops.transpose_2d(weight)
+    return weight.detach().t().contiguous()
 
 
-def _transposed_weight(weight: torch.Tensor) -> torch.Tensor:
-    """A contiguous ``[K, V]`` copy of the head's ``[V, K]`` weight, remade when the weight has been
-    written since (an optimizer step bumps its version) and dropped with the weight.
+class _TransposedOnce:
+    """The ``[K, V]`` copy of the head's weight for ONE replay.
 
     The gradient of the hidden states is ``dL [rows, V] @ W [V, K]``, a product with both operands
     read across their rows; the GEMM library runs it at 0.65 - 0.75 of the speed it reaches on
     ``dL @ Wt.T`` with ``Wt`` stored ``[K, V]`` (measured on the MI355X, Qwen3-4B head: 7.3 against
-    4.8 ms at 8192 rows, 1.84 against 1.51 ms at 2048).  One transposition per weight version (0.8 GB
-    moved) buys that for every chunk of every replay until the next optimizer step."""
-    key = id(weight)
-    hit = _TRANSPOSED.get(key)
-    if hit is not None and hit[0]() is weight and hit[1] == weight._version and hit[2] == weight.data_ptr():
-        return hit[3]
-    if weight.dim() == 2 and weight.is_cuda and weight.element_size() in (2, 4) and weight.stride(1) == 1:
-        wt = ops.transpose_2d(weight)  # 0.5 ms for the Qwen3-4B head where torch's strided copy takes 6 ms
-    else:
-        wt = weight.detach().t().contiguous()
-    _TRANSPOSED[key] = (weakref.ref(weight, lambda _r, key=key: _TRANSPOSED.pop(key, None)), weight._version,
-                        weight.data_ptr(), wt)
-    return wt
+    4.8 ms at 8192 rows, 1.84 against 1.51 ms at 2048).  The copy is made in the backward, by the
+    first chunk that needs it, from the weight's values at that moment, shared by the replay's
+    other chunks and dropped with the replay's graph.  Nothing outlives the replay, so no write
+    to the weight can leave a stale copy behind -- in particular not one made through ``.data``
+    (``p.data.copy_(...)``: EMA, weight sync and parameter injection all write that way), which
+    changes neither the tensor's version counter nor its address and therefore cannot be seen by
+    a cache that is keyed on them.  The price is one transposition per replay (0.3 ms against a
+    backward of 11 ms at 8192 rows) instead of one per optimizer step.  A second backward through
+    a retained graph remakes the copy if the version counter has moved in between."""
+
+    __slots__ = ("weight", "version", "copy")
+
+    def __init__(self, weight: torch.Tensor) -> None:
+        self.weight, self.version, self.copy = weight, None, None
+
+    def get(self) -> torch.Tensor:
+        if self.copy is None or self.version != self.weight._version:
+            self.copy, self.version = transpose_weight(self.weight), self.weight._version
+        return self.copy
+
+    def release(self) -> None:
+        self.copy = None
 
 
 class _LinearHeadChunkFn(torch.autograd.Function):
@@ -159,7 +170,8 @@ class _LinearHeadChunkFn(torch.autograd.Function):
     the two gradient GEMMs are issued in the operand layouts the GEMM library is fastest on."""
 
     @staticmethod
-    def forward(ctx, hidden, tokens, weight, bias, temperature: float, keep: bool, fused_head: bool, transposed: bool):
+    def forward(ctx, hidden, tokens, weight, bias, temperature: float, keep: bool, fused_head: bool, transposed):
+        # transposed: None, or the replay's _TransposedOnce plus whether this chunk runs last in the backward
         logits = None
         with torch.no_grad():
             if fused_head:
@@ -191,7 +203,13 @@ class _LinearHeadChunkFn(torch.autograd.Function):
         d2 = d_logits.reshape(-1, d_logits.shape[-1])
         g_hidden = g_weight = g_bias = None
         if ctx.needs_input_grad[0]:
-            g_hidden = torch.mm(d2, _transposed_weight(weight).t() if ctx.transposed else weight).view(hidden.shape)
+            if ctx.transposed is not None:
+                once, last = ctx.transposed
+                g_hidden = torch.mm(d2, once.get().t()).view(hidden.shape)
+                if last:
+                    once.release()  # the replay's backward is complete: the copy's memory goes back now
+            else:
+                g_hidden = torch.mm(d2, weight).view(hidden.shape)
         if ctx.needs_input_grad[2]:
             g_weight = torch.mm(d2.t(), hidden.reshape(-1, hidden.shape[-1]))
         if bias is not None and ctx.needs_input_grad[3]:
@@ -282,10 +300,13 @@ def chunked_replay_logp(
 
     For a plain ``nn.Linear`` head on hidden states of its own dtype (no autocast) the head and
     its backward run inside one autograd node, which issues the gradient GEMMs itself.
-    ``transposed_head`` lets it compute the hidden states' gradient on a cached ``[K, V]`` copy of
-    the weight (one transposition per weight version, ``V * K`` elements of memory): the GEMM
-    library is 1.2 - 1.5 times faster on that layout.  Left at ``None`` it is used for replays of
-    at least ``TRANSPOSED_HEAD_MIN_ROWS`` rows.
+    ``transposed_head`` lets it compute the hidden states' gradient on a ``[K, V]`` copy of the
+    weight: the GEMM library is 1.2 - 1.5 times faster on that layout.  The copy is made once per
+    replay, in its backward, from the weight's values at that moment (``V * K`` elements held while
+    the backward runs), and dropped with it: no copy survives a replay, so a weight written between
+    replays in any way -- an optimizer step, or a write through ``.data`` that no version counter
+    records -- is always read afresh.  Left at ``None`` it is used for replays of at least
+    ``TRANSPOSED_HEAD_MIN_ROWS`` rows.
     """
     bsz, t_max = int(resp_hidden.size(0)), int(response_tokens.size(1))
     if t_max == 0:
@@ -326,12 +347,14 @@ def chunked_replay_logp(
     if transposed_head is None:
         transposed_head = bsz * t_max >= TRANSPOSED_HEAD_MIN_ROWS
     recompute = not keep_logits and wants_grad
+    once = _TransposedOnce(lm_head.weight) if (own_linear and transposed_head and resp_hidden.requires_grad) else None
     parts: List[torch.Tensor] = []
     for s in range(0, t_max, step):
         h, tok = resp_hidden[:, s : s + step, :], response_tokens[:, s : s + step]
         if own_linear:
+            # autograd runs the chunks' backwards in reverse order of creation: the first chunk is the last
             parts.append(_LinearHeadChunkFn.apply(h, tok, lm_head.weight, lm_head.bias, T, bool(keep_logits), fused_head,
-                                                  bool(transposed_head and resp_hidden.requires_grad)))
+                                                  None if once is None else (once, s == 0)))
         elif recompute:
             parts.append(_RecomputedChunkFn.apply(h, tok, lm_head, T, fused_head, *params))
         elif fused_head:

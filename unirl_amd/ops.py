@@ -282,6 +282,19 @@ def _replay_slot_arrays(slots_x: tuple, slots_p: tuple, K: int):
     return (ctypes.c_int64 * S)(*slots_x), (ctypes.c_int64 * S)(*slots_p), S
 
 
+def _blocks_disjoint(stride_a: int, n_a: int, stride_b: int, n_b: int, block: int) -> bool:
+    """Whether the ``n_a x n_b`` blocks of ``block`` contiguous elements at offsets
+    ``i * stride_a + j * stride_b`` are pairwise disjoint (positive strides; an extent of 1 leaves
+    its stride free)."""
+    dims = sorted((s, n) for s, n in ((stride_a, n_a), (stride_b, n_b)) if n > 1)
+    span = block
+    for stride, n in dims:  # inner dimension first: each must step past everything nested inside it
+        if stride < span:
+            return False
+        span = (n - 1) * stride + span
+    return True
+
+
 def _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next, kind, eta, sigma_max, step_major):
     """Checked operands and the filled ``unirl_sde_replay_desc`` of a batched replay; returns
     ``(desc, keepalive, B, S, D, shape_tail)``."""
@@ -307,7 +320,10 @@ def _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next,
     # are free, except that 0 means "dense" in the C ABI: a tensor broadcast over the samples or the
     # steps is copied, as is a stack whose slots overlap
     b_dim, s_dim = (1, 0) if step_major else (0, 1)
-    if B and not (_dense_from(v, 2) and (B == 1 or v.stride(b_dim) >= 1) and (S == 1 or v.stride(s_dim) >= D)):
+    # The velocities' gradient is written in the velocities' own layout, so their (sample, step)
+    # blocks must also be pairwise disjoint: a view whose samples (or steps) overlap would have its
+    # overlapping gradient rows written concurrently, where autograd expects their sum.
+    if B and not (_dense_from(v, 2) and _blocks_disjoint(v.stride(b_dim), B, v.stride(s_dim), S, D)):
         v = v.contiguous()
     if B and not (_dense_from(x, 2) and (B == 1 or x.stride(0) >= 1) and (K == 1 or x.stride(1) >= D)):
         x = x.contiguous()
