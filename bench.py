@@ -238,6 +238,26 @@ def make_shapes(torch, dev):
                 strat.denoise_into(v_[:, j], st_[:, slot_x[j]], sg_d[k], sg_d[k + 1], eta=0.7, prev_sample=st_[:, slot_p[j]],
                                    sigma_max=smax_r, mean_out=out_mean[:, j], logp_out=out_lp[:, j])
 
+        # the Flow-DPPO micro-step's forward on the same transitions: replay log-probs + KL against the frozen
+        # means + masks, loss, metrics, gradient -- fused (one streaming pass over 4 reads + one finishing
+        # workgroup) against the pair it replaces (batched replay writing the means, then the KL / loss step)
+        old_means = [torch.randn((B, S) + tail, generator=g).to(tdt).to(dev) for _ in range(nsr)]
+        old_lp = torch.randn(B, S, generator=g).to(dev)
+        adv_bs = torch.randn(B, 1, generator=g).expand(B, S).contiguous().to(dev)
+        sig_t = torch.full((S,), 0.1, device=dev)
+
+        def run_dppo_fused(i, stacks=stacks, vels=vels, nsr=nsr, slot_x=slot_x, slot_p=slot_p, sg_a=sg_a, sg_b=sg_b,
+                           smax_r=smax_r, old_means=old_means, old_lp=old_lp, adv_bs=adv_bs, sig_t=sig_t):
+            return ops.flowdppo_replay_step(vels[i % nsr], stacks[i % nsr], slot_x, slot_p, sg_a, sg_b, old_lp,
+                                            old_means[i % nsr], adv_bs, sig_t, 1.0, kind="flow", eta=0.7,
+                                            sigma_max=smax_r, loss_scale=1.0)
+
+        def run_dppo_pair(i, stacks=stacks, vels=vels, nsr=nsr, slot_x=slot_x, slot_p=slot_p, sg_a=sg_a, sg_b=sg_b,
+                          smax_r=smax_r, old_means=old_means, old_lp=old_lp, adv_bs=adv_bs, sig_t=sig_t):
+            lp, means = ops.sde_replay_logp(vels[i % nsr], stacks[i % nsr], slot_x, slot_p, sg_a, sg_b, kind="flow",
+                                            eta=0.7, sigma_max=smax_r)
+            return ops.flowdppo_step(lp, old_lp, means, old_means[i % nsr], adv_bs, sig_t, 1.0, loss_scale=1.0)
+
         shape_txt = f"{str(tdt).split('.')[-1]} stack [{B},{K},{','.join(map(str, tail))}], bf16 velocities, S'={S} steps"
         shapes.append(dict(
             name=f"sde_replay_BxS_{tag}", config=1, shape=shape_txt + ": one launch over the B*S' transitions",
@@ -247,6 +267,18 @@ def make_shapes(torch, dev):
         shapes.append(dict(
             name=f"sde_replay_per_step_{tag}", config=1, shape=shape_txt + ": one call per step (S' launch pairs)",
             bytes=bytes_r, read_bytes=bytes_r * 3 // 4, write_bytes=bytes_r // 4, elements=B * S * D, run=run_loop,
+            sets=nsr,
+        ))
+        shapes.append(dict(
+            name=f"flowdppo_replay_step_{tag}", config=4,
+            shape=shape_txt + " + frozen means [B,S',...]: replay log-prob + KL + loss + metrics + grad, 4 reads, 2 launches",
+            bytes=bytes_r, read_bytes=bytes_r, write_bytes=0, elements=B * S * D, run=run_dppo_fused, sets=nsr,
+        ))
+        shapes.append(dict(
+            name=f"flowdppo_replay_pair_{tag}", config=4,
+            shape=shape_txt + " + frozen means: the same job as sde_replay_logp (means written) then flowdppo_step "
+                              "(means re-read): 5 reads + 1 write, 4 launches; GB/s on the fused job's 4 reads",
+            bytes=bytes_r, read_bytes=bytes_r * 5 // 4, write_bytes=bytes_r // 4, elements=B * S * D, run=run_dppo_pair,
             sets=nsr,
         ))
 

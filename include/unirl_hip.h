@@ -38,7 +38,8 @@ extern "C" {
 /* 2: typed gradient outputs in unirl_sde_step_logp_bwd; unirl_ratio_loss_fwd_bwd and
  * unirl_flowdppo_step added.  3: unirl_dpm2_step added.  4: unirl_gaussian_kl_mask_static
  * added.  5: unirl_sde_replay_logp, unirl_sde_replay_logp_bwd, unirl_lmhead_logp added.
- * 6: the unirl_calib_* measurement aids left the library (they live in the measurement build). */
+ * 6: the unirl_calib_* measurement aids left the library (they live in the measurement build);
+ * unirl_flowdppo_replay_step added. */
 #define UNIRL_ABI_VERSION 6
 
 enum unirl_dtype { UNIRL_F32 = 0, UNIRL_BF16 = 1, UNIRL_F16 = 2 };
@@ -320,6 +321,42 @@ int unirl_flowdppo_step(const void* p, const void* q, int dtype, const float* si
                         float loss_scale, float* kl_out, float* loss_elem, float* grad_new,
                         float* metrics /* [16] f32, as unirl_flowdppo_loss */, void* workspace,
                         size_t workspace_bytes, void* stream);
+
+/* ------------------------------------------------------------------------
+ * The forward of a Flow-DPPO micro-step straight from the model's velocities:
+ * unirl_sde_replay_logp and unirl_flowdppo_step as ONE streaming pass plus one
+ * finishing workgroup.  Replaces the replay loop of
+ * unirl/models/sd3/diffusion.py:467-497 (per step: denoise with the stored
+ * next latent -> log-prob and mean, stacked to [B,S'] / [B,S',...]) followed
+ * by FlowDPPO.compute_loss_and_backward's loss (unirl/algorithms/flowdppo.py:
+ * 286-320: gather the frozen old log-probs and means, _flowdppo_kl_adv_loss).
+ * The new mean of every element is in registers while the log-prob residual is
+ * summed; it is rounded to the trajectory dtype as the reference stores it
+ * (`.to(trajectory_dtype)`) and the Gaussian-KL numerator against the old mean
+ * is summed beside it with torch's type promotion (flowdppo.py:51), so the new
+ * means are never written and never re-read: 4 reads per element and 2 launches,
+ * where replay + KL take 5 reads, 1 write and 4 launches.
+ *   desc        as unirl_sde_replay_logp; desc->logp_out (required) receives the
+ *               new log-probs [B,S]; desc->mean_out only if the caller wants the
+ *               means as well (NULL otherwise)
+ *   old_means   [B,S,D] dense, in the dtype of desc->latents (the trajectory dtype)
+ *   sigma_t     f32 [n_sigma_t], row r = b*S + j uses sigma_t[r % n_sigma_t]
+ *               (FlowDPPO._compute_sigma_t, flowdppo.py:342-368)
+ *   old_logp, advantages, kl_out, loss_elem   f32 [B*S]
+ *   mask_out    NULL or u8 [B*S]: kl < threshold
+ *   grad_logp   NULL or f32 [B*S]: loss_scale * loss_elem / (B*S), what
+ *               `(loss_elem.mean() * loss_scale).backward()` leaves in the new
+ *               log-probs; hand it to unirl_sde_replay_logp_bwd as g_logp
+ *   metrics     f32 [16] as unirl_flowdppo_loss
+ * Limits: B*S <= 2048 rows (UNIRL_E_LIMIT); eta >= 1e-7 (UNIRL_E_SHAPE: a
+ * deterministic step has no log-prob).
+ * ---------------------------------------------------------------------- */
+int unirl_flowdppo_replay_step(const struct unirl_sde_replay_desc* desc /* host */,
+                               const void* old_means, const float* sigma_t, int64_t n_sigma_t,
+                               const float* old_logp, const float* advantages, float threshold,
+                               float loss_scale, float* kl_out, uint8_t* mask_out,
+                               float* loss_elem, float* grad_logp, float* metrics,
+                               void* workspace, size_t workspace_bytes, void* stream);
 
 /* Element-wise form of the same quantity (unirl/algorithms/flowdppo.py:51), f32 output [R,D]. */
 int unirl_gaussian_kl_elem(const void* p, const void* q, int dtype, const float* sigma,

@@ -1,0 +1,234 @@
+"""The fused Flow-DPPO forward (`unirl_flowdppo_replay_step`: replay log-probs and the KL against the
+frozen means in one streaming pass, then masks, loss, the twelve metrics and the gradient in one
+finishing workgroup) against the oracle's per-step replay loop followed by its KL-ADV loss -- the
+loop of unirl/models/sd3/diffusion.py:467-497 and unirl/algorithms/flowdppo.py:286-320."""
+
+import types
+
+import pytest
+import torch
+
+from oracle import flowdppo as ofd
+from oracle import schedule as osch
+from oracle import sde as osde
+from tests._util import BF16_RTOL, FP32_RTOL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+KEYS = ("ratio_mean", "ratio_std", "ratio_min", "ratio_max", "approx_kl", "kl_new_old_mean", "kl_new_old_max",
+        "kl_mask_fraction", "pos_rm_fraction", "neg_rm_fraction", "masked_fraction", "unmasked_fraction")
+
+
+def oracle_step(kind, sig, stack, v_new, v_old, steps, stored, traj_dtype, adv, eta, thr_pick):
+    """Old policy (v_old) frozen per step, then the new policy's replay and the KL-ADV loss, on the CPU."""
+    def replay(v):
+        lps, means = [], []
+        for j, i in enumerate(steps):
+            _, lp, mean = osde.sde_denoise(kind, v[:, j], stack[:, stored.index(i)], sig[i], sig[i + 1], eta=eta,
+                                           prev_sample=stack[:, stored.index(i + 1)], sigma_max=sig[1], ieee_sqrt=True)
+            lps.append(lp)
+            means.append(mean)
+        return torch.stack(lps, 1), torch.stack(means, 1).to(traj_dtype)
+
+    old_lp, old_means = replay(v_old)
+    new_lp, new_means = replay(v_new)
+    sigma_t = ofd.sigma_t(sig, steps, eta).reshape((1, -1) + (1,) * (new_means.dim() - 2))  # video latents have one more axis
+    kl = ofd.kl_per_sample(new_means, old_means, sigma_t)
+    thr = thr_pick(kl)
+    adv_b = adv.reshape(-1, 1).expand_as(new_lp)
+    leaf = new_lp.clone().requires_grad_(True)
+    elem, m = ofd.flowdppo_loss(leaf, old_lp, new_means, old_means, adv_b, sigma_t, thr)
+    (elem.mean() * 0.5).backward()
+    return dict(old_lp=old_lp, old_means=old_means, new_lp=new_lp, new_means=new_means, sigma_t=sigma_t, kl=kl, thr=thr,
+                elem=elem.detach(), metrics=m, grad_lp=leaf.grad, adv_b=adv_b)
+
+
+def run_case(dev, kind, n_sched, shift, B, tail, stored, steps, traj_dtype, v_dtype, seed, step_major=False,
+             thr_pick=lambda kl: float(kl.flatten().sort().values[kl.numel() // 2])):
+    from unirl_amd import ops, sde
+
+    sig = osch.sigma_schedule(n_sched, shift)
+    g = torch.Generator().manual_seed(seed)
+    stack = torch.randn((B, len(stored)) + tail, generator=g).to(traj_dtype)
+    v_old = torch.randn((B, len(steps)) + tail, generator=g).to(v_dtype)
+    # the policy has moved a little, by a different amount per (sample, step): KLs on both sides of the threshold
+    bump = 0.02 * torch.rand(B, len(steps), generator=g).reshape((B, len(steps)) + (1,) * len(tail))
+    v_new = (v_old.float() + bump * torch.randn(v_old.shape, generator=g)).to(v_dtype)
+    adv = torch.randn(B, generator=g)
+    ref = oracle_step(kind, sig, stack, v_new, v_old, steps, stored, traj_dtype, adv, 0.7, thr_pick)
+    slot_x, slot_p = sde.replay_slots(stored, steps)
+    sa = torch.stack([sig[i] for i in steps]).to(dev)
+    sb = torch.stack([sig[i + 1] for i in steps]).to(dev)
+    v_dev = v_new.to(dev)
+    if step_major:
+        v_dev = v_dev.transpose(0, 1).contiguous()
+    out = ops.flowdppo_replay_step(
+        v_dev, stack.to(dev), slot_x, slot_p, sa, sb, ref["old_lp"].to(dev), ref["old_means"].to(dev),
+        ref["adv_b"].to(dev), ref["sigma_t"].reshape(-1).to(dev), ref["thr"], kind=kind, eta=0.7, sigma_max=sig[1].to(dev),
+        step_major=step_major, loss_scale=0.5, want_means=True, want_mask=True)
+    rtol = FP32_RTOL if traj_dtype == torch.float32 and v_dtype == torch.float32 else BF16_RTOL
+    assert torch.equal(out["means"].cpu(), ref["new_means"]), "means written on request differ from the oracle's"
+    assert_close(out["logp"], ref["new_lp"], rtol, 2e-6, "new log-probs")
+    assert_close(out["kl"], ref["kl"], 1e-5, 1e-12, "row KL")
+    # masks bit-exact, except rows whose KL lies within an ulp or two of the threshold (counted)
+    kl64 = ref["kl"].double()
+    near = (kl64 - ref["thr"]).abs() <= 4e-7 * abs(ref["thr"])
+    want_mask = ref["kl"] < ref["thr"]
+    got_mask = out["mask"].cpu()
+    assert torch.equal(got_mask[~near], want_mask[~near]), "KL mask differs away from the threshold"
+    print(f"rows within 4e-7 of the threshold (either side allowed): {int(near.sum())} of {near.numel()}")
+    keep = ~near
+    # the loss is -A exp(new - old): a log-prob that moves by d moves it by d relative, and two fp32
+    # evaluations of a log-prob may differ by 1e-5 of its size (DanceGRPO's log-probs are large)
+    lp_tol = 1e-5 * max(1.0, float(ref["new_lp"].abs().max()))
+    assert_close(out["loss_elem"].cpu()[keep], ref["elem"][keep], max(rtol, lp_tol), 1e-7, "loss elements")
+    assert_close(out["grad_logp"].cpu()[keep], ref["grad_lp"][keep], max(rtol, lp_tol), 1e-9, "gradient w.r.t. the new log-probs")
+    vals = out["metrics"].tolist()
+    slack = float(near.sum()) / near.numel()
+    for k in KEYS:
+        got, want = vals[ops.FLOWDPPO_METRIC_SLOTS[k]], float(ref["metrics"][k])
+        if k.endswith("fraction"):
+            assert abs(got - want) <= slack + 1e-7, (k, got, want)
+        elif k.startswith("ratio_"):
+            # statistics of ratios of magnitude 1: a log-prob that moves by d moves its ratio by d, and the
+            # std -- a small difference of those -- by as much in absolute terms; d is 1e-5 of a log-prob
+            assert abs(got - want) <= lp_tol, (k, got, want)
+        elif k == "approx_kl":
+            # mean(ld^2 / 2) moves by |ld| * d when a log-prob moves by d
+            assert abs(got - want) <= lp_tol * (2.0 * want) ** 0.5 + 1e-5 * want + 1e-9, (k, got, want)
+        else:
+            assert abs(got - want) <= 1e-5 * abs(want) + 1e-9, (k, got, want)
+    assert 0.0 < float(want_mask.float().mean()) < 1.0, "the case must exercise both mask values"
+    # the unfused call gives the same means bit for bit (same per-element arithmetic) and the same log-probs up
+    # to the order in which the workgroups' partial sums are added (the two launches split a row differently)
+    lp2, means2 = ops.sde_replay_logp(v_dev, stack.to(dev), slot_x, slot_p, sa, sb, kind=kind, eta=0.7,
+                                      sigma_max=sig[1].to(dev), step_major=step_major)
+    assert torch.equal(means2, out["means"])
+    assert_close(lp2, out["logp"], 1e-6, 1e-7, "fused vs unfused log-probs")
+    return out, ref
+
+
+@pytest.mark.parametrize("kind", ["flow", "dance", "cps"])
+@pytest.mark.parametrize("traj_dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_small_shapes_match_the_oracle(dev, kind, traj_dtype):
+    run_case(dev, kind, 28, 3.0, 3, (4, 12, 10), [0, 1, 2, 3, 5, 6, 9, 10], [2, 0, 5, 9], traj_dtype, traj_dtype, 41)
+
+
+def test_step_major_velocities_and_odd_extent(dev):
+    run_case(dev, "flow", 28, 3.0, 4, (3, 7, 5), list(range(8)), [1, 3, 4], torch.bfloat16, torch.bfloat16, 42,
+             step_major=True)
+    run_case(dev, "flow", 28, 3.0, 2, (5, 9, 3), list(range(6)), [4, 0], torch.float32, torch.bfloat16, 43)
+
+
+def test_sd3_recipe_shape(dev):
+    """SD3: bf16 trajectory of 10 steps, 3 trained steps, micro-batch 8, latents [16,128,128]."""
+    run_case(dev, "flow", 10, 3.0, 8, (16, 128, 128), list(range(11)), [0, 2, 4], torch.bfloat16, torch.bfloat16, 44)
+
+
+def test_wan_recipe_shape(dev):
+    """WAN 2.1: fp16 trajectory of 14 steps, the 7 first-half steps trained, micro-batch 2, latents [16,21,60,104]."""
+    run_case(dev, "flow", 14, 5.0, 2, (16, 21, 60, 104), list(range(15)), list(range(7)), torch.float16, torch.bfloat16, 45)
+
+
+def test_all_masked_and_none_masked(dev):
+    for pick in (lambda kl: float(kl.min()) * 0.5, lambda kl: float(kl.max()) * 2.0):
+        try:
+            run_case(dev, "flow", 28, 3.0, 3, (4, 8, 8), list(range(6)), [0, 2, 3], torch.bfloat16, torch.bfloat16, 46,
+                     thr_pick=pick)
+        except AssertionError as e:
+            assert "both mask values" in str(e)
+
+
+def test_argument_errors(dev):
+    from unirl_amd import ops
+
+    stack = torch.randn(2, 4, 8, device=dev)
+    v = torch.randn(2, 2, 8, device=dev)
+    z = torch.zeros(2, 2, device=dev)
+    om = torch.zeros(2, 2, 8, device=dev)
+    st = torch.ones(2, device=dev)
+    with pytest.raises(RuntimeError, match="deterministic"):
+        ops.flowdppo_replay_step(v, stack, [0, 1], [1, 2], [0.9, 0.8], [0.8, 0.7], z, om, z, st, 0.1, eta=0.0)
+    with pytest.raises(ValueError, match="old_means"):
+        ops.flowdppo_replay_step(v, stack, [0, 1], [1, 2], [0.9, 0.8], [0.8, 0.7], z, om[:, :1], z, st, 0.1, eta=0.7)
+    with pytest.raises(ValueError, match="sigma_t"):
+        ops.flowdppo_replay_step(v, stack, [0, 1], [1, 2], [0.9, 0.8], [0.8, 0.7], z, om, z, torch.ones(3, device=dev), 0.1,
+                                 eta=0.7)
+
+
+class VelocityStage:
+    """A stage that hands over the velocities of all target steps at once (the opt-in protocol), and,
+    for the comparison, the reference's per-step replay."""
+
+    def __init__(self, fields, device, strategy):
+        self.fields = [f.to(device) for f in fields]
+        self.w = torch.tensor(1.0, device=device, requires_grad=True)
+        self.strategy = strategy
+        self.device = device
+
+    def replay_velocities(self, conditions, *, segment, params, step_indices):
+        return types.SimpleNamespace(noise_pred=torch.stack([self.w * self.fields[k] for k in step_indices], dim=1))
+
+    def replay(self, conditions, *, segment, params, step_indices):
+        lps, means = [], []
+        sig = segment.sigmas
+        for step in step_indices:
+            _, lp, mean = self.strategy.denoise(self.w * self.fields[step], segment.latents[:, step], sig[step],
+                                                sig[step + 1], eta=params.eta, prev_sample=segment.latents[:, step + 1],
+                                                sigma_max=sig[1])
+            lps.append(lp)
+            means.append(mean)
+        return types.SimpleNamespace(log_probs=torch.stack(lps, 1), prev_sample_means=torch.stack(means, 1))
+
+
+def test_flowdppo_uses_the_fused_step_when_the_stage_hands_over_velocities(dev):
+    """FlowDPPO on a stage with `replay_velocities`: same loss, metrics and parameter gradient as on a
+    stage that loops `denoise` per step (the reference's replay), through three launches."""
+    from unirl_amd import ops
+    from unirl_amd.algorithms import FlowDPPO
+    from unirl_amd.sde import FlowSDEStrategy
+
+    sig = osch.sigma_schedule(10, 3.0)
+    g = torch.Generator().manual_seed(47)
+    B, T, shape = 6, 10, (4, 8, 8)
+    fields = [torch.randn((B,) + shape, generator=g) for _ in range(T)]
+    latents = torch.randn((B, T + 1) + shape, generator=g)
+    adv = torch.randn(B, generator=g)
+    params = types.SimpleNamespace(eta=0.7)
+    # a threshold between the row KLs of this move of the policy (oracle means at w = 1 and w = 1.03)
+    steps = [4, 1, 2]
+    means = {}
+    for w in (1.0, 1.03):
+        means[w] = torch.stack([osde.sde_denoise("flow", w * fields[k], latents[:, k], sig[k], sig[k + 1], eta=0.7,
+                                                 prev_sample=latents[:, k + 1], sigma_max=sig[1], ieee_sqrt=True)[2]
+                                for k in steps], dim=1)
+    thr = float(ofd.kl_per_sample(means[1.03], means[1.0], ofd.sigma_t(sig, steps, 0.7)).median())
+    results = {}
+    for name, with_hook in (("fused", True), ("loop", False)):
+        stage = VelocityStage(fields, dev, FlowSDEStrategy())
+        if not with_hook:
+            stage.replay_velocities = None
+        seg = types.SimpleNamespace(latents=latents.to(dev), sigmas=sig.to(dev), indices=torch.arange(T + 1),
+                                    sde_indices=torch.tensor([4, 1, 2]), sde_logp=None, sde_means=None)
+        algo = FlowDPPO(params=params, stage=stage, kl_mask_threshold=thr, old_logp_source="replay")
+        algo.prepare_segment(conditions={}, segment=seg)
+        with torch.no_grad():
+            stage.w.fill_(1.03)
+        calls = []
+        real = ops.flowdppo_replay_step
+        ops.flowdppo_replay_step = lambda *a, **k: (calls.append(1), real(*a, **k))[1]
+        try:
+            res = algo.compute_loss_and_backward(conditions={}, segment=seg, advantages=adv.to(dev), training_progress=0.0,
+                                                 loss_scale=0.25)
+        finally:
+            ops.flowdppo_replay_step = real
+        assert len(calls) == (1 if with_hook else 0)
+        results[name] = (res, stage.w.grad.clone(), seg.sde_logp.clone(), seg.sde_means.clone())
+    (rf, gf, lpf, mf), (rl, gl, lpl, ml) = results["fused"], results["loop"]
+    assert torch.equal(mf, ml), "frozen means differ between the batched and the per-step anchor replay"
+    assert_close(lpf, lpl, 1e-6, 1e-7, "frozen log-probs")
+    assert abs(rf.loss - rl.loss) <= 1e-5 * abs(rl.loss) + 1e-7
+    for k, v in rl.metrics.items():
+        assert abs(rf.metrics[k] - v) <= 1e-5 * abs(v) + 1e-7, (k, rf.metrics[k], v)
+    assert 0.0 < rf.metrics["kl_mask_fraction"] < 1.0
+    assert_close(gf, gl, 1e-5, 1e-9, "d loss / d w")

@@ -179,6 +179,11 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_float,
          c_float, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
     ),
+    "unirl_flowdppo_replay_step": (
+        c_int,
+        [POINTER(SdeReplayDesc), c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_float, c_float, c_void_p, c_void_p,
+         c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    ),
     "unirl_expand_per_seq": (
         c_int,
         [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_void_p],

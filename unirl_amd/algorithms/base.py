@@ -197,7 +197,51 @@ class SdeStepAlgorithm(StageAlgorithm):
         indices = segment.sde_indices
         return [] if indices is None else [int(i) for i in indices.tolist()]
 
+    def _velocity_replay(self, conditions: Mapping[str, Any], segment: Any, steps: List[int]) -> Optional[Dict[str, Any]]:
+        """The operands of a batched replay, when the stage can hand over the model's velocities of
+        all target steps at once instead of looping ``denoise`` itself.
+
+        Opt-in protocol (no counterpart in the reference, whose stages loop step by step,
+        ``unirl/models/sd3/diffusion.py:467-497``): a stage with a ``replay_velocities(conditions, *,
+        segment, params, step_indices)`` method returns an object whose ``noise_pred`` holds the
+        velocities as ``[B, S', ...]`` (or ``[S', B, ...]`` with ``step_major=True``: a model pass
+        over the steps stacked into the batch); its SDE strategy is ``stage.strategy`` (or the
+        result's ``strategy``).  Everything else is read from the segment as the reference's loop
+        reads it: ``latents_at(step)`` / ``latents_at(step + 1)`` become slot tables into
+        ``segment.latents``, sigma pairs come from ``segment.sigmas``, ``sigma_max = sigmas[1]``.
+        Returns ``None`` for a stage without the method."""
+        hook = getattr(self.stage, "replay_velocities", None)
+        if hook is None:
+            return None
+        from ..sde.kernels import replay_slots
+
+        out = hook(typed_conditions(conditions, self.conditions_cls), segment=segment, params=self.params,
+                   step_indices=steps)
+        v = out.noise_pred
+        strategy = getattr(out, "strategy", None) or getattr(self.stage, "strategy", None)
+        if strategy is None or getattr(strategy, "_kind", None) is None:
+            raise RuntimeError(f"{type(self).__name__}: replay_velocities needs a stage.strategy with a fused SDE kernel")
+        device = v.device
+        latents = segment.latents if segment.latents.device == device else segment.latents.to(device)
+        sigmas = segment.sigmas.detach().to(device=device, dtype=torch.float32)
+        idx = torch.tensor(steps, dtype=torch.long, device=device)
+        slot_x, slot_p = replay_slots(segment.indices, steps)
+        return dict(
+            noise_pred=v, latents=latents, slot_sample=slot_x, slot_prev=slot_p, sigma=sigmas[idx], sigma_next=sigmas[idx + 1],
+            sigma_max=sigmas[1] if int(sigmas.shape[0]) > 1 else 0.99, eta=float(self.params.eta), strategy=strategy,
+            step_major=bool(getattr(out, "step_major", False)),
+        )
+
     def _replay(self, conditions: Mapping[str, Any], segment: Any, steps: List[int]) -> Any:
+        vr = self._velocity_replay(conditions, segment, steps)
+        if vr is not None:
+            # every (sample, step) transition in one launch pair, differentiable w.r.t. the velocities
+            import types
+
+            lp, means = vr["strategy"].replay_steps(
+                vr["noise_pred"], vr["latents"], vr["slot_sample"], vr["slot_prev"], vr["sigma"], vr["sigma_next"],
+                eta=vr["eta"], sigma_max=vr["sigma_max"], step_major=vr["step_major"])
+            return types.SimpleNamespace(log_probs=lp, prev_sample_means=means)
         return self.stage.replay(
             typed_conditions(conditions, self.conditions_cls), segment=segment, params=self.params, step_indices=steps
         )

@@ -197,6 +197,9 @@ class FlowDPPO(SdeStepAlgorithm):
         steps = self._resolve_target_steps(segment)
         if not steps:
             return NO_STEP
+        fused = self._step_from_velocities(conditions, segment, steps, advantages, loss_scale)
+        if fused is not None:
+            return fused
         replay = self._replay(conditions, segment, steps)
         new_logp, new_means = replay.log_probs, replay.prev_sample_means
         if new_means is None:
@@ -234,6 +237,47 @@ class FlowDPPO(SdeStepAlgorithm):
         metrics.update(policy_loss=loss_value, kl_mask_threshold=float(self.kl_mask_threshold))
         return AlgorithmStepResult(loss=loss_value, metrics=metrics, num_steps_or_tokens=len(steps),
                                    has_backward=True)
+
+    def _step_from_velocities(self, conditions, segment, steps, advantages, loss_scale) -> Optional[AlgorithmStepResult]:
+        """The whole micro-step from the model's stacked velocities (a stage with ``replay_velocities``):
+        replay log-probs, the KL against the frozen means, masks, loss, metrics and the gradient with
+        respect to the new log-probs in one streaming pass plus one finishing workgroup
+        (``unirl_flowdppo_replay_step`` -- the new means are never written), then the replay's
+        backward kernel hands the velocities their gradient.  Three launches for what the reference
+        does in ``S'`` ``denoise`` chains, a stack, a KL pass and autograd (``unirl/models/sd3/
+        diffusion.py:467-497``, ``unirl/algorithms/flowdppo.py:286-320``).  ``None`` when the stage
+        has no such method or the problem is beyond the fused kernel's row limit."""
+        if len(steps) == 0 or getattr(self.stage, "replay_velocities", None) is None:
+            return None
+        B = int(segment.latents.shape[0])
+        if not 0 < B * len(steps) <= ops.FLOWDPPO_REPLAY_MAX_ROWS:
+            return None
+        vr = self._velocity_replay(conditions, segment, steps)
+        v = vr["noise_pred"]
+        device = v.device
+
+        def frozen(name):
+            return gather_sde_field(getattr(segment, name), segment.sde_indices, steps, field_name=name).to(device)
+
+        old_logp, old_means = frozen("sde_logp"), frozen("sde_means")
+        sigma_t = self._compute_sigma_t(segment, steps, device=device).reshape(-1)
+        adv_b = advantages.detach().to(dtype=torch.float32, device=device).reshape(-1, 1).expand(B, len(steps))
+        need_grad = torch.is_grad_enabled() and v.requires_grad
+        kw = dict(kind=vr["strategy"]._kind, eta=vr["eta"], sigma_max=vr["sigma_max"], step_major=vr["step_major"])
+        out = ops.flowdppo_replay_step(
+            v, vr["latents"], vr["slot_sample"], vr["slot_prev"], vr["sigma"], vr["sigma_next"], old_logp, old_means,
+            adv_b, sigma_t, self.kl_mask_threshold, loss_scale=loss_scale if need_grad else None, **kw)
+        if need_grad:
+            grad_v = ops.sde_replay_logp_bwd(
+                v, vr["latents"], vr["slot_sample"], vr["slot_prev"], vr["sigma"], vr["sigma_next"],
+                g_logp=out["grad_logp"], g_mean=None, **kw)
+            v.backward(grad_v)
+        vals = out["metrics"].tolist()  # the step's only device-to-host copy
+        slots = dict(ops.FLOWDPPO_METRIC_SLOTS)
+        loss_value = vals[slots.pop("loss_mean")]
+        metrics: Dict[str, Any] = {k: vals[slot] for k, slot in slots.items()}
+        metrics.update(policy_loss=loss_value, kl_mask_threshold=float(self.kl_mask_threshold))
+        return AlgorithmStepResult(loss=loss_value, metrics=metrics, num_steps_or_tokens=len(steps), has_backward=True)
 
     def _loss_with_metrics(self, new_logp, old_logp, new_means, old_means, adv_b, sigma_t):
         kl, _ = ops.gaussian_kl_mask(

@@ -489,6 +489,32 @@ __device__ __forceinline__ double lane_ordered_sum(const double* __restrict__ p,
   if (rem <= 4 * kWave) return lane_ordered_sum_batched<4>(p, n, first);
   return lane_ordered_sum_batched<8>(p, n, first);
 }
+// Two arrays of `n` partials at once (per-lane sums as lane_ordered_sum gives them): both batches of
+// loads are in flight before either is used.
+__device__ __forceinline__ void lane_ordered_sum2(const double* __restrict__ p1, const double* __restrict__ p2,
+                                                  int64_t n, double& q1, double& q2) {
+  const int lane = threadIdx.x & (kWave - 1);
+  constexpr int kBatch = 8;
+  q1 = 0.0;
+  q2 = 0.0;
+  for (int64_t j0 = lane; j0 - lane < n; j0 += kWave * kBatch) {
+    double y1[kBatch], y2[kBatch];
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const int64_t j = j0 + b * kWave;
+      const int64_t jc = j < n ? j : n - 1;
+      y1[b] = p1[jc];
+      y2[b] = p2[jc];
+    }
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int b = 0; b < kBatch; ++b) {
+      const bool ok = j0 + b * kWave < n;
+      q1 += ok ? y1[b] : 0.0;
+      q2 += ok ? y2[b] : 0.0;
+    }
+  }
+}
 // The whole sum, valid in every lane.
 __device__ __forceinline__ double wave_ordered_sum(const double* __restrict__ p, int64_t n) {
   return wave_sum(lane_ordered_sum(p, n, 0));

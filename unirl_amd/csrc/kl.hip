@@ -14,6 +14,7 @@
 #include <mutex>
 
 #include "common_hip.h"
+#include "dppo_body.h"
 #include "unirl_internal.h"
 
 namespace unirl {
@@ -37,12 +38,6 @@ struct KlArgs {
   int always_partials;  // store workgroup partials even when one workgroup covers a row
   UNIRL_TRACE_FIELD
 };
-
-template <typename T>
-__device__ __forceinline__ float kl_sq(float p, float q) {
-  const float d = Elem<T>::round_trip(p - q);
-  return Elem<T>::round_trip(d * d);
-}
 
 __device__ __forceinline__ float kl_den(const KlArgs& A, int64_t row) {
   const float s = A.sigma[(A.row0 + row) % A.n_sigma];
@@ -227,116 +222,7 @@ static int launch_kl_elem(const KlArgs& A, int64_t R, int vec, hipStream_t st) {
   return (int)hipGetLastError();
 }
 
-// ---------------------------------------------------------------------------
-// KL-ADV masked loss over the [B,S'] log-probs (unirl/algorithms/flowdppo.py:86-137):
-// ratio, masks, where(keep, -A*r, 0) and the twelve logged metrics, one workgroup.
-// ---------------------------------------------------------------------------
-struct DppoArgs {
-  const float* nw;
-  const float* od;
-  const float* adv;
-  const float* kl;
-  int64_t n;
-  float threshold;
-  float* loss_elem;
-  float* metrics;
-  float* grad_new;  // NULL, or receives grad_scale * loss_elem (the gradient of grad_scale * n * mean)
-  float grad_scale;
-};
-
-enum { D_SR = 0, D_SR2, D_LD2, D_KL, D_LOSS, D_NKL, D_POS, D_NEG, D_RM, D_SUMS, D_RMIN = D_SUMS, D_RMAX, D_KLMAX, D_VALS };
-
-struct DppoAcc {
-  double acc[D_SUMS];
-  float rmin = INFINITY, rmax = -INFINITY, klmax = -INFINITY;
-  __device__ __forceinline__ DppoAcc() {
-#pragma unroll
-    for (int v = 0; v < D_SUMS; ++v) acc[v] = 0.0;
-  }
-};
-
-// Element i of the [B,S'] problem: ratio, the two removal masks, the kept loss (and its gradient).
-__device__ __forceinline__ void dppo_elem_of(const DppoArgs& A, int64_t i, float nw, float od, float a, float kl,
-                                             DppoAcc& s) {
-  const float ld = nw - od;
-  const float r = expf(ld);
-  const bool low_kl = kl < A.threshold;
-  const bool pos = !low_kl && (r > 1.0f) && (a > 0.0f);
-  const bool neg = !low_kl && (r < 1.0f) && (a < 0.0f);
-  const bool rm = pos || neg;
-  const float loss = rm ? 0.0f : (-a) * r;
-  A.loss_elem[i] = loss;
-  if (A.grad_new) A.grad_new[i] = A.grad_scale * loss;  // d(-a*exp(new-old))/dnew = the loss itself
-  s.acc[D_SR] += (double)r;
-  s.acc[D_SR2] += (double)r * (double)r;
-  s.acc[D_LD2] += (double)(0.5f * (ld * ld));
-  s.acc[D_KL] += (double)kl;
-  s.acc[D_LOSS] += (double)loss;
-  s.acc[D_NKL] += low_kl ? 0.0 : 1.0;
-  s.acc[D_POS] += pos ? 1.0 : 0.0;
-  s.acc[D_NEG] += neg ? 1.0 : 0.0;
-  s.acc[D_RM] += rm ? 1.0 : 0.0;
-  s.rmin = fminf(s.rmin, r);
-  s.rmax = fmaxf(s.rmax, r);
-  s.klmax = fmaxf(s.klmax, kl);
-}
-
-__device__ __forceinline__ void dppo_elem(const DppoArgs& A, int64_t i, float kl, DppoAcc& s) {
-  dppo_elem_of(A, i, A.nw[i], A.od[i], A.adv[i], kl, s);
-}
-
-// The twelve metrics from the totals; one thread.
-__device__ __forceinline__ void dppo_metrics(const DppoArgs& A, const double (&tot)[D_SUMS], float rmin, float rmax,
-                                             float klmax) {
-  const double N = (double)A.n;
-  // one reciprocal for every mean (x * (1/N) and x / N agree to an ulp of fp64, far below fp32)
-  const double inv_n = 1.0 / N;
-  double var = 0.0;
-  if (A.n > 1) {
-    var = (tot[D_SR2] - tot[D_SR] * tot[D_SR] * inv_n) / (N - 1.0);
-    if (var < 0.0) var = 0.0;
-  }
-  float* M = A.metrics;
-  M[0] = (float)(tot[D_SR] * inv_n);
-  M[1] = (float)sqrt(var);
-  // min()/max() of the reference return NaN when any element is NaN; ratios and KL values are
-  // >= 0, so their sums are NaN exactly then
-  const bool r_nan = tot[D_SR] != tot[D_SR], kl_nan = tot[D_KL] != tot[D_KL];
-  M[2] = r_nan ? quiet_nan() : rmin;
-  M[3] = r_nan ? quiet_nan() : rmax;
-  M[4] = (float)(tot[D_LD2] * inv_n);
-  M[5] = (float)(tot[D_KL] * inv_n);
-  M[6] = kl_nan ? quiet_nan() : klmax;
-  M[7] = (float)(tot[D_NKL] * inv_n);
-  M[8] = (float)(tot[D_POS] * inv_n);
-  M[9] = (float)(tot[D_NEG] * inv_n);
-  M[10] = (float)(tot[D_RM] * inv_n);
-  M[11] = (float)((N - tot[D_RM]) * inv_n);
-  M[12] = (float)(tot[D_LOSS] * inv_n);
-  M[13] = M[14] = M[15] = 0.0f;
-}
-
-// The whole [B,S'] problem on one wavefront (it is a few dozen elements): no barriers, the
-// reductions are DPP only.  `kl` points at global or LDS memory.  Every lane must call.
-// `first`: the lane's first element (new, old, advantage), already loaded by the caller, or null.
-__device__ __forceinline__ void dppo_on_one_wave(const DppoArgs& A, const float* kl, const float* first = nullptr) {
-  const int lane = threadIdx.x & (kWave - 1);
-  DppoAcc s;
-  int64_t i = lane;
-  if (first && i < A.n) {
-    dppo_elem_of(A, i, first[0], first[1], first[2], kl[i], s);
-    i += kWave;
-  }
-  for (; i < A.n; i += kWave) dppo_elem(A, i, kl[i], s);
-  double tot[D_SUMS];
-#pragma unroll
-  for (int v = 0; v < D_SUMS; ++v) tot[v] = wave_sum(s.acc[v]);
-  const float rmin = wave_min(s.rmin), rmax = wave_max(s.rmax), klmax = wave_max(s.klmax);
-  if (lane == 0) dppo_metrics(A, tot, rmin, rmax, klmax);
-}
-
 // Launched with one wavefront for up to kDppoWaveMax elements, with a workgroup beyond.
-constexpr int64_t kDppoWaveMax = 4096;
 
 __global__ __launch_bounds__(kKlThreads) void flowdppo_loss_kernel(DppoArgs A) {
   if (blockDim.x == kWave) {

@@ -17,6 +17,7 @@
 // = 20 bytes; replay with the mean kept: read v, x, prev; write mean = 16.
 
 #include "common_hip.h"
+#include "dppo_body.h"
 #include "unirl_internal.h"
 
 namespace unirl {
@@ -131,6 +132,11 @@ struct SdeStepArgs {
   float* logp_out;
   int64_t stride_logp;
   double* partials;        // [B][gridDim.x]
+  // fused Flow-DPPO replay only: the old policy's means [rows, D] (dense, the latents' dtype), whose
+  // Gaussian-KL numerator against this pass's means is summed beside the log-prob residual
+  const void* kl_old;
+  double* partials_kl;     // [rows][gridDim.x]
+  float* coef_out;         // [rows][2]: the row's log-prob denominator and log(std), for the finish kernel
   unsigned int nblk;       // host only: grid.x
   int items;               // host only: vectors in flight per lane
   UNIRL_TRACE_FIELD
@@ -160,9 +166,14 @@ __device__ __forceinline__ void sde_store_as(void* base, int dtype, int64_t idx,
     Vec<f16_t, VEC>::store(reinterpret_cast<f16_t*>(base) + idx, o);
 }
 
-template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING, bool ROWS>
+// KL (replay rows only): also read the old policy's mean of every element and accumulate
+// (round(mean) - old)^2 in the means' dtype beside the log-prob residual -- the numerator of
+// _gaussian_kl_div (unirl/algorithms/flowdppo.py:51) on the means the reference would have stored
+// (`.to(trajectory_dtype)`, unirl/models/sd3/diffusion.py:496) -- so that the Flow-DPPO loss needs
+// no second pass over the means.  Both partials go to the workspace whatever the grid.
+template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING, bool ROWS, bool KL = false>
 __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRowMap* M) {
-  __shared__ double lds[kSdeThreads / kWave];
+  __shared__ double lds[(KL ? 2 : 1) * (kSdeThreads / kWave)];
   using T3 = typename std::conditional<SAMPLING, float, TX>::type;
   UNIRL_TRACE_T0();
 
@@ -183,6 +194,7 @@ __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRow
   const TV* __restrict__ vp = reinterpret_cast<const TV*>(A.v) + b * A.stride_v + off_v;
   const TX* __restrict__ xp = reinterpret_cast<const TX*>(A.x) + b * A.stride_x + off_x;
   const T3* __restrict__ tp = A.third ? reinterpret_cast<const T3*>(A.third) + b * A.stride_third + off_t : nullptr;
+  const TX* __restrict__ qp = KL ? reinterpret_cast<const TX*>(A.kl_old) + row * A.D : nullptr;
   void* const po = A.prev_out;
   void* const mo = A.mean_out;
   const int64_t po0 = row * A.stride_prev, mo0 = row * A.stride_mean;
@@ -190,9 +202,9 @@ __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRow
 
   const int64_t nvec = D / VEC;  // VEC == 1 or D % VEC == 0 (checked on the host)
   const int64_t stride = (int64_t)gridDim.x * kSdeThreads;
-  float acc = 0.0f;
+  float acc = 0.0f, acc_kl = 0.0f;
 
-  float v[ITEMS][VEC], x[ITEMS][VEC], t[ITEMS][VEC];
+  float v[ITEMS][VEC], x[ITEMS][VEC], t[ITEMS][VEC], q[KL ? ITEMS : 1][VEC];
   auto load_pass = [&](int64_t i0) {
 #pragma unroll
     for (int it = 0; it < ITEMS; ++it) {
@@ -200,6 +212,7 @@ __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRow
       if (i < nvec) {
         Vec<TV, VEC>::load(vp + i * VEC, v[it]);
         Vec<TX, VEC>::load(xp + i * VEC, x[it]);
+        if (KL) Vec<TX, VEC>::load(qp + i * VEC, q[KL ? it : 0]);
         if (tp) {
           Vec<T3, VEC>::load(tp + i * VEC, t[it]);
         } else {
@@ -230,6 +243,7 @@ __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRow
         for (int k = 0; k < VEC; ++k) {
           const float d = sde_elem<TX, SAMPLING>(kind, c, v[it][k], x[it][k], t[it][k], mean[k], prev[k]);
           acc = fmaf(d, d, acc);
+          if (KL) acc_kl += kl_sq<TX>(Elem<TX>::round_trip(mean[k]), q[KL ? it : 0][k]);
         }
         if (po) sde_store_as<VEC>(po, pdt, po0 + i * VEC, prev);
         if (mo) sde_store_as<VEC>(mo, mdt, mo0 + i * VEC, mean);
@@ -245,6 +259,33 @@ __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRow
     return;
   }
 
+  if (KL) {
+    // both sums through one barrier: wavefront totals side by side, added in wavefront order
+    const double w_lp = wave_sum((double)acc), w_kl = wave_sum((double)acc_kl);
+    constexpr int kWaves = kSdeThreads / kWave;
+    const int wid = threadIdx.x / kWave;
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      lds[wid] = w_lp;
+      lds[kWaves + wid] = w_kl;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      double p_lp = lds[0], p_kl = lds[kWaves];
+#pragma unroll
+      for (int w = 1; w < kWaves; ++w) {
+        p_lp += lds[w];
+        p_kl += lds[kWaves + w];
+      }
+      A.partials[row * gridDim.x + blockIdx.x] = p_lp;     // both summed by flowdppo_replay_finish_kernel
+      A.partials_kl[row * gridDim.x + blockIdx.x] = p_kl;
+      if (blockIdx.x == 0) {  // the coefficients are worked out here anyway: the finish kernel only reads them
+        A.coef_out[2 * row] = c.den;
+        A.coef_out[2 * row + 1] = c.logs;
+      }
+    }
+    UNIRL_TRACE_END(A.trace);
+    return;
+  }
   const double part = block_sum<double>((double)acc, lds);
   if (threadIdx.x != 0) return;
   if (gridDim.x == 1) {
@@ -264,6 +305,123 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
 template <typename TV, typename TX, int VEC, int ITEMS>
 __global__ __launch_bounds__(kSdeThreads) void sde_replay_kernel(SdeStepArgs A, SdeRowMap M) {
   sde_step_body<TV, TX, VEC, ITEMS, false, true>(A, &M);
+}
+
+// The same replay with the Flow-DPPO KL numerator against the old means accumulated in the pass.
+template <typename TV, typename TX, int VEC, int ITEMS>
+__global__ __launch_bounds__(kSdeThreads) void sde_replay_kl_kernel(SdeStepArgs A, SdeRowMap M) {
+  sde_step_body<TV, TX, VEC, ITEMS, false, true, true>(A, &M);
+}
+
+// Finish of the fused Flow-DPPO replay step: one workgroup, arranged so that nothing is evaluated
+// twice -- on a single compute unit the fp64 divide / sqrt / log behind the coefficients and the
+// per-row divisions are what a replicated finish would spend its time on:
+//   1. every wavefront takes rows in turn and adds the row's log-prob and KL partials (fixed order;
+//      with one partial per lane the loads of four rows are in flight at once), leaving the two
+//      sums in LDS;
+//   2. the rows' coefficients (log-prob denominator, log std) are not worked out again: the streaming
+//      kernel, which needs them anyway, has left them in the workspace;
+//   3. after one barrier the first wavefront finishes the rows, lane = row (log-prob as
+//      sde_step_finalize_kernel, KL as gaussian_kl_finalize_kernel), and runs the [B,S'] KL-ADV
+//      problem on them (unirl/algorithms/flowdppo.py:86-137): masks, loss, the twelve metrics, the
+//      gradient with respect to the new log-probs.
+// R <= kReplayKlMaxRows.
+struct ReplayKlFinish {
+  const float* sigma_t;  // the KL's noise scale: row r uses sigma_t[r % n_sigma_t]
+  int64_t n_sigma_t;
+  float threshold;
+  float* kl_out;
+  uint8_t* mask_out;
+};
+constexpr int kReplayFinishThreads = 1024;
+constexpr int64_t kReplayKlMaxRows = 2048;
+
+__global__ __launch_bounds__(kReplayFinishThreads) void flowdppo_replay_finish_kernel(SdeStepArgs A, DppoArgs P,
+                                                                                     ReplayKlFinish F, unsigned int nblk) {
+  __shared__ double lds_q[2][kReplayKlMaxRows];  // per row: the two sums of partials
+  __shared__ float lds_lp[kReplayKlMaxRows];
+  __shared__ float lds_kl[kReplayKlMaxRows];
+  UNIRL_TRACE_T0();
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  const int64_t R = P.n;
+  constexpr int kWaves = kReplayFinishThreads / kWave;
+  // the first wavefront's share of the [B,S'] problem and of the KL scales is loaded now, with the partials
+  float first_od = 0.0f, first_adv = 0.0f, first_st = 1.0f, first_den = 1.0f, first_logs = 0.0f;
+  if (wave == 0 && lane < R) {
+    first_od = P.od[lane];
+    first_adv = P.adv[lane];
+    first_st = F.sigma_t[lane % F.n_sigma_t];
+    first_den = A.coef_out[2 * lane];
+    first_logs = A.coef_out[2 * lane + 1];
+  }
+
+  auto store_row = [&](int64_t row, double q_lp, double q_kl) {
+    q_lp = wave_sum(q_lp);
+    q_kl = wave_sum(q_kl);
+    if (lane == 0) {
+      lds_q[0][row] = q_lp;
+      lds_q[1][row] = q_kl;
+    }
+  };
+  if (nblk <= kWave) {
+    // One partial per lane and row: a wavefront keeps the loads of four of its rows in flight at once
+    // (every trip to memory that waits for the one before costs about a microsecond here).  A row
+    // past the end repeats the last row's loads and is dropped.
+    constexpr int kRows = 4;
+    const unsigned int jl = (unsigned int)lane < nblk ? lane : nblk - 1;
+    for (int64_t base = wave; base < R; base += kWaves * kRows) {
+      double y_lp[kRows], y_kl[kRows];
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        const int64_t row = base + r * kWaves;
+        const int64_t rc = row < R ? row : R - 1;
+        y_lp[r] = A.partials[rc * nblk + jl];
+        y_kl[r] = A.partials_kl[rc * nblk + jl];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        const int64_t row = base + r * kWaves;
+        if (row < R) {  // wave-uniform
+          const bool ok = (unsigned int)lane < nblk;
+          store_row(row, ok ? y_lp[r] : 0.0, ok ? y_kl[r] : 0.0);
+        }
+      }
+    }
+  } else {
+    // many partials per row means few rows (rows * nblk is capped by the launch): one row at a time
+    for (int64_t row = wave; row < R; row += kWaves) {
+      double q_lp, q_kl;
+      lane_ordered_sum2(A.partials + row * nblk, A.partials_kl + row * nblk, nblk, q_lp, q_kl);
+      store_row(row, q_lp, q_kl);
+    }
+  }
+  UNIRL_TRACE_MARK1();
+  __syncthreads();
+  if (wave != 0) return;
+  // lane = row: the log-prob and the KL of 64 rows per pass, then the loss on them
+  for (int64_t row = lane; row < R; row += kWave) {
+    const bool head = (row == lane);  // the lane's first row: its operands were loaded at kernel entry
+    SdeCoef c;
+    c.den = head ? first_den : A.coef_out[2 * row];
+    c.logs = head ? first_logs : A.coef_out[2 * row + 1];
+    const float lp = sde_finish_logp(A.kind, c, lds_q[0][row], (double)A.D, A.logp_sum);
+    const float st = head ? first_st : F.sigma_t[row % F.n_sigma_t];
+    const float den = 2.0f * (st * st);
+    const float kl = (float)((lds_q[1][row] / (double)den) / (double)A.D);
+    A.logp_out[row * A.stride_logp] = lp;
+    F.kl_out[row] = kl;
+    if (F.mask_out) F.mask_out[row] = (kl < F.threshold) ? 1 : 0;
+    lds_lp[row] = lp;
+    lds_kl[row] = kl;
+  }
+  UNIRL_TRACE_MARK2();
+  DppoArgs Q = P;
+  Q.nw = lds_lp;  // the new log-probs never leave the workgroup before the loss has used them
+  float first[3] = {0.0f, first_od, first_adv};
+  if (lane < R) first[0] = lds_lp[lane];
+  dppo_on_one_wave(Q, lds_kl, first);
+  UNIRL_TRACE_END(A.trace);
 }
 
 // One wavefront per row: adds the workgroup partials in index order and finishes the log-prob.
@@ -704,6 +862,33 @@ static int launch_replay_x(const SdeStepArgs& A, const SdeRowMap& M, int dtype_x
 }
 
 template <typename TV, typename TX>
+static int launch_replay_kl(const SdeStepArgs& A, const SdeRowMap& M, int64_t rows, int vec, hipStream_t st) {
+  dim3 grid(A.nblk, (unsigned int)rows), block(kSdeThreads);
+  if (vec == 8) {
+    if constexpr (sizeof(TV) == 2 || sizeof(TX) == 2)
+      hipLaunchKernelGGL((sde_replay_kl_kernel<TV, TX, 8, 2>), grid, block, 0, st, A, M);
+    else
+      return UNIRL_E_DTYPE;
+  } else if (vec == 4) {
+    hipLaunchKernelGGL((sde_replay_kl_kernel<TV, TX, 4, 4>), grid, block, 0, st, A, M);
+  } else {
+    hipLaunchKernelGGL((sde_replay_kl_kernel<TV, TX, 1, 2>), grid, block, 0, st, A, M);
+  }
+  return (int)hipGetLastError();
+}
+
+template <typename TV>
+static int launch_replay_kl_x(const SdeStepArgs& A, const SdeRowMap& M, int dtype_x, int64_t rows, int vec,
+                              hipStream_t st) {
+  switch (dtype_x) {
+    case UNIRL_F32: return launch_replay_kl<TV, float>(A, M, rows, vec, st);
+    case UNIRL_BF16: return launch_replay_kl<TV, bf16_t>(A, M, rows, vec, st);
+    case UNIRL_F16: return launch_replay_kl<TV, f16_t>(A, M, rows, vec, st);
+  }
+  return UNIRL_E_DTYPE;
+}
+
+template <typename TV, typename TX>
 static int launch_replay_bwd(const SdeBwdArgs& A, const SdeRowMap& M, int64_t rows, int vec, hipStream_t st) {
   const unsigned int nblk = sde_blocks_per_sample(A.D / vec, 1, rows);
   dim3 grid(nblk, (unsigned int)rows), block(kSdeThreads);
@@ -1015,6 +1200,105 @@ extern "C" int unirl_sde_replay_logp(const unirl_sde_replay_desc* d, void* works
     }
   }
   return UNIRL_OK;
+}
+
+extern "C" int unirl_flowdppo_replay_step(const unirl_sde_replay_desc* d, const void* old_means, const float* sigma_t,
+                                          int64_t n_sigma_t, const float* old_logp, const float* advantages,
+                                          float threshold, float loss_scale, float* kl_out, uint8_t* mask_out,
+                                          float* loss_elem, float* grad_logp, float* metrics, void* workspace,
+                                          size_t workspace_bytes, void* stream) {
+  if (!d) return UNIRL_E_NULL;
+  ReplayPlan P;
+  const size_t sx = dtype_ok(d->latents.dtype) ? dtype_size(d->latents.dtype) : 4;
+  int rc = plan_replay(d, nullptr, old_means, sx, P);
+  if (rc != 0) return rc;
+  const int64_t B = d->B, S = d->S, D = d->D, R = B * S;
+  if (R <= 0 || n_sigma_t <= 0) return UNIRL_E_SHAPE;
+  if (d->eta < 1e-7) return UNIRL_E_SHAPE;  // a deterministic step has no log-prob to build a ratio from
+  if (R > kReplayKlMaxRows) return UNIRL_E_LIMIT;
+  if (!d->noise_pred.ptr || !d->latents.ptr || !d->sigma || !d->sigma_next || !d->logp_out || !old_means || !sigma_t ||
+      !old_logp || !advantages || !kl_out || !loss_elem || !metrics)
+    return UNIRL_E_NULL;
+  if (!aligned_to(sigma_t, 4) || !aligned_to(old_logp, 4) || !aligned_to(advantages, 4) || !aligned_to(kl_out, 4) ||
+      !aligned_to(loss_elem, 4) || !aligned_to(grad_logp, 4) || !aligned_to(metrics, 4))
+    return UNIRL_E_ALIGN;
+  if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
+  const int vec = P.vec;
+  const int items = (vec == 8) ? 2 : (vec == 4) ? 4 : 2;
+  // Workgroups: at most 768 in all -- with its fourth operand in flight the kernel holds 136 - 157 vector
+  // registers, three wavefronts per SIMD, so 3 x 256 workgroups are resident at once and a 769th would
+  // wait for a whole workgroup's lifetime (896 at the WAN shape: 50 us per call, 728: 43 us) -- at most
+  // 64 per row (the finish kernel then has one partial per lane and keeps several rows in flight),
+  // and the fewest that keep the number of passes, so that every pass of a lane is a full one.
+  unsigned int nblk = sde_blocks_per_sample(D / vec, items, R, 768);
+  if (nblk > (unsigned int)kWave) nblk = kWave;
+  {
+    const int64_t per_lane = (int64_t)kSdeThreads * items, nvec = D / vec;
+    const int64_t passes = (nvec + nblk * per_lane - 1) / (nblk * per_lane);
+    const int64_t even = (nvec + passes * per_lane - 1) / (passes * per_lane);
+    if (even >= 1 && even < (int64_t)nblk) nblk = (unsigned int)even;
+  }
+  if ((2 * (int64_t)nblk + 1) * R > kPartialCapacity) return UNIRL_E_LIMIT;
+  hipStream_t st = (hipStream_t)stream;
+  SdeStepArgs A = {};
+  A.v = d->noise_pred.ptr;
+  A.x = d->latents.ptr;
+  A.third = A.x;  // the stored next latent lives in the same stack
+  A.stride_v = P.stride_v;
+  A.stride_x = P.stride_x;
+  A.stride_third = P.stride_x;
+  A.sigma = d->sigma;
+  A.sigma_next = d->sigma_next;
+  A.sigma_max_ptr = d->sigma_max_ptr;
+  A.sigma_max_val = d->sigma_max_val;
+  A.sigma_stride = 0;
+  A.sc = make_scalars(d->eta);
+  A.kind = d->kind;
+  A.want_logp = 1;
+  A.logp_sum = d->logp_sum;
+  A.D = D;
+  A.prev_out = nullptr;
+  A.mean_out = d->mean_out;  // only on request: the loss itself never needs the means in memory
+  A.prev_dtype = UNIRL_F32;
+  A.mean_dtype = d->mean_dtype;
+  A.stride_prev = D;
+  A.stride_mean = D;
+  A.logp_out = d->logp_out;
+  A.stride_logp = 1;
+  A.partials = ws_partials(workspace);
+  A.partials_kl = ws_partials(workspace) + (int64_t)nblk * R;
+  A.coef_out = reinterpret_cast<float*>(ws_partials(workspace) + 2 * (int64_t)nblk * R);
+  A.kl_old = old_means;
+  A.nblk = nblk;
+  A.items = items;
+  UNIRL_TRACE_SET(A, "sde_replay_kl", nblk * (unsigned int)R);
+  rc = UNIRL_E_DTYPE;
+  switch (d->noise_pred.dtype) {
+    case UNIRL_F32: rc = launch_replay_kl_x<float>(A, P.M, d->latents.dtype, R, vec, st); break;
+    case UNIRL_BF16: rc = launch_replay_kl_x<bf16_t>(A, P.M, d->latents.dtype, R, vec, st); break;
+    case UNIRL_F16: rc = launch_replay_kl_x<f16_t>(A, P.M, d->latents.dtype, R, vec, st); break;
+  }
+  if (rc != 0) return rc;
+  DppoArgs Q;
+  Q.nw = nullptr;  // taken from the finish kernel's LDS
+  Q.od = old_logp;
+  Q.adv = advantages;
+  Q.kl = nullptr;
+  Q.n = R;
+  Q.threshold = threshold;
+  Q.loss_elem = loss_elem;
+  Q.metrics = metrics;
+  Q.grad_new = grad_logp;
+  Q.grad_scale = loss_scale / (float)R;
+  ReplayKlFinish F;
+  F.sigma_t = sigma_t;
+  F.n_sigma_t = n_sigma_t;
+  F.threshold = threshold;
+  F.kl_out = kl_out;
+  F.mask_out = mask_out;
+  UNIRL_TRACE_SET(A, "flowdppo_replay_finish", 1);
+  hipLaunchKernelGGL(flowdppo_replay_finish_kernel, dim3(1), dim3(kReplayFinishThreads), 0, st, A, Q, F, nblk);
+  return (int)hipGetLastError();
 }
 
 extern "C" int unirl_sde_replay_logp_bwd(const unirl_sde_replay_desc* d, const float* g_logp, const float* g_mean,

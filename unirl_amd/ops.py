@@ -715,6 +715,7 @@ def flowdppo_loss(
 
 
 FLOWDPPO_STEP_MAX_ROWS = 4096
+FLOWDPPO_REPLAY_MAX_ROWS = 2048  # unirl_flowdppo_replay_step: (sample, step) rows per call
 
 
 def flowdppo_step(
@@ -778,6 +779,83 @@ def flowdppo_step(
         )
     N.check(rc, "unirl_flowdppo_step")
     return kl, elem, metrics, grad
+
+
+def flowdppo_replay_step(
+    noise_pred: torch.Tensor,
+    latents: torch.Tensor,
+    slot_sample: Sequence[int],
+    slot_prev: Sequence[int],
+    sigma,
+    sigma_next,
+    old_logp: torch.Tensor,
+    old_means: torch.Tensor,
+    advantages: torch.Tensor,
+    sigma_t: torch.Tensor,
+    threshold: float,
+    *,
+    kind: str = "flow",
+    eta: float = 1.0,
+    sigma_max: Union[float, torch.Tensor] = 0.99,
+    step_major: bool = False,
+    loss_scale: Optional[float] = None,
+    want_means: bool = False,
+    want_mask: bool = False,
+):
+    """The forward of a Flow-DPPO micro-step from the model's velocities, as one streaming pass and
+    one finishing workgroup: :func:`sde_replay_logp` and :func:`flowdppo_step` without the new means
+    ever being written or re-read.
+
+    Arguments as :func:`sde_replay_logp` (velocities ``[B, S, ...]``, the ``[B, K, ...]`` stack and
+    its slot tables, one sigma pair per step) plus the frozen ``old_logp`` ``[B, S]`` and
+    ``old_means`` ``[B, S, ...]``, the advantages (``[B, S]`` or broadcastable), the KL's
+    ``sigma_t`` (one value or one per step) and the KL threshold.  Returns a dict with ``logp``
+    ``[B, S]``, ``kl`` ``[B, S]``, ``loss_elem`` ``[B, S]``, ``metrics`` ``[16]`` (all fp32), ``grad_logp``
+    ``[B, S]`` (``loss_scale`` given: what ``(loss_elem.mean() * loss_scale).backward()`` leaves in the
+    new log-probs; hand it to :func:`sde_replay_logp_bwd`), and on request ``means`` (the stack's
+    dtype) and ``mask`` (bool, ``kl < threshold``).  At most ``FLOWDPPO_REPLAY_MAX_ROWS`` rows."""
+    d, keep, B, S, D, tail = _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next, kind, eta,
+                                          sigma_max, step_major)
+    device = latents.device
+    x = keep[1]
+    R = B * S
+    if R == 0 or D == 0 or R > FLOWDPPO_REPLAY_MAX_ROWS:
+        raise ValueError(f"flowdppo_replay_step handles 1..{FLOWDPPO_REPLAY_MAX_ROWS} (sample, step) rows; got {R}")
+    if eta < 1e-7:
+        raise RuntimeError(f"flowdppo_replay_step: eta={eta} is a deterministic step (no log-prob)")
+    if tuple(old_means.shape) != (B, S) + tail:
+        raise ValueError(f"old_means {tuple(old_means.shape)} != {(B, S) + tail}")
+    qm = old_means.detach()
+    if qm.dtype is not x.dtype or qm.device != device or not qm.is_contiguous():
+        qm = qm.to(device=device, dtype=x.dtype).contiguous()  # the KL is taken in the trajectory dtype
+    sig_t = N.as_operand(sigma_t, torch.float32, device)
+    if sig_t.numel() not in (1, S):
+        raise ValueError(f"sigma_t must hold 1 or {S} values; got {tuple(sigma_t.shape)}")
+
+    def f32c(t):
+        if tuple(t.shape) != (B, S):
+            t = t.detach().expand((B, S))
+        return N.as_operand(t, torch.float32, device)
+
+    od, ad = f32c(old_logp), f32c(advantages)
+    logp, kl, elem, grad = torch.empty((4, B, S), dtype=torch.float32, device=device).unbind(0)
+    if loss_scale is None:
+        grad = None
+    metrics = torch.empty(N.M_COUNT, dtype=torch.float32, device=device)
+    means = torch.empty((B, S) + tail, dtype=x.dtype, device=device) if want_means else None
+    mask = torch.empty((B, S), dtype=torch.bool, device=device) if want_mask else None
+    d.mean_out, d.mean_dtype = N.ptr(means), (N.dtype_code(x.dtype) if want_means else 0)
+    d.logp_out, d.logp_sum = N.ptr(logp), 0
+    stream = N.current_stream(device)
+    ws, ws_bytes = N.workspace(device, stream)
+    with N.on_device(device):
+        rc = N.F.unirl_flowdppo_replay_step(
+            ctypes.byref(d), N.ptr(qm), N.ptr(sig_t), sig_t.numel(), N.ptr(od), N.ptr(ad), float(threshold),
+            float(loss_scale or 0.0), N.ptr(kl), N.ptr(mask), N.ptr(elem), N.ptr(grad), N.ptr(metrics), N.ptr(ws),
+            ws_bytes, stream,
+        )
+    N.check(rc, "unirl_flowdppo_replay_step")
+    return dict(logp=logp, kl=kl, loss_elem=elem, metrics=metrics, grad_logp=grad, means=means, mask=mask)
 
 
 def expand_per_seq(values: torch.Tensor, cu_seqlens: torch.Tensor, n_tok: int) -> torch.Tensor:
