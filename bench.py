@@ -179,6 +179,36 @@ def make_shapes(torch, dev):
         cpu_bytes=bytes1,
     ))
 
+    # the same sampling step with the noise drawn inside the kernel (Philox + Box-Muller in registers):
+    # 2 reads + 2 writes, no noise tensor written by torch.randn and read back
+    bytes1g = 4 * numel * 4
+
+    def run1g(i):
+        x, v, _ = sets1[i % ns]
+        return ops.sde_step_logp(v, x, s10, s11, kind="flow", eta=0.7, sigma_max=smax, rng=(1001, 4 * i))
+
+    shapes.append(dict(
+        name="sde_step_logp_sample_rng", config=1,
+        shape="fp32 [8,16,128,128], step 10/28, sampling, noise drawn in the kernel (2 reads, 2 writes)",
+        bytes=bytes1g, read_bytes=2 * numel * 4, write_bytes=2 * numel * 4, elements=numel, run=run1g, sets=ns,
+    ))
+
+    # what that replaces: the noise drawn by torch.randn into a tensor (one more launch, one more write),
+    # then the 3-read step -- the sampling step of a rollout as denoise() ran it before
+    noise_buf = [torch.empty(shp, device=dev) for _ in range(ns)]
+
+    def run1n(i):
+        x, v, _ = sets1[i % ns]
+        n = noise_buf[i % ns].normal_()
+        return ops.sde_step_logp(v, x, s10, s11, kind="flow", eta=0.7, noise=n, sigma_max=smax)
+
+    shapes.append(dict(
+        name="sde_step_logp_sample_randn", config=1,
+        shape="fp32 [8,16,128,128], step 10/28, sampling: torch's normal_() into a noise tensor, then the step "
+              "(GB/s on the drawing kernel's 2 reads + 2 writes)",
+        bytes=bytes1g, read_bytes=3 * numel * 4, write_bytes=3 * numel * 4, elements=numel, run=run1n, sets=ns,
+    ))
+
     # the same step in replay mode: the stored next latent is given, mean and log-prob come back
     prev_dev = run1(0)[0]
     prev_host = prev_dev.cpu()

@@ -39,7 +39,8 @@ extern "C" {
  * unirl_flowdppo_step added.  3: unirl_dpm2_step added.  4: unirl_gaussian_kl_mask_static
  * added.  5: unirl_sde_replay_logp, unirl_sde_replay_logp_bwd, unirl_lmhead_logp added.
  * 6: the unirl_calib_* measurement aids left the library (they live in the measurement build);
- * unirl_flowdppo_replay_step added. */
+ * unirl_flowdppo_replay_step added; in-kernel sampling noise (struct unirl_rng in
+ * unirl_sde_step_desc, two more arguments of unirl_sde_rollout_logp). */
 #define UNIRL_ABI_VERSION 6
 
 enum unirl_dtype { UNIRL_F32 = 0, UNIRL_BF16 = 1, UNIRL_F16 = 2 };
@@ -110,9 +111,20 @@ struct unirl_sde_tensor {
   int dtype;             /* unirl_dtype */
   int64_t sample_stride; /* elements; 0 = D */
 };
+/* Sampling noise drawn inside the kernel instead of read from memory -- the reference draws it
+ * inside FlowSDEStrategy.step with randn_tensor(generator=None) (unirl/sde/kernels.py:230-232),
+ * i.e. from a generator no bit pattern of which has to be matched.  Counter-based: Philox-4x32-10
+ * keyed by `seed`, counter {element index / 4, offset (+ the step index in a rollout)}, two
+ * Box-Muller pairs per block; the draw of an element depends only on (seed, offset, step,
+ * b * D + i), never on the launch shape.  The caller moves `offset` on between calls. */
+struct unirl_rng {
+  int enabled;
+  uint64_t seed;
+  uint64_t offset;
+};
 struct unirl_sde_step_desc {
   struct unirl_sde_tensor noise_pred, sample, prev_sample;
-  const float* noise;    /* sampling only; NULL = no noise */
+  const float* noise;    /* sampling only; NULL = no noise (or drawn in the kernel, see rng) */
   int64_t noise_stride;
   const float* sigma;
   const float* sigma_next;
@@ -131,6 +143,9 @@ struct unirl_sde_step_desc {
   float* logp_out;       /* element b at logp_out[b * logp_stride] */
   int64_t logp_stride;   /* 0 = 1 */
   int logp_sum;
+  struct unirl_rng rng;  /* sampling with noise == NULL: draw N(0,1) noise in the kernel */
+  float* noise_out;      /* NULL, or f32 [B,D]: receives the drawn noise (one more write) */
+  int64_t noise_out_stride; /* elements between samples; 0 = D */
 };
 int unirl_sde_step_logp_ex(const struct unirl_sde_step_desc* desc /* host */, void* workspace,
                            size_t workspace_bytes, void* stream);
@@ -217,14 +232,20 @@ int unirl_sde_step_logp_bwd(const void* noise_pred, int dtype_v, const void* sam
  *   x0          [B,D] dtype_x
  *   v_steps     host array of S device pointers, each [B,D] dtype_v
  *   noise_steps host array of S device pointers, each [B,D] f32 (entries may
- *               be NULL for steps with eta < 1e-7)
+ *               be NULL: no noise for that step, or noise drawn in the kernel
+ *               when rng is given); NULL altogether with rng
+ *   rng         host, NULL or the generator: a step without a noise pointer and
+ *               with eta >= 1e-7 draws its noise in the kernel (step k uses
+ *               offset + k); noise_out_steps: NULL, or host array of S device
+ *               pointers (entries may be NULL), each f32 [B,D], receiving it
  *   sigmas      device f32 [S+1];  etas  host double [S]
  *   x_out       [B,D] f32  final latent
  *   traj_out    NULL or [S,B,D] f32: latent after every step
  *   logp_out    [B,S] f32; steps with eta < 1e-7 hold NaN
  * ---------------------------------------------------------------------- */
 int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* const* v_steps, int dtype_v,
-                           const float* const* noise_steps, const float* sigmas,
+                           const float* const* noise_steps, const struct unirl_rng* rng /* host */,
+                           float* const* noise_out_steps, const float* sigmas,
                            const double* etas, int S, const float* sigma_max_ptr,
                            float sigma_max_val, int kind, int64_t B, int64_t D, float* x_out,
                            float* traj_out, float* logp_out, int logp_sum, void* workspace,

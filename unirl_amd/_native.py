@@ -61,6 +61,12 @@ class SdeTensor(Structure):
     _fields_ = [("ptr", c_void_p), ("dtype", c_int), ("sample_stride", c_int64)]
 
 
+class Rng(Structure):
+    """struct unirl_rng."""
+
+    _fields_ = [("enabled", c_int), ("seed", ctypes.c_uint64), ("offset", ctypes.c_uint64)]
+
+
 class SdeStepDesc(Structure):
     """struct unirl_sde_step_desc."""
 
@@ -88,6 +94,9 @@ class SdeStepDesc(Structure):
         ("logp_out", c_void_p),
         ("logp_stride", c_int64),
         ("logp_sum", c_int),
+        ("rng", Rng),
+        ("noise_out", c_void_p),
+        ("noise_out_stride", c_int64),
     ]
 
 
@@ -153,9 +162,9 @@ _SIGNATURES = {
     ),
     "unirl_sde_rollout_logp": (
         c_int,
-        [c_void_p, c_int, POINTER(c_void_p), c_int, POINTER(c_void_p), c_void_p, POINTER(c_double), c_int,
-         c_void_p, c_float, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_size_t,
-         c_void_p],
+        [c_void_p, c_int, POINTER(c_void_p), c_int, POINTER(c_void_p), POINTER(Rng), POINTER(c_void_p), c_void_p,
+         POINTER(c_double), c_int, c_void_p, c_float, c_int, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_int,
+         c_void_p, c_size_t, c_void_p],
     ),
     "unirl_dpm2_step": (
         c_int,

@@ -428,6 +428,73 @@ __device__ __forceinline__ float block_min(float v, float* lds) {
 }
 
 // ---------------------------------------------------------------------------
+// Counter-based normal draws: Philox-4x32-10 (Salmon et al., "Parallel random numbers: as easy as
+// 1, 2, 3", SC'11) keyed by a 64-bit seed, with the 128-bit counter {element index / 4, offset};
+// one block yields the standard normals of four consecutive elements through two Box-Muller
+// pairs.  A draw depends only on (seed, offset, element index): not on the launch shape, the
+// vector width or which lane computes it.
+// ---------------------------------------------------------------------------
+struct RngKey {
+  uint32_t k0, k1;  // seed
+  uint32_t o0, o1;  // offset: counter words 2 and 3
+};
+
+__device__ __forceinline__ void philox4x32_10(uint32_t (&c)[4], uint32_t k0, uint32_t k1) {
+  constexpr uint32_t kM0 = 0xD2511F53u, kM1 = 0xCD9E8D57u, kW0 = 0x9E3779B9u, kW1 = 0xBB67AE85u;
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi0 = __umulhi(kM0, c[0]), lo0 = kM0 * c[0];
+    const uint32_t hi1 = __umulhi(kM1, c[2]), lo1 = kM1 * c[2];
+    c[0] = hi1 ^ c[1] ^ k0;
+    c[1] = lo1;
+    c[2] = hi0 ^ c[3] ^ k1;
+    c[3] = lo0;
+    k0 += kW0;
+    k1 += kW1;
+  }
+}
+
+// Two independent standard normals from two 32-bit words: u1 = (a + 1/2) / 2^32 in (0, 1],
+// u2 = b / 2^32 in [0, 1]; r = sqrt(-2 ln u1); (r cos 2 pi u2, r sin 2 pi u2).  The hardware
+// log2 / sin / cos (arguments in revolutions, so no range reduction) are accurate to about an ulp;
+// |z| <= 6.7.
+__device__ __forceinline__ void box_muller(uint32_t a, uint32_t b, float& z0, float& z1) {
+  const float u1 = fmaf((float)a, 2.3283064365386963e-10f, 1.1641532182693481e-10f);
+  const float u2 = (float)b * 2.3283064365386963e-10f;
+  const float r = __builtin_amdgcn_sqrtf(-1.3862943611198906f * __builtin_amdgcn_logf(u1));  // -2 ln2 * log2(u1)
+  z0 = r * __builtin_amdgcn_cosf(u2);
+  z1 = r * __builtin_amdgcn_sinf(u2);
+}
+
+// The normals of elements [4 * block, 4 * block + 4).
+__device__ __forceinline__ void rng_normal4(const RngKey& K, uint64_t block, uint32_t step, float (&z)[4]) {
+  uint32_t c[4] = {(uint32_t)block, (uint32_t)(block >> 32), K.o0 + step, K.o1};
+  philox4x32_10(c, K.k0, K.k1);
+  box_muller(c[0], c[1], z[0], z[1]);
+  box_muller(c[2], c[3], z[2], z[3]);
+}
+
+// VEC normals for the elements starting at index e (a multiple of VEC when VEC is 4 or 8).
+template <int VEC>
+__device__ __forceinline__ void rng_normals(const RngKey& K, uint64_t e, uint32_t step, float (&out)[VEC]) {
+  if constexpr (VEC == 1) {
+    float z[4];
+    rng_normal4(K, e >> 2, step, z);
+    const int w = (int)(e & 3);
+    out[0] = w == 0 ? z[0] : (w == 1 ? z[1] : (w == 2 ? z[2] : z[3]));
+  } else {
+    static_assert(VEC % 4 == 0, "whole Philox blocks");
+#pragma unroll
+    for (int g = 0; g < VEC / 4; ++g) {
+      float z[4];
+      rng_normal4(K, (e >> 2) + g, step, z);
+#pragma unroll
+      for (int k = 0; k < 4; ++k) out[4 * g + k] = z[k];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Timeline marks of measurement builds (-DUNIRL_TRACE); nothing otherwise.  T0 reads the clock
 // at kernel entry, MARK reads it again, END has thread 0 of the workgroup store
 // {start, mark1, mark2, end} at slot (workgroup index) of the launch's trace slice.

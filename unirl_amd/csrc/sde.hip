@@ -134,6 +134,12 @@ struct SdeStepArgs {
   double* partials;        // [B][gridDim.x]
   // fused Flow-DPPO replay only: the old policy's means [rows, D] (dense, the latents' dtype), whose
   // Gaussian-KL numerator against this pass's means is summed beside the log-prob residual
+  // sampling only: noise drawn in the kernel (third == nullptr), optionally stored
+  int rng;
+  RngKey rng_key;
+  int64_t rng_row0;        // index of the launch's first sample within the call
+  float* noise_out;
+  int64_t stride_noise_out;
   const void* kl_old;
   double* partials_kl;     // [rows][gridDim.x]
   float* coef_out;         // [rows][2]: the row's log-prob denominator and log(std), for the finish kernel
@@ -171,8 +177,10 @@ __device__ __forceinline__ void sde_store_as(void* base, int dtype, int64_t idx,
 // _gaussian_kl_div (unirl/algorithms/flowdppo.py:51) on the means the reference would have stored
 // (`.to(trajectory_dtype)`, unirl/models/sd3/diffusion.py:496) -- so that the Flow-DPPO loss needs
 // no second pass over the means.  Both partials go to the workspace whatever the grid.
-template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING, bool ROWS, bool KL = false>
+// RNG (sampling only): the noise is drawn in the kernel (A.rng_key) instead of read through `third`.
+template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING, bool ROWS, bool KL = false, bool RNG = false>
 __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRowMap* M) {
+  static_assert(!RNG || (SAMPLING && !ROWS && !KL), "noise is drawn for the plain sampling step only");
   __shared__ double lds[(KL ? 2 : 1) * (kSdeThreads / kWave)];
   using T3 = typename std::conditional<SAMPLING, float, TX>::type;
   UNIRL_TRACE_T0();
@@ -215,9 +223,20 @@ __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRow
         if (KL) Vec<TX, VEC>::load(qp + i * VEC, q[KL ? it : 0]);
         if (tp) {
           Vec<T3, VEC>::load(tp + i * VEC, t[it]);
-        } else {
+        } else if (!RNG) {
 #pragma unroll
           for (int k = 0; k < VEC; ++k) t[it][k] = 0.0f;
+        }
+      }
+    }
+    if (RNG) {
+      // the noise of the pass is worked out while its loads are in flight
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) {
+        const int64_t i = i0 + it * stride;
+        if (i < nvec) {
+          rng_normals<VEC>(A.rng_key, (uint64_t)((A.rng_row0 + row) * D + i * VEC), 0u, t[it]);
+          if (A.noise_out) Vec<float, VEC>::store(A.noise_out + row * A.stride_noise_out + i * VEC, t[it]);
         }
       }
     }
@@ -296,9 +315,9 @@ __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRow
   UNIRL_TRACE_END(A.trace);
 }
 
-template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING>
+template <typename TV, typename TX, int VEC, int ITEMS, bool SAMPLING, bool RNG = false>
 __global__ __launch_bounds__(kSdeThreads) void sde_step_kernel(SdeStepArgs A) {
-  sde_step_body<TV, TX, VEC, ITEMS, SAMPLING, false>(A, nullptr);
+  sde_step_body<TV, TX, VEC, ITEMS, SAMPLING, false, false, RNG>(A, nullptr);
 }
 
 // The replay of S recorded steps per sample as one launch over the (sample, step) rows.
@@ -602,8 +621,16 @@ struct SdeRolloutArgs {
   int items;               // host only: vectors per lane (one pass covers a sample)
 };
 
-template <typename TV, typename TX, int VEC, int ITEMS>
-__global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs A) {
+// What the drawing variant of the rollout kernel needs beside SdeRolloutArgs.
+struct SdeRolloutRng {
+  RngKey key;
+  int64_t row0;                                  // index of the launch's first sample within the call
+  unsigned char draw[UNIRL_MAX_ROLLOUT_STEPS];   // the step's noise is drawn in the kernel
+  float* n_out[UNIRL_MAX_ROLLOUT_STEPS];         // where a step's drawn noise is stored, or null
+};
+
+template <typename TV, typename TX, int VEC, int ITEMS, bool RNG>
+__device__ __forceinline__ void sde_rollout_body(const SdeRolloutArgs& A, const SdeRolloutRng* G) {
   constexpr int NW = kSdeThreads / kWave;
   __shared__ double lds_q[UNIRL_MAX_ROLLOUT_STEPS][NW];
   __shared__ SdeCoef lds_c[UNIRL_MAX_ROLLOUT_STEPS];
@@ -649,9 +676,20 @@ __global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs
         Vec<TV, VEC>::load(vp + i * VEC, v[it]);
         if (np) {
           Vec<float, VEC>::load(np + i * VEC, n[it]);
-        } else {
+        } else if (!RNG || !G->draw[k]) {
 #pragma unroll
           for (int e = 0; e < VEC; ++e) n[it][e] = 0.0f;
+        }
+      }
+    }
+    if (RNG && G->draw[k]) {  // wave-uniform: the step's noise, worked out while its velocity loads are in flight
+      float* __restrict__ no = G->n_out[k] ? G->n_out[k] + b * D : nullptr;
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) {
+        const int64_t i = i_first + it * stride;
+        if (i < nvec) {
+          rng_normals<VEC>(G->key, (uint64_t)((G->row0 + b) * D + i * VEC), (uint32_t)k, n[it]);
+          if (no) Vec<float, VEC>::store(no + i * VEC, n[it]);
         }
       }
     }
@@ -699,6 +737,16 @@ __global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs
       A.partials[((int64_t)b * S + threadIdx.x) * nblk + blockIdx.x] = q;  // summed by sde_rollout_finalize_kernel
     }
   }
+}
+
+template <typename TV, typename TX, int VEC, int ITEMS>
+__global__ __launch_bounds__(kSdeThreads) void sde_rollout_kernel(SdeRolloutArgs A) {
+  sde_rollout_body<TV, TX, VEC, ITEMS, false>(A, nullptr);
+}
+// The same with the noise of some (or all) steps drawn in the kernel.
+template <typename TV, typename TX, int VEC, int ITEMS>
+__global__ __launch_bounds__(kSdeThreads) void sde_rollout_rng_kernel(SdeRolloutArgs A, SdeRolloutRng G) {
+  sde_rollout_body<TV, TX, VEC, ITEMS, true>(A, &G);
 }
 
 // One wavefront per (sample, step).
@@ -766,31 +814,32 @@ static int launch_step_finalize(const SdeStepArgs& A, int64_t rows, unsigned int
   return (int)hipGetLastError();
 }
 
-template <typename TV, typename TX, bool SAMPLING>
+template <typename TV, typename TX, bool SAMPLING, bool RNG = false>
 static int launch_step(const SdeStepArgs& A, int64_t B, int vec, hipStream_t st) {
   const int items = A.items;
   dim3 grid(A.nblk, (unsigned int)B), block(kSdeThreads);
   if (vec == 8) {
     // sixteen-byte accesses on the 16-bit operands; only built where there is one
     if constexpr (sizeof(TV) == 2 || sizeof(TX) == 2)
-      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 8, 2, SAMPLING>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 8, 2, SAMPLING, RNG>), grid, block, 0, st, A);
     else
       return UNIRL_E_DTYPE;
   } else if (vec == 4) {
-    if (items >= 4)
-      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 4, SAMPLING>), grid, block, 0, st, A);
+    if (items >= 4 || RNG)  // the drawing variant is built for four vectors per lane only
+      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 4, SAMPLING, RNG>), grid, block, 0, st, A);
     else if (items >= 2)
-      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 2, SAMPLING>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 2, SAMPLING, false>), grid, block, 0, st, A);
     else
-      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 1, SAMPLING>), grid, block, 0, st, A);
+      hipLaunchKernelGGL((sde_step_kernel<TV, TX, 4, 1, SAMPLING, false>), grid, block, 0, st, A);
   } else {
-    hipLaunchKernelGGL((sde_step_kernel<TV, TX, 1, 2, SAMPLING>), grid, block, 0, st, A);
+    hipLaunchKernelGGL((sde_step_kernel<TV, TX, 1, 2, SAMPLING, RNG>), grid, block, 0, st, A);
   }
   return (int)hipGetLastError();
 }
 
 template <typename TV, typename TX>
 static int launch_step_mode(const SdeStepArgs& A, int64_t B, int vec, bool sampling, hipStream_t st) {
+  if (sampling && A.rng) return launch_step<TV, TX, true, true>(A, B, vec, st);
   return sampling ? launch_step<TV, TX, true>(A, B, vec, st) : launch_step<TV, TX, false>(A, B, vec, st);
 }
 
@@ -981,33 +1030,34 @@ static int plan_replay(const unirl_sde_replay_desc* d, const void* extra_f32_a, 
 }
 
 template <typename TV, typename TX>
-static int launch_rollout(const SdeRolloutArgs& A, int64_t B, int vec, hipStream_t st) {
+static int launch_rollout(const SdeRolloutArgs& A, const SdeRolloutRng* G, int64_t B, int vec, hipStream_t st) {
   dim3 grid(A.nblk, (unsigned int)B), block(kSdeThreads);
   const int items = A.items;
+#define UNIRL_LAUNCH_ROLLOUT(VEC, ITEMS)                                                                   \
+  do {                                                                                                     \
+    if (G) hipLaunchKernelGGL((sde_rollout_rng_kernel<TV, TX, VEC, ITEMS>), grid, block, 0, st, A, *G);    \
+    else hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, VEC, ITEMS>), grid, block, 0, st, A);              \
+  } while (0)
   if (vec == 4) {
-    if (items >= 4)
-      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 4, 4>), grid, block, 0, st, A);
-    else if (items == 2)
-      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 4, 2>), grid, block, 0, st, A);
-    else
-      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 4, 1>), grid, block, 0, st, A);
+    if (items >= 4) UNIRL_LAUNCH_ROLLOUT(4, 4);
+    else if (items == 2) UNIRL_LAUNCH_ROLLOUT(4, 2);
+    else UNIRL_LAUNCH_ROLLOUT(4, 1);
   } else {
-    if (items >= 4)
-      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 1, 4>), grid, block, 0, st, A);
-    else if (items == 2)
-      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 1, 2>), grid, block, 0, st, A);
-    else
-      hipLaunchKernelGGL((sde_rollout_kernel<TV, TX, 1, 1>), grid, block, 0, st, A);
+    if (items >= 4) UNIRL_LAUNCH_ROLLOUT(1, 4);
+    else if (items == 2) UNIRL_LAUNCH_ROLLOUT(1, 2);
+    else UNIRL_LAUNCH_ROLLOUT(1, 1);
   }
+#undef UNIRL_LAUNCH_ROLLOUT
   return (int)hipGetLastError();
 }
 
 template <typename TV>
-static int launch_rollout_x(const SdeRolloutArgs& A, int dtype_x, int64_t B, int vec, hipStream_t st) {
+static int launch_rollout_x(const SdeRolloutArgs& A, const SdeRolloutRng* G, int dtype_x, int64_t B, int vec,
+                            hipStream_t st) {
   switch (dtype_x) {
-    case UNIRL_F32: return launch_rollout<TV, float>(A, B, vec, st);
-    case UNIRL_BF16: return launch_rollout<TV, bf16_t>(A, B, vec, st);
-    case UNIRL_F16: return launch_rollout<TV, f16_t>(A, B, vec, st);
+    case UNIRL_F32: return launch_rollout<TV, float>(A, G, B, vec, st);
+    case UNIRL_BF16: return launch_rollout<TV, bf16_t>(A, G, B, vec, st);
+    case UNIRL_F16: return launch_rollout<TV, f16_t>(A, G, B, vec, st);
   }
   return UNIRL_E_DTYPE;
 }
@@ -1045,11 +1095,15 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
   if (!sampling && d->prev_sample.dtype != dtype_x) return UNIRL_E_DTYPE;
   const bool want_logp = (d->logp_out != nullptr) && !(d->eta < 1e-7);
   if (want_logp && (!workspace || workspace_bytes < kWorkspaceBytes)) return UNIRL_E_WORKSPACE;
+  // noise drawn in the kernel: sampling, no noise tensor given, a stochastic step
+  const bool draw = sampling && d->rng.enabled && !d->noise && !(d->eta < 1e-7);
+  const int64_t stride_no = d->noise_out_stride ? d->noise_out_stride : D;
+  if (draw && d->noise_out && stride_no < D) return UNIRL_E_SHAPE;
   const size_t sv = dtype_size(dtype_v), sx = dtype_size(dtype_x);
   const size_t spo = d->prev_out ? dtype_size(d->prev_dtype) : 4, smo = d->mean_out ? dtype_size(d->mean_dtype) : 4;
   if (!aligned_to(noise_pred, sv) || !aligned_to(sample, sx) || !aligned_to(prev_sample, sx) ||
       !aligned_to(d->noise, 4) || !aligned_to(d->prev_out, spo) || !aligned_to(d->mean_out, smo) ||
-      !aligned_to(d->logp_out, 4))
+      !aligned_to(d->logp_out, 4) || (draw && !aligned_to(d->noise_out, 4)))
     return UNIRL_E_ALIGN;
 
   // 4-element vectors need every per-sample base to keep the vector alignment.
@@ -1057,7 +1111,8 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
   if (D % 4 != 0 || !aligned_to(noise_pred, 4 * sv) || !aligned_to(sample, 4 * sx) ||
       !aligned_to(prev_sample, 4 * sx) || !aligned_to(d->noise, 16) || !aligned_to(d->prev_out, 4 * spo) ||
       !aligned_to(d->mean_out, 4 * smo) || stride_v % 4 || stride_x % 4 || (!sampling && stride_p % 4) ||
-      (sampling && d->noise && stride_n % 4) || (d->prev_out && stride_po % 4) || (d->mean_out && stride_mo % 4))
+      (sampling && d->noise && stride_n % 4) || (d->prev_out && stride_po % 4) || (d->mean_out && stride_mo % 4) ||
+      (draw && d->noise_out && (stride_no % 4 || !aligned_to(d->noise_out, 16))))
     vec = 1;
 
   // 16-bit operands: eight elements per lane make their accesses sixteen bytes too, while an
@@ -1077,6 +1132,7 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
     visit(noise_pred, sv, stride_v);
     visit(sample, sx, stride_x);
     if (sampling) visit(d->noise, 4, stride_n); else visit(prev_sample, sx, stride_p);
+    if (draw) visit(d->noise_out, 4, stride_no);
     visit(d->prev_out, spo, stride_po);
     visit(d->mean_out, smo, stride_mo);
     if (ok && narrow >= wide) vec = 8;
@@ -1088,7 +1144,7 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
 
   for (int64_t b0 = 0; b0 < B; b0 += per_launch) {
     const int64_t nb = (B - b0 < per_launch) ? (B - b0) : per_launch;
-    SdeStepArgs A;
+    SdeStepArgs A = {};
     A.v = offset_ptr(noise_pred, b0 * stride_v, sv);
     A.x = offset_ptr(sample, b0 * stride_x, sx);
     A.third = sampling ? (const void*)offset_f32(d->noise, b0 * stride_n) : offset_ptr(prev_sample, b0 * stride_p, sx);
@@ -1116,6 +1172,14 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
     A.partials = ws_partials(workspace);
     A.nblk = nblk;
     A.items = items;
+    if (draw) {
+      A.rng = 1;
+      A.rng_key = RngKey{(uint32_t)d->rng.seed, (uint32_t)(d->rng.seed >> 32), (uint32_t)d->rng.offset,
+                         (uint32_t)(d->rng.offset >> 32)};
+      A.rng_row0 = b0;
+      A.noise_out = offset_f32(d->noise_out, b0 * stride_no);
+      A.stride_noise_out = stride_no;
+    }
     UNIRL_TRACE_SET(A, "sde_step", nblk * (unsigned int)nb);
     int rc = UNIRL_E_DTYPE;
     switch (dtype_v) {
@@ -1452,7 +1516,8 @@ extern "C" int unirl_sde_step_logp_bwd(const void* noise_pred, int dtype_v, cons
 }
 
 extern "C" int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* const* v_steps, int dtype_v,
-                                      const float* const* noise_steps, const float* sigmas, const double* etas,
+                                      const float* const* noise_steps, const unirl_rng* rng,
+                                      float* const* noise_out_steps, const float* sigmas, const double* etas,
                                       int S, const float* sigma_max_ptr, float sigma_max_val, int kind, int64_t B,
                                       int64_t D, float* x_out, float* traj_out, float* logp_out, int logp_sum,
                                       void* workspace, size_t workspace_bytes, void* stream) {
@@ -1461,7 +1526,8 @@ extern "C" int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* c
   if (B < 0 || D <= 0 || S < 1) return UNIRL_E_SHAPE;
   if (S > UNIRL_MAX_ROLLOUT_STEPS) return UNIRL_E_LIMIT;
   if (B == 0) return UNIRL_OK;
-  if (!x0 || !x_out || !logp_out || !v_steps || !noise_steps || !sigmas || !etas) return UNIRL_E_NULL;
+  const bool has_rng = rng && rng->enabled;
+  if (!x0 || !x_out || !logp_out || !v_steps || (!noise_steps && !has_rng) || !sigmas || !etas) return UNIRL_E_NULL;
   if (!workspace || workspace_bytes < kWorkspaceBytes) return UNIRL_E_WORKSPACE;
   const size_t sv = dtype_size(dtype_v), sx = dtype_size(dtype_x);
   if (!aligned_to(x0, sx) || !aligned_to(x_out, 4) || !aligned_to(traj_out, 4)) return UNIRL_E_ALIGN;
@@ -1470,8 +1536,10 @@ extern "C" int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* c
   if (D % 4 != 0 || !aligned_to(x0, 4 * sx) || !aligned_to(x_out, 16) || !aligned_to(traj_out, 16)) vec = 1;
   for (int k = 0; k < S; ++k) {
     if (!v_steps[k]) return UNIRL_E_NULL;
-    if (!aligned_to(v_steps[k], sv) || !aligned_to(noise_steps[k], 4)) return UNIRL_E_ALIGN;
-    if (!aligned_to(v_steps[k], 4 * sv) || !aligned_to(noise_steps[k], 16)) vec = 1;
+    const float* nz = noise_steps ? noise_steps[k] : nullptr;
+    const float* no = (has_rng && noise_out_steps) ? noise_out_steps[k] : nullptr;
+    if (!aligned_to(v_steps[k], sv) || !aligned_to(nz, 4) || !aligned_to(no, 4)) return UNIRL_E_ALIGN;
+    if (!aligned_to(v_steps[k], 4 * sv) || !aligned_to(nz, 16) || !aligned_to(no, 16)) vec = 1;
   }
 
   // One pass must cover a sample (the latent lives in registers): pick the
@@ -1491,12 +1559,23 @@ extern "C" int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* c
   for (int64_t b0 = 0; b0 < B; b0 += per_launch) {
     const int64_t nb = (B - b0 < per_launch) ? (B - b0) : per_launch;
     const int64_t off = b0 * D;
-    SdeRolloutArgs A;
+    SdeRolloutArgs A = {};
+    SdeRolloutRng G = {};
+    bool any_draw = false;
     for (int k = 0; k < S; ++k) {
       A.v[k] = offset_ptr(v_steps[k], off, sv);
-      A.n[k] = offset_f32(noise_steps[k], off);
+      A.n[k] = offset_f32(noise_steps ? noise_steps[k] : nullptr, off);
       A.sc[k] = make_scalars(etas[k]);
       A.want_logp[k] = !(etas[k] < 1e-7);
+      // a stochastic step without a noise tensor draws its noise when a generator is given
+      G.draw[k] = (has_rng && !A.n[k] && A.want_logp[k]) ? 1 : 0;
+      G.n_out[k] = (G.draw[k] && noise_out_steps) ? offset_f32(noise_out_steps[k], off) : nullptr;
+      any_draw = any_draw || G.draw[k];
+    }
+    if (has_rng) {
+      G.key = RngKey{(uint32_t)rng->seed, (uint32_t)(rng->seed >> 32), (uint32_t)rng->offset,
+                     (uint32_t)(rng->offset >> 32)};
+      G.row0 = b0;
     }
     A.x0 = offset_ptr(x0, off, sx);
     A.sigmas = sigmas;
@@ -1515,9 +1594,9 @@ extern "C" int unirl_sde_rollout_logp(const void* x0, int dtype_x, const void* c
     A.items = items;
     int rc = UNIRL_E_DTYPE;
     switch (dtype_v) {
-      case UNIRL_F32: rc = launch_rollout_x<float>(A, dtype_x, nb, vec, st); break;
-      case UNIRL_BF16: rc = launch_rollout_x<bf16_t>(A, dtype_x, nb, vec, st); break;
-      case UNIRL_F16: rc = launch_rollout_x<f16_t>(A, dtype_x, nb, vec, st); break;
+      case UNIRL_F32: rc = launch_rollout_x<float>(A, any_draw ? &G : nullptr, dtype_x, nb, vec, st); break;
+      case UNIRL_BF16: rc = launch_rollout_x<bf16_t>(A, any_draw ? &G : nullptr, dtype_x, nb, vec, st); break;
+      case UNIRL_F16: rc = launch_rollout_x<f16_t>(A, any_draw ? &G : nullptr, dtype_x, nb, vec, st); break;
     }
     if (rc != 0) return rc;
     if (nblk > 1) {

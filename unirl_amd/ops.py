@@ -74,18 +74,34 @@ def sde_step_logp(
     want_mean: bool = True,
     want_logp: bool = True,
     logp_sum: bool = False,
+    rng: Optional[Tuple[int, int]] = None,
 ) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor], Optional[torch.Tensor]]:
     """One fused SDE transition. Returns ``(prev f32, logp [B] f32 or None, mean f32)``.
 
     ``prev_sample`` given = replay, else sampling with ``noise`` (f32, same shape;
-    ``None`` adds no noise).  ``sample.dtype`` is the dtype of the round trip applied
-    to ``prev`` before the log-prob.
+    ``None`` adds no noise, or -- with ``rng = (seed, offset)`` -- standard normal noise drawn
+    inside the kernel: no noise tensor is written or read).  ``sample.dtype`` is the dtype of the
+    round trip applied to ``prev`` before the log-prob.
     """
     if sample.dim() < 2:
         raise ValueError(f"sample needs a batch dimension and at least one more; got {tuple(sample.shape)}")
     if noise_pred.shape != sample.shape:
         raise ValueError(f"noise_pred {tuple(noise_pred.shape)} != sample {tuple(sample.shape)}")
     device = sample.device
+    if rng is not None and prev_sample is None and noise is None:
+        # the generator rides in the descriptor of the strided entry point; the outputs are fresh fp32 tensors
+        B = sample.shape[0]
+        logp_wanted = want_logp and not (eta < 1e-7)
+        prev_out = torch.empty(sample.shape, dtype=torch.float32, device=device) if want_prev else None
+        mean_out = torch.empty(sample.shape, dtype=torch.float32, device=device) if want_mean else None
+        logp_out = torch.empty(B, dtype=torch.float32, device=device) if logp_wanted else None
+        if B == 0 or sample.numel() == 0:
+            if logp_out is not None:
+                logp_out.fill_(float("nan"))
+            return prev_out, logp_out, mean_out
+        sde_step_logp_into(noise_pred, sample, sigma, sigma_next, kind=kind, eta=eta, sigma_max=sigma_max,
+                           prev_out=prev_out, mean_out=mean_out, logp_out=logp_out, logp_sum=logp_sum, rng=rng)
+        return prev_out, logp_out, mean_out
     v = _kernel_dtype(_flat2(noise_pred, "noise_pred"))
     x = _kernel_dtype(_flat2(sample, "sample"))
     B = x.shape[0]
@@ -168,9 +184,16 @@ def sde_step_logp_into(
     mean_out: Optional[torch.Tensor] = None,
     logp_out: Optional[torch.Tensor] = None,
     logp_sum: bool = False,
+    rng: Optional[Tuple[int, int]] = None,
+    noise_out: Optional[torch.Tensor] = None,
 ) -> None:
     """One fused SDE transition that reads strided ``[B, ...]`` views in place and writes into
     caller-owned views (``unirl_sde_step_logp_ex``), no gradient.
+
+    Sampling without a ``noise`` tensor and with ``rng = (seed, offset)`` draws the noise inside the
+    kernel (Philox-4x32-10 keyed by ``seed``, counter ``(element index / 4, offset)``, Box-Muller):
+    the draw of an element depends on nothing but ``(seed, offset, element index)``.  ``noise_out``
+    (fp32, ``sample``'s shape) receives it when given.
 
     ``sample`` / ``prev_sample`` may be ``stack[:, k]`` slices of a ``[B, K, ...]`` trajectory in
     fp32, bf16 or fp16; ``prev_out`` / ``mean_out`` may be slices of such stacks in any of the
@@ -250,6 +273,13 @@ def sde_step_logp_into(
     d.prev_out, d.prev_dtype, d.prev_stride = N.ptr(po), (N.dtype_code(po.dtype) if po is not None else 0), spo
     d.mean_out, d.mean_dtype, d.mean_stride = N.ptr(mo), (N.dtype_code(mo.dtype) if mo is not None else 0), smo
     d.logp_out, d.logp_stride, d.logp_sum = N.ptr(lp), slp, int(bool(logp_sum))
+    if rng is not None and prev_sample is None and noise is None:
+        d.rng = N.Rng(1, int(rng[0]) & 0xFFFFFFFFFFFFFFFF, int(rng[1]) & 0xFFFFFFFFFFFFFFFF)
+        if noise_out is not None:
+            if noise_out.dtype != torch.float32 or tuple(noise_out.shape) != tuple(sample.shape) or noise_out.device != device:
+                raise ValueError(f"noise_out must be float32 {tuple(sample.shape)} on {device}")
+            no, sno = _per_sample_view(noise_out, "noise_out", writable=True)
+            d.noise_out, d.noise_out_stride = N.ptr(no), sno
     ws, ws_bytes = N.workspace(device)
     with N.on_device(device):
         rc = N.F.unirl_sde_step_logp_ex(ctypes.byref(d), N.ptr(ws), ws_bytes, N.current_stream(device))
@@ -516,17 +546,26 @@ def sde_rollout_logp(
     sigma_max: Union[float, torch.Tensor, None] = None,
     want_trajectory: bool = False,
     logp_sum: bool = False,
+    rng: Optional[Tuple[int, int]] = None,
+    noise_out: Optional[Sequence[Optional[torch.Tensor]]] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
     """``S = len(velocities)`` chained transitions in one launch.
 
     Step ``k`` moves ``sigmas[k] -> sigmas[k+1]`` with ``velocities[k]``, ``noises[k]``
     and ``etas[k]``.  ``sigma_max=None`` takes ``sigmas[1]`` like the reference's stage
-    loop.  Returns ``(x_final f32, logp [B,S] f32 (NaN where eta<1e-7), trajectory
-    [S,B,...] f32 or None)``.
+    loop.  With ``rng = (seed, offset)`` a stochastic step whose ``noises[k]`` is ``None`` (or all
+    of them: ``noises=None``) draws its noise inside the kernel, step ``k`` with ``offset + k`` --
+    the draws of ``k`` single steps called with those offsets; ``noise_out[k]`` (fp32, ``x0``'s
+    shape) receives a step's drawn noise when given.  Returns ``(x_final f32, logp [B,S] f32 (NaN
+    where eta<1e-7), trajectory [S,B,...] f32 or None)``.
     """
     S = len(velocities)
     if S < 1 or S > N.MAX_ROLLOUT_STEPS:
         raise ValueError(f"number of steps must be in [1, {N.MAX_ROLLOUT_STEPS}]; got {S}")
+    if noises is None:
+        if rng is None:
+            raise ValueError("noises=None needs rng=(seed, offset)")
+        noises = [None] * S
     if len(noises) != S:
         raise ValueError(f"{S} velocities but {len(noises)} noises")
     if isinstance(etas, (int, float)):
@@ -574,10 +613,21 @@ def sde_rollout_logp(
     v_arr = (ctypes.c_void_p * S)(*[t.data_ptr() for t in vs])
     n_arr = (ctypes.c_void_p * S)(*[(t.data_ptr() if t is not None else None) for t in ns])
     e_arr = (ctypes.c_double * S)(*[float(e) for e in etas])
+    rng_s, no_arr = None, None
+    if rng is not None:
+        rng_s = ctypes.byref(N.Rng(1, int(rng[0]) & 0xFFFFFFFFFFFFFFFF, int(rng[1]) & 0xFFFFFFFFFFFFFFFF))
+        if noise_out is not None:
+            if len(noise_out) != S:
+                raise ValueError(f"{S} steps but {len(noise_out)} noise_out entries")
+            for k, t in enumerate(noise_out):
+                if t is not None and (t.dtype != torch.float32 or tuple(t.shape) != tuple(x0.shape) or not t.is_contiguous()
+                                      or t.device != device):
+                    raise ValueError(f"noise_out[{k}] must be a contiguous float32 tensor of x0's shape on {device}")
+            no_arr = (ctypes.c_void_p * S)(*[(t.data_ptr() if t is not None else None) for t in noise_out])
     ws, ws_bytes = N.workspace(device)
     with N.on_device(device):
         rc = N.F.unirl_sde_rollout_logp(
-            N.ptr(x), N.dtype_code(x.dtype), v_arr, N.dtype_code(vdtype), n_arr, N.ptr(sig), e_arr, S,
+            N.ptr(x), N.dtype_code(x.dtype), v_arr, N.dtype_code(vdtype), n_arr, rng_s, no_arr, N.ptr(sig), e_arr, S,
             N.ptr(smax_t), smax_v, SDE_KINDS[kind], B, D, N.ptr(x_out), N.ptr(traj), N.ptr(logp),
             int(bool(logp_sum)), N.ptr(ws), ws_bytes, N.current_stream(device),
         )

@@ -109,6 +109,22 @@ class _SdeReplayFn(torch.autograd.Function):
         return (grad_v,) + (None,) * 9
 
 
+def next_rng(device: torch.device) -> Optional[Tuple[int, int]]:
+    """``(seed, offset)`` for one in-kernel noise draw, taken from -- and advancing -- the device's
+    default torch generator, so that ``torch.manual_seed`` governs the sampling noise as it governs
+    ``torch.randn``: same seed, same sequence of calls, same noise.  (The kernel keys its own
+    Philox stream with the seed; torch's offset is only the counter that tells calls apart.)
+    ``None`` while a HIP graph is being captured: the generator's state then belongs to the graph."""
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    gen = torch.cuda.default_generators[index]
+    offset = gen.get_offset()
+    gen.set_offset(offset + 4)  # torch keeps its offsets multiples of four
+    # another key than torch's own kernels use with this seed: the two streams never meet
+    return (gen.initial_seed() ^ 0x9E3779B97F4A7C15) & 0xFFFFFFFFFFFFFFFF, offset
+
+
 class StepStrategy(ABC):
     """Base class of all sampling step strategies."""
 
@@ -164,10 +180,17 @@ class StepStrategy(ABC):
                 f"{type(self).__name__}.denoise: sample lives on {sample.device}; the fused SDE kernel "
                 "runs on a HIP device only and there is no CPU fallback"
             )
-        if prev_sample is None and noise is None and float(eta) != 0.0:
-            # the reference draws with generator=None on noise_pred's device, in fp32
-            noise = torch.randn(sample.shape, device=sample.device, dtype=torch.float32)
         needs_grad = torch.is_grad_enabled() and (noise_pred.requires_grad or sample.requires_grad)
+        rng = None
+        if prev_sample is None and noise is None and float(eta) != 0.0:
+            # The reference draws with generator=None on noise_pred's device, in fp32
+            # (unirl/sde/kernels.py:230-232).  Here the kernel draws the noise itself from the device's
+            # default generator state (seed, offset) -- no noise tensor is written and read back --
+            # except under autograd, whose backward wants the noise tensor, and under graph capture,
+            # where the generator's state is the graph's business.
+            rng = None if needs_grad else next_rng(sample.device)
+            if rng is None:
+                noise = torch.randn(sample.shape, device=sample.device, dtype=torch.float32)
         # fp32 replay: the reference's .float() / .to(float32) round trip is the identity, so the
         # caller's own tensor is handed back and the kernel need not write a copy of it
         reuse_prev = (
@@ -182,7 +205,7 @@ class StepStrategy(ABC):
         else:
             prev, logp, mean = ops.sde_step_logp(
                 noise_pred, sample, sigma, sigma_next, kind=kind, eta=float(eta), prev_sample=prev_sample,
-                noise=noise, sigma_max=sigma_max, want_prev=not reuse_prev,
+                noise=noise, sigma_max=sigma_max, want_prev=not reuse_prev, rng=rng,
             )
         if reuse_prev:
             prev = prev_sample
@@ -222,11 +245,14 @@ class StepStrategy(ABC):
                 f"{type(self).__name__}.denoise_into: sample lives on {sample.device}; the fused SDE kernel "
                 "runs on a HIP device only and there is no CPU fallback"
             )
+        rng = None
         if prev_sample is None and noise is None and float(eta) != 0.0:
-            noise = torch.randn(sample.shape, device=sample.device, dtype=torch.float32)
+            rng = next_rng(sample.device)  # the kernel draws the noise itself (see denoise)
+            if rng is None:
+                noise = torch.randn(sample.shape, device=sample.device, dtype=torch.float32)
         ops.sde_step_logp_into(
             noise_pred, sample, sigma, sigma_next, kind=self._kind, eta=float(eta), prev_sample=prev_sample,
-            noise=noise, sigma_max=sigma_max, prev_out=prev_out, mean_out=mean_out, logp_out=logp_out,
+            noise=noise, sigma_max=sigma_max, prev_out=prev_out, mean_out=mean_out, logp_out=logp_out, rng=rng,
         )
         return not (eta < 1e-7)
 
