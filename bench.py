@@ -617,6 +617,33 @@ def head_probe(torch, dev, vocab: int, hidden: int = 2560, row_counts=(64, 256, 
     return out
 
 
+def head_counters_probe(torch, dev, vocab: int, rows: int = 8192, hidden: int = 2560, calls: int = 6):
+    """The command the matrix-core counters are collected on (`rocprofv3 --pmc ... -- python3 bench.py
+    --head-counters-probe`): after a spin-up that brings the device to its sustained clocks, `calls`
+    back-to-back calls of the fused lm_head kernel, then `calls` of the library GEMM on the same
+    operands (`linear(h, w)`: the kernel the fused one is measured against).  Cycle counters of the two
+    kernels divided by their durations give the shader clock each one ran at."""
+    from unirl_amd import ops
+
+    g = torch.Generator(device=dev).manual_seed(0)
+    w = (torch.randn(vocab, hidden, generator=g, device=dev) * (3.0 / math.sqrt(hidden))).bfloat16()
+    h = torch.randn(rows, hidden, generator=g, device=dev).bfloat16()
+    ids = torch.randint(0, vocab, (rows,), generator=g, device=dev)
+    t_end = time.perf_counter() + 0.5
+    while time.perf_counter() < t_end:
+        ops.lmhead_logp(h, w, None, ids, 1.0, want_entropy=True, want_lse=True)
+        torch.nn.functional.linear(h, w)
+        torch.cuda.synchronize()
+    for _ in range(calls):
+        ops.lmhead_logp(h, w, None, ids, 1.0, want_entropy=True, want_lse=True)
+    torch.cuda.synchronize()
+    for _ in range(calls):
+        torch.nn.functional.linear(h, w)
+    torch.cuda.synchronize()
+    return {"rows": rows, "vocab": vocab, "hidden": hidden, "calls_each": calls,
+            "flop_per_call": 2.0 * rows * hidden * vocab}
+
+
 def tail_probe(torch, dev):
     """What finishing a grid-wide reduction costs after its streaming part, at the byte counts of the
     three small reducing shapes: the streaming kernel alone, plus a dependent second launch (the
@@ -770,6 +797,9 @@ def main() -> int:
                     help="device-side timeline (launch gaps, kernel bodies) of the small shapes inside the 64-launch "
                          "graph, from the measurement build's own clock readings; optional comma-separated shape "
                          "names; needs `python -m unirl_amd.build --tune`")
+    ap.add_argument("--head-counters-probe", action="store_true",
+                    help="spin up, then 6 calls of the fused lm_head kernel and 6 of the library GEMM at 8192 rows: "
+                         "the command the matrix-core cycle counters are collected on")
     ap.add_argument("--head-probe", action="store_true",
                     help="the fused lm_head + log-softmax kernel (logits never written) against the library GEMM + "
                          "token kernel for a bf16 Linear(2560, --vocab) head at 64 / 2048 / 8192 rows, then exit")
@@ -808,6 +838,10 @@ def main() -> int:
     if args.timeline is not None:
         names = [n for n in args.timeline.split(",") if n]
         print(json.dumps({"timeline": timeline_probe(torch, dev, names)}), flush=True)
+        return 0
+
+    if args.head_counters_probe:
+        print(json.dumps({"head_counters_probe": head_counters_probe(torch, dev, args.vocab)}), flush=True)
         return 0
 
     if args.head_probe:
