@@ -82,6 +82,7 @@ struct RatioConsts {
   float drpo_eps;            // (float)epsilon
   float drpo_two_eps;        // (float)(2.0 * epsilon)
   float inv_two_eps;         // 1 / drpo_two_eps, correctly rounded
+  float inv_eps;             // 1 / drpo_eps, correctly rounded
   float horizon;
   // DRPO, token-adaptive boundary: with epsilon >= 1 a token with mu <= 1 and r <= fast_hi =
   // fl(1 + epsilon) can be on neither side of its trust region (see drpo_flags_provably_clear)
@@ -111,6 +112,7 @@ struct RatioArgs {
   float loss_scale;      // gradient arriving at the aggregated loss
   int64_t n_valid_host;  // token-mean denominator when the host knows it, else < 0
   int64_t per_wave;      // packed kernel: vectors in a wavefront's run (a multiple of 64)
+  double inv_seq_scale;  // sequence-mean modes: 1 / n_seq or 1 / (n_seq * horizon), the loss's factor
   UNIRL_TRACE_FIELD
 #ifdef UNIRL_TUNE
   int synth_len;  // timing experiment: row lengths from a hash of the row instead of the load
@@ -313,7 +315,7 @@ __device__ __forceinline__ float accumulate_token(float nw, float od, float A, f
     acc.pen += pen;
     if (GRAD) {
       const bool clamped = (d0 < -20.0f) || (d0 > 20.0f);
-      dl = clamped ? 0.0f : ((-A) + (fabsf(A) * w) * d / C.drpo_eps) * r;
+      dl = clamped ? 0.0f : ((-A) + div_by_const((fabsf(A) * w) * d, C.drpo_eps, C.inv_eps)) * r;
     }
   }
   acc.loss += loss * lw;
@@ -1010,27 +1012,30 @@ __global__ __launch_bounds__(kFinThreads) void ratio_loss_finalize_kernel(RatioA
   const int v = t;
   const double N = lds_tot[P_CNT], sr = lds_tot[P_SR], sr2 = lds_tot[P_SR2], sab = lds_tot[P_ABS];
   const double x = lds_tot[v];
-  // One fp64 reciprocal serves every mean: x * (1/N) and x / N differ by at most an ulp of fp64,
-  // far below the fp32 result's rounding.
-  const double inv_n = 1.0 / N;
+  // One reciprocal serves every mean.  N is a whole number below 2^32: the hardware's fp32
+  // reciprocal refined by two Newton steps in fp64 is within an ulp of fp64's 1/N (the error
+  // squares twice from 2^-23), far below the fp32 result's rounding, at a third of the division's
+  // instructions.  N = 0 gives inf * 0 = NaN in the step; the estimate (inf) is kept, as 1.0 / 0.
+  const double r0 = (double)__builtin_amdgcn_rcpf((float)N);
+  const double r1 = fma(fma(-N, r0, 1.0), r0, r0);
+  const double r2 = fma(fma(-N, r1, 1.0), r1, r1);
+  const double inv_n = (r2 == r2) ? r2 : r0;
   double loss_scale = inv_n;
-  if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_SUM)
-    loss_scale = 1.0 / ((double)A.n_seq * (double)C.horizon);
-  else if (C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_MEAN)
-    loss_scale = 1.0 / (double)A.n_seq;
-  // sr, sr2: sums of (r-1) and (r-1)^2
-  double var = 0.0;
+  if (C.agg_mode != UNIRL_AGG_TOKEN_MEAN) loss_scale = (double)A.inv_seq_scale;
+  // sr, sr2: sums of (r-1) and (r-1)^2.  The numerator cancels, so it is formed in fp64; the
+  // quotient and the root are fp32 operations on an fp32 result.
+  float sd = 0.0f;
   if (N > 1.0) {
-    var = (sr2 - sr * sr * inv_n) / (N - 1.0);
-    if (var < 0.0) var = 0.0;
+    const double num = sr2 - sr * sr * inv_n;
+    sd = sqrtf(fmaxf((float)num, 0.0f) / (float)(N - 1.0));
+    if (num != num) sd = quiet_nan();  // fmaxf would drop it
   }
-  const double sd = sqrt(var);
   double y = x * inv_n;  // the means: penalty, |new-old|, the three clip fractions
   if (v == P_SR) y = 1.0 + y;
   // GRPO accumulates ld^2; mean(0.5*ld^2) = 0.5*sum/N exactly (halving commutes with rounding)
   if (v == P_KL && C.kind == UNIRL_LOSS_GRPO) y = 0.5 * y;
   if (v == P_LOSS) y = x * loss_scale;
-  if (v == P_SR2) y = sd;
+  if (v == P_SR2) y = (double)sd;
   if (v == P_CNT) y = x;
   // min()/max() of the reference return NaN when any ratio is NaN; the ratios are >= 0, so their
   // sum is NaN exactly then (likewise the absolute differences)
@@ -1158,6 +1163,7 @@ static int fill_consts(const unirl_ratio_loss_params* p, RatioConsts& C) {
   C.drpo_eps = (float)p->drpo_epsilon;
   C.drpo_two_eps = (float)(2.0 * p->drpo_epsilon);
   C.inv_two_eps = (float)(1.0 / (double)C.drpo_two_eps);
+  C.inv_eps = (float)(1.0 / (double)C.drpo_eps);
   C.horizon = (float)p->horizon;
   C.fast_ok = (p->kind == UNIRL_LOSS_DRPO && p->mu_weighted && C.drpo_eps >= 1.0f) ? 1 : 0;
   C.fast_hi = 1.0f + C.drpo_eps;  // fp32, as the kernel would form it
@@ -1227,6 +1233,8 @@ static int check_common(const float* new_logp, const float* old_logp, const floa
   A.n_seq = n_seq;
   A.seq_stride = seq_stride;
   A.n_tok = n_tok;
+  A.inv_seq_scale = (A.C.agg_mode == UNIRL_AGG_SEQ_MEAN_TOKEN_SUM) ? 1.0 / ((double)n_seq * (double)A.C.horizon)
+                                                                   : 1.0 / (double)n_seq;
 #ifdef UNIRL_TUNE
   A.synth_len = (int)tune_int("UNIRL_RATIO_SYNTH_LEN", 0);
 #endif
