@@ -34,6 +34,10 @@ def _kernel_dtype(t: torch.Tensor) -> torch.Tensor:
 def _sigma_arg(sigma: torch.Tensor, B: int, device: torch.device, name: str) -> Tuple[torch.Tensor, int]:
     """f32 device tensor with 1 or B values, and the per-sample stride (0 or 1)."""
     s = sigma
+    if s.dtype is torch.float32 and s.dim() == 1 and s.device == device and s.stride(0) == 1 and not s.requires_grad:
+        n = s.shape[0]  # already what the kernel reads: no view is made
+        if n == 1 or n == B:
+            return s, (0 if n == 1 else 1)
     if s.dtype != torch.float32 or s.device != device or s.requires_grad:
         s = s.detach().to(device=device, dtype=torch.float32)
     n = s.numel()
@@ -158,6 +162,8 @@ def _per_sample_view(t: torch.Tensor, name: str, *, writable: bool = False) -> T
     N.require_device(t, name)
     B = t.shape[0]
     D = t.numel() // B if B else 0
+    if t.is_contiguous():
+        return t, D
     inner_ok = B == 0 or _dense_from(t, 1)
     # A sample stride of 0 means "densely packed" in the C ABI, so a tensor broadcast over the
     # samples (expand(B, ...), stride 0) cannot be handed over as it is: it is copied.
@@ -208,10 +214,11 @@ def sde_step_logp_into(
     B = sample.shape[0]
     D = sample.numel() // B if B else 0
 
-    def as_input(t, name):
-        t = t.detach()
+    def as_input(t, name):  # only the address is used: a tensor that requires grad needs no detach
         if t.dtype not in N._DTYPE_CODE:
-            t = t.float()
+            t = t.detach().float()
+        elif t.requires_grad and not t.is_contiguous():
+            t = t.detach()  # a copy may follow; keep it out of the autograd graph
         return _per_sample_view(t, name)
 
     v, sv = as_input(noise_pred, "noise_pred")
@@ -220,15 +227,18 @@ def sde_step_logp_into(
     if prev_sample is not None:
         if prev_sample.shape != sample.shape:
             raise ValueError(f"prev_sample {tuple(prev_sample.shape)} != sample {tuple(sample.shape)}")
-        pin = prev_sample.detach()
+        pin = prev_sample
         if pin.dtype != x.dtype:
-            pin = pin.to(x.dtype)  # the reference's round trip through the input dtype
+            pin = pin.detach().to(x.dtype)  # the reference's round trip through the input dtype
+        elif pin.requires_grad and not pin.is_contiguous():
+            pin = pin.detach()
         pin, sp = _per_sample_view(pin, "prev_sample")
     nz, sn = None, 0
     if noise is not None and prev_sample is None:
         if noise.shape != sample.shape:
             raise ValueError(f"noise {tuple(noise.shape)} != sample {tuple(sample.shape)}")
-        nz, sn = _per_sample_view(noise.detach().float(), "noise")
+        nz, sn = _per_sample_view(noise if noise.dtype is torch.float32 and not noise.requires_grad
+                                  else noise.detach().float(), "noise")
 
     def as_output(t, name, shape):
         if t is None:
@@ -340,10 +350,11 @@ def _replay_desc(noise_pred, latents, slot_sample, slot_prev, sigma, sigma_next,
     want = ((S, B) if step_major else (B, S)) + tail
     if tuple(noise_pred.shape) != want:
         raise ValueError(f"noise_pred {tuple(noise_pred.shape)} != {want}")
-    v = noise_pred.detach()
+    # only addresses are used: a detached alias is made only where a cast or a copy may follow
+    v = noise_pred.detach() if noise_pred.requires_grad else noise_pred
     if v.dtype not in N._DTYPE_CODE:
         v = v.float()
-    x = latents.detach()
+    x = latents.detach() if latents.requires_grad else latents
     if x.dtype not in N._DTYPE_CODE:
         x = x.float()
     # every (sample, step) block must be one contiguous run of D elements.  The two leading strides
