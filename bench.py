@@ -521,7 +521,7 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
             torch.cuda.synchronize()
         stats = {"forward_ms": round(a.elapsed_time(b), 2), "backward_ms": round(b.elapsed_time(c), 2),
                  "total_ms": round(a.elapsed_time(c), 2),
-                 "peak_transient_gib": round((torch.cuda.max_memory_allocated() - base) / 2**30, 2)}
+                 "peak_transient_gib": round((torch.cuda.max_memory_allocated() - base) / 2**30, 3)}
         return stats, out.detach(), h.grad.detach().float(), head.weight.grad.detach().float()
 
     out = {"rows": rows, "vocab": vocab, "hidden": hidden}
@@ -532,6 +532,8 @@ def replay_probe(torch, dev, rows: int, vocab: int, hidden: int = 2560):
                      ("fused_keep_logits", dict(transposed_head=False)), ("fused_default", dict()),
                      ("fused_head_chunk4096", dict(keep_logits=False, transposed_head=False)),
                      ("fused_head_chunk2048_transposed", dict(keep_logits=False, chunk=2048)),
+                     ("fused_head_chunk1024_transposed", dict(keep_logits=False, chunk=1024)),
+                     ("fused_head_chunk512_transposed", dict(keep_logits=False, chunk=512)),
                      ("fused_recompute_chunk2048_transposed", dict(chunk=2048, keep_logits=False, fused_head=False))):
         got = timed(lambda h: models.chunked_replay_logp(head, h, tokens, 1.0, **kw))
         got[0]["max_abs_logp_diff"] = float((got[1] - ref[1]).abs().max())
@@ -749,12 +751,15 @@ def timeline_probe(torch, dev, names):
                 if t.numel() == 0:
                     continue
                 start, end = int(t[:, 0].min()), int(t[:, 3].max())
-                d = per.setdefault(name, dict(gap=[], body=[], first_wg_done=[], stream_done=[]))
+                d = per.setdefault(name, dict(gap=[], body=[], first_wg_done=[], stream_done=[], second_mark=[]))
                 d["body"].append((end - start) * tick_ns)
                 d["first_wg_done"].append((int(t[:, 3].min()) - start) * tick_ns)
                 marks = t[:, 1][t[:, 1] > 0]
                 if marks.numel():
                     d["stream_done"].append((int(marks.max()) - start) * tick_ns)
+                marks2 = t[:, 2][t[:, 2] > 0]
+                if marks2.numel():
+                    d["second_mark"].append((int(marks2.max()) - start) * tick_ns)
                 if prev_end is not None:
                     d["gap"].append((start - prev_end) * tick_ns)
                 prev_end = end
@@ -766,6 +771,7 @@ def timeline_probe(torch, dev, names):
                 "gap_before_us": med(d["gap"]), "body_us": med(d["body"]),
                 "first_workgroup_done_at_us": med(d["first_wg_done"]),
                 "last_workgroup_past_its_loop_at_us": med(d["stream_done"]),
+                "second_mark_at_us": med(d["second_mark"]),
             }
             total += (med(d["gap"]) or 0.0) + (med(d["body"]) or 0.0)
         row["sum_of_gaps_and_bodies_us"] = round(total, 2)

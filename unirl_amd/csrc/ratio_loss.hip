@@ -917,12 +917,17 @@ __global__ __launch_bounds__(kRlThreads) void ratio_loss_packed_kernel(RatioArgs
   UNIRL_TRACE_END(A.trace);
 }
 
-// One workgroup of five wavefronts: wavefront c reads the c-th 16-byte chunk of every workgroup's
-// partial vector (two sums; two sums; two sums; the four counters; the three extrema),
-// lane l the vectors l, l + 64, ... in that order, every load of a lane in flight at once; one
-// wavefront reduction per value then leaves the thirteen totals in LDS and sixteen lanes turn them
-// into the metrics.  Fixed order throughout.
-constexpr int kFinThreads = 5 * kWave;
+// One workgroup of six wavefronts.  Wavefronts 0-2 read the three chunks of sums, wavefronts 3 and
+// 4 the counter chunk (two counters each: no wavefront reduces more than two 64-bit values),
+// wavefront 5 the extrema; lane l takes the vectors l, l + 64, ... of its chunk, every load of a
+// lane in flight at once; the lane adds its values pairwise (a tree of fixed shape), one wavefront
+// reduction per value then leaves the thirteen totals in LDS and sixteen lanes turn them into the
+// metrics.  Fixed order throughout.
+// kBatch: loads a lane has in flight per trip, chosen by the host to cover the positions in one trip
+// where it can (4, 8 or 16 for up to 256, 512 or more positions): a surplus load costs as much as
+// a useful one.
+constexpr int kFinThreads = 6 * kWave;
+template <int kBatch>
 __global__ __launch_bounds__(kFinThreads) void ratio_loss_finalize_kernel(RatioArgs A, unsigned int nblk) {
   __shared__ double lds_tot[kRlVals];
   UNIRL_TRACE_T0();
@@ -930,13 +935,13 @@ __global__ __launch_bounds__(kFinThreads) void ratio_loss_finalize_kernel(RatioA
   const int t = threadIdx.x;
   {
     const int lane = t & (kWave - 1);
-    const int chunk = __builtin_amdgcn_readfirstlane(t) / kWave;  // wave-uniform
+    const int wave = __builtin_amdgcn_readfirstlane(t) / kWave;  // wave-uniform
+    const int chunk = wave < 4 ? wave : wave - 1;                // wavefronts 3 and 4 share the counters
     const unsigned int per = partial_per_xcd(nblk), npos = per * kXcds;
     const u32x4* src = reinterpret_cast<const u32x4*>(A.partials) + (size_t)chunk * npos;
-    constexpr int kBatch = 16;
     const unsigned int idw = (chunk == 4) ? 0xff800000u : 0u;  // -inf for the maxima, 0 for the sums
     const u32x4 ident = {idw, idw, idw, idw};
-    double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
+    double a0 = 0.0, a1 = 0.0;
     float m0 = -INFINITY, m1 = -INFINITY, m2 = -INFINITY;
     for (unsigned int j0 = 0; j0 < npos; j0 += kWave * kBatch) {
       u32x4 y[kBatch];
@@ -952,20 +957,41 @@ __global__ __launch_bounds__(kFinThreads) void ratio_loss_finalize_kernel(RatioA
 #pragma unroll
       for (int b = 0; b < kBatch; ++b)
         if (j0 + b * kWave + lane >= npos) y[b] = ident;
+      double u[kBatch], w[kBatch];
+      auto add_pairwise = [&]() {
+#pragma unroll
+        for (int width = kBatch / 2; width >= 1; width /= 2) {
+#pragma unroll
+          for (int b = 0; b < width; ++b) {
+            u[b] += u[b + width];
+            w[b] += w[b + width];
+          }
+        }
+        a0 += u[0];
+        a1 += w[0];
+      };
+      // one straight-line block per kind of wavefront (the kind is wave-uniform)
       if (chunk < 3) {
 #pragma unroll
         for (int b = 0; b < kBatch; ++b) {
-          a0 += __longlong_as_double((long long)(((unsigned long long)y[b].y << 32) | y[b].x));
-          a1 += __longlong_as_double((long long)(((unsigned long long)y[b].w << 32) | y[b].z));
+          u[b] = __longlong_as_double((long long)(((unsigned long long)y[b].y << 32) | y[b].x));
+          w[b] = __longlong_as_double((long long)(((unsigned long long)y[b].w << 32) | y[b].z));
         }
-      } else if (chunk == 3) {
+        add_pairwise();
+      } else if (wave == 3) {  // counters are exact in fp64
 #pragma unroll
         for (int b = 0; b < kBatch; ++b) {
-          a0 += (double)y[b].x;
-          a1 += (double)y[b].y;
-          a2 += (double)y[b].z;
-          a3 += (double)y[b].w;
+          u[b] = (double)y[b].x;
+          w[b] = (double)y[b].y;
         }
+        add_pairwise();
+      } else if (wave == 4) {
+#pragma unroll
+        for (int b = 0; b < kBatch; ++b) {
+          u[b] = (double)y[b].z;
+          w[b] = (double)y[b].w;
+        }
+        add_pairwise();
       } else {
 #pragma unroll
         for (int b = 0; b < kBatch; ++b) {
@@ -976,23 +1002,13 @@ __global__ __launch_bounds__(kFinThreads) void ratio_loss_finalize_kernel(RatioA
       }
     }
     UNIRL_TRACE_MARK1();
-    if (chunk < 3) {
+    if (chunk < 4) {
       a0 = wave_sum(a0);
       a1 = wave_sum(a1);
       if (lane == 0) {
-        lds_tot[2 * chunk] = a0;
-        lds_tot[2 * chunk + 1] = a1;
-      }
-    } else if (chunk == 3) {
-      a0 = wave_sum(a0);
-      a1 = wave_sum(a1);
-      a2 = wave_sum(a2);
-      a3 = wave_sum(a3);
-      if (lane == 0) {
-        lds_tot[kFirstCnt] = a0;
-        lds_tot[kFirstCnt + 1] = a1;
-        lds_tot[kFirstCnt + 2] = a2;
-        lds_tot[kFirstCnt + 3] = a3;
+        const int slot = chunk < 3 ? 2 * chunk : kFirstCnt + 2 * (wave - 3);
+        lds_tot[slot] = a0;
+        lds_tot[slot + 1] = a1;
       }
     } else {
       m0 = wave_max(m0);
@@ -1007,6 +1023,7 @@ __global__ __launch_bounds__(kFinThreads) void ratio_loss_finalize_kernel(RatioA
     }
   }
   __syncthreads();
+  UNIRL_TRACE_MARK2();
   if (t >= kRlVals) return;
   // Lane v turns slot v into its metric; the lanes run the same straight-line code.
   const int v = t;
@@ -1322,7 +1339,13 @@ static int launch_forward(RatioArgs& A, hipStream_t st) {
   if (launch_rc != 0 || !A.metrics) return launch_rc;
   const unsigned int nblk = S.grid.x * S.grid.y;
   UNIRL_TRACE_SET(A, "ratio_finalize", 1);
-  hipLaunchKernelGGL(ratio_loss_finalize_kernel, dim3(1), dim3(kFinThreads), 0, st, A, nblk);
+  const unsigned int npos = partial_per_xcd(nblk) * kXcds;
+  if (npos <= 4 * kWave)
+    hipLaunchKernelGGL(ratio_loss_finalize_kernel<4>, dim3(1), dim3(kFinThreads), 0, st, A, nblk);
+  else if (npos <= 8 * kWave)
+    hipLaunchKernelGGL(ratio_loss_finalize_kernel<8>, dim3(1), dim3(kFinThreads), 0, st, A, nblk);
+  else
+    hipLaunchKernelGGL(ratio_loss_finalize_kernel<16>, dim3(1), dim3(kFinThreads), 0, st, A, nblk);
   return (int)hipGetLastError();
 }
 
