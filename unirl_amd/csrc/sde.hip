@@ -311,6 +311,10 @@ __device__ __forceinline__ void sde_step_body(const SdeStepArgs& A, const SdeRow
     A.logp_out[row * A.stride_logp] = sde_finish_logp(kind, c, part, (double)D, A.logp_sum);
   } else {
     A.partials[row * gridDim.x + blockIdx.x] = part;  // summed by sde_step_finalize_kernel
+    if (blockIdx.x == 0) {  // worked out here anyway, behind the first pass of loads: the finalize only reads them
+      A.coef_out[2 * row] = c.den;
+      A.coef_out[2 * row + 1] = c.logs;
+    }
   }
   UNIRL_TRACE_END(A.trace);
 }
@@ -444,17 +448,16 @@ __global__ __launch_bounds__(kReplayFinishThreads) void flowdppo_replay_finish_k
 }
 
 // One wavefront per row: adds the workgroup partials in index order and finishes the log-prob.
-// sigma_mod: rows per sample of a batched replay (sigma is then indexed by the step, row modulo
-// sigma_mod), 0 for the plain step (sigma indexed by the sample through sigma_stride).
+// The row's coefficients (log-prob denominator, log std) come from the workspace, where the
+// streaming kernel has left them: worked out here they would follow the sigma loads -- a trip to
+// memory, then an fp64 divide, square root and logarithm with nothing to overlap them.
 // kBatch: partial loads a lane has in flight, chosen by the host from nblk (1, 2, 4 or 8 cover 64,
 // 128, 256 and more partials per row: surplus loads of a short row cost more than they hide).
 template <int kBatch>
-__global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepArgs A, int64_t B, unsigned int nblk,
-                                                                       int sigma_mod) {
+__global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepArgs A, int64_t B, unsigned int nblk) {
   UNIRL_TRACE_T0();
   const int64_t b = (int64_t)blockIdx.x * (kSdeThreads / kWave) + threadIdx.x / kWave;
   if (b >= B) return;
-  // the partial loads are issued first; the coefficients are worked out while they are in flight
   const int lane = threadIdx.x & (kWave - 1);
   const double* __restrict__ pp = A.partials + b * nblk;
   double y[kBatch];  // lane l adds partials l, l + 64, ... in that order
@@ -463,12 +466,10 @@ __global__ __launch_bounds__(kSdeThreads) void sde_step_finalize_kernel(SdeStepA
     const unsigned int j = lane + k * kWave;
     y[k] = pp[j < nblk ? j : nblk - 1];  // past the end: a harmless repeat, discarded below
   }
-  const int64_t sig_idx = sigma_mod ? b % sigma_mod : b * A.sigma_stride;
-  const float s = A.sigma[sig_idx];
-  const float sn = A.sigma_next[sig_idx];
-  const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
+  SdeCoef c;
+  c.den = A.coef_out[2 * b];
+  c.logs = A.coef_out[2 * b + 1];
   __builtin_amdgcn_sched_barrier(0);  // all of the above in flight before the first value is used
-  const SdeCoef c = sde_coef(A.kind, s, sn, smax, A.sc);
   double q = 0.0;
 #pragma unroll
   for (int k = 0; k < kBatch; ++k) q += (lane + k * kWave < (int)nblk) ? y[k] : 0.0;
@@ -793,24 +794,25 @@ static unsigned int sde_blocks_per_sample(int64_t nvec, int items, int64_t B, in
 
 // Samples per launch so that the partials fit the workspace (and grid.y its limit).
 static int64_t sde_samples_per_launch(int64_t B, int64_t partials_per_sample) {
-  int64_t nb = kPartialCapacity / (partials_per_sample > 0 ? partials_per_sample : 1);
+  // one more slot per row: its two fp32 coefficients, stored behind the launch's partials
+  int64_t nb = kPartialCapacity / ((partials_per_sample > 0 ? partials_per_sample : 1) + 1);
   if (nb > 32768) nb = 32768;
   if (nb > B) nb = B;
   return nb < 1 ? 1 : nb;
 }
 
 // Finalize launch of a step / replay call: one wavefront per row, the in-flight batch picked from nblk.
-static int launch_step_finalize(const SdeStepArgs& A, int64_t rows, unsigned int nblk, int sigma_mod, hipStream_t st) {
+static int launch_step_finalize(const SdeStepArgs& A, int64_t rows, unsigned int nblk, hipStream_t st) {
   const int per_block = kSdeThreads / kWave;
   const dim3 grid((unsigned int)((rows + per_block - 1) / per_block)), block(kSdeThreads);
   if (nblk <= kWave)
-    hipLaunchKernelGGL(sde_step_finalize_kernel<1>, grid, block, 0, st, A, rows, nblk, sigma_mod);
+    hipLaunchKernelGGL(sde_step_finalize_kernel<1>, grid, block, 0, st, A, rows, nblk);
   else if (nblk <= 2 * kWave)
-    hipLaunchKernelGGL(sde_step_finalize_kernel<2>, grid, block, 0, st, A, rows, nblk, sigma_mod);
+    hipLaunchKernelGGL(sde_step_finalize_kernel<2>, grid, block, 0, st, A, rows, nblk);
   else if (nblk <= 4 * kWave)
-    hipLaunchKernelGGL(sde_step_finalize_kernel<4>, grid, block, 0, st, A, rows, nblk, sigma_mod);
+    hipLaunchKernelGGL(sde_step_finalize_kernel<4>, grid, block, 0, st, A, rows, nblk);
   else
-    hipLaunchKernelGGL(sde_step_finalize_kernel<8>, grid, block, 0, st, A, rows, nblk, sigma_mod);
+    hipLaunchKernelGGL(sde_step_finalize_kernel<8>, grid, block, 0, st, A, rows, nblk);
   return (int)hipGetLastError();
 }
 
@@ -1170,6 +1172,7 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
     A.logp_out = offset_f32(d->logp_out, b0 * stride_lp);
     A.stride_logp = stride_lp;
     A.partials = ws_partials(workspace);
+    A.coef_out = reinterpret_cast<float*>(A.partials + nb * (int64_t)nblk);
     A.nblk = nblk;
     A.items = items;
     if (draw) {
@@ -1190,7 +1193,7 @@ extern "C" int unirl_sde_step_logp_ex(const unirl_sde_step_desc* d, void* worksp
     if (rc != 0) return rc;
     if (want_logp && nblk > 1) {
       UNIRL_TRACE_SET(A, "sde_finalize", (unsigned int)((nb + kSdeThreads / kWave - 1) / (kSdeThreads / kWave)));
-      rc = launch_step_finalize(A, nb, nblk, 0, st);
+      rc = launch_step_finalize(A, nb, nblk, st);
       if (rc != 0) return rc;
     }
   }
@@ -1247,6 +1250,7 @@ extern "C" int unirl_sde_replay_logp(const unirl_sde_replay_desc* d, void* works
     A.logp_out = offset_f32(d->logp_out, b0 * S);
     A.stride_logp = 1;
     A.partials = ws_partials(workspace);
+    A.coef_out = reinterpret_cast<float*>(A.partials + nb * S * (int64_t)nblk);
     A.nblk = nblk;
     A.items = items;
     UNIRL_TRACE_SET(A, "sde_replay", nblk * (unsigned int)(nb * S));
@@ -1259,7 +1263,7 @@ extern "C" int unirl_sde_replay_logp(const unirl_sde_replay_desc* d, void* works
     if (rc != 0) return rc;
     if (want_logp && nblk > 1) {
       UNIRL_TRACE_SET(A, "sde_finalize", (unsigned int)((nb * S + kSdeThreads / kWave - 1) / (kSdeThreads / kWave)));
-      rc = launch_step_finalize(A, nb * S, nblk, (int)S, st);
+      rc = launch_step_finalize(A, nb * S, nblk, st);
       if (rc != 0) return rc;
     }
   }
