@@ -33,10 +33,14 @@ struct DppoArgs {
   float grad_scale;
 };
 
-enum { D_SR = 0, D_SR2, D_LD2, D_KL, D_LOSS, D_NKL, D_POS, D_NEG, D_RM, D_SUMS, D_RMIN = D_SUMS, D_RMAX, D_KLMAX, D_VALS };
+// Five fp64 sums per lane; the four counters are wave-wide from the start (a comparison is a lane
+// mask and counting it is one scalar instruction, where a sum over lanes is six shifts and adds).
+enum { D_SR = 0, D_SR2, D_LD2, D_KL, D_LOSS, D_SUMS };
+enum { C_NKL = 0, C_POS, C_NEG, C_RM, C_VALS };
 
 struct DppoAcc {
   double acc[D_SUMS];
+  unsigned long long cnt[C_VALS] = {0ull, 0ull, 0ull, 0ull};  // wave-uniform
   float rmin = INFINITY, rmax = -INFINITY, klmax = -INFINITY;
   __device__ __forceinline__ DppoAcc() {
 #pragma unroll
@@ -45,8 +49,9 @@ struct DppoAcc {
 };
 
 // Element i of the [B,S'] problem: ratio, the two removal masks, the kept loss (and its gradient).
-__device__ __forceinline__ void dppo_elem_of(const DppoArgs& A, int64_t i, float nw, float od, float a, float kl,
-                                             DppoAcc& s) {
+// The whole wavefront calls together; `valid` is false for a lane past the end.
+__device__ __forceinline__ void dppo_elem_of(const DppoArgs& A, int64_t i, bool valid, float nw, float od, float a,
+                                             float kl, DppoAcc& s) {
   const float ld = nw - od;
   const float r = expf(ld);
   const bool low_kl = kl < A.threshold;
@@ -54,6 +59,11 @@ __device__ __forceinline__ void dppo_elem_of(const DppoArgs& A, int64_t i, float
   const bool neg = !low_kl && (r < 1.0f) && (a < 0.0f);
   const bool rm = pos || neg;
   const float loss = rm ? 0.0f : (-a) * r;
+  s.cnt[C_NKL] += (unsigned long long)__builtin_popcountll(__builtin_amdgcn_ballot_w64(valid && !low_kl));
+  s.cnt[C_POS] += (unsigned long long)__builtin_popcountll(__builtin_amdgcn_ballot_w64(valid && pos));
+  s.cnt[C_NEG] += (unsigned long long)__builtin_popcountll(__builtin_amdgcn_ballot_w64(valid && neg));
+  s.cnt[C_RM] += (unsigned long long)__builtin_popcountll(__builtin_amdgcn_ballot_w64(valid && rm));
+  if (!valid) return;
   A.loss_elem[i] = loss;
   if (A.grad_new) A.grad_new[i] = A.grad_scale * loss;  // d(-a*exp(new-old))/dnew = the loss itself
   s.acc[D_SR] += (double)r;
@@ -61,33 +71,31 @@ __device__ __forceinline__ void dppo_elem_of(const DppoArgs& A, int64_t i, float
   s.acc[D_LD2] += (double)(0.5f * (ld * ld));
   s.acc[D_KL] += (double)kl;
   s.acc[D_LOSS] += (double)loss;
-  s.acc[D_NKL] += low_kl ? 0.0 : 1.0;
-  s.acc[D_POS] += pos ? 1.0 : 0.0;
-  s.acc[D_NEG] += neg ? 1.0 : 0.0;
-  s.acc[D_RM] += rm ? 1.0 : 0.0;
   s.rmin = fminf(s.rmin, r);
   s.rmax = fmaxf(s.rmax, r);
   s.klmax = fmaxf(s.klmax, kl);
 }
 
-__device__ __forceinline__ void dppo_elem(const DppoArgs& A, int64_t i, float kl, DppoAcc& s) {
-  dppo_elem_of(A, i, A.nw[i], A.od[i], A.adv[i], kl, s);
-}
-
 // The twelve metrics from the totals; one thread.
-__device__ __forceinline__ void dppo_metrics(const DppoArgs& A, const double (&tot)[D_SUMS], float rmin, float rmax,
+__device__ __forceinline__ void dppo_metrics(const DppoArgs& A, const double (&tot)[D_SUMS],
+                                             const unsigned long long (&cnt)[C_VALS], float rmin, float rmax,
                                              float klmax) {
   const double N = (double)A.n;
-  // one reciprocal for every mean (x * (1/N) and x / N agree to an ulp of fp64, far below fp32)
-  const double inv_n = 1.0 / N;
-  double var = 0.0;
+  // One reciprocal for every mean (x * (1/N) and x / N agree to an ulp of fp64, far below fp32): the
+  // hardware's fp32 estimate and two Newton steps in fp64 (the error squares twice from 2^-23).
+  const double r0 = (double)__builtin_amdgcn_rcpf((float)N);
+  const double r1 = fma(fma(-N, r0, 1.0), r0, r0);
+  const double inv_n = fma(fma(-N, r1, 1.0), r1, r1);
+  // the variance's numerator cancels and is formed in fp64; quotient and root are fp32 operations
+  float sd = 0.0f;
   if (A.n > 1) {
-    var = (tot[D_SR2] - tot[D_SR] * tot[D_SR] * inv_n) / (N - 1.0);
-    if (var < 0.0) var = 0.0;
+    const double num = tot[D_SR2] - tot[D_SR] * tot[D_SR] * inv_n;
+    sd = sqrtf(fmaxf((float)num, 0.0f) / (float)(N - 1.0));
+    if (num != num) sd = quiet_nan();  // fmaxf would drop it
   }
   float* M = A.metrics;
   M[0] = (float)(tot[D_SR] * inv_n);
-  M[1] = (float)sqrt(var);
+  M[1] = sd;
   // min()/max() of the reference return NaN when any element is NaN; ratios and KL values are
   // >= 0, so their sums are NaN exactly then
   const bool r_nan = tot[D_SR] != tot[D_SR], kl_nan = tot[D_KL] != tot[D_KL];
@@ -96,11 +104,11 @@ __device__ __forceinline__ void dppo_metrics(const DppoArgs& A, const double (&t
   M[4] = (float)(tot[D_LD2] * inv_n);
   M[5] = (float)(tot[D_KL] * inv_n);
   M[6] = kl_nan ? quiet_nan() : klmax;
-  M[7] = (float)(tot[D_NKL] * inv_n);
-  M[8] = (float)(tot[D_POS] * inv_n);
-  M[9] = (float)(tot[D_NEG] * inv_n);
-  M[10] = (float)(tot[D_RM] * inv_n);
-  M[11] = (float)((N - tot[D_RM]) * inv_n);
+  M[7] = (float)((double)cnt[C_NKL] * inv_n);
+  M[8] = (float)((double)cnt[C_POS] * inv_n);
+  M[9] = (float)((double)cnt[C_NEG] * inv_n);
+  M[10] = (float)((double)cnt[C_RM] * inv_n);
+  M[11] = (float)((N - (double)cnt[C_RM]) * inv_n);
   M[12] = (float)(tot[D_LOSS] * inv_n);
   M[13] = M[14] = M[15] = 0.0f;
 }
@@ -111,17 +119,30 @@ __device__ __forceinline__ void dppo_metrics(const DppoArgs& A, const double (&t
 __device__ __forceinline__ void dppo_on_one_wave(const DppoArgs& A, const float* kl, const float* first = nullptr) {
   const int lane = threadIdx.x & (kWave - 1);
   DppoAcc s;
-  int64_t i = lane;
-  if (first && i < A.n) {
-    dppo_elem_of(A, i, first[0], first[1], first[2], kl[i], s);
-    i += kWave;
+  // wave-uniform trip count: every lane runs every pass (the counters are taken across the wavefront)
+  for (int64_t base = 0; base < A.n; base += kWave) {
+    const int64_t i = base + lane;
+    const bool valid = i < A.n;
+    float nw = 0.0f, od = 0.0f, a = 0.0f, k = 0.0f;
+    if (valid) {
+      k = kl[i];
+      if (first && base == 0) {
+        nw = first[0];
+        od = first[1];
+        a = first[2];
+      } else {
+        nw = A.nw[i];
+        od = A.od[i];
+        a = A.adv[i];
+      }
+    }
+    dppo_elem_of(A, i, valid, nw, od, a, k, s);
   }
-  for (; i < A.n; i += kWave) dppo_elem(A, i, kl[i], s);
   double tot[D_SUMS];
 #pragma unroll
   for (int v = 0; v < D_SUMS; ++v) tot[v] = wave_sum(s.acc[v]);
   const float rmin = wave_min(s.rmin), rmax = wave_max(s.rmax), klmax = wave_max(s.klmax);
-  if (lane == 0) dppo_metrics(A, tot, rmin, rmax, klmax);
+  if (lane == 0) dppo_metrics(A, tot, s.cnt, rmin, rmax, klmax);
 }
 
 }  // namespace unirl

@@ -232,12 +232,23 @@ __global__ __launch_bounds__(kKlThreads) void flowdppo_loss_kernel(DppoArgs A) {
   __shared__ double lds[kKlThreads / kWave];
   __shared__ float ldsf[kKlThreads / kWave];
   DppoAcc s;
-  for (int64_t i = threadIdx.x; i < A.n; i += kKlThreads) dppo_elem(A, i, A.kl[i], s);
+  // every wavefront makes the same number of trips as a whole (its counters are taken across the lanes)
+  for (int64_t base = 0; base < A.n; base += kKlThreads) {
+    const int64_t i = base + threadIdx.x;
+    const bool valid = i < A.n;
+    dppo_elem_of(A, i, valid, valid ? A.nw[i] : 0.0f, valid ? A.od[i] : 0.0f, valid ? A.adv[i] : 0.0f,
+                 valid ? A.kl[i] : 0.0f, s);
+  }
   double tot[D_SUMS];
 #pragma unroll
   for (int v = 0; v < D_SUMS; ++v) tot[v] = block_sum<double>(s.acc[v], lds);
+  // the wavefronts' counters (exact in fp64), carried by each wavefront's first lane
+  unsigned long long cnt[C_VALS];
+  const bool lead = (threadIdx.x & (kWave - 1)) == 0;
+#pragma unroll
+  for (int v = 0; v < C_VALS; ++v) cnt[v] = (unsigned long long)block_sum<double>(lead ? (double)s.cnt[v] : 0.0, lds);
   const float rmin = block_min(s.rmin, ldsf), rmax = block_max(s.rmax, ldsf), klmax = block_max(s.klmax, ldsf);
-  if (threadIdx.x == 0) dppo_metrics(A, tot, rmin, rmax, klmax);
+  if (threadIdx.x == 0) dppo_metrics(A, tot, cnt, rmin, rmax, klmax);
 }
 
 // KL finalize and the KL-ADV loss in one launch: the wavefronts of one workgroup add the
