@@ -251,13 +251,18 @@ __global__ __launch_bounds__(kKlThreads) void flowdppo_loss_kernel(DppoArgs A) {
   if (threadIdx.x == 0) dppo_metrics(A, tot, cnt, rmin, rmax, klmax);
 }
 
-// KL finalize and the KL-ADV loss in one launch: the wavefronts of one workgroup add the
+// KL finalize and the KL-ADV loss in one launch: the sixteen wavefronts of one workgroup add the
 // streaming kernel's partials row by row (fixed order), leave the per-row KL in LDS, and the
-// first wavefront runs the [B,S'] problem on it.  R <= kDppoWaveMax.
-__global__ __launch_bounds__(kKlThreads) void flowdppo_finish_kernel(KlArgs K, DppoArgs A, unsigned int nblk) {
+// first wavefront runs the [B,S'] problem on it.  With one partial per lane a wavefront keeps the
+// loads of four of its rows in flight at once: every trip to memory that waits for the one before
+// costs about a microsecond here, and a row per trip made this kernel 5.5 us at 24 rows.
+// R <= kDppoWaveMax.
+constexpr int kDppoFinishThreads = 1024;
+__global__ __launch_bounds__(kDppoFinishThreads) void flowdppo_finish_kernel(KlArgs K, DppoArgs A, unsigned int nblk) {
   __shared__ float lds_kl[kDppoWaveMax];
   UNIRL_TRACE_T0();
-  const int wave = threadIdx.x / kWave;
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x & (kWave - 1);
+  constexpr int kWaves = kDppoFinishThreads / kWave;
   const int64_t R = A.n;
   // the first wavefront's share of the [B,S'] problem is loaded now, with the partials, not after them
   float first[3] = {0.0f, 0.0f, 0.0f};
@@ -266,14 +271,39 @@ __global__ __launch_bounds__(kKlThreads) void flowdppo_finish_kernel(KlArgs K, D
     first[1] = A.od[threadIdx.x];
     first[2] = A.adv[threadIdx.x];
   }
-  for (int64_t row = wave; row < R; row += kKlThreads / kWave) {
-    const float den = kl_den(K, row);  // issued with the partial loads, not after them
-    const double q = wave_ordered_sum(K.partials + row * nblk, nblk);
+  auto finish_row = [&](int64_t row, double q, float den) {
     const float kl = (float)((q / (double)den) / (double)K.D);
-    if ((threadIdx.x & (kWave - 1)) == 0) {
+    if (lane == 0) {
       K.kl[row] = kl;
       if (K.mask) K.mask[row] = (kl < K.threshold) ? 1 : 0;
       lds_kl[row] = kl;
+    }
+  };
+  if (nblk <= kWave) {
+    constexpr int kRows = 4;
+    const unsigned int jl = (unsigned int)lane < nblk ? lane : nblk - 1;
+    for (int64_t base = wave; base < R; base += kWaves * kRows) {
+      double y[kRows];
+      float den[kRows];
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        const int64_t row = base + r * kWaves;
+        const int64_t rc = row < R ? row : R - 1;  // past the end: the last row again, dropped below
+        y[r] = K.partials[rc * nblk + jl];
+        den[r] = kl_den(K, rc);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // every load issued before the first value is used
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        const int64_t row = base + r * kWaves;
+        if (row < R) finish_row(row, wave_sum((unsigned int)lane < nblk ? y[r] : 0.0), den[r]);  // wave-uniform
+      }
+    }
+  } else {
+    // many partials per row means few rows (rows * nblk is capped by the launch): one row at a time
+    for (int64_t row = wave; row < R; row += kWaves) {
+      const float den = kl_den(K, row);  // issued with the partial loads, not after them
+      finish_row(row, wave_ordered_sum(K.partials + row * nblk, nblk), den);
     }
   }
   UNIRL_TRACE_MARK1();
@@ -475,7 +505,7 @@ extern "C" int unirl_flowdppo_step(const void* p, const void* q, int dtype, cons
   A.grad_new = grad_new;
   A.grad_scale = loss_scale / (float)R;  // d(loss_scale * mean(elem)) / d elem
   UNIRL_TRACE_SET(K, "dppo_finish", 1);
-  hipLaunchKernelGGL(flowdppo_finish_kernel, dim3(1), dim3(kKlThreads), 0, st, K, A, nblk);
+  hipLaunchKernelGGL(flowdppo_finish_kernel, dim3(1), dim3(kDppoFinishThreads), 0, st, K, A, nblk);
   return (int)hipGetLastError();
 }
 
