@@ -750,21 +750,39 @@ __global__ __launch_bounds__(kSdeThreads) void sde_rollout_rng_kernel(SdeRollout
   sde_rollout_body<TV, TX, VEC, ITEMS, true>(A, &G);
 }
 
-// One wavefront per (sample, step).
+// One wavefront per (sample, step).  The step's sigma pair is requested first and the partials right
+// behind it, so that the coefficients (an fp64 divide, square root and logarithm) are worked out
+// while the partials are still on their way, instead of a second trip to memory after the sum.
 __global__ __launch_bounds__(kSdeThreads) void sde_rollout_finalize_kernel(SdeRolloutArgs A, int64_t B,
                                                                            unsigned int nblk) {
   const int64_t row = (int64_t)blockIdx.x * (kSdeThreads / kWave) + threadIdx.x / kWave;  // b * S + k
   if (row >= B * A.S) return;
-  const double q = wave_ordered_sum(A.partials + row * nblk, nblk);
-  if ((threadIdx.x & (kWave - 1)) != 0) return;
+  const int lane = threadIdx.x & (kWave - 1);
   const int k = (int)(row % A.S);
-  if (A.want_logp[k]) {
-    const float smax = A.sigma_max_ptr ? *A.sigma_max_ptr : A.sigma_max_val;
-    const SdeCoef c = sde_coef(A.kind, A.sigmas[k], A.sigmas[k + 1], smax, A.sc[k]);
-    A.logp_out[row] = sde_finish_logp(A.kind, c, q, (double)A.D, A.logp_sum);
-  } else {
-    A.logp_out[row] = __uint_as_float(0x7fc00000u);
+  const bool want = A.want_logp[k] != 0;  // wave-uniform
+  float s = 0.5f, sn = 0.25f, smax = A.sigma_max_val;
+  if (want) {
+    s = A.sigmas[k];
+    sn = A.sigmas[k + 1];
+    if (A.sigma_max_ptr) smax = *A.sigma_max_ptr;
   }
+  constexpr int kBatch = 2;
+  const double* __restrict__ pp = A.partials + row * nblk;
+  double y[kBatch];  // lane l adds partials l, l + 64, ... in that order
+#pragma unroll
+  for (int j = 0; j < kBatch; ++j) {
+    const unsigned int i = lane + j * kWave;
+    y[j] = pp[i < nblk ? i : nblk - 1];  // past the end: a harmless repeat, discarded below
+  }
+  __builtin_amdgcn_sched_barrier(0);  // everything above in flight before the first value is used
+  const SdeCoef c = sde_coef(A.kind, s, sn, smax, A.sc[k]);
+  double q = 0.0;
+#pragma unroll
+  for (int j = 0; j < kBatch; ++j) q += (lane + j * kWave < (int)nblk) ? y[j] : 0.0;
+  if (nblk > kBatch * kWave) q += lane_ordered_sum(pp, nblk, kBatch * kWave);
+  q = wave_sum(q);
+  if (lane != 0) return;
+  A.logp_out[row] = want ? sde_finish_logp(A.kind, c, q, (double)A.D, A.logp_sum) : __uint_as_float(0x7fc00000u);
 }
 
 // ---------------------------------------------------------------------------
