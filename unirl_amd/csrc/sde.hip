@@ -131,18 +131,18 @@ struct SdeStepArgs {
   int64_t stride_prev, stride_mean;
   float* logp_out;
   int64_t stride_logp;
-  double* partials;        // [B][gridDim.x]
-  // fused Flow-DPPO replay only: the old policy's means [rows, D] (dense, the latents' dtype), whose
-  // Gaussian-KL numerator against this pass's means is summed beside the log-prob residual
+  double* partials;        // [rows][gridDim.x]
+  float* coef_out;         // [rows][2]: the row's log-prob denominator and log(std), left for the finalize / finish kernel
   // sampling only: noise drawn in the kernel (third == nullptr), optionally stored
   int rng;
   RngKey rng_key;
   int64_t rng_row0;        // index of the launch's first sample within the call
   float* noise_out;
   int64_t stride_noise_out;
+  // fused Flow-DPPO replay only: the old policy's means [rows, D] (dense, the latents' dtype), whose
+  // Gaussian-KL numerator against this pass's means is summed beside the log-prob residual
   const void* kl_old;
   double* partials_kl;     // [rows][gridDim.x]
-  float* coef_out;         // [rows][2]: the row's log-prob denominator and log(std), for the finish kernel
   unsigned int nblk;       // host only: grid.x
   int items;               // host only: vectors in flight per lane
   UNIRL_TRACE_FIELD
