@@ -120,6 +120,31 @@ def test_step_major_velocities_and_odd_extent(dev):
     run_case(dev, "flow", 28, 3.0, 2, (5, 9, 3), list(range(6)), [4, 0], torch.float32, torch.bfloat16, 43)
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_cases(dev, seed):
+    """Seeded draws of batch, latent shape, stored and trained steps, dtypes, strategy and velocity layout."""
+    import random
+
+    rng = random.Random(7100 + seed)
+    for _ in range(3):
+        n_stored = rng.randint(3, 9)
+        stored = sorted(rng.sample(range(0, 12), n_stored))
+        can = [i for i in stored if i + 1 in stored]
+        if not can:
+            continue
+        steps = rng.sample(can, rng.randint(1, min(4, len(can))))  # distinct: repeated steps give rows with equal KLs
+        B = rng.randint(1, 5)
+        if B * len(steps) < 2:
+            B = 2  # both mask values need two rows
+        # at least a few dozen elements per row: with fewer, 16-bit rows often have equal (or zero) KLs and no
+        # threshold separates them
+        tail = (rng.randint(2, 5), rng.randint(3, 9), rng.randint(4, 11)) if rng.random() < 0.6 else (rng.randint(5, 40), rng.randint(5, 17))
+        traj = rng.choice([torch.bfloat16, torch.float16, torch.float32])
+        vdt = rng.choice([traj, torch.float32]) if traj is not torch.float32 else rng.choice([torch.float32, torch.bfloat16])
+        run_case(dev, rng.choice(["flow", "dance", "cps"]), 28, rng.choice([3.0, 5.0]), B, tail, stored, steps, traj, vdt,
+                 rng.randint(0, 10 ** 6), step_major=rng.random() < 0.4)
+
+
 def test_sd3_recipe_shape(dev):
     """SD3: bf16 trajectory of 10 steps, 3 trained steps, micro-batch 8, latents [16,128,128]."""
     run_case(dev, "flow", 10, 3.0, 8, (16, 128, 128), list(range(11)), [0, 2, 4], torch.bfloat16, torch.bfloat16, 44)
