@@ -8,6 +8,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -379,6 +380,180 @@ void check_sde_replay(hipStream_t st, void* ws, size_t ws_bytes) {
   std::printf("batched replay: %lld x %lld transitions equal the single-step calls\n", (long long)B, (long long)S);
 }
 
+// The Flow-DPPO forward straight from the velocities (unirl/models/sd3/diffusion.py:467-497 followed by
+// unirl/algorithms/flowdppo.py:43-51,86-137): the frozen policy's log-probs and means come from one replay
+// call, the new policy's from the fused entry point, and the KL rows, masks, loss elements and gradient are
+// checked against a float64 evaluation of the reference's formulas on the means the unfused replay writes.
+void check_flowdppo_replay(hipStream_t st, void* ws, size_t ws_bytes) {
+  const int64_t B = 3, K = 4, S = 2, D = 520, R = B * S;
+  const double eta = 0.7, sigma_max = 0.98780483;
+  Rng rng(16);
+  std::vector<float> stack(B * K * D), v_old(B * S * D), v_new(B * S * D), adv(R);
+  for (auto& e : stack) e = (float)rng.normal();
+  for (auto& e : v_old) e = (float)rng.normal();
+  for (int64_t r = 0; r < R; ++r) {
+    const double bump = 0.002 + 0.03 * rng.uniform();  // the policy has moved by a different amount per row
+    for (int64_t i = 0; i < D; ++i) v_new[r * D + i] = v_old[r * D + i] + (float)(bump * rng.normal());
+    adv[r] = (float)rng.normal();
+  }
+  const std::vector<float> sg = {0.84375006f, 0.5f}, sn = {0.82258058f, 0.4f}, sig_t = {0.31f, 0.22f};
+  const int64_t slot_x[2] = {2, 0}, slot_p[2] = {3, 1};
+  DevBuf<float> dstack(stack), dvo(v_old), dvn(v_new), dsg(sg), dsn(sn), dst(sig_t), dadv(adv);
+  DevBuf<float> old_mean(R * D), old_lp(R), new_mean(R * D), new_lp(R), lp_f(R), kl(R), elem(R), grad(R), met(16);
+  DevBuf<uint8_t> mask(R);
+  unirl_sde_replay_desc d;
+  std::memset(&d, 0, sizeof(d));
+  d.noise_pred = {dvo.p, UNIRL_F32, S * D};
+  d.noise_pred_step_stride = D;
+  d.latents = {dstack.p, UNIRL_F32, K * D};
+  d.latents_slot_stride = D;
+  d.K = K;
+  d.slot_sample = slot_x;
+  d.slot_prev = slot_p;
+  d.sigma = dsg.p;
+  d.sigma_next = dsn.p;
+  d.sigma_max_val = (float)sigma_max;
+  d.eta = eta;
+  d.kind = UNIRL_SDE_FLOW;
+  d.B = B;
+  d.S = S;
+  d.D = D;
+  d.mean_dtype = UNIRL_F32;
+  d.mean_out = old_mean.p;
+  d.logp_out = old_lp.p;
+  expect_status("unirl_sde_replay_logp (frozen policy)", unirl_sde_replay_logp(&d, ws, ws_bytes, st));
+  d.noise_pred.ptr = dvn.p;
+  d.mean_out = new_mean.p;
+  d.logp_out = new_lp.p;
+  expect_status("unirl_sde_replay_logp (new policy)", unirl_sde_replay_logp(&d, ws, ws_bytes, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto om = old_mean.host(), nm = new_mean.host(), olp = old_lp.host(), nlp = new_lp.host();
+  // float64 KL rows, and a threshold halfway between two of them so that both mask values occur
+  std::vector<double> kl_ref(R);
+  for (int64_t r = 0; r < R; ++r) {
+    double q = 0.0;
+    for (int64_t i = 0; i < D; ++i) {
+      const double df = (double)nm[r * D + i] - (double)om[r * D + i];
+      q += df * df;
+    }
+    const double s_t = sig_t[r % S];
+    kl_ref[r] = q / (2.0 * s_t * s_t) / (double)D;
+  }
+  std::vector<double> sorted = kl_ref;
+  std::sort(sorted.begin(), sorted.end());
+  const float thr = (float)(0.5 * (sorted[R / 2 - 1] + sorted[R / 2]));
+  const float loss_scale = 0.37f;
+  d.mean_out = nullptr;  // the new means are not wanted: nothing but the partials is written
+  d.logp_out = lp_f.p;
+  expect_status("unirl_flowdppo_replay_step",
+                unirl_flowdppo_replay_step(&d, old_mean.p, dst.p, S, old_lp.p, dadv.p, thr, loss_scale, kl.p, mask.p, elem.p,
+                                           grad.p, met.p, ws, ws_bytes, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto lpf = lp_f.host(), klg = kl.host(), el = elem.host(), gr = grad.host(), mt = met.host();
+  const auto mk = mask.host();
+  int kept = 0, low = 0;
+  for (int64_t r = 0; r < R; ++r) {
+    expect_close("fused step: new log-prob vs the replay's", lpf[r], nlp[r], 1e-6, 1e-7);
+    expect_close("fused step: KL row", klg[r], kl_ref[r], 1e-5, 1e-12);
+    const bool low_kl = kl_ref[r] < (double)thr;
+    if ((mk[r] != 0) != low_kl) {
+      std::printf("FAIL fused step: mask of row %lld\n", (long long)r);
+      ++g_failures;
+    }
+    const double ratio = std::exp((double)nlp[r] - (double)olp[r]);
+    const bool rm = !low_kl && ((ratio > 1.0 && adv[r] > 0.0f) || (ratio < 1.0 && adv[r] < 0.0f));
+    const double loss = rm ? 0.0 : -(double)adv[r] * ratio;
+    // a log-prob of magnitude L carries fp32 rounding of 6e-8 L, which the exponential turns into that much
+    // relative error of the ratio
+    const double tol = 1e-5 + 2e-7 * std::fabs((double)nlp[r]);
+    expect_close("fused step: loss element", el[r], loss, tol, 1e-9);
+    expect_close("fused step: gradient", gr[r], (double)loss_scale * loss / (double)R, tol, 1e-10);
+    kept += rm ? 0 : 1;
+    low += low_kl ? 1 : 0;
+  }
+  expect_close("fused step: kl_mask_fraction", mt[7], 1.0 - (double)low / (double)R, 1e-6, 1e-7);
+  expect_close("fused step: unmasked_fraction", mt[11], (double)kept / (double)R, 1e-6, 1e-7);
+  std::printf("fused Flow-DPPO replay step: %lld rows, %d below the KL threshold, %d kept\n", (long long)R, low, kept);
+}
+
+// Sampling noise drawn inside the step (the reference draws it inside FlowSDEStrategy.step,
+// unirl/sde/kernels.py:219-233): the drawn noise, stored on request, fed back as a given noise tensor must
+// reproduce the step bit for bit; the same (seed, offset) must give the same draw and another offset another;
+// and the draw must look standard normal.
+void check_sde_rng(hipStream_t st, void* ws, size_t ws_bytes) {
+  const int64_t B = 4, D = 4096;
+  Rng rng(17);
+  std::vector<float> x(B * D), v(B * D);
+  for (auto& e : x) e = (float)rng.normal();
+  for (auto& e : v) e = (float)rng.normal();
+  const std::vector<float> sg = {0.84375006f}, sn = {0.82258058f};
+  DevBuf<float> dx(x), dv(v), dsg(sg), dsn(sn), prev_a(B * D), prev_b(B * D), nz_a(B * D), nz_b(B * D), nz_c(B * D), lp_a(B),
+      lp_b(B);
+  unirl_sde_step_desc d;
+  std::memset(&d, 0, sizeof(d));
+  d.noise_pred = {dv.p, UNIRL_F32, 0};
+  d.sample = {dx.p, UNIRL_F32, 0};
+  d.prev_sample = {nullptr, UNIRL_F32, 0};
+  d.sigma = dsg.p;
+  d.sigma_next = dsn.p;
+  d.sigma_max_val = 0.98780483f;
+  d.eta = 0.7;
+  d.kind = UNIRL_SDE_FLOW;
+  d.B = B;
+  d.D = D;
+  d.prev_dtype = UNIRL_F32;
+  d.prev_out = prev_a.p;
+  d.logp_out = lp_a.p;
+  d.rng.enabled = 1;
+  d.rng.seed = 20241125ull;
+  d.rng.offset = 40ull;
+  d.noise_out = nz_a.p;
+  expect_status("unirl_sde_step_logp_ex (noise drawn in the kernel)", unirl_sde_step_logp_ex(&d, ws, ws_bytes, st));
+  d.prev_out = nullptr;
+  d.logp_out = nullptr;
+  d.noise_out = nz_b.p;
+  expect_status("unirl_sde_step_logp_ex (same seed and offset)", unirl_sde_step_logp_ex(&d, ws, ws_bytes, st));
+  d.rng.offset = 41ull;
+  d.noise_out = nz_c.p;
+  expect_status("unirl_sde_step_logp_ex (next offset)", unirl_sde_step_logp_ex(&d, ws, ws_bytes, st));
+  // the same step with the drawn noise handed over as a tensor
+  d.rng.enabled = 0;
+  d.noise = nz_a.p;
+  d.noise_out = nullptr;
+  d.prev_out = prev_b.p;
+  d.logp_out = lp_b.p;
+  expect_status("unirl_sde_step_logp_ex (given noise)", unirl_sde_step_logp_ex(&d, ws, ws_bytes, st));
+  HIP_OK(hipStreamSynchronize(st));
+  const auto na = nz_a.host(), nb = nz_b.host(), nc = nz_c.host(), pa = prev_a.host(), pb = prev_b.host();
+  const auto la = lp_a.host(), lb = lp_b.host();
+  if (std::memcmp(na.data(), nb.data(), na.size() * 4) != 0) {
+    std::printf("FAIL drawn noise is not a function of (seed, offset)\n");
+    ++g_failures;
+  }
+  if (std::memcmp(na.data(), nc.data(), na.size() * 4) == 0) {
+    std::printf("FAIL another offset gave the same noise\n");
+    ++g_failures;
+  }
+  if (std::memcmp(pa.data(), pb.data(), pa.size() * 4) != 0) {
+    std::printf("FAIL the step from drawn noise differs from the step from the same noise given\n");
+    ++g_failures;
+  }
+  for (int64_t b = 0; b < B; ++b) expect_close("log-prob from drawn noise vs given noise", la[b], lb[b], 1e-6, 1e-7);
+  double m1 = 0.0, m2 = 0.0, cross = 0.0;
+  const double n = (double)na.size();
+  for (size_t i = 0; i < na.size(); ++i) {
+    m1 += na[i];
+    m2 += (double)na[i] * na[i];
+    cross += (double)na[i] * nc[i];
+  }
+  const double se = 1.0 / std::sqrt(n);
+  expect_close("drawn noise: mean", m1 / n, 0.0, 0.0, 5.0 * se);
+  expect_close("drawn noise: variance", m2 / n, 1.0, 0.0, 5.0 * std::sqrt(2.0) * se);
+  expect_close("drawn noise: correlation between two offsets", cross / n, 0.0, 0.0, 5.0 * se);
+  std::printf("in-kernel noise: %lld draws reproducible, standard normal, step equal to the step from the same noise\n",
+              (long long)na.size());
+}
+
 // lm_head + log-softmax with the logits never written (unirl/models/qwen3/ar.py:82-99), and the
 // transposed copy of the weight used by its backward: against a float64 product of the same bf16
 // operands rounded to bf16 (a logit one bf16 ulp off moves a log-prob by that ulp at most).
@@ -458,6 +633,8 @@ int main() {
   check_grpo(st, ws, ws_bytes);
   check_advantages(st);
   check_sde_replay(st, ws, ws_bytes);
+  check_flowdppo_replay(st, ws, ws_bytes);
+  check_sde_rng(st, ws, ws_bytes);
   check_lmhead(st);
   HIP_OK(hipStreamSynchronize(st));
   HIP_OK(hipFree(ws));
